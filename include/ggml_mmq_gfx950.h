@@ -1,0 +1,134 @@
+/* C ABI of libggml_mmq_gfx950.so: packed GGUF-weight matmul kernels for LoRA training on gfx950.
+ *
+ * The library replaces, behind plain pointers and sizes, the native operators the reference reaches
+ * through torch.ops.torch_ggml_ops (un-vendored wheel), AITER gmm/ptgmm, its Triton routing kernels and
+ * Liger's cross-entropy kernel.  Each declaration names the reference call site it stands in for
+ * (file:line in the reference repository).
+ *
+ * Conventions
+ *   - every pointer is a device pointer unless it is a `stream` (a hipStream_t passed as void*);
+ *   - matrices are row-major and contiguous; activations and LoRA factors are bf16 (uint16 storage);
+ *   - packed weights are the raw GGUF blocks of a [N, K] tensor, row after row, read-only, never
+ *     copied or repacked; supported GGML type ids: 8 (Q8_0), 12 (Q4_K), 14 (Q6_K), 16 (IQ2_XXS);
+ *     K must be a multiple of 64 and of the type's block size;
+ *   - nothing is allocated inside: the caller passes outputs and, where stated, a workspace whose size
+ *     comes from the matching *_workspace_bytes function (256-byte aligned carving inside);
+ *   - work is enqueued on `stream` and the call returns without synchronising;
+ *   - return value 0 = success; negative = error (-1 type id, -2 shape, -3 alignment, -4 null pointer,
+ *     -5 HIP runtime, -6 workspace too small) with text available from ggq_last_error() (thread-local).
+ *     Errors are detected before any launch; nothing is repaired silently (no hidden operand copies).
+ *   - expert groups: `expert_ids[g]` (int64) is the expert of group g and `end_offsets[g]` (int32) the
+ *     cumulative END row of group g in the expert-sorted row order (test_fast_moe_lora.py:136-137:
+ *     experts [0,2,5], offsets [2,5,6]).  groups == 0 means one dense group that uses expert 0.
+ */
+#ifndef GGML_MMQ_GFX950_H
+#define GGML_MMQ_GFX950_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* ggq_last_error(void);
+
+/* fast_lora.py:24-31 (_NATIVE_MMQ_QUANT_TYPES / supports_native_mmq): 1 if this library has kernels
+ * for the GGML type id. */
+int ggq_supports_quant_type(int qt);
+
+/* Bytes of one packed row of K elements (gguf GGML_QUANT_SIZES, test_deepseek_v4_moe_lora.py:58);
+ * -1 if K is not a whole number of blocks or the type is unknown. */
+int64_t ggq_row_bytes(int qt, int64_t k);
+
+/* dequantize_gguf_tensor (transformers gguf fork; used at fast_moe_lora.py:163-165, 235-240 and as the
+ * oracle of test_fast_lora.py:110-115): packed [rows, K] -> bf16 (out_is_f32 = 0) or fp32 values,
+ * bit-exact with ggml's dequantize_row_* followed by round-to-nearest-even to bf16. */
+int ggq_dequantize(int qt, const void* packed, int64_t rows, int64_t k, void* out, int out_is_f32, void* stream);
+
+/* torch.ops.torch_ggml_ops.mmq (fast_lora.py:155-160, gguf_liger_loss.py:109-114): y[M,N] = x[M,K] . W^T. */
+int ggq_mmq(const void* x, const void* packed, int qt, int64_t m, int64_t n, int64_t k, void* y, void* stream);
+
+/* torch.ops.torch_ggml_ops.mmq_grad_input (gguf_liger_loss.py:172-177; autograd of mmq,
+ * test_fast_lora.py:104-105): dx[M,K] = dy[M,N] . W with W decoded to bf16, fp32 accumulation. */
+int ggq_mmq_grad_input(const void* dy, const void* packed, int qt, int64_t m, int64_t n, int64_t k, void* dx, void* stream);
+
+/* Workspace bound for the four LoRA entry points below (n_total = N, or 2N for a pair). */
+int64_t ggq_lora_workspace_bytes(int64_t rows, int64_t groups, int64_t experts, int64_t n_total, int64_t k, int r);
+
+/* FastGGUFLoraLinear._base_layer_forward + _fused_lora_add (fast_lora.py:34-65, 134-163) in one call:
+ *   xa_out[M, r16] = bf16(x . A^T)  (r16 = r rounded up to 16, zero padded),
+ *   y[M,N] = x . W^T + scale * xa . B^T.      A [r,K], B [N,r].  A = B = NULL gives plain mmq. */
+int ggq_lora_mmq_forward(const void* x, const void* packed, int qt, int64_t m, int64_t n, int64_t k, const void* lora_a,
+                         const void* lora_b, int r, float scale, void* xa_out, void* y, void* ws, int64_t ws_bytes,
+                         void* stream);
+
+/* Autograd of the above (test_fast_lora.py:101-134): dx = dy . W + scale * (dy . B) . A,
+ * dB[N,r] = scale * dy^T . xa, dA[r,K] = scale * (dy . B)^T . x; dA / dB may be NULL. */
+int ggq_lora_mmq_backward(const void* dy, const void* packed, int qt, int64_t m, int64_t n, int64_t k, const void* x,
+                          const void* xa, const void* lora_a, const void* lora_b, int r, float scale, void* dx,
+                          void* d_lora_a, void* d_lora_b, void* ws, int64_t ws_bytes, void* stream);
+
+/* torch.ops.torch_ggml_ops.grouped_mmq / grouped_mmq_pair (fast_moe_lora.py:221-228, 339-347) fused with
+ * the per-expert LoRA delta that the reference computes with AITER gmm (_lora_grouped_linear,
+ * fast_moe_lora.py:675-682, added at :743-745 / :763).  packed1/packed2 [E,N,bytes]; packed2 != NULL
+ * selects the pair form (two outputs y1, y2 from one x; LoRA B is [E,2N,r], first N rows for y1).
+ * A [E,r,K].  A = B = NULL gives the plain grouped ops. */
+int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void* packed2, const int64_t* expert_ids,
+                                 const int32_t* end_offsets, int64_t groups, int64_t experts, int qt, int64_t rows, int64_t n,
+                                 int64_t k, const void* lora_a, const void* lora_b, int r, float scale, void* xa_out, void* y1,
+                                 void* y2, void* ws, int64_t ws_bytes, void* stream);
+
+/* torch.ops.torch_ggml_ops.grouped_mmq_grad_input / grouped_mmq_pair_grad_input
+ * (fast_moe_lora.py:255-262, 364-375: both cotangents of a pair land in one fp32 accumulator and are
+ * rounded once) plus the LoRA input gradient (gmm with transposed rhs, fast_moe_lora.py:56-73) and the
+ * factor gradients (ptgmm, fast_moe_lora.py:76-87; all E planes written, inactive experts exactly zero,
+ * test_fast_moe_lora.py:331-333).  dA [E,r,K], dB [E,N or 2N,r]; may be NULL. */
+int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* packed1, const void* packed2,
+                                  const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts, int qt,
+                                  int64_t rows, int64_t n, int64_t k, const void* x, const void* xa, const void* lora_a,
+                                  const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b, void* ws,
+                                  int64_t ws_bytes, void* stream);
+
+/* prepare_expert_routing (fast_moe_routing.py:379-428: torch.sort of the flat top-k ids + inverse
+ * permutation kernel :88-98) and the grouped-execution offsets of the expert module
+ * (fast_moe_lora.py:709-719, 652-672).  Stable order: ties keep ascending route index.
+ *   sorted_ids, permutation, inverse: int64 [tokens*top_k];  counts, end_offsets: int32 [num_experts];
+ *   active_ids int64 / active_end_offsets int32 [num_experts]: compact list of experts with rows (tail
+ *   entries repeat the total);  status int32[2] = {number of active experts, 1 if an id was outside
+ *   [0,num_experts) (such ids are clamped)}. */
+int64_t ggq_route_plan_workspace_bytes(int64_t tokens, int top_k, int num_experts);
+int ggq_route_plan(const void* topk_ids, int ids_are_int64, int64_t tokens, int top_k, int num_experts, int64_t* sorted_ids,
+                   int64_t* permutation, int64_t* inverse, int32_t* counts, int32_t* end_offsets, int64_t* active_ids,
+                   int32_t* active_end_offsets, int32_t* status, void* ws, int64_t ws_bytes, void* stream);
+
+/* _route_gather_forward_kernel (fast_moe_routing.py:101-123): selected[s] = hidden[permutation[s] / k]. */
+int ggq_route_gather_forward(const void* hidden, const int64_t* permutation, void* selected, int64_t tokens, int top_k, int hidden_dim, void* stream);
+
+/* _route_gather_backward_kernel (fast_moe_routing.py:126-159): per token, routes added in ascending
+ * sorted position with a bf16 rounding after every add. */
+int ggq_route_gather_backward(const void* grad_selected, const int64_t* inverse, void* grad_hidden, int64_t tokens, int top_k, int hidden_dim, void* stream);
+
+/* _route_combine_forward_kernel (fast_moe_routing.py:162-194); weights [tokens, top_k] fp32 or bf16. */
+int ggq_route_combine_forward(const void* expert_out, const void* weights, int weights_are_bf16, const int64_t* inverse, void* out, int64_t tokens, int top_k, int hidden_dim, void* stream);
+
+/* _route_combine_backward_kernel (fast_moe_routing.py:197-226); either gradient may be NULL. */
+int ggq_route_combine_backward(const void* expert_out, const void* weights, int weights_are_bf16, const int64_t* permutation, const void* grad_out, void* grad_expert_out, void* grad_weights, int64_t tokens, int top_k, int hidden_dim, void* stream);
+
+/* GGUFExperts._apply_split_gate (fork; called at fast_moe_lora.py:747): h = silu(gate) * up, and its
+ * autograd.  elems = rows * intermediate. */
+int ggq_swiglu_forward(const void* gate, const void* up, void* h, int64_t elems, void* stream);
+int ggq_swiglu_backward(const void* gate, const void* up, const void* dh, void* dgate, void* dup, int64_t elems, void* stream);
+
+/* _packed_q8_linear_cross_entropy_forward (gguf_liger_loss.py:38-186): chunked mmq -> Liger
+ * cross-entropy -> mmq_grad_input, without the [chunk, vocab] logits tensor.  labels int64 [rows];
+ * loss_per_row fp32 [rows] (already divided by the number of non-ignored rows when reduction_mean);
+ * grad_hidden bf16 [rows, hidden]; lse_out fp32 [rows] or NULL; n_valid_out int32[1] or NULL. */
+int64_t ggq_lmhead_ce_workspace_bytes(int64_t rows, int64_t vocab, int64_t hidden_dim, int64_t chunk);
+int ggq_lmhead_cross_entropy(int qt, const void* hidden, const void* packed, const int64_t* labels, int64_t rows, int64_t vocab,
+                             int64_t hidden_dim, int64_t chunk, int64_t ignore_index, int reduction_mean, float* loss_per_row,
+                             void* grad_hidden, float* lse_out, int32_t* n_valid_out, void* ws, int64_t ws_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,223 @@
+"""Grouped expert projections and the full expert layer against the per-expert oracle loop
+(relations of test_fast_moe_lora.py:133-279, 282-348, 406-511 and test_deepseek_v4_moe_lora.py:67-118)."""
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import ALL_TYPES, TYPE_NAMES, assert_close_bf16, bf16_randn, make_payload
+from oracle import gguf_blocks as gb
+from oracle import lora_matmul as ref
+from oracle import routing as rref
+
+pytestmark = pytest.mark.gpu
+
+
+def _expert_payload(seed, qt, experts, n, k, kind="quantized"):
+    return np.stack([make_payload(seed + e, qt, n, k, kind) for e in range(experts)])
+
+
+def _to(dev, *ts):
+    return [t.to(dev) for t in ts]
+
+
+@pytest.mark.parametrize("qt", ALL_TYPES, ids=[TYPE_NAMES[q] for q in ALL_TYPES])
+def test_grouped_pair_and_single_projection_jacobian(pkg, dev, qt):
+    # experts [0, 2, 5], cumulative end offsets [2, 5, 6] (test_fast_moe_lora.py:136-137)
+    ml = pkg.fast_moe_lora
+    experts = torch.tensor([0, 2, 5], dtype=torch.int64)
+    offsets = torch.tensor([2, 5, 6], dtype=torch.int32)
+    gen = torch.Generator().manual_seed(2468)
+    k, n = 2048, 64
+    pg, pu = _expert_payload(10, qt, 8, n, k), _expert_payload(50, qt, 8, n, k)
+    wg, wu = ref.weights_bf16(pg, qt), ref.weights_bf16(pu, qt)
+    hidden = bf16_randn(gen, 6, k)
+    g1, g2 = bf16_randn(gen, 6, n), bf16_randn(gen, 6, n)
+    want_g = ref.grouped_lora_linear(hidden, wg, experts, offsets, dy=g1)
+    want_u = ref.grouped_lora_linear(hidden, wu, experts, offsets, dy=g2)
+    h = hidden.to(dev).requires_grad_(True)
+    e_d, o_d = _to(dev, experts, offsets)
+    pg_d, pu_d = torch.from_numpy(pg).to(dev), torch.from_numpy(pu).to(dev)
+    gate, up = ml.grouped_mmq_pair(h, pg_d, pu_d, e_d, o_d, qt, n)
+    torch.autograd.backward((gate, up), _to(dev, g1, g2))
+    assert_close_bf16(gate, want_g["y"], "gate")
+    assert_close_bf16(up, want_u["y"], "up")
+    # both cotangents in one accumulator, rounded once (test_fast_moe_lora.py:199-203: atol 1e-4 there)
+    assert_close_bf16(h.grad, want_g["dx"] + want_u["dx"], "pair dX")
+    # pair == two single projections, bit for bit (test_fast_moe_lora.py:207-236)
+    assert torch.equal(gate, ml.grouped_mmq(h.detach(), pg_d, e_d, o_d, qt, n))
+    assert torch.equal(up, ml.grouped_mmq(h.detach(), pu_d, e_d, o_d, qt, n))
+    # single projection backward (down-proj shape of the reference test: K = 512)
+    pd = _expert_payload(90, qt, 8, 64, 512)
+    wd = ref.weights_bf16(pd, qt)
+    inter = bf16_randn(gen, 6, 512)
+    gd = bf16_randn(gen, 6, 64)
+    want_d = ref.grouped_lora_linear(inter, wd, experts, offsets, dy=gd)
+    it = inter.to(dev).requires_grad_(True)
+    out = ml.grouped_mmq(it, torch.from_numpy(pd).to(dev), e_d, o_d, qt, 64)
+    out.backward(gd.to(dev))
+    assert_close_bf16(out, want_d["y"], "down")
+    assert_close_bf16(it.grad, want_d["dx"], "down dX")
+    dx_op = ml.grouped_mmq_grad_input(gd.to(dev), torch.from_numpy(pd).to(dev), e_d, o_d, qt, 512)
+    assert torch.equal(dx_op, it.grad)
+
+
+def test_constant_byte_iq2_xxs_experts(pkg, dev):
+    # test_deepseek_v4_moe_lora.py:55-118: payload of all bytes 32, experts [0,1], offsets [3,7]
+    ml = pkg.fast_moe_lora
+    payload = np.full((2, 256, 66), 32, dtype=np.uint8)
+    w = ref.weights_bf16(payload, gb.IQ2_XXS)
+    experts = torch.tensor([0, 1], dtype=torch.int64)
+    offsets = torch.tensor([3, 7], dtype=torch.int32)
+    gen = torch.Generator().manual_seed(5)
+    hidden, gout = bf16_randn(gen, 7, 256), bf16_randn(gen, 7, 256)
+    want = ref.grouped_lora_linear(hidden, w, experts, offsets, dy=gout)
+    h = hidden.to(dev).requires_grad_(True)
+    out = ml.grouped_mmq(h, torch.from_numpy(payload).to(dev), experts.to(dev), offsets.to(dev), gb.IQ2_XXS, 256)
+    out.backward(gout.to(dev))
+    torch.testing.assert_close(out.double().cpu(), want["y"], rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(h.grad.double().cpu(), want["dx"], rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("qt,r", [(gb.Q4_K, 16), (gb.Q8_0, 4), (gb.Q6_K, 8), (gb.IQ2_XXS, 16)])
+def test_grouped_lora_projection_all_gradients(pkg, dev, qt, r):
+    # ragged groups including empty experts, a group larger than one 128-row tile, and inactive planes
+    ml = pkg.fast_moe_lora
+    e_total, n, k = 8, 192, 512
+    sizes = [0, 150, 3, 0, 129, 1, 64, 0]
+    rows = sum(sizes)
+    all_ids = torch.arange(e_total, dtype=torch.int64)
+    ends = torch.tensor(np.cumsum(sizes), dtype=torch.int32)
+    gen = torch.Generator().manual_seed(8642 + r)
+    p1, p2 = _expert_payload(300, qt, e_total, n, k), _expert_payload(400, qt, e_total, n, k)
+    w1, w2 = ref.weights_bf16(p1, qt), ref.weights_bf16(p2, qt)
+    x = bf16_randn(gen, rows, k)
+    a = bf16_randn(gen, e_total, r, k, std=k ** -0.5)
+    b = bf16_randn(gen, e_total, 2 * n, r, std=0.02)
+    dy = bf16_randn(gen, rows, 2 * n)
+    s = 2.0
+    want = ref.grouped_lora_linear(x, torch.cat([w1, w2], dim=1), all_ids, ends, a, b, s, dy)
+    xd, ad, bd = (t.to(dev).requires_grad_(True) for t in (x, a, b))
+    y1, y2 = ml.grouped_lora_mmq_pair(xd, torch.from_numpy(p1).to(dev), torch.from_numpy(p2).to(dev), all_ids.to(dev), ends.to(dev), qt, n, ad, bd, s)
+    torch.autograd.backward((y1, y2), (dy[:, :n].contiguous().to(dev), dy[:, n:].contiguous().to(dev)))
+    assert_close_bf16(torch.cat([y1, y2], dim=1), want["y"], "pair Y")
+    assert_close_bf16(xd.grad, want["dx"], "pair dX")
+    assert_close_bf16(ad.grad, want["da"], "dA")
+    assert_close_bf16(bd.grad, want["db"], "dB")
+    inactive = torch.tensor([sz == 0 for sz in sizes])
+    assert torch.count_nonzero(ad.grad[inactive.to(dev)]) == 0 and torch.count_nonzero(bd.grad[inactive.to(dev)]) == 0
+    # compact active-expert form gives the same bits as the full list with empty groups
+    active = torch.tensor([e for e, sz in enumerate(sizes) if sz], dtype=torch.int64)
+    active_ends = torch.tensor(np.cumsum([sz for sz in sizes if sz]), dtype=torch.int32)
+    z1, z2 = ml.grouped_lora_mmq_pair(xd.detach(), torch.from_numpy(p1).to(dev), torch.from_numpy(p2).to(dev), active.to(dev), active_ends.to(dev), qt, n, ad.detach(), bd.detach(), s)
+    assert torch.equal(z1, y1) and torch.equal(z2, y2)
+    # single (down-like) projection with LoRA
+    want1 = ref.grouped_lora_linear(x, w1, all_ids, ends, a, b[:, :n].contiguous(), s, dy[:, :n].contiguous())
+    xd2, ad2, bd2 = (t.to(dev).requires_grad_(True) for t in (x, a, b[:, :n].contiguous()))
+    y = ml.grouped_lora_mmq(xd2, torch.from_numpy(p1).to(dev), all_ids.to(dev), ends.to(dev), qt, n, ad2, bd2, s)
+    y.backward(dy[:, :n].contiguous().to(dev))
+    assert_close_bf16(y, want1["y"], "single Y")
+    assert_close_bf16(xd2.grad, want1["dx"], "single dX")
+    assert_close_bf16(ad2.grad, want1["da"], "single dA")
+    assert_close_bf16(bd2.grad, want1["db"], "single dB")
+
+
+def _layer_case(seed, tokens, hidden, inter, experts, k, r, qt):
+    gen = torch.Generator().manual_seed(seed)
+    pg, pu = _expert_payload(seed, qt, experts, inter, hidden), _expert_payload(seed + 1000, qt, experts, inter, hidden)
+    pd = _expert_payload(seed + 2000, qt, experts, hidden, inter)
+    x = bf16_randn(gen, tokens, hidden)
+    logits = torch.randn(tokens, experts, generator=gen)
+    idx, w = rref.router_topk(logits, k)
+    a_gu = bf16_randn(gen, experts, r, hidden, std=hidden ** -0.5)
+    b_gu = bf16_randn(gen, experts, 2 * inter, r, std=0.01)
+    a_d = bf16_randn(gen, experts, r, inter, std=inter ** -0.5)
+    b_d = bf16_randn(gen, experts, hidden, r, std=0.01)
+    dy = bf16_randn(gen, tokens, hidden)
+    return pg, pu, pd, x, idx, w, a_gu, b_gu, a_d, b_d, dy
+
+
+def _oracle_layer(pg, pu, pd, x, idx, w, a_gu, b_gu, a_d, b_d, dy, qt, s, experts):
+    tokens, k = idx.shape
+    sorted_ids, perm, inv = rref.plan(idx)
+    counts = rref.expert_counts(idx, experts)
+    ends = torch.cumsum(counts.long(), 0).int()
+    sel = rref.gather_forward(x, perm, k)
+    # backward through combine first: dO rows for the sorted layout
+    d_o = (dy.float()[perm // k] * rref.bf16(w).reshape(-1)[perm][:, None]).to(torch.bfloat16)
+    res = ref.expert_layer(sel, torch.arange(experts), ends, ref.weights_bf16(pg, qt), ref.weights_bf16(pu, qt),
+                           ref.weights_bf16(pd, qt), a_gu, b_gu, a_d, b_d, s, d_o)
+    out = rref.combine_forward(ref.bf16_round(res["out"]).to(torch.bfloat16), w, inv)
+    dx_tok = rref.gather_backward(ref.bf16_round(res["dx"]).to(torch.bfloat16), inv, tokens, k)
+    _, dw = rref.combine_backward(dy, ref.bf16_round(res["out"]).to(torch.bfloat16), w, perm)
+    return out, dx_tok, dw, res
+
+
+@pytest.mark.parametrize("qt,tokens,hidden,inter,experts,k,r", [
+    (gb.Q4_K, 8, 2048, 512, 8, 4, 4),        # the reference's one-layer test geometry (test_fast_moe_lora.py:409-470)
+    (gb.Q4_K, 300, 512, 256, 16, 8, 16),     # ragged groups, some experts idle, r = 16
+    (gb.IQ2_XXS, 64, 512, 512, 8, 2, 16),
+    (gb.Q8_0, 40, 256, 128, 4, 2, 8),
+])
+def test_expert_layer_forward_backward(pkg, dev, qt, tokens, hidden, inter, experts, k, r):
+    ml, G = pkg.fast_moe_lora, pkg.gguf.GGUFQuantizedTensor
+    s = 32.0 / r
+    pg, pu, pd, x, idx, w, a_gu, b_gu, a_d, b_d, dy = _layer_case(97531, tokens, hidden, inter, experts, k, r, qt)
+    want_out, want_dx, want_dw, res = _oracle_layer(pg, pu, pd, x, idx, w, a_gu, b_gu, a_d, b_d, dy, qt, s, experts)
+    mod = ml.GGUFExperts(G(torch.from_numpy(pg).to(dev), qt, (experts, inter, hidden)), G(torch.from_numpy(pu).to(dev), qt, (experts, inter, hidden)),
+                         G(torch.from_numpy(pd).to(dev), qt, (experts, hidden, inter)))
+    layer = ml.FastGGUFMoeLora(mod, r=r, lora_alpha=32)
+    with torch.no_grad():
+        layer.lora_A["default"].copy_(a_gu.to(dev)); layer.lora_B["default"].copy_(b_gu.to(dev))
+        layer.lora_A_down["default"].copy_(a_d.to(dev)); layer.lora_B_down["default"].copy_(b_d.to(dev))
+    xd = x.to(dev).requires_grad_(True)
+    wd = w.to(dev).requires_grad_(True)
+    out = layer(xd, idx.to(dev), wd)
+    out.backward(dy.to(dev))
+    assert out.shape == x.shape
+    assert_close_bf16(out, want_out.double(), "layer output", ulps=4)
+    assert_close_bf16(xd.grad, want_dx.double(), "dHidden", ulps=6)
+    assert_close_bf16(wd.grad, want_dw, "dRoutingWeights", ulps=6)
+    for name, param, key in (("dA_gate_up", layer.lora_A, "da_gu"), ("dB_gate_up", layer.lora_B, "db_gu"),
+                             ("dA_down", layer.lora_A_down, "da_d"), ("dB_down", layer.lora_B_down, "db_d")):
+        assert_close_bf16(param["default"].grad, res[key], name, ulps=6)
+    active = torch.unique(idx)
+    inactive = torch.ones(experts, dtype=torch.bool)
+    inactive[active] = False
+    for p in layer.parameters():
+        assert torch.count_nonzero(p.grad[inactive.to(dev)]) == 0
+    for t in (mod.gate_proj, mod.up_proj, mod.down_proj):
+        assert t.grad is None
+    # a recomputed forward/backward (activation checkpointing) reproduces the same bits
+    grads1 = [p.grad.clone() for p in layer.parameters()] + [xd.grad.clone()]
+    for p in layer.parameters():
+        p.grad = None
+    xd.grad = None
+    out2 = layer(xd, idx.to(dev), wd)
+    out2.backward(dy.to(dev))
+    assert torch.equal(out2, out)
+    for g1, g2 in zip(grads1, [p.grad for p in layer.parameters()] + [xd.grad]):
+        assert torch.equal(g1, g2)
+
+
+def test_moe_guards(pkg, dev):
+    ml = pkg.fast_moe_lora
+    x = torch.zeros(6, 256, dtype=torch.bfloat16, device=dev)
+    p = torch.zeros(4, 32, 144, dtype=torch.uint8, device=dev)
+    ids = torch.tensor([0, 1], dtype=torch.int64, device=dev)
+    offs = torch.tensor([3, 6], dtype=torch.int32, device=dev)
+    with pytest.raises(TypeError):
+        ml.grouped_mmq(x, p, ids.int(), offs, gb.Q4_K, 32)
+    with pytest.raises(TypeError):
+        ml.grouped_mmq(x, p, ids, offs.long(), gb.Q4_K, 32)
+    with pytest.raises(ValueError):
+        ml.grouped_mmq(x, p, ids, offs, 11, 32)
+    with pytest.raises(ValueError):
+        ml.grouped_mmq(x, p, ids, offs, gb.Q4_K, 33)
+    with pytest.raises(RuntimeError):
+        ml.grouped_mmq_pair(x, p, p[:, :16].contiguous(), ids, offs, gb.Q4_K, 32)
+    sizes = ml._group_sizes_from_offsets(offs)
+    assert sizes.tolist() == [3, 3]
+    assert ml._complete_group_sizes(sizes, ids, 4).tolist() == [3, 3, 0, 0]
+    with pytest.raises(ValueError):
+        ml._group_sizes_from_offsets(offs.long())

@@ -1,0 +1,136 @@
+"""Pins for the block-decoder oracle: hand-computed known-answer blocks (derived on paper from the
+published ggml block layouts, not by re-running the decoder's formula), the independent scalar C
+restatement, format invariants and structural checks of the IQ2_XXS codebook."""
+
+import numpy as np
+import pytest
+
+from oracle import c_oracle
+from oracle import gguf_blocks as gb
+from oracle.iq2xxs_grid import IQ2XXS_GRID
+
+F16 = {1.0: (0x00, 0x3C), 0.5: (0x00, 0x38), 0.25: (0x00, 0x34)}
+
+
+def both(payload, qt):
+    a = gb.dequantize(payload, qt)
+    b = c_oracle.dequantize(payload, qt)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), "numpy and C restatements disagree"
+    return a
+
+
+def test_q8_0_known_answer():
+    blk = np.zeros(34, dtype=np.uint8)
+    blk[0:2] = F16[0.5]
+    q = np.zeros(32, dtype=np.int8)
+    q[:5] = [-128, -1, 0, 1, 127]
+    q[31] = 64
+    blk[2:] = q.view(np.uint8)
+    y = both(blk[None, :], gb.Q8_0)[0]
+    assert y[:5].tolist() == [-64.0, -0.5, 0.0, 0.5, 63.5]
+    assert y[31] == 32.0 and np.all(y[5:31] == 0)
+
+
+def test_q4_k_known_answer():
+    # d = 1, dmin = 0.5; sub-block scales sc = 1,2,3,4,33,34,35,36 and mins m = 5,6,7,8,37,38,39,40
+    # packed by hand into the 12 scale bytes (6-bit fields, upper two bits of sc[4..7] / m[4..7] in the
+    # tops of bytes 0..7); qs[i] = (i % 16) | ((15 - i % 16) << 4).
+    blk = np.zeros(144, dtype=np.uint8)
+    blk[0:2] = F16[1.0]
+    blk[2:4] = F16[0.5]
+    blk[4:16] = [129, 130, 131, 132, 133, 134, 135, 136, 81, 98, 115, 132]
+    i = np.arange(128)
+    blk[16:] = (i % 16) | ((15 - i % 16) << 4)
+    y = both(blk[None, :], gb.Q4_K)[0]
+    want = {0: -2.5, 5: 2.5, 32: 27.0, 47: -3.0, 64: -3.5, 79: 41.5, 128: -18.5, 131: 80.5, 224: 520.0, 255: -20.0}
+    for e, v in want.items():
+        assert y[e] == v, (e, y[e], v)
+
+
+def test_q6_k_known_answer():
+    # d = 0.25; int8 sub-scales 1,-2,3,-4,...,15,-16; ql = 0x21 for l < 32 and 0x43 for l >= 32 of each
+    # 64-byte half; qh = 0xE4 (bit pairs 0,1,2,3 from the bottom).
+    blk = np.zeros(210, dtype=np.uint8)
+    ql = np.empty(128, dtype=np.uint8)
+    ql[0:32] = 0x21
+    ql[32:64] = 0x43
+    ql[64:96] = 0x21
+    ql[96:128] = 0x43
+    blk[0:128] = ql
+    blk[128:192] = 0xE4
+    sc = np.array([(j + 1) * (1 if j % 2 == 0 else -1) for j in range(16)], dtype=np.int8)
+    blk[192:208] = sc.view(np.uint8)
+    blk[208:210] = F16[0.25]
+    y = both(blk[None, :], gb.Q6_K)[0]
+    want = {0: -7.75, 16: 15.5, 32: -9.75, 64: 2.5, 96: 35.0, 127: -40.0, 128: -69.75, 255: -80.0}
+    for e, v in want.items():
+        assert y[e] == v, (e, y[e], v)
+
+
+def test_iq2_xxs_constant_byte_payload_known_answer():
+    # every byte 32: the synthetic expert payload of test_deepseek_v4_moe_lora.py:55-64.
+    # d = half(0x2020) = 2^-7 * (1 + 32/1024); scale nibble 2 -> db = d * 2.5 / 4; all four codebook
+    # indices are 32 -> bytes 25,8,8,8,8,25,8,8; sign indices 32, 64, 0, 1 (+ parity bit 7).
+    payload = np.full((1, 66), 32, dtype=np.uint8)
+    y = both(payload, gb.IQ2_XXS)[0]
+    a, b = 0.125885009765625, 0.040283203125  # db * 25, db * 8
+    run0 = [a, b, b, b, b, -a, b, -b]
+    run1 = [a, b, b, b, b, a, -b, -b]
+    run2 = [a, b, b, b, b, a, b, b]
+    run3 = [-a, b, b, b, b, a, b, -b]
+    assert y[:32].tolist() == run0 + run1 + run2 + run3
+    assert np.array_equal(y[:32], y[224:256])  # all eight groups are identical
+
+
+def test_iq2xxs_grid_structure():
+    g = np.array(IQ2XXS_GRID, dtype=np.uint64)
+    assert g.shape == (256,) and np.all(g[1:] > g[:-1]) and int(g[0]) == 0x0808080808080808
+    b = g.view(np.uint8).reshape(256, 8)
+    assert set(np.unique(b).tolist()) == {0x08, 0x19, 0x2B}
+    assert np.all((b == 0x19).sum(axis=1) % 2 == 0)  # E8 lattice points (half-integer coset)
+    n19, n2b = (b == 0x19).sum(axis=1), (b == 0x2B).sum(axis=1)
+    assert int(((n19 == 2) & (n2b == 0)).sum()) == 28 and int(((n19 == 0) & (n2b == 1)).sum()) == 8
+
+
+@pytest.mark.parametrize("qt", [gb.Q8_0, gb.Q4_K, gb.Q6_K, gb.IQ2_XXS])
+def test_numpy_and_c_agree_on_arbitrary_bytes(qt):
+    payload = gb.random_payload(np.random.default_rng(qt), qt, 23, 1024)
+    y = both(payload, qt)
+    assert np.isfinite(y).all()
+    assert np.array_equal(gb.to_bf16_bits(y), c_oracle.to_bf16_bits(y))
+
+
+def test_format_invariants():
+    rng = np.random.default_rng(3)
+    # Q4_K with all-zero quants decodes to -dmin*m per sub-block, whatever d is
+    p = gb.random_payload(rng, gb.Q4_K, 1, 256)
+    p[0, 16:] = 0
+    y = gb.dequantize(p, gb.Q4_K)[0].reshape(8, 32)
+    _, m = gb.unpack_q4_k_scales(p[0, 4:16])
+    dmin = p[0, 2:4].copy().view(np.float16).astype(np.float32)[0]
+    assert np.array_equal(y, np.repeat((-(dmin * m.astype(np.float32)))[:, None], 32, axis=1))
+    # negating an IQ2_XXS block scale negates every weight; Q8_0 is linear in d
+    p = gb.random_payload(rng, gb.IQ2_XXS, 1, 256)
+    q = p.copy()
+    q[0, 1] ^= 0x80
+    assert np.array_equal(gb.dequantize(q, gb.IQ2_XXS), -gb.dequantize(p, gb.IQ2_XXS))
+    # each IQ2_XXS run of eight has an even number of minus signs relative to |w|
+    w = gb.dequantize(p, gb.IQ2_XXS)[0].reshape(32, 8)
+    assert np.all((w < 0).sum(axis=1) % 2 == 0)
+
+
+def test_bf16_rounding_is_nearest_even():
+    x = np.array([1.0, 1.00390625, 1.005859375, 1.01171875, -1.00390625, 3.0e38], dtype=np.float32)
+    # 1 + 2^-8 is a tie -> even (1.0); 1 + 1.5*2^-8 rounds up; 1 + 3*2^-8 is a tie -> even (1.015625)
+    want = np.array([0x3F80, 0x3F80, 0x3F81, 0x3F82, 0xBF80, 0x7F62], dtype=np.uint16)
+    assert np.array_equal(gb.to_bf16_bits(x), want)
+
+
+@pytest.mark.parametrize("qt,bound", [(gb.Q8_0, 0.01), (gb.Q4_K, 0.12), (gb.Q6_K, 0.03), (gb.IQ2_XXS, 0.6)])
+def test_quantizer_round_trip_error(qt, bound):
+    rng = np.random.default_rng(11)
+    w = (rng.standard_normal((16, 1024)) * 0.02).astype(np.float32)
+    p = gb.quantize(w, qt)
+    assert p.shape == (16, gb.row_bytes(qt, 1024))
+    err = np.sqrt(((gb.dequantize(p, qt) - w) ** 2).mean()) / 0.02
+    assert err < bound

@@ -1,0 +1,294 @@
+// extern "C" surface of libggml_mmq_gfx950.so.  Declarations and the reference interface each entry
+// point replaces are in include/ggml_mmq_gfx950.h.  Plain device pointers and sizes only.
+#include "../../include/ggml_mmq_gfx950.h"
+
+#include "launch.h"
+#include "mmq_host.h"
+
+using namespace ggq;
+
+namespace {
+
+inline hipStream_t as_stream(void* s) { return (hipStream_t)s; }
+inline int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
+inline int rank_pad(int r) { return (r + 15) / 16 * 16; }
+
+struct Bump {  // carve 256-byte aligned pieces out of the caller's workspace
+    char* base;
+    int64_t size, used;
+    void* take(int64_t bytes) {
+        const int64_t at = used;
+        used += align256(bytes);
+        return used <= size ? base + at : nullptr;
+    }
+};
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+int check_weights(const char* what, int qt, const void* w, int64_t k) {
+    if (!w) return set_error(GGQ_ERR_NULL, "%s: packed weight pointer is null", what);
+    if (packed_row_bytes(qt, k) < 0) return set_error(GGQ_ERR_QTYPE, "%s: unsupported GGML type id %d (supported: 8, 12, 14, 16)", what, qt);
+    if (!aligned16(w)) return set_error(GGQ_ERR_ALIGN, "%s: packed weights must be 16-byte aligned", what);
+    return GGQ_OK;
+}
+
+int check_lora(const char* what, const void* a, const void* b, int r) {
+    if ((a == nullptr) != (b == nullptr)) return set_error(GGQ_ERR_NULL, "%s: LoRA factors must both be given or both be null", what);
+    if (a && (r < 1 || r > 64)) return set_error(GGQ_ERR_SHAPE, "%s: LoRA rank %d outside 1..64", what, r);
+    if (a && (!aligned16(a) || !aligned16(b))) return set_error(GGQ_ERR_ALIGN, "%s: LoRA factors must be 16-byte aligned", what);
+    return GGQ_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* ggq_last_error(void) { return last_error(); }
+
+int ggq_supports_quant_type(int qt) { return packed_row_bytes(qt, 256) > 0 ? 1 : 0; }
+
+int64_t ggq_row_bytes(int qt, int64_t k) { return block_multiple(qt, k) ? packed_row_bytes(qt, k) : -1; }
+
+int ggq_dequantize(int qt, const void* packed, int64_t rows, int64_t k, void* out, int out_is_f32, void* stream) {
+    if (!packed || !out) return set_error(GGQ_ERR_NULL, "dequantize: null pointer");
+    return dequantize(qt, packed, rows, k, out, out_is_f32, as_stream(stream));
+}
+
+// ---------------------------------------------------------------------------------------------------
+int64_t ggq_lora_workspace_bytes(int64_t rows, int64_t groups, int64_t experts, int64_t n_total, int64_t k, int r) {
+    const int rp = rank_pad(r > 0 ? r : 1);
+    if (experts < 1) experts = 1;
+    const int64_t tiles = rows / 64 + groups + 2;
+    return 2 * align256(tiles * (int64_t)sizeof(TileDesc)) + align256(16) + align256(experts * 2 * 4) +
+           align256(experts * n_total * rp * 2) * 2 + align256(experts * k * rp * 2) + align256(rows * rp * 2) + 4096;
+}
+
+int ggq_lora_mmq_forward(const void* x, const void* packed, int qt, int64_t m, int64_t n, int64_t k, const void* lora_a,
+                         const void* lora_b, int r, float scale, void* xa_out, void* y, void* ws, int64_t ws_bytes,
+                         void* stream) {
+    return ggq_grouped_lora_mmq_forward(x, packed, nullptr, nullptr, nullptr, 0, 1, qt, m, n, k, lora_a, lora_b, r,
+                                        scale, xa_out, y, nullptr, ws, ws_bytes, stream);
+}
+
+int ggq_lora_mmq_backward(const void* dy, const void* packed, int qt, int64_t m, int64_t n, int64_t k, const void* x,
+                          const void* xa, const void* lora_a, const void* lora_b, int r, float scale, void* dx,
+                          void* d_lora_a, void* d_lora_b, void* ws, int64_t ws_bytes, void* stream) {
+    return ggq_grouped_lora_mmq_backward(dy, nullptr, packed, nullptr, nullptr, nullptr, 0, 1, qt, m, n, k, x, xa, lora_a,
+                                         lora_b, r, scale, dx, d_lora_a, d_lora_b, ws, ws_bytes, stream);
+}
+
+int ggq_mmq(const void* x, const void* packed, int qt, int64_t m, int64_t n, int64_t k, void* y, void* stream) {
+    return ggq_grouped_lora_mmq_forward(x, packed, nullptr, nullptr, nullptr, 0, 1, qt, m, n, k, nullptr, nullptr, 0, 0.f,
+                                        nullptr, y, nullptr, nullptr, 0, stream);
+}
+
+int ggq_mmq_grad_input(const void* dy, const void* packed, int qt, int64_t m, int64_t n, int64_t k, void* dx, void* stream) {
+    return ggq_grouped_lora_mmq_backward(dy, nullptr, packed, nullptr, nullptr, nullptr, 0, 1, qt, m, n, k, nullptr, nullptr,
+                                         nullptr, nullptr, 0, 0.f, dx, nullptr, nullptr, nullptr, 0, stream);
+}
+
+// Forward of one projection (or a gate/up pair) over expert-sorted rows, optional LoRA fused.
+// groups == 0 means dense: one group of all rows using expert 0.
+int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void* packed2, const int64_t* expert_ids,
+                                 const int32_t* end_offsets, int64_t groups, int64_t experts, int qt, int64_t rows, int64_t n,
+                                 int64_t k, const void* lora_a, const void* lora_b, int r, float scale, void* xa_out, void* y1,
+                                 void* y2, void* ws, int64_t ws_bytes, void* stream) {
+    const char* what = "grouped_lora_mmq_forward";
+    hipStream_t s = as_stream(stream);
+    if (rows < 0 || n <= 0 || k <= 0 || rows >= (1ll << 31) || n >= (1ll << 30) || k >= (1ll << 30)) return set_error(GGQ_ERR_SHAPE, "%s: bad shape rows=%lld n=%lld k=%lld", what, (long long)rows, (long long)n, (long long)k);
+    if (int rc = check_weights(what, qt, packed1, k)) return rc;
+    if (packed2 && !aligned16(packed2)) return set_error(GGQ_ERR_ALIGN, "%s: packed weights must be 16-byte aligned", what);
+    if (int rc = check_lora(what, lora_a, lora_b, r)) return rc;
+    if (!x || !y1 || (packed2 && !y2)) return set_error(GGQ_ERR_NULL, "%s: null activation or output pointer", what);
+    if (groups > 0 && (!expert_ids || !end_offsets)) return set_error(GGQ_ERR_NULL, "%s: expert ids / offsets are null", what);
+    if (lora_a && !xa_out) return set_error(GGQ_ERR_NULL, "%s: xa_out is required with LoRA", what);
+    if (rows == 0) return GGQ_OK;
+    const int nseg = packed2 ? 2 : 1;
+    const int rp = lora_a ? rank_pad(r) : 0;
+    Bump bump{(char*)ws, ws_bytes, 0};
+
+    MmqParams p;
+    if (int rc = init_params(p, qt, kModeNT, (int)rows, (int)n, (int)k, nseg)) return rc;
+    p.a[0] = (const bf16_t*)x, p.lda = k;
+    p.w[0] = (const uint8_t*)packed1, p.w[1] = (const uint8_t*)packed2;
+    p.c[0] = y1, p.c[1] = y2, p.ldc = n;
+
+    const TileDesc* tiles64 = nullptr;
+    const int* num_tiles64 = nullptr;
+    int max_tiles64 = (int)((rows + 63) / 64);
+    if (groups > 0) {
+        const int max128 = (int)(rows / kBM + groups);
+        max_tiles64 = (int)(rows / 64 + groups);
+        TileDesc* t128 = (TileDesc*)bump.take((int64_t)max128 * sizeof(TileDesc));
+        TileDesc* t64 = lora_a ? (TileDesc*)bump.take((int64_t)max_tiles64 * sizeof(TileDesc)) : nullptr;
+        int* counts = (int*)bump.take(16);
+        if (!t128 || !counts || (lora_a && !t64)) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
+        if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, kBM, t128, counts, nullptr, 0, s)) return rc;
+        if (lora_a) {
+            if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, 64, t64, counts + 1, nullptr, 0, s)) return rc;
+        }
+        p.expert_ids = expert_ids, p.tiles = t128, p.num_tiles = counts, p.max_row_tiles = max128;
+        tiles64 = t64, num_tiles64 = counts + 1;
+    }
+    if (lora_a) {
+        SkinnyNtParams sp{};
+        sp.in[0] = (const bf16_t*)x, sp.ld_in = k;
+        sp.f = (const bf16_t*)lora_a, sp.ldf = k, sp.f_expert_elems = (int64_t)r * k;
+        sp.out = (bf16_t*)xa_out;
+        sp.m = (int)rows, sp.c = (int)k, sp.r = r, sp.nseg = 1;
+        sp.expert_ids = groups > 0 ? expert_ids : nullptr, sp.tiles = tiles64, sp.num_tiles = num_tiles64;
+        if (int rc = skinny_nt(sp, rp, max_tiles64, s)) return rc;
+        const bf16_t* lb = (const bf16_t*)lora_b;
+        if (rp != r) {
+            bf16_t* padded = (bf16_t*)bump.take(experts * nseg * n * rp * 2);
+            if (!padded) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
+            if (int rc = pad_factor(lb, padded, experts, (int)(nseg * n), r, rp, false, s)) return rc;
+            lb = padded;
+        }
+        p.la = (const bf16_t*)xa_out, p.lb = lb, p.lb_expert_elems = (int64_t)nseg * n * rp, p.r_pad = rp, p.lora_scale = scale;
+    }
+    return launch_mmq(qt, kModeNT, kEpiStore, p, s);
+}
+
+// Backward: dx = dy . W (+ LoRA term), and the factor gradients over all `experts` planes.
+int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* packed1, const void* packed2,
+                                  const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts, int qt,
+                                  int64_t rows, int64_t n, int64_t k, const void* x, const void* xa, const void* lora_a,
+                                  const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b, void* ws,
+                                  int64_t ws_bytes, void* stream) {
+    const char* what = "grouped_lora_mmq_backward";
+    hipStream_t s = as_stream(stream);
+    if (rows < 0 || n <= 0 || k <= 0 || rows >= (1ll << 31) || n >= (1ll << 30) || k >= (1ll << 30)) return set_error(GGQ_ERR_SHAPE, "%s: bad shape rows=%lld n=%lld k=%lld", what, (long long)rows, (long long)n, (long long)k);
+    if (int rc = check_weights(what, qt, packed1, k)) return rc;
+    if (packed2 && !aligned16(packed2)) return set_error(GGQ_ERR_ALIGN, "%s: packed weights must be 16-byte aligned", what);
+    if ((packed2 == nullptr) != (dy2 == nullptr)) return set_error(GGQ_ERR_NULL, "%s: a pair needs both cotangents and both weights", what);
+    if (int rc = check_lora(what, lora_a, lora_b, r)) return rc;
+    if (!dy1 || !dx) return set_error(GGQ_ERR_NULL, "%s: null cotangent or output pointer", what);
+    if (groups > 0 && (!expert_ids || !end_offsets)) return set_error(GGQ_ERR_NULL, "%s: expert ids / offsets are null", what);
+    if (lora_a && (!x || !xa)) return set_error(GGQ_ERR_NULL, "%s: x and xa are required with LoRA", what);
+    if ((d_lora_a || d_lora_b) && !lora_a) return set_error(GGQ_ERR_NULL, "%s: factor gradients requested without factors", what);
+    const int nseg = packed2 ? 2 : 1;
+    const int rp = lora_a ? rank_pad(r) : 0;
+    const int64_t ntot = nseg * n;
+    Bump bump{(char*)ws, ws_bytes, 0};
+
+    MmqParams p;
+    if (int rc = init_params(p, qt, kModeNN, (int)rows, (int)n, (int)k, nseg)) return rc;
+    p.a[0] = (const bf16_t*)dy1, p.a[1] = (const bf16_t*)dy2, p.lda = n;
+    p.w[0] = (const uint8_t*)packed1, p.w[1] = (const uint8_t*)packed2;
+    p.c[0] = dx, p.ldc = k;
+
+    const TileDesc* tiles64 = nullptr;
+    const int* num_tiles64 = nullptr;
+    const int* ranges = nullptr;
+    int max_tiles64 = (int)((rows + 63) / 64);
+    if (groups > 0) {
+        const int max128 = (int)(rows / kBM + groups);
+        max_tiles64 = (int)(rows / 64 + groups);
+        TileDesc* t128 = (TileDesc*)bump.take((int64_t)max128 * sizeof(TileDesc));
+        TileDesc* t64 = lora_a ? (TileDesc*)bump.take((int64_t)max_tiles64 * sizeof(TileDesc)) : nullptr;
+        int* counts = (int*)bump.take(16);
+        int* rg = lora_a ? (int*)bump.take(experts * 2 * 4) : nullptr;
+        if (!t128 || !counts || (lora_a && (!t64 || !rg))) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
+        if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, kBM, t128, counts, rg, (int)experts, s)) return rc;
+        if (lora_a) {
+            if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, 64, t64, counts + 1, nullptr, 0, s)) return rc;
+        }
+        p.expert_ids = expert_ids, p.tiles = t128, p.num_tiles = counts, p.max_row_tiles = max128;
+        tiles64 = t64, num_tiles64 = counts + 1, ranges = rg;
+    }
+    if (lora_a) {
+        // t = dy . B  (through B^T so both operands are contraction-contiguous)
+        bf16_t* bt = (bf16_t*)bump.take(experts * ntot * r * 2);
+        bf16_t* dyb = (bf16_t*)bump.take(rows * rp * 2);
+        bf16_t* atp = (bf16_t*)bump.take(experts * k * rp * 2);
+        if (!bt || !dyb || !atp) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
+        if (int rc = transpose_factor((const bf16_t*)lora_b, bt, experts, (int)ntot, r, s)) return rc;
+        if (int rc = pad_factor((const bf16_t*)lora_a, atp, experts, (int)k, r, rp, true, s)) return rc;
+        if (rows > 0) {
+            SkinnyNtParams sp{};
+            sp.in[0] = (const bf16_t*)dy1, sp.in[1] = (const bf16_t*)dy2, sp.ld_in = n;
+            sp.f = bt, sp.ldf = ntot, sp.f_expert_elems = (int64_t)r * ntot;
+            sp.out = dyb;
+            sp.m = (int)rows, sp.c = (int)n, sp.r = r, sp.nseg = nseg;
+            sp.expert_ids = groups > 0 ? expert_ids : nullptr, sp.tiles = tiles64, sp.num_tiles = num_tiles64;
+            if (int rc = skinny_nt(sp, rp, max_tiles64, s)) return rc;
+        }
+        p.la = dyb, p.lb = atp, p.lb_expert_elems = k * rp, p.r_pad = rp, p.lora_scale = scale;
+        if (d_lora_b) {
+            FactorGradParams fp{};
+            fp.in[0] = (const bf16_t*)dy1, fp.in[1] = (const bf16_t*)dy2, fp.ld_in = n;
+            fp.s = (const bf16_t*)xa, fp.out = (bf16_t*)d_lora_b, fp.out_expert_elems = ntot * r;
+            fp.ranges = ranges, fp.m = (int)rows, fp.c = (int)n, fp.r = r, fp.nseg = nseg, fp.out_j_major = 0, fp.scale = scale;
+            if (int rc = factor_grad(fp, rp, experts, s)) return rc;
+        }
+        if (d_lora_a) {
+            FactorGradParams fp{};
+            fp.in[0] = (const bf16_t*)x, fp.ld_in = k;
+            fp.s = dyb, fp.out = (bf16_t*)d_lora_a, fp.out_expert_elems = (int64_t)r * k;
+            fp.ranges = ranges, fp.m = (int)rows, fp.c = (int)k, fp.r = r, fp.nseg = 1, fp.out_j_major = 1, fp.scale = scale;
+            if (int rc = factor_grad(fp, rp, experts, s)) return rc;
+        }
+    }
+    if (rows == 0) return GGQ_OK;
+    return launch_mmq(qt, kModeNN, kEpiStore, p, s);
+}
+
+// ---------------------------------------------------------------------------------------------------
+int64_t ggq_route_plan_workspace_bytes(int64_t tokens, int top_k, int num_experts) {
+    return route_plan_workspace_bytes(tokens * top_k, num_experts) + 256;
+}
+
+int ggq_route_plan(const void* topk_ids, int ids_are_int64, int64_t tokens, int top_k, int num_experts, int64_t* sorted_ids,
+                   int64_t* permutation, int64_t* inverse, int32_t* counts, int32_t* end_offsets, int64_t* active_ids,
+                   int32_t* active_end_offsets, int32_t* status, void* ws, int64_t ws_bytes, void* stream) {
+    if (!topk_ids || !sorted_ids || !permutation || !inverse || !counts || !end_offsets || !active_ids || !active_end_offsets || !status || !ws)
+        return set_error(GGQ_ERR_NULL, "route_plan: null pointer");
+    return route_plan(topk_ids, ids_are_int64, tokens, top_k, num_experts, sorted_ids, permutation, inverse, counts, end_offsets,
+                      active_ids, active_end_offsets, status, ws, ws_bytes, as_stream(stream));
+}
+
+int ggq_route_gather_forward(const void* hidden, const int64_t* permutation, void* selected, int64_t tokens, int top_k, int hidden_dim, void* stream) {
+    if (!hidden || !permutation || !selected) return set_error(GGQ_ERR_NULL, "route_gather_forward: null pointer");
+    return route_gather_fwd(hidden, permutation, selected, tokens, top_k, hidden_dim, as_stream(stream));
+}
+
+int ggq_route_gather_backward(const void* grad_selected, const int64_t* inverse, void* grad_hidden, int64_t tokens, int top_k, int hidden_dim, void* stream) {
+    if (!grad_selected || !inverse || !grad_hidden) return set_error(GGQ_ERR_NULL, "route_gather_backward: null pointer");
+    return route_gather_bwd(grad_selected, inverse, grad_hidden, tokens, top_k, hidden_dim, as_stream(stream));
+}
+
+int ggq_route_combine_forward(const void* expert_out, const void* weights, int weights_are_bf16, const int64_t* inverse, void* out, int64_t tokens, int top_k, int hidden_dim, void* stream) {
+    if (!expert_out || !weights || !inverse || !out) return set_error(GGQ_ERR_NULL, "route_combine_forward: null pointer");
+    return route_combine_fwd(expert_out, weights, weights_are_bf16, inverse, out, tokens, top_k, hidden_dim, as_stream(stream));
+}
+
+int ggq_route_combine_backward(const void* expert_out, const void* weights, int weights_are_bf16, const int64_t* permutation, const void* grad_out, void* grad_expert_out, void* grad_weights, int64_t tokens, int top_k, int hidden_dim, void* stream) {
+    if (!expert_out || !weights || !permutation || !grad_out) return set_error(GGQ_ERR_NULL, "route_combine_backward: null pointer");
+    return route_combine_bwd(expert_out, weights, weights_are_bf16, permutation, grad_out, grad_expert_out, grad_weights, tokens, top_k, hidden_dim, as_stream(stream));
+}
+
+int ggq_swiglu_forward(const void* gate, const void* up, void* h, int64_t elems, void* stream) {
+    if (!gate || !up || !h) return set_error(GGQ_ERR_NULL, "swiglu_forward: null pointer");
+    return swiglu_fwd(gate, up, h, elems, as_stream(stream));
+}
+
+int ggq_swiglu_backward(const void* gate, const void* up, const void* dh, void* dgate, void* dup, int64_t elems, void* stream) {
+    if (!gate || !up || !dh || !dgate || !dup) return set_error(GGQ_ERR_NULL, "swiglu_backward: null pointer");
+    return swiglu_bwd(gate, up, dh, dgate, dup, elems, as_stream(stream));
+}
+
+// ---------------------------------------------------------------------------------------------------
+int64_t ggq_lmhead_ce_workspace_bytes(int64_t rows, int64_t vocab, int64_t hidden_dim, int64_t chunk) {
+    return lmhead_ce_workspace_bytes(rows, vocab, hidden_dim, chunk);
+}
+
+int ggq_lmhead_cross_entropy(int qt, const void* hidden, const void* packed, const int64_t* labels, int64_t rows, int64_t vocab,
+                             int64_t hidden_dim, int64_t chunk, int64_t ignore_index, int reduction_mean, float* loss_per_row,
+                             void* grad_hidden, float* lse_out, int32_t* n_valid_out, void* ws, int64_t ws_bytes, void* stream) {
+    if (int rc = check_weights("lmhead_cross_entropy", qt, packed, hidden_dim)) return rc;
+    return lmhead_ce(qt, hidden, packed, labels, rows, vocab, hidden_dim, chunk, ignore_index, reduction_mean, loss_per_row,
+                     grad_hidden, lse_out, n_valid_out, ws, ws_bytes, as_stream(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,68 @@
+// Shared device helpers for the gfx950 quantized-weight matmul kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ggq {
+
+// GGML type ids of the supported block formats.
+enum : int { kQ8_0 = 8, kQ4_K = 12, kQ6_K = 14, kIQ2_XXS = 16 };
+
+// Decoder helpers are host+device so the bit unpacking can also be exercised in a CPU build.
+#define GGQ_HD __host__ __device__ __forceinline__
+
+typedef uint16_t bf16_t;  // raw bf16 bits
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+// Two floats -> packed bf16 pair (lo in bits 0..15), round to nearest even (v_cvt_pk_bf16_f32).
+GGQ_HD uint32_t pack_bf16(float lo, float hi) {
+    f32x2_t v = {lo, hi};
+    bf16x2_t r = __builtin_convertvector(v, bf16x2_t);
+    return __builtin_bit_cast(uint32_t, r);
+}
+GGQ_HD bf16_t to_bf16(float x) { return (bf16_t)(pack_bf16(x, 0.0f) & 0xFFFFu); }
+GGQ_HD float bf16_to_f32(bf16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
+GGQ_HD float bf16_lo(uint32_t p) { return __builtin_bit_cast(float, p << 16); }
+GGQ_HD float bf16_hi(uint32_t p) { return __builtin_bit_cast(float, p & 0xFFFF0000u); }
+
+GGQ_HD float half_bits_to_f32(uint32_t h16) {
+    _Float16 h = __builtin_bit_cast(_Float16, (uint16_t)h16);
+    return (float)h;
+}
+
+// Hides the value's known bits from the optimizer so that a following
+// (float)((x >> 8*i) & 0xff) stays a single v_cvt_f32_ubyte<i> instead of bfe + cvt.
+GGQ_HD uint32_t opaque(uint32_t x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm("" : "+v"(x));
+#endif
+    return x;
+}
+GGQ_HD float ubyte0(uint32_t x) { return (float)(x & 0xFFu); }
+GGQ_HD float ubyte1(uint32_t x) { return (float)((x >> 8) & 0xFFu); }
+GGQ_HD float ubyte2(uint32_t x) { return (float)((x >> 16) & 0xFFu); }
+GGQ_HD float ubyte3(uint32_t x) { return (float)(x >> 24); }
+
+// Unaligned (2-byte aligned) global loads: the target allows unaligned vector memory access, so
+// these stay single global_load instructions.
+GGQ_HD uint32_t ld_u32(const uint8_t* p) {
+    uint32_t v;
+    __builtin_memcpy(&v, p, 4);
+    return v;
+}
+GGQ_HD uint4 ld_u128(const uint8_t* p) {
+    uint4 v;
+    __builtin_memcpy(&v, p, 16);
+    return v;
+}
+GGQ_HD uint32_t ld_u16(const uint8_t* p) {
+    uint16_t v;
+    __builtin_memcpy(&v, p, 2);
+    return v;
+}
+
+}  // namespace ggq

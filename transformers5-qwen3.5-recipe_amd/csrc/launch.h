@@ -1,0 +1,38 @@
+// Host-side plumbing shared by the C-ABI entry points: error codes, last-error text, launch checks.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ggq {
+
+enum : int {
+    GGQ_OK = 0,
+    GGQ_ERR_QTYPE = -1,    // unsupported GGML type id
+    GGQ_ERR_SHAPE = -2,    // negative / inconsistent / unsupported shape
+    GGQ_ERR_ALIGN = -3,    // pointer or leading dimension not aligned as required
+    GGQ_ERR_NULL = -4,     // required pointer is null
+    GGQ_ERR_RUNTIME = -5,  // HIP runtime reported an error
+    GGQ_ERR_WORKSPACE = -6 // workspace too small
+};
+
+int set_error(int code, const char* fmt, ...);
+int check_launch(const char* what);
+
+inline bool block_multiple(int qt, int64_t k) {
+    switch (qt) {
+        case 8: return k % 32 == 0;
+        case 12: case 14: case 16: return k % 256 == 0;
+    }
+    return true;  // unknown types are rejected by the callers' switch
+}
+inline int64_t packed_row_bytes(int qt, int64_t k) {
+    switch (qt) {
+        case 8: return k / 32 * 34;
+        case 12: return k / 256 * 144;
+        case 14: return k / 256 * 210;
+        case 16: return k / 256 * 66;
+    }
+    return -1;
+}
+
+}  // namespace ggq

@@ -1,0 +1,142 @@
+// Host launchers for the packed-weight tile kernel, the expert row-tile table and the error state.
+#include "mmq_tile.h"
+#include "launch.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+
+namespace ggq {
+
+// ------------------------------------------------------------------------------------------------
+static thread_local char g_last_error[512] = "";
+
+int set_error(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+const char* last_error() { return g_last_error; }
+
+int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return set_error(GGQ_ERR_RUNTIME, "%s: %s", what, hipGetErrorString(e));
+    return GGQ_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Row-tile table.  One workgroup; groups are walked 256 at a time with an LDS prefix sum, so the table
+// is in group order and identical from run to run.
+__global__ __launch_bounds__(256) void build_row_tiles_kernel(const int64_t* expert_ids, const int32_t* end_offsets,
+                                                              int groups, int bm, TileDesc* tiles, int* num_tiles,
+                                                              int* expert_ranges, int num_experts) {
+    __shared__ int scan[256];
+    __shared__ int base;
+    const int tid = threadIdx.x;
+    if (expert_ranges) {
+        for (int e = tid; e < num_experts; e += 256) expert_ranges[2 * e] = expert_ranges[2 * e + 1] = 0;
+    }
+    if (tid == 0) base = 0;
+    __syncthreads();
+    for (int g0 = 0; g0 < groups; g0 += 256) {
+        const int g = g0 + tid;
+        int r0 = 0, r1 = 0, count = 0;
+        if (g < groups) {
+            r0 = g == 0 ? 0 : end_offsets[g - 1];
+            r1 = end_offsets[g];
+            count = r1 > r0 ? (r1 - r0 + bm - 1) / bm : 0;
+            if (expert_ranges) {
+                const int64_t e = expert_ids ? expert_ids[g] : g;
+                if (e >= 0 && e < num_experts) expert_ranges[2 * e] = r0, expert_ranges[2 * e + 1] = r1;
+            }
+        }
+        scan[tid] = count;
+        __syncthreads();
+        for (int off = 1; off < 256; off <<= 1) {  // inclusive Hillis-Steele scan
+            int v = tid >= off ? scan[tid - off] : 0;
+            __syncthreads();
+            scan[tid] += v;
+            __syncthreads();
+        }
+        const int first = base + scan[tid] - count;
+        for (int t = 0; t < count; t++) {
+            TileDesc d;
+            d.group = g, d.row_begin = r0 + t * bm, d.row_end = min(r1, r0 + (t + 1) * bm), d.pad = 0;
+            tiles[first + t] = d;
+        }
+        __syncthreads();
+        if (tid == 255) base += scan[255];
+        __syncthreads();
+    }
+    if (tid == 0) *num_tiles = base;
+}
+
+int build_row_tiles(const int64_t* expert_ids, const int32_t* end_offsets, int groups, int bm, TileDesc* tiles,
+                    int* num_tiles, int* expert_ranges, int num_experts, hipStream_t s) {
+    hipLaunchKernelGGL(build_row_tiles_kernel, dim3(1), dim3(256), 0, s, expert_ids, end_offsets, groups, bm, tiles,
+                       num_tiles, expert_ranges, num_experts);
+    return check_launch("build_row_tiles");
+}
+
+// ------------------------------------------------------------------------------------------------
+template <int QT, int MODE, int EPI>
+static int launch_one(const MmqParams& p, hipStream_t s) {
+    const int col_tiles = (MODE == kModeNT ? p.nseg : 1) * p.col_tiles_per_seg;
+    const int64_t total = (int64_t)p.max_row_tiles * col_tiles;
+    if (total <= 0) return GGQ_OK;
+    const int64_t grid = (total + 7) / 8 * 8;  // the XCD remap inside the kernel needs a multiple of 8
+    if (grid > 0x7FFFFFF0) return set_error(GGQ_ERR_SHAPE, "mmq: too many tiles for one launch");
+    hipLaunchKernelGGL((mmq_tile_kernel<QT, MODE, EPI>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+    return check_launch("mmq_tile_kernel");
+}
+
+template <int QT>
+static int launch_qt(int mode, int epi, const MmqParams& p, hipStream_t s) {
+    if (mode == kModeNT) {
+        switch (epi) {
+            case kEpiStore: return launch_one<QT, kModeNT, kEpiStore>(p, s);
+            case kEpiCeStats: return launch_one<QT, kModeNT, kEpiCeStats>(p, s);
+            case kEpiCeGrad: return launch_one<QT, kModeNT, kEpiCeGrad>(p, s);
+        }
+    } else {
+        switch (epi) {
+            case kEpiStore: return launch_one<QT, kModeNN, kEpiStore>(p, s);
+            case kEpiAccumF32: return launch_one<QT, kModeNN, kEpiAccumF32>(p, s);
+        }
+    }
+    return set_error(GGQ_ERR_SHAPE, "mmq: unsupported mode/epilogue combination");
+}
+
+int launch_mmq(int qt, int mode, int epi, const MmqParams& p, hipStream_t s) {
+    switch (qt) {
+        case kQ8_0: return launch_qt<kQ8_0>(mode, epi, p, s);
+        case kQ4_K: return launch_qt<kQ4_K>(mode, epi, p, s);
+        case kQ6_K: return launch_qt<kQ6_K>(mode, epi, p, s);
+        case kIQ2_XXS: return launch_qt<kIQ2_XXS>(mode, epi, p, s);
+    }
+    return set_error(GGQ_ERR_QTYPE, "unsupported GGML type id %d (supported: 8 Q8_0, 12 Q4_K, 14 Q6_K, 16 IQ2_XXS)", qt);
+}
+
+// Fills the shape-derived fields of a parameter block.  n, k describe one weight segment [n, k].
+int init_params(MmqParams& p, int qt, int mode, int m, int n, int k, int nseg) {
+    if (m < 0 || n <= 0 || k <= 0) return set_error(GGQ_ERR_SHAPE, "mmq: bad shape m=%d n=%d k=%d", m, n, k);
+    if (packed_row_bytes(qt, k) < 0) return set_error(GGQ_ERR_QTYPE, "unsupported GGML type id %d", qt);
+    if (!block_multiple(qt, k)) return set_error(GGQ_ERR_SHAPE, "mmq: K=%d is not a multiple of the block size of type %d", k, qt);
+    if (k % 64) return set_error(GGQ_ERR_SHAPE, "mmq: K=%d must be a multiple of 64", k);
+    p = MmqParams{};
+    p.m = m, p.n = n, p.k = k, p.nseg = nseg;
+    p.w_row_bytes = packed_row_bytes(qt, k);
+    p.w_expert_bytes = p.w_row_bytes * n;
+    if (mode == kModeNT) {
+        p.col_tiles_per_seg = (n + kBN - 1) / kBN;
+        p.steps_per_seg = k / kBK;
+    } else {
+        p.col_tiles_per_seg = (k + kBN - 1) / kBN;
+        p.steps_per_seg = (n + kBK - 1) / kBK;
+    }
+    p.max_row_tiles = (m + kBM - 1) / kBM;
+    return GGQ_OK;
+}
+
+}  // namespace ggq

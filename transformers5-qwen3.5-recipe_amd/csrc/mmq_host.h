@@ -1,0 +1,113 @@
+// Parameter blocks and host launchers shared between the translation units of the library.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ggq {
+
+typedef uint16_t bf16_t;
+
+struct TileDesc {  // one row tile of an expert group: rows [row_begin, row_end) of group `group`
+    int group, row_begin, row_end, pad;
+};
+
+struct SkinnyNtParams {
+    const bf16_t* in[2];  // [m, c] per segment
+    int64_t ld_in;
+    const bf16_t* f;      // per expert [r][ldf], contraction contiguous
+    int64_t ldf, f_expert_elems;
+    bf16_t* out;          // [m, r_pad]
+    int m, c, r, nseg;
+    const int64_t* expert_ids;
+    const TileDesc* tiles;  // 64-row tiles (null: dense)
+    const int* num_tiles;
+};
+
+struct FactorGradParams {
+    const bf16_t* in[2];  // [m, c] per segment
+    int64_t ld_in;
+    const bf16_t* s;      // [m, r_pad]
+    bf16_t* out;          // per expert: [nseg*c][r] (out_j_major = 0) or [r][nseg*c] (= 1)
+    int64_t out_expert_elems;
+    const int* ranges;    // per expert (row_begin, row_end); null: all m rows, one expert
+    int m, c, r, nseg, out_j_major;
+    float scale;
+};
+
+constexpr int kBM = 128, kBN = 256, kBK = 64;
+constexpr int kLdsStride = kBK + 8;  // bf16 elements per LDS row: 144 bytes keeps 128-bit reads conflict-free
+constexpr int kThreads = 256;
+
+enum : int { kModeNT = 0, kModeNN = 1 };
+enum : int {
+    kEpiStore = 0,     // C (bf16) = acc
+    kEpiAccumF32 = 1,  // C32 (fp32) += acc
+    kEpiCeStats = 2,   // per-row partial (max, sum exp) over the tile's columns + target logit
+    kEpiCeGrad = 3     // C (bf16) = (exp(acc - lse[m]) - [col == label[m]]) * row_scale[m]
+};
+
+struct MmqParams {
+    const bf16_t* a[2];   // activations; [1] only for a pair in NN mode
+    int64_t lda;
+    const uint8_t* w[2];  // packed weights; [1] only for a pair
+    int64_t w_row_bytes, w_expert_bytes;
+    void* c[2];           // outputs; [1] only for a pair in NT mode
+    int64_t ldc;
+    int m, n, k;          // W segment is [n, k]
+    int nseg;             // 1, or 2 for a pair
+    int col_tiles_per_seg;  // NT: ceil(n/256); NN: ceil(k/256) (nseg applies to contraction there)
+    int steps_per_seg;      // NT: k/64; NN: ceil(n/64)
+    // expert groups (null tiles => one dense group of m rows)
+    const int64_t* expert_ids;
+    const TileDesc* tiles;
+    const int* num_tiles;
+    int max_row_tiles;
+    // LoRA
+    const bf16_t* la;     // [rows, r_pad]  (x A^T in NT, dY B in NN)
+    const bf16_t* lb;     // per expert [cols_total, r_pad] (B rows in NT, A^T rows in NN)
+    int64_t lb_expert_elems;
+    int r_pad;            // multiple of 16, <= 64; 0 = no LoRA
+    float lora_scale;
+    // cross-entropy epilogues
+    const int64_t* labels;     // [m]
+    const float* lse;          // [m]
+    const float* row_scale;    // [m]  (1/n_non_ignore or 1, 0 for ignored rows)
+    float2* ce_partials;       // [m, ce_partials_ld] (max, sumexp)
+    float* ce_target_logit;    // [m]
+    int ce_partials_ld, ce_col_offset, ce_partial_offset;
+    int64_t ignore_index;
+};
+
+const char* last_error();
+int launch_mmq(int qt, int mode, int epi, const MmqParams& p, hipStream_t s);
+int init_params(MmqParams& p, int qt, int mode, int m, int n, int k, int nseg);
+
+int pad_factor(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int r, int r_pad, bool transpose, hipStream_t s);
+int transpose_factor(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int r, hipStream_t s);
+int skinny_nt(const SkinnyNtParams& p, int r_pad, int grid_tiles, hipStream_t s);
+int factor_grad(const FactorGradParams& p, int r_pad, int64_t experts, hipStream_t s);
+
+// Builds the row-tile table of an expert-sorted layout on the device (no host sync):
+// tiles[0..*num_tiles) in group order, tile height bm; optionally per-expert row ranges.
+int build_row_tiles(const int64_t* expert_ids, const int32_t* end_offsets, int groups, int bm, TileDesc* tiles,
+                    int* num_tiles, int* expert_ranges, int num_experts, hipStream_t s);
+
+int64_t route_plan_workspace_bytes(int64_t routes, int num_experts);
+int route_plan(const void* topk_ids, int ids_are_int64, int64_t tokens, int top_k, int num_experts,
+               int64_t* sorted_ids, int64_t* permutation, int64_t* inverse, int* counts, int* end_offsets,
+               int64_t* active_ids, int* active_end, int* num_active, void* ws, int64_t ws_bytes, hipStream_t s);
+int route_gather_fwd(const void* hidden, const int64_t* permutation, void* selected, int64_t tokens, int top_k, int hidden_dim, hipStream_t s);
+int route_gather_bwd(const void* grad_selected, const int64_t* inverse, void* grad_hidden, int64_t tokens, int top_k, int hidden_dim, hipStream_t s);
+int route_combine_fwd(const void* expert_out, const void* weights, int w_is_bf16, const int64_t* inverse, void* out, int64_t tokens, int top_k, int hidden_dim, hipStream_t s);
+int route_combine_bwd(const void* expert_out, const void* weights, int w_is_bf16, const int64_t* permutation, const void* grad_out, void* grad_expert_out, void* grad_weights, int64_t tokens, int top_k, int hidden_dim, hipStream_t s);
+int swiglu_fwd(const void* gate, const void* up, void* h, int64_t elems, hipStream_t s);
+int swiglu_bwd(const void* gate, const void* up, const void* dh, void* dgate, void* dup, int64_t elems, hipStream_t s);
+
+int64_t lmhead_ce_workspace_bytes(int64_t rows, int64_t vocab, int64_t hidden, int64_t chunk);
+int lmhead_ce(int qt, const void* hidden, const void* packed, const int64_t* labels, int64_t rows, int64_t vocab,
+              int64_t hidden_dim, int64_t chunk, int64_t ignore_index, int reduction_mean, float* loss_1d,
+              void* grad_hidden, float* lse_out, int* n_valid_out, void* ws, int64_t ws_bytes, hipStream_t s);
+
+int dequantize(int qt, const void* payload, int64_t rows, int64_t k, void* out, int out_f32, hipStream_t stream);
+
+}  // namespace ggq

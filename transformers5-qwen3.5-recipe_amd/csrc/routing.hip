@@ -1,0 +1,413 @@
+// Expert-sorted routing layout: stable counting sort of the flat top-k expert ids, per-expert offsets,
+// row gather / weighted combine and their backward passes.  Pure integer and byte work, HBM-bound;
+// everything is deterministic (no atomics) so a recomputed forward reproduces the same bits.
+//
+// Route r = token * k + rank.  permutation[s] = route at sorted position s; inverse[r] = s.
+#include "common.h"
+#include "launch.h"
+#include "mmq_host.h"
+
+namespace ggq {
+
+constexpr int kChunk = 256;  // routes per workgroup in the sort
+
+template <typename IdT>
+__device__ __forceinline__ int load_id(const IdT* ids, int64_t i, int num_experts, int* bad) {
+    int64_t v = (int64_t)ids[i];
+    if (v < 0 || v >= num_experts) {
+        *bad = 1;
+        v = v < 0 ? 0 : num_experts - 1;
+    }
+    return (int)v;
+}
+
+// Pass 1: per chunk of 256 routes, the rank of every route among equal ids inside the chunk and the
+// chunk's histogram.
+template <typename IdT>
+__global__ __launch_bounds__(kChunk) void route_rank_kernel(const IdT* ids, int64_t routes, int num_experts,
+                                                            int* local_rank, int* chunk_hist, int* chunk_bad) {
+    __shared__ int sid[kChunk];
+    __shared__ int any_bad;
+    const int tid = threadIdx.x;
+    const int64_t i = (int64_t)blockIdx.x * kChunk + tid;
+    int bad = 0;
+    const int my = i < routes ? load_id(ids, i, num_experts, &bad) : -1;
+    if (tid == 0) any_bad = 0;
+    sid[tid] = my;
+    __syncthreads();
+    if (bad) any_bad = 1;  // benign race: every writer stores 1
+    __syncthreads();
+    if (tid == 0) chunk_bad[blockIdx.x] = any_bad;
+    if (i < routes) {
+        int rank = 0;
+        for (int j = 0; j < tid; j++) rank += (sid[j] == my);
+        local_rank[i] = rank;
+    }
+    for (int e = tid; e < num_experts; e += kChunk) {
+        int c = 0;
+        for (int j = 0; j < kChunk; j++) c += (sid[j] == e);
+        chunk_hist[(int64_t)blockIdx.x * num_experts + e] = c;
+    }
+}
+
+// Pass 2 (one workgroup): turn chunk histograms into chunk bases, expert counts, cumulative end
+// offsets and the compact list of active experts.
+__global__ __launch_bounds__(256) void route_scan_kernel(int* chunk_hist, int chunks, int num_experts, int* counts,
+                                                         int* end_offsets, int64_t* active_ids, int* active_end,
+                                                         int* num_active, int* expert_base, const int* chunk_bad) {
+    __shared__ int scan[256];
+    __shared__ int carry_rows, carry_active;
+    const int tid = threadIdx.x;
+    if (tid == 0) carry_rows = 0, carry_active = 0;
+    __syncthreads();
+    for (int e0 = 0; e0 < num_experts; e0 += 256) {
+        const int e = e0 + tid;
+        int total = 0;
+        if (e < num_experts) {
+            for (int c = 0; c < chunks; c++) {
+                int* h = &chunk_hist[(int64_t)c * num_experts + e];
+                const int v = *h;
+                *h = total;  // becomes the chunk's base inside the expert
+                total += v;
+            }
+            counts[e] = total;
+        }
+        // prefix over experts: rows
+        scan[tid] = total;
+        __syncthreads();
+        for (int off = 1; off < 256; off <<= 1) {
+            int v = tid >= off ? scan[tid - off] : 0;
+            __syncthreads();
+            scan[tid] += v;
+            __syncthreads();
+        }
+        const int end = carry_rows + scan[tid];
+        const int chunk_rows = scan[255];
+        __syncthreads();
+        // prefix over experts: active flags
+        const int active = total > 0 ? 1 : 0;
+        scan[tid] = active;
+        __syncthreads();
+        for (int off = 1; off < 256; off <<= 1) {
+            int v = tid >= off ? scan[tid - off] : 0;
+            __syncthreads();
+            scan[tid] += v;
+            __syncthreads();
+        }
+        if (e < num_experts) {
+            end_offsets[e] = end;
+            expert_base[e] = end - total;
+            if (active) {
+                const int slot = carry_active + scan[tid] - 1;
+                active_ids[slot] = e;
+                active_end[slot] = end;
+            }
+        }
+        const int chunk_active = scan[255];
+        __syncthreads();
+        if (tid == 0) carry_rows += chunk_rows, carry_active += chunk_active;
+        __syncthreads();
+    }
+    // status word pair: number of active experts, and whether any id was outside [0, num_experts)
+    // (such ids are clamped so that no access leaves the buffers; the caller decides what to do).
+    int bad = 0;
+    for (int c = tid; c < chunks; c += 256) bad |= chunk_bad[c];
+    scan[tid] = bad;
+    __syncthreads();
+    if (tid == 0) {
+        for (int j = 1; j < 256; j++) bad |= scan[j];
+        num_active[0] = carry_active;
+        num_active[1] = bad;
+    }
+    // unused tail of the compact lists: repeat the total so that "offsets" stay monotone
+    for (int s = carry_active + tid; s < num_experts; s += 256) {
+        active_ids[s] = 0;
+        active_end[s] = carry_rows;
+    }
+}
+
+// Pass 3: scatter.
+template <typename IdT>
+__global__ __launch_bounds__(kChunk) void route_scatter_kernel(const IdT* ids, int64_t routes, int num_experts,
+                                                               const int* local_rank, const int* chunk_base,
+                                                               const int* expert_base, int64_t* sorted_ids,
+                                                               int64_t* permutation, int64_t* inverse) {
+    const int64_t i = (int64_t)blockIdx.x * kChunk + threadIdx.x;
+    if (i >= routes) return;
+    int bad = 0;
+    const int e = load_id(ids, i, num_experts, &bad);
+    const int64_t pos = (int64_t)expert_base[e] + chunk_base[(int64_t)blockIdx.x * num_experts + e] + local_rank[i];
+    sorted_ids[pos] = e;
+    permutation[pos] = i;
+    inverse[i] = pos;
+}
+
+int64_t route_plan_workspace_bytes(int64_t routes, int num_experts) {
+    const int64_t chunks = (routes + kChunk - 1) / kChunk;
+    return (routes + chunks * num_experts + num_experts + chunks + 4) * (int64_t)sizeof(int);
+}
+
+int route_plan(const void* topk_ids, int ids_are_int64, int64_t tokens, int top_k, int num_experts,
+               int64_t* sorted_ids, int64_t* permutation, int64_t* inverse, int* counts, int* end_offsets,
+               int64_t* active_ids, int* active_end, int* num_active, void* ws, int64_t ws_bytes, hipStream_t s) {
+    const int64_t routes = tokens * top_k;
+    if (tokens < 0 || top_k <= 0 || num_experts <= 0) return set_error(GGQ_ERR_SHAPE, "route_plan: bad shape");
+    if (routes >= (int64_t)1 << 31) return set_error(GGQ_ERR_SHAPE, "route_plan: more than 2^31 routes");
+    if (ws_bytes < route_plan_workspace_bytes(routes, num_experts)) return set_error(GGQ_ERR_WORKSPACE, "route_plan: workspace too small");
+    const int chunks = (int)((routes + kChunk - 1) / kChunk);
+    int* local_rank = (int*)ws;
+    int* chunk_hist = local_rank + routes;
+    int* expert_base = chunk_hist + (int64_t)chunks * num_experts;
+    int* chunk_bad = expert_base + num_experts;
+    if (chunks > 0) {
+        if (ids_are_int64)
+            hipLaunchKernelGGL(route_rank_kernel<int64_t>, dim3(chunks), dim3(kChunk), 0, s, (const int64_t*)topk_ids, routes, num_experts, local_rank, chunk_hist, chunk_bad);
+        else
+            hipLaunchKernelGGL(route_rank_kernel<int32_t>, dim3(chunks), dim3(kChunk), 0, s, (const int32_t*)topk_ids, routes, num_experts, local_rank, chunk_hist, chunk_bad);
+    }
+    hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(256), 0, s, chunk_hist, chunks, num_experts, counts, end_offsets, active_ids, active_end, num_active, expert_base, chunk_bad);
+    if (chunks > 0) {
+        if (ids_are_int64)
+            hipLaunchKernelGGL(route_scatter_kernel<int64_t>, dim3(chunks), dim3(kChunk), 0, s, (const int64_t*)topk_ids, routes, num_experts, local_rank, chunk_hist, expert_base, sorted_ids, permutation, inverse);
+        else
+            hipLaunchKernelGGL(route_scatter_kernel<int32_t>, dim3(chunks), dim3(kChunk), 0, s, (const int32_t*)topk_ids, routes, num_experts, local_rank, chunk_hist, expert_base, sorted_ids, permutation, inverse);
+    }
+    return check_launch("route_plan");
+}
+
+// ------------------------------------------------------------------------------------------------
+// gather forward: selected[s, :] = hidden[permutation[s] / k, :]   (16-byte copies)
+__global__ __launch_bounds__(256) void route_gather_fwd_kernel(const uint4* hidden, const int64_t* permutation, uint4* selected,
+                                                               int64_t routes, int top_k, int chunks_per_row) {
+    const int64_t total = routes * chunks_per_row;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t srow = i / chunks_per_row;
+        const int ch = (int)(i - srow * chunks_per_row);
+        const int64_t token = permutation[srow] / top_k;
+        selected[i] = hidden[token * chunks_per_row + ch];
+    }
+}
+
+// gather backward: grad_hidden[t] = sum over the token's routes, visited in ascending sorted position,
+// with the running sum rounded to bf16 after every add.
+template <int MAXK>
+__global__ __launch_bounds__(256) void route_gather_bwd_kernel(const uint4* grad_selected, const int64_t* inverse, uint4* grad_hidden,
+                                                               int64_t tokens, int top_k, int chunks_per_row) {
+    const int64_t total = tokens * chunks_per_row;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t t = i / chunks_per_row;
+        const int ch = (int)(i - t * chunks_per_row);
+        int64_t pos[MAXK];
+#pragma unroll
+        for (int j = 0; j < MAXK; j++) pos[j] = j < top_k ? inverse[t * top_k + j] : INT64_MAX;
+        // insertion sort (k is tiny)
+#pragma unroll
+        for (int a = 1; a < MAXK; a++)
+#pragma unroll
+            for (int b = a; b > 0; b--)
+                if (pos[b] < pos[b - 1]) {
+                    const int64_t tmp = pos[b];
+                    pos[b] = pos[b - 1];
+                    pos[b - 1] = tmp;
+                }
+        float acc[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] = 0.f;
+#pragma unroll
+        for (int j = 0; j < MAXK; j++) {
+            if (j < top_k) {
+                const uint4 g = grad_selected[pos[j] * chunks_per_row + ch];
+                const uint32_t w[4] = {g.x, g.y, g.z, g.w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    acc[2 * e] = bf16_to_f32(to_bf16(acc[2 * e] + bf16_lo(w[e])));
+                    acc[2 * e + 1] = bf16_to_f32(to_bf16(acc[2 * e + 1] + bf16_hi(w[e])));
+                }
+            }
+        }
+        uint4 o;
+        o.x = pack_bf16(acc[0], acc[1]), o.y = pack_bf16(acc[2], acc[3]);
+        o.z = pack_bf16(acc[4], acc[5]), o.w = pack_bf16(acc[6], acc[7]);
+        grad_hidden[i] = o;
+    }
+}
+
+__device__ __forceinline__ float load_weight(const void* w, int w_is_bf16, int64_t i) {
+    const float v = w_is_bf16 ? bf16_to_f32(((const bf16_t*)w)[i]) : ((const float*)w)[i];
+    return bf16_to_f32(to_bf16(v));  // the layout applies routing weights at bf16 precision
+}
+
+// combine forward: out[t] = bf16( sum_rank fp32(o[inverse[t*k+rank]]) * w[t, rank] ), ranks in order.
+__global__ __launch_bounds__(256) void route_combine_fwd_kernel(const uint4* expert_out, const void* weights, int w_is_bf16,
+                                                                const int64_t* inverse, uint4* out, int64_t tokens, int top_k,
+                                                                int chunks_per_row) {
+    const int64_t total = tokens * chunks_per_row;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t t = i / chunks_per_row;
+        const int ch = (int)(i - t * chunks_per_row);
+        float acc[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] = 0.f;
+        for (int rank = 0; rank < top_k; rank++) {
+            const int64_t route = t * top_k + rank;
+            const float w = load_weight(weights, w_is_bf16, route);
+            const uint4 g = expert_out[inverse[route] * chunks_per_row + ch];
+            const uint32_t v[4] = {g.x, g.y, g.z, g.w};
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                acc[2 * e] = fmaf(bf16_lo(v[e]), w, acc[2 * e]);
+                acc[2 * e + 1] = fmaf(bf16_hi(v[e]), w, acc[2 * e + 1]);
+            }
+        }
+        uint4 o;
+        o.x = pack_bf16(acc[0], acc[1]), o.y = pack_bf16(acc[2], acc[3]);
+        o.z = pack_bf16(acc[4], acc[5]), o.w = pack_bf16(acc[6], acc[7]);
+        out[i] = o;
+    }
+}
+
+// combine backward: one wave per sorted route.  dO[s] = bf16(g[t] * w); dW[route] = sum_h g * o in
+// fp32 with a fixed lane-strided order and a butterfly reduction.
+__global__ __launch_bounds__(256) void route_combine_bwd_kernel(const uint4* expert_out, const void* weights, int w_is_bf16,
+                                                                const int64_t* permutation, const uint4* grad_out, uint4* grad_expert_out,
+                                                                void* grad_weights, int64_t routes, int top_k, int chunks_per_row) {
+    const int lane = threadIdx.x & 63;
+    const int64_t s = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (s >= routes) return;
+    const int64_t route = permutation[s];
+    const int64_t t = route / top_k;
+    const float w = load_weight(weights, w_is_bf16, route);
+    float dot = 0.f;
+    for (int ch = lane; ch < chunks_per_row; ch += 64) {
+        const uint4 g = grad_out[t * chunks_per_row + ch];
+        const uint4 o = expert_out[s * chunks_per_row + ch];
+        const uint32_t gv[4] = {g.x, g.y, g.z, g.w}, ov[4] = {o.x, o.y, o.z, o.w};
+        uint32_t r[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const float g0 = bf16_lo(gv[e]), g1 = bf16_hi(gv[e]);
+            r[e] = pack_bf16(g0 * w, g1 * w);
+            dot = fmaf(g0, bf16_lo(ov[e]), dot);
+            dot = fmaf(g1, bf16_hi(ov[e]), dot);
+        }
+        if (grad_expert_out) grad_expert_out[s * chunks_per_row + ch] = make_uint4(r[0], r[1], r[2], r[3]);
+    }
+    if (grad_weights) {
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) dot += __shfl_xor(dot, off, 64);
+        if (lane == 0) {
+            if (w_is_bf16) ((bf16_t*)grad_weights)[route] = to_bf16(dot);
+            else ((float*)grad_weights)[route] = dot;
+        }
+    }
+}
+
+static inline unsigned stream_grid(int64_t items) {
+    int64_t g = (items + 255) / 256;
+    return (unsigned)(g < 1 ? 1 : (g > 256 * 64 ? 256 * 64 : g));
+}
+
+static int check_rows(const void* a, const void* b, int hidden, const char* what) {
+    if (hidden <= 0 || hidden % 8) return set_error(GGQ_ERR_SHAPE, "%s: hidden size must be a positive multiple of 8", what);
+    if (((uintptr_t)a | (uintptr_t)b) & 15) return set_error(GGQ_ERR_ALIGN, "%s: row buffers must be 16-byte aligned", what);
+    return GGQ_OK;
+}
+
+int route_gather_fwd(const void* hidden, const int64_t* permutation, void* selected, int64_t tokens, int top_k, int hidden_dim, hipStream_t s) {
+    if (int rc = check_rows(hidden, selected, hidden_dim, "route_gather_forward")) return rc;
+    const int64_t routes = tokens * top_k;
+    if (routes == 0) return GGQ_OK;
+    hipLaunchKernelGGL(route_gather_fwd_kernel, dim3(stream_grid(routes * (hidden_dim / 8))), dim3(256), 0, s, (const uint4*)hidden, permutation, (uint4*)selected, routes, top_k, hidden_dim / 8);
+    return check_launch("route_gather_forward");
+}
+
+int route_gather_bwd(const void* grad_selected, const int64_t* inverse, void* grad_hidden, int64_t tokens, int top_k, int hidden_dim, hipStream_t s) {
+    if (int rc = check_rows(grad_selected, grad_hidden, hidden_dim, "route_gather_backward")) return rc;
+    if (tokens == 0) return GGQ_OK;
+    const unsigned grid = stream_grid(tokens * (hidden_dim / 8));
+    if (top_k <= 8)
+        hipLaunchKernelGGL(route_gather_bwd_kernel<8>, dim3(grid), dim3(256), 0, s, (const uint4*)grad_selected, inverse, (uint4*)grad_hidden, tokens, top_k, hidden_dim / 8);
+    else if (top_k <= 16)
+        hipLaunchKernelGGL(route_gather_bwd_kernel<16>, dim3(grid), dim3(256), 0, s, (const uint4*)grad_selected, inverse, (uint4*)grad_hidden, tokens, top_k, hidden_dim / 8);
+    else
+        return set_error(GGQ_ERR_SHAPE, "route_gather_backward: top_k above 16 is not supported");
+    return check_launch("route_gather_backward");
+}
+
+int route_combine_fwd(const void* expert_out, const void* weights, int w_is_bf16, const int64_t* inverse, void* out, int64_t tokens, int top_k, int hidden_dim, hipStream_t s) {
+    if (int rc = check_rows(expert_out, out, hidden_dim, "route_combine_forward")) return rc;
+    if (tokens == 0) return GGQ_OK;
+    hipLaunchKernelGGL(route_combine_fwd_kernel, dim3(stream_grid(tokens * (hidden_dim / 8))), dim3(256), 0, s, (const uint4*)expert_out, weights, w_is_bf16, inverse, (uint4*)out, tokens, top_k, hidden_dim / 8);
+    return check_launch("route_combine_forward");
+}
+
+int route_combine_bwd(const void* expert_out, const void* weights, int w_is_bf16, const int64_t* permutation, const void* grad_out, void* grad_expert_out, void* grad_weights, int64_t tokens, int top_k, int hidden_dim, hipStream_t s) {
+    if (int rc = check_rows(expert_out, grad_out, hidden_dim, "route_combine_backward")) return rc;
+    if (grad_expert_out && ((uintptr_t)grad_expert_out & 15)) return set_error(GGQ_ERR_ALIGN, "route_combine_backward: output must be 16-byte aligned");
+    const int64_t routes = tokens * top_k;
+    if (routes == 0) return GGQ_OK;
+    const int64_t grid = (routes + 3) / 4;
+    if (grid > 0x7FFFFFFF) return set_error(GGQ_ERR_SHAPE, "route_combine_backward: too many routes");
+    hipLaunchKernelGGL(route_combine_bwd_kernel, dim3((unsigned)grid), dim3(256), 0, s, (const uint4*)expert_out, weights, w_is_bf16, permutation, (const uint4*)grad_out, (uint4*)grad_expert_out, grad_weights, routes, top_k, hidden_dim / 8);
+    return check_launch("route_combine_backward");
+}
+
+// ------------------------------------------------------------------------------------------------
+// SiLU-gated product of the expert FFN: h = silu(gate) * up, and its backward.
+__global__ __launch_bounds__(256) void swiglu_fwd_kernel(const uint4* gate, const uint4* up, uint4* h, int64_t chunks) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < chunks; i += (int64_t)gridDim.x * 256) {
+        const uint4 g = gate[i], u = up[i];
+        const uint32_t gv[4] = {g.x, g.y, g.z, g.w}, uv[4] = {u.x, u.y, u.z, u.w};
+        uint32_t r[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const float g0 = bf16_lo(gv[e]), g1 = bf16_hi(gv[e]);
+            const float s0 = g0 / (1.0f + __expf(-g0)), s1 = g1 / (1.0f + __expf(-g1));
+            r[e] = pack_bf16(s0 * bf16_lo(uv[e]), s1 * bf16_hi(uv[e]));
+        }
+        h[i] = make_uint4(r[0], r[1], r[2], r[3]);
+    }
+}
+
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint4* gate, const uint4* up, const uint4* dh, uint4* dgate, uint4* dup, int64_t chunks) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < chunks; i += (int64_t)gridDim.x * 256) {
+        const uint4 g = gate[i], u = up[i], d = dh[i];
+        const uint32_t gv[4] = {g.x, g.y, g.z, g.w}, uv[4] = {u.x, u.y, u.z, u.w}, dv[4] = {d.x, d.y, d.z, d.w};
+        uint32_t rg[4], ru[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            float og[2], ou[2];
+#pragma unroll
+            for (int hlf = 0; hlf < 2; hlf++) {
+                const float x = hlf ? bf16_hi(gv[e]) : bf16_lo(gv[e]);
+                const float uu = hlf ? bf16_hi(uv[e]) : bf16_lo(uv[e]);
+                const float dd = hlf ? bf16_hi(dv[e]) : bf16_lo(dv[e]);
+                const float sig = 1.0f / (1.0f + __expf(-x));
+                og[hlf] = dd * uu * (sig * (1.0f + x * (1.0f - sig)));
+                ou[hlf] = dd * x * sig;
+            }
+            rg[e] = pack_bf16(og[0], og[1]);
+            ru[e] = pack_bf16(ou[0], ou[1]);
+        }
+        dgate[i] = make_uint4(rg[0], rg[1], rg[2], rg[3]);
+        dup[i] = make_uint4(ru[0], ru[1], ru[2], ru[3]);
+    }
+}
+
+int swiglu_fwd(const void* gate, const void* up, void* h, int64_t elems, hipStream_t s) {
+    if (elems % 8) return set_error(GGQ_ERR_SHAPE, "swiglu: element count must be a multiple of 8");
+    if (((uintptr_t)gate | (uintptr_t)up | (uintptr_t)h) & 15) return set_error(GGQ_ERR_ALIGN, "swiglu: buffers must be 16-byte aligned");
+    if (elems == 0) return GGQ_OK;
+    hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(stream_grid(elems / 8)), dim3(256), 0, s, (const uint4*)gate, (const uint4*)up, (uint4*)h, elems / 8);
+    return check_launch("swiglu_forward");
+}
+
+int swiglu_bwd(const void* gate, const void* up, const void* dh, void* dgate, void* dup, int64_t elems, hipStream_t s) {
+    if (elems % 8) return set_error(GGQ_ERR_SHAPE, "swiglu: element count must be a multiple of 8");
+    if (((uintptr_t)gate | (uintptr_t)up | (uintptr_t)dh | (uintptr_t)dgate | (uintptr_t)dup) & 15) return set_error(GGQ_ERR_ALIGN, "swiglu: buffers must be 16-byte aligned");
+    if (elems == 0) return GGQ_OK;
+    hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(stream_grid(elems / 8)), dim3(256), 0, s, (const uint4*)gate, (const uint4*)up, (const uint4*)dh, (uint4*)dgate, (uint4*)dup, elems / 8);
+    return check_launch("swiglu_backward");
+}
+
+}  // namespace ggq

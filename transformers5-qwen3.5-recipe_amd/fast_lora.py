@@ -1,0 +1,226 @@
+"""Dense LoRA linear over a frozen packed GGUF weight:  Y = X W^T + s (X A^T) B^T.
+
+Host-side mirror of the reference's ``fast_lora.py``: the same operator names (``mmq``,
+``mmq_grad_input``, ``supports_native_mmq``) and module surface (``GGUFLinear`` base layer wrapped by
+``FastGGUFLoraLinear`` with ``lora_A`` / ``lora_B`` / ``scaling``), but the base matmul, the LoRA
+residual (``_fused_lora_add``, fast_lora.py:34-65) and the whole backward (dX, dA, dB;
+test_fast_lora.py:101-134) each run as one call into the gfx950 kernel library.  PEFT is not a
+dependency; the wrapper keeps PEFT's attribute names so adapter state dicts line up.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Any
+
+import torch
+
+from . import _lib
+from .gguf import GGML_QUANT_SIZES, GGUFQuantizedTensor, row_bytes
+
+# GGML type ids with native kernels here (the reference's wheel also lists 10, 11, 13, 22:
+# fast_lora.py:24-27; those are not implemented and are rejected, never routed elsewhere).
+_NATIVE_MMQ_QUANT_TYPES = frozenset(GGML_QUANT_SIZES)
+
+
+def supports_native_mmq(weight: Any) -> bool:
+    return int(weight.quant_type) in _NATIVE_MMQ_QUANT_TYPES
+
+
+def _check_packed(payload: torch.Tensor, quant_type: int, rows: int, k: int, what: str) -> None:
+    _lib.require_device_tensor(payload, f"{what} payload", torch.uint8)
+    if quant_type not in _NATIVE_MMQ_QUANT_TYPES:
+        raise ValueError(f"{what}: GGML type id {quant_type} has no native MMQ kernel (supported: {sorted(_NATIVE_MMQ_QUANT_TYPES)})")
+    if payload.ndim != 2 or payload.shape[0] != rows or payload.shape[1] != row_bytes(quant_type, k):
+        raise ValueError(f"{what}: payload shape {tuple(payload.shape)} does not describe a [{rows}, {k}] weight of type {quant_type}")
+    if k % 64:
+        raise ValueError(f"{what}: in_features {k} must be a multiple of 64")
+
+
+def _flat_bf16(x: torch.Tensor, name: str) -> torch.Tensor:
+    _lib.require_device_tensor(x, name, torch.bfloat16)
+    return x.reshape(-1, x.shape[-1])
+
+
+def _mmq_forward(x: torch.Tensor, payload: torch.Tensor, quant_type: int, out_features: int) -> torch.Tensor:
+    x2 = _flat_bf16(x, "mmq input")
+    m, k = x2.shape
+    _check_packed(payload, quant_type, out_features, k, "mmq")
+    y = torch.empty(m, out_features, dtype=torch.bfloat16, device=x.device)
+    if m:
+        _lib.check(_lib.load().ggq_mmq(x2.data_ptr(), payload.data_ptr(), quant_type, m, out_features, k, y.data_ptr(), _lib.stream_handle(x.device)))
+    return y.reshape(*x.shape[:-1], out_features)
+
+
+def mmq_grad_input(grad_output: torch.Tensor, payload: torch.Tensor, quant_type: int, in_features: int) -> torch.Tensor:
+    """dX = dY . W with W decoded to bf16 and fp32 accumulation (no quantization of the cotangent)."""
+    payload = payload.as_subclass(torch.Tensor)
+    quant_type = int(quant_type)
+    g2 = _flat_bf16(grad_output, "mmq_grad_input cotangent")
+    m, n = g2.shape
+    _check_packed(payload, quant_type, n, in_features, "mmq_grad_input")
+    dx = torch.empty(m, in_features, dtype=torch.bfloat16, device=grad_output.device)
+    if m:
+        _lib.check(_lib.load().ggq_mmq_grad_input(g2.data_ptr(), payload.data_ptr(), quant_type, m, n, in_features, dx.data_ptr(), _lib.stream_handle(g2.device)))
+    return dx.reshape(*grad_output.shape[:-1], in_features)
+
+
+class _Mmq(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, payload, quant_type, out_features):
+        ctx.save_for_backward(payload)
+        ctx.quant_type, ctx.in_features = quant_type, x.shape[-1]
+        return _mmq_forward(x, payload, quant_type, out_features)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        if torch.is_grad_enabled():
+            raise RuntimeError("packed MMQ does not support higher-order gradients")
+        (payload,) = ctx.saved_tensors
+        dx = mmq_grad_input(grad_output.contiguous(), payload, ctx.quant_type, ctx.in_features) if ctx.needs_input_grad[0] else None
+        return dx, None, None, None
+
+
+def mmq(x: torch.Tensor, payload: torch.Tensor, quant_type: int, out_features: int) -> torch.Tensor:
+    """Y = X . W^T over packed rows (the reference's ``torch_ggml_ops.mmq``, fast_lora.py:155-160)."""
+    payload = payload.as_subclass(torch.Tensor)
+    return _Mmq.apply(x, payload, int(quant_type), int(out_features))
+
+
+def _workspace(device, rows: int, groups: int, experts: int, n_total: int, k: int, r: int) -> torch.Tensor:
+    nbytes = _lib.load().ggq_lora_workspace_bytes(rows, groups, experts, n_total, k, r)
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+class _LoraMmq(torch.autograd.Function):
+    """Base matmul + LoRA residual in one forward call; dX, dA, dB in one backward call."""
+
+    @staticmethod
+    def forward(ctx, x, payload, quant_type, out_features, lora_a, lora_b, scaling):
+        x2 = _flat_bf16(x, "LoRA linear input")
+        m, k = x2.shape
+        _check_packed(payload, quant_type, out_features, k, "LoRA linear")
+        _lib.require_device_tensor(lora_a, "lora_A", torch.bfloat16)
+        _lib.require_device_tensor(lora_b, "lora_B", torch.bfloat16)
+        r = lora_a.shape[0]
+        if tuple(lora_a.shape) != (r, k) or tuple(lora_b.shape) != (out_features, r):
+            raise ValueError(f"LoRA factors must be A [r,{k}] and B [{out_features},r], got {tuple(lora_a.shape)} and {tuple(lora_b.shape)}")
+        r_pad = (r + 15) // 16 * 16
+        xa = torch.empty(m, r_pad, dtype=torch.bfloat16, device=x.device)
+        y = torch.empty(m, out_features, dtype=torch.bfloat16, device=x.device)
+        if m:
+            ws = _workspace(x.device, m, 0, 1, out_features, k, r)
+            _lib.check(_lib.load().ggq_lora_mmq_forward(
+                x2.data_ptr(), payload.data_ptr(), quant_type, m, out_features, k, lora_a.data_ptr(), lora_b.data_ptr(), r,
+                float(scaling), xa.data_ptr(), y.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_handle(x.device)))
+        ctx.save_for_backward(x2, xa, payload, lora_a, lora_b)
+        ctx.meta = (quant_type, out_features, float(scaling), x.shape)
+        return y.reshape(*x.shape[:-1], out_features)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        if torch.is_grad_enabled():
+            raise RuntimeError("packed MMQ LoRA linear does not support higher-order gradients")
+        x2, xa, payload, lora_a, lora_b = ctx.saved_tensors
+        quant_type, n, scaling, x_shape = ctx.meta
+        g2 = _flat_bf16(grad_output.contiguous(), "LoRA linear cotangent")
+        m, k = x2.shape
+        r = lora_a.shape[0]
+        dx = torch.empty_like(x2)
+        da = torch.empty_like(lora_a) if ctx.needs_input_grad[4] else None
+        db = torch.empty_like(lora_b) if ctx.needs_input_grad[5] else None
+        ws = _workspace(x2.device, m, 0, 1, n, k, r)
+        _lib.check(_lib.load().ggq_lora_mmq_backward(
+            g2.data_ptr(), payload.data_ptr(), quant_type, m, n, k, x2.data_ptr(), xa.data_ptr(), lora_a.data_ptr(),
+            lora_b.data_ptr(), r, scaling, dx.data_ptr(), _lib.ptr(da), _lib.ptr(db), ws.data_ptr(), ws.numel(),
+            _lib.stream_handle(x2.device)))
+        return (dx.reshape(x_shape) if ctx.needs_input_grad[0] else None), None, None, None, da, db, None
+
+
+def lora_mmq(x, payload, quant_type, out_features, lora_a, lora_b, scaling) -> torch.Tensor:
+    return _LoraMmq.apply(x, payload.as_subclass(torch.Tensor), int(quant_type), int(out_features), lora_a, lora_b, float(scaling))
+
+
+def _fused_lora_add(result, x, lora_A: torch.nn.Linear, lora_B: torch.nn.Linear, dropout: torch.nn.Module, scaling: float):
+    """``result + scaling * lora_B(lora_A(dropout(x)))`` with framework ops, for base layers that are
+    not packed (ordinary float linears); same composition as fast_lora.py:34-65."""
+    dt = result.dtype
+    x_a = torch.matmul(dropout(x).to(dt), lora_A.weight.to(dt).transpose(0, 1))
+    shape = result.shape
+    out = torch.addmm(result.reshape(-1, shape[-1]), x_a.reshape(-1, x_a.shape[-1]), lora_B.weight.to(dt).transpose(0, 1), beta=1, alpha=scaling).reshape(shape)
+    if lora_B.bias is not None:
+        out = torch.add(out, lora_B.bias.to(dt), alpha=scaling)
+    return out
+
+
+class GGUFLinear(torch.nn.Module):
+    """Frozen linear layer whose weight stays packed (stand-in for the fork's ``GGUFLinear``; exposes
+    the attributes fast_lora.py:137-162 and gguf_liger_loss.py:305-324 read)."""
+
+    def __init__(self, in_features: int, out_features: int, weight: GGUFQuantizedTensor, bias: torch.Tensor | None = None,
+                 compute_dtype: torch.dtype = torch.bfloat16):
+        super().__init__()
+        if tuple(weight.logical_shape) != (out_features, in_features):
+            raise ValueError(f"weight logical shape {weight.logical_shape} != ({out_features}, {in_features})")
+        self.in_features, self.out_features = in_features, out_features
+        self.weight = weight
+        self.bias = bias
+        self.compute_dtype = compute_dtype
+        self.input_permutation = None
+        self.output_permutation = None
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self.compute_dtype != torch.bfloat16:
+            raise RuntimeError("The packed GGUF MMQ linear path requires BF16 compute_dtype.")
+        y = mmq(x, self.weight, self.weight.quant_type, self.out_features)
+        if self.bias is not None:
+            y = y + self.bias.to(device=y.device, dtype=y.dtype)
+        return y
+
+
+class FastGGUFLoraLinear(torch.nn.Module):
+    """LoRA wrapper for a frozen packed ``GGUFLinear`` (counterpart of fast_lora.py:127-175).
+
+    One adapter, no dropout, no DoRA: the configurations the reference's fast path accepts
+    (fast_lora.py:82-94); anything else is rejected rather than served by a slower route."""
+
+    def __init__(self, base_layer: GGUFLinear, r: int, lora_alpha: float, adapter_name: str = "default",
+                 use_rslora: bool = False, lora_dropout: float = 0.0):
+        super().__init__()
+        if r <= 0 or r > 64:
+            raise ValueError(f"LoRA rank must be in 1..64, got {r}")
+        if lora_dropout != 0.0:
+            raise ValueError("the packed LoRA linear requires lora_dropout=0")
+        if not isinstance(base_layer.weight, GGUFQuantizedTensor) or not supports_native_mmq(base_layer.weight):
+            raise TypeError("FastGGUFLoraLinear requires a packed weight of a natively supported GGML type")
+        if base_layer.input_permutation is not None or base_layer.output_permutation is not None:
+            raise RuntimeError("the packed GGUF MMQ linear path does not support layout permutations")
+        self.base_layer = base_layer
+        dev, dt = base_layer.weight.device, base_layer.compute_dtype
+        self.lora_A = torch.nn.ModuleDict({adapter_name: torch.nn.Linear(base_layer.in_features, r, bias=False, device=dev, dtype=dt)})
+        self.lora_B = torch.nn.ModuleDict({adapter_name: torch.nn.Linear(r, base_layer.out_features, bias=False, device=dev, dtype=dt)})
+        torch.nn.init.kaiming_uniform_(self.lora_A[adapter_name].weight, a=math.sqrt(5))
+        torch.nn.init.zeros_(self.lora_B[adapter_name].weight)
+        self.scaling = {adapter_name: lora_alpha / (math.sqrt(r) if use_rslora else r)}
+        self.active_adapter = adapter_name
+        self.disable_adapters = False
+
+    def forward(self, x: torch.Tensor, *args: Any, **kwargs: Any) -> torch.Tensor:
+        if args or kwargs:
+            raise TypeError("The packed GGUF MMQ linear path accepts only its input tensor.")
+        base = self.base_layer
+        if base.compute_dtype != torch.bfloat16:
+            raise RuntimeError("The packed GGUF MMQ linear path requires BF16 compute_dtype.")
+        if self.disable_adapters:
+            return base(x)
+        name = self.active_adapter
+        y = lora_mmq(x, base.weight, base.weight.quant_type, base.out_features, self.lora_A[name].weight, self.lora_B[name].weight, self.scaling[name])
+        if base.bias is not None:
+            y = y + base.bias.to(device=y.device, dtype=y.dtype)
+        return y
+
+    def merge(self, *args: Any, **kwargs: Any) -> None:
+        raise RuntimeError("GGUF LoRA adapters cannot be merged into packed base weights.")
+
+    def unmerge(self) -> None:
+        raise RuntimeError("GGUF LoRA adapters cannot be unmerged because merging is unsupported.")

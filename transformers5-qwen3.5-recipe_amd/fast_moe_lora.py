@@ -1,0 +1,371 @@
+"""Grouped-expert MoE LoRA over frozen packed GGUF expert weights.
+
+Host-side mirror of the reference's ``fast_moe_lora.py``.  Operator names follow the reference's native
+boundary (``grouped_mmq``, ``grouped_mmq_pair`` and their ``_grad_input`` twins, fast_moe_lora.py:221,
+255, 339, 364); the expert-layer forward keeps its structure (route -> gate/up pair -> SiLU gate -> down
+-> combine, fast_moe_lora.py:685-770).  What differs is the fusion: the per-expert LoRA delta that the
+reference computes with separate AITER grouped GEMMs (fast_moe_lora.py:42-151, 675-682) is folded into
+the packed-weight kernels, so each projection is one forward call (base + s (x A^T) B^T) and one backward
+call (dX plus dA, dB for all expert planes, zeros for experts without rows).
+
+Expert groups are passed as ``expert_indices`` (int64) and cumulative END ``expert_offsets`` (int32), as
+in the reference (test_fast_moe_lora.py:136-137).  The layer itself uses the full list of experts with
+the device-computed offsets, so no host synchronisation is needed to learn which experts are active.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Any
+
+import torch
+
+from . import _lib
+from .fast_lora import _NATIVE_MMQ_QUANT_TYPES, supports_native_mmq
+from .fast_moe_routing import ExpertRoutingPlan, finalize_expert_routing, prepare_expert_routing
+from .gguf import GGUFQuantizedTensor, row_bytes
+
+EXPERTS_IMPLEMENTATION = "qwen3_5_moe_gguf_mmq_lora"
+
+
+# ------------------------------------------------------------------------------------------------
+def _check_grouped(x, payload, expert_indices, expert_offsets, quant_type, n, k, what):
+    _lib.require_device_tensor(x, f"{what} rows", torch.bfloat16)
+    _lib.require_device_tensor(payload, f"{what} payload", torch.uint8)
+    _lib.require_device_tensor(expert_indices, f"{what} expert_indices", torch.int64)
+    _lib.require_device_tensor(expert_offsets, f"{what} expert_offsets", torch.int32)
+    if quant_type not in _NATIVE_MMQ_QUANT_TYPES:
+        raise ValueError(f"{what}: GGML type id {quant_type} has no native grouped MMQ kernel")
+    if x.ndim != 2 or payload.ndim != 3 or expert_indices.ndim != 1 or expert_offsets.shape != expert_indices.shape:
+        raise ValueError(f"{what}: expects rows [R,K], payload [E,N,bytes], expert_indices [G] and expert_offsets [G]")
+    if payload.shape[1] != n or payload.shape[2] != row_bytes(quant_type, k):
+        raise ValueError(f"{what}: payload shape {tuple(payload.shape)} does not describe [E,{n},{k}] of type {quant_type}")
+    if k % 64:
+        raise ValueError(f"{what}: in_features {k} must be a multiple of 64")
+
+
+def _lora_ws(device, rows, groups, experts, n_total, k, r):
+    nbytes = _lib.load().ggq_lora_workspace_bytes(rows, groups, experts, n_total, k, max(r, 1))
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+def _grouped_forward(x, p1, p2, expert_indices, expert_offsets, quant_type, n, lora_a, lora_b, scaling):
+    rows, k = x.shape
+    experts = p1.shape[0]
+    _check_grouped(x, p1, expert_indices, expert_offsets, quant_type, n, k, "grouped_mmq")
+    if p2 is not None:
+        if p2.shape != p1.shape:
+            raise RuntimeError("Paired grouped GGUF MMQ requires matching logical shapes.")
+        _lib.require_device_tensor(p2, "grouped_mmq second payload", torch.uint8)
+    nseg = 1 if p2 is None else 2
+    r = 0
+    xa = None
+    if lora_a is not None:
+        _lib.require_device_tensor(lora_a, "expert lora_A", torch.bfloat16)
+        _lib.require_device_tensor(lora_b, "expert lora_B", torch.bfloat16)
+        r = lora_a.shape[1]
+        if tuple(lora_a.shape) != (experts, r, k) or tuple(lora_b.shape) != (experts, nseg * n, r):
+            raise ValueError(f"expert LoRA factors must be A [{experts},r,{k}] and B [{experts},{nseg * n},r], got {tuple(lora_a.shape)}, {tuple(lora_b.shape)}")
+        xa = torch.empty(rows, (r + 15) // 16 * 16, dtype=torch.bfloat16, device=x.device)
+    y1 = torch.empty(rows, n, dtype=torch.bfloat16, device=x.device)
+    y2 = torch.empty(rows, n, dtype=torch.bfloat16, device=x.device) if p2 is not None else None
+    if rows:
+        ws = _lora_ws(x.device, rows, expert_indices.numel(), experts, nseg * n, k, r)
+        _lib.check(_lib.load().ggq_grouped_lora_mmq_forward(
+            x.data_ptr(), p1.data_ptr(), _lib.ptr(p2), expert_indices.data_ptr(), expert_offsets.data_ptr(), expert_indices.numel(),
+            experts, quant_type, rows, n, k, _lib.ptr(lora_a), _lib.ptr(lora_b), r, float(scaling), _lib.ptr(xa), y1.data_ptr(),
+            _lib.ptr(y2), ws.data_ptr(), ws.numel(), _lib.stream_handle(x.device)))
+    return y1, y2, xa
+
+
+def _grouped_backward(dy1, dy2, p1, p2, expert_indices, expert_offsets, quant_type, k, x, xa, lora_a, lora_b, scaling, want_da, want_db):
+    rows, n = dy1.shape
+    experts = p1.shape[0]
+    _check_grouped(dy1, p1, expert_indices, expert_offsets, quant_type, n, k, "grouped_mmq_grad_input")
+    nseg = 1 if p2 is None else 2
+    if p2 is not None:
+        _lib.require_device_tensor(dy2, "grouped_mmq_grad_input second cotangent", torch.bfloat16)
+    r = 0 if lora_a is None else lora_a.shape[1]
+    dx = torch.empty(rows, k, dtype=torch.bfloat16, device=dy1.device)
+    da = torch.empty_like(lora_a) if (lora_a is not None and want_da) else None
+    db = torch.empty_like(lora_b) if (lora_b is not None and want_db) else None
+    ws = _lora_ws(dy1.device, rows, expert_indices.numel(), experts, nseg * n, k, r)
+    _lib.check(_lib.load().ggq_grouped_lora_mmq_backward(
+        dy1.data_ptr(), _lib.ptr(dy2), p1.data_ptr(), _lib.ptr(p2), expert_indices.data_ptr(), expert_offsets.data_ptr(),
+        expert_indices.numel(), experts, quant_type, rows, n, k, _lib.ptr(x), _lib.ptr(xa), _lib.ptr(lora_a), _lib.ptr(lora_b), r,
+        float(scaling), dx.data_ptr(), _lib.ptr(da), _lib.ptr(db), ws.data_ptr(), ws.numel(), _lib.stream_handle(dy1.device)))
+    return dx, da, db
+
+
+def grouped_mmq_grad_input(grad_output, payload, expert_indices, expert_offsets, quant_type, in_features):
+    """dX[r0:r1] = dY[r0:r1] . W[expert] per group (fast_moe_lora.py:255-262)."""
+    payload = payload.as_subclass(torch.Tensor)
+    dx, _, _ = _grouped_backward(grad_output, None, payload, None, expert_indices, expert_offsets, int(quant_type), int(in_features),
+                                 None, None, None, None, 0.0, False, False)
+    return dx
+
+
+def grouped_mmq_pair_grad_input(first_grad, second_grad, first_payload, second_payload, expert_indices, expert_offsets, quant_type, in_features):
+    """dX = dY1 . W1 + dY2 . W2 in one fp32 accumulator, rounded once (fast_moe_lora.py:364-375)."""
+    dx, _, _ = _grouped_backward(first_grad, second_grad, first_payload.as_subclass(torch.Tensor), second_payload.as_subclass(torch.Tensor),
+                                 expert_indices, expert_offsets, int(quant_type), int(in_features), None, None, None, None, 0.0, False, False)
+    return dx
+
+
+class _GroupedLoraProjection(torch.autograd.Function):
+    """One expert projection (or a gate/up pair) with the LoRA delta fused in."""
+
+    @staticmethod
+    def forward(ctx, x, p1, p2, expert_indices, expert_offsets, quant_type, n, lora_a, lora_b, scaling):
+        y1, y2, xa = _grouped_forward(x, p1, p2, expert_indices, expert_offsets, quant_type, n, lora_a, lora_b, scaling)
+        tensors = [x, expert_indices, expert_offsets, p1]
+        ctx.has_pair, ctx.has_lora = p2 is not None, lora_a is not None
+        if ctx.has_pair:
+            tensors.append(p2)
+        if ctx.has_lora:
+            tensors += [xa, lora_a, lora_b]
+        ctx.save_for_backward(*tensors)
+        ctx.meta = (quant_type, n, float(scaling))
+        if ctx.has_pair:
+            return y1, y2
+        return y1
+
+    @staticmethod
+    def backward(ctx, *grads):
+        if torch.is_grad_enabled():
+            raise RuntimeError("packed grouped MMQ does not support higher-order gradients")
+        saved = list(ctx.saved_tensors)
+        x, expert_indices, expert_offsets, p1 = saved[:4]
+        rest = saved[4:]
+        p2 = rest.pop(0) if ctx.has_pair else None
+        xa, lora_a, lora_b = rest if ctx.has_lora else (None, None, None)
+        quant_type, n, scaling = ctx.meta
+        g1 = grads[0]
+        g2 = grads[1] if ctx.has_pair else None
+        if ctx.has_pair and (g1 is None or g2 is None):
+            if g1 is None and g2 is None:
+                return (None,) * 10
+            like = g1 if g1 is not None else g2
+            g1 = torch.zeros_like(like) if g1 is None else g1
+            g2 = torch.zeros_like(like) if g2 is None else g2
+        g1 = g1.contiguous()
+        g2 = g2.contiguous() if g2 is not None else None
+        want_da, want_db = ctx.needs_input_grad[7], ctx.needs_input_grad[8]
+        dx, da, db = _grouped_backward(g1, g2, p1, p2, expert_indices, expert_offsets, quant_type, x.shape[1], x, xa, lora_a, lora_b,
+                                       scaling, want_da, want_db)
+        return (dx if ctx.needs_input_grad[0] else None), None, None, None, None, None, None, da, db, None
+
+
+def _as_payload(w):
+    return w.as_subclass(torch.Tensor) if w is not None else None
+
+
+def grouped_mmq(hidden_states, payload, expert_indices, expert_offsets, quant_type, out_features):
+    """Y[r0:r1] = X[r0:r1] . W[expert]^T per group (fast_moe_lora.py:221-228); differentiable in X."""
+    return _GroupedLoraProjection.apply(hidden_states, _as_payload(payload), None, expert_indices, expert_offsets, int(quant_type),
+                                        int(out_features), None, None, 0.0)
+
+
+def grouped_mmq_pair(hidden_states, first_payload, second_payload, expert_indices, expert_offsets, quant_type, out_features):
+    """(gate, up) from one pass over X (fast_moe_lora.py:339-347); differentiable in X."""
+    return _GroupedLoraProjection.apply(hidden_states, _as_payload(first_payload), _as_payload(second_payload), expert_indices,
+                                        expert_offsets, int(quant_type), int(out_features), None, None, 0.0)
+
+
+def grouped_lora_mmq(hidden_states, payload, expert_indices, expert_offsets, quant_type, out_features, lora_a, lora_b, scaling):
+    return _GroupedLoraProjection.apply(hidden_states, _as_payload(payload), None, expert_indices, expert_offsets, int(quant_type),
+                                        int(out_features), lora_a, lora_b, float(scaling))
+
+
+def grouped_lora_mmq_pair(hidden_states, first_payload, second_payload, expert_indices, expert_offsets, quant_type, out_features,
+                          lora_a, lora_b, scaling):
+    return _GroupedLoraProjection.apply(hidden_states, _as_payload(first_payload), _as_payload(second_payload), expert_indices,
+                                        expert_offsets, int(quant_type), int(out_features), lora_a, lora_b, float(scaling))
+
+
+class _SwiGLU(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, gate, up):
+        _lib.require_device_tensor(gate, "gate", torch.bfloat16)
+        _lib.require_device_tensor(up, "up", torch.bfloat16)
+        h = torch.empty_like(gate)
+        _lib.check(_lib.load().ggq_swiglu_forward(gate.data_ptr(), up.data_ptr(), h.data_ptr(), gate.numel(), _lib.stream_handle(gate.device)))
+        ctx.save_for_backward(gate, up)
+        return h
+
+    @staticmethod
+    def backward(ctx, dh):
+        gate, up = ctx.saved_tensors
+        dh = dh.contiguous()
+        dgate, dup = torch.empty_like(gate), torch.empty_like(up)
+        _lib.check(_lib.load().ggq_swiglu_backward(gate.data_ptr(), up.data_ptr(), dh.data_ptr(), dgate.data_ptr(), dup.data_ptr(),
+                                                   gate.numel(), _lib.stream_handle(gate.device)))
+        return dgate, dup
+
+
+def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """silu(gate) * up (the fork's ``_apply_split_gate`` for ``hidden_act="silu"``, fast_moe_lora.py:747)."""
+    return _SwiGLU.apply(gate, up)
+
+
+# ------------------------------------------------------------------------------------------------
+def _group_sizes_from_offsets(offsets: torch.Tensor) -> torch.Tensor:
+    if offsets.ndim != 1:
+        raise ValueError(f"GGUF grouped execution requires one-dimensional offsets, got {offsets.shape}.")
+    if offsets.dtype != torch.int32 or offsets.stride() != (1,):
+        raise ValueError("GGUF grouped offsets must be contiguous int32.")
+    return torch.diff(offsets, prepend=offsets.new_zeros(1))
+
+
+def _complete_group_sizes(active_group_sizes: torch.Tensor, expert_indices: torch.Tensor, num_experts: int) -> torch.Tensor:
+    if expert_indices.numel() == num_experts:
+        return active_group_sizes
+    return active_group_sizes.new_zeros(num_experts).index_copy(0, expert_indices, active_group_sizes)
+
+
+@dataclass(frozen=True)
+class _ExpertLoraWeights:
+    gate_up_a: torch.Tensor  # [experts, rank, hidden]
+    gate_up_b: torch.Tensor  # [experts, 2 * intermediate, rank]
+    down_a: torch.Tensor     # [experts, rank, intermediate]
+    down_b: torch.Tensor     # [experts, hidden, rank]
+    scaling: float
+
+
+@dataclass(frozen=True)
+class _ExpertExecutionPlan:
+    expert_indices: torch.Tensor
+    offsets: torch.Tensor
+    output_mask: torch.Tensor | None = None
+
+
+class GGUFExperts(torch.nn.Module):
+    """Packed expert weights of one MoE layer (stand-in for the fork's ``GGUFExperts``; exposes what
+    fast_moe_lora.py:541-545, 698-709, 747 reads)."""
+
+    projection_layout = "split_gate_up"
+    has_bias = False
+    has_gate = True
+
+    def __init__(self, gate_proj: GGUFQuantizedTensor, up_proj: GGUFQuantizedTensor, down_proj: GGUFQuantizedTensor,
+                 compute_dtype: torch.dtype = torch.bfloat16):
+        super().__init__()
+        e, i, h = gate_proj.logical_shape
+        if tuple(up_proj.logical_shape) != (e, i, h) or tuple(down_proj.logical_shape) != (e, h, i):
+            raise ValueError("expert projections must be gate/up [E,I,H] and down [E,H,I]")
+        self.gate_proj, self.up_proj, self.down_proj = gate_proj, up_proj, down_proj
+        self.num_experts, self.hidden_dim, self.intermediate_dim = e, h, i
+        self.compute_dtype = compute_dtype
+        self._all_experts = torch.arange(e, dtype=torch.int64, device=gate_proj.device)
+
+    def _prepare_expert_hidden_states(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        return hidden_states.reshape(-1, self.hidden_dim).to(self.compute_dtype).contiguous()
+
+    def _prepare_expert_execution(self, routing_plan: ExpertRoutingPlan, mode: str) -> _ExpertExecutionPlan:
+        if mode != "grouped_mm":
+            raise RuntimeError(f"unsupported expert execution mode {mode!r}")
+        return _ExpertExecutionPlan(self._all_experts, routing_plan.expert_end_offsets, None)
+
+    def _apply_split_gate(self, gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+        return swiglu(gate, up)
+
+    def forward(self, hidden_states, top_k_index, top_k_weights, lora_weights: _ExpertLoraWeights | None = None):
+        return qwen3_5_moe_gguf_mmq_lora_forward(self, hidden_states, top_k_index, top_k_weights, lora_weights)
+
+
+def qwen3_5_moe_gguf_mmq_lora_forward(self: GGUFExperts, hidden_states: torch.Tensor, top_k_index: torch.Tensor,
+                                      top_k_weights: torch.Tensor, lora_weights: _ExpertLoraWeights | None = None) -> torch.Tensor:
+    """Packed expert FFN with LoRA on gate/up and down (orchestration of fast_moe_lora.py:685-770)."""
+    if not isinstance(self, GGUFExperts):
+        raise TypeError(f"{EXPERTS_IMPLEMENTATION} requires GGUFExperts, got {type(self).__name__}.")
+    if self.projection_layout != "split_gate_up" or self.has_bias or not self.has_gate:
+        raise RuntimeError("The GGUF LoRA path requires split, bias-free gate/up expert projections.")
+    for w in (self.gate_proj, self.up_proj, self.down_proj):
+        if w.requires_grad:
+            raise RuntimeError("Fast GGUF expert execution requires frozen packed base weights.")
+        if not supports_native_mmq(w):
+            raise RuntimeError(f"GGML type id {w.quant_type} has no native grouped MMQ kernel.")
+    if self.compute_dtype != torch.bfloat16:
+        raise RuntimeError("Grouped GGUF MMQ requires BF16 compute dtype.")
+    if self.gate_proj.quant_type != self.up_proj.quant_type:
+        raise RuntimeError("Paired grouped GGUF MMQ requires one quantization type.")
+
+    compute_hidden_states = self._prepare_expert_hidden_states(hidden_states)
+    routing_plan = prepare_expert_routing(compute_hidden_states, top_k_index, top_k_weights, self.num_experts)
+    execution_plan = self._prepare_expert_execution(routing_plan, "grouped_mm")
+    if execution_plan.offsets is None:
+        raise RuntimeError("GGUF LoRA requires grouped expert offsets.")
+    selected = routing_plan.selected_hidden_states
+    expert_indices, expert_offsets = execution_plan.expert_indices, execution_plan.offsets
+    lw = lora_weights
+    s = lw.scaling if lw is not None else 0.0
+
+    gate, up = _GroupedLoraProjection.apply(
+        selected, _as_payload(self.gate_proj), _as_payload(self.up_proj), expert_indices, expert_offsets,
+        int(self.gate_proj.quant_type), self.intermediate_dim, lw.gate_up_a if lw else None, lw.gate_up_b if lw else None, s)
+    intermediate = self._apply_split_gate(gate, up)
+    output = _GroupedLoraProjection.apply(
+        intermediate, _as_payload(self.down_proj), None, expert_indices, expert_offsets, int(self.down_proj.quant_type),
+        self.hidden_dim, lw.down_a if lw else None, lw.down_b if lw else None, s)
+    return finalize_expert_routing(output, hidden_states, routing_plan, execution_plan.output_mask).reshape(hidden_states.shape)
+
+
+class FastGGUFMoeLora(torch.nn.Module):
+    """LoRA wrapper owning the four factor families of one packed ``GGUFExperts`` module
+    (counterpart of fast_moe_lora.py:482-646; same parameter names and shapes)."""
+
+    adapter_layer_names = ("lora_A", "lora_B", "lora_A_down", "lora_B_down")
+
+    def __init__(self, base_layer: GGUFExperts, adapter_name: str = "default", *, r: int, lora_alpha: float,
+                 use_rslora: bool = False, lora_dropout: float = 0.0, init_lora_weights: bool | str = True):
+        super().__init__()
+        if not isinstance(base_layer, GGUFExperts):
+            raise TypeError(f"Fast GGUF MoE LoRA requires GGUFExperts, got {type(base_layer).__name__}.")
+        if r <= 0 or r > 64:
+            raise ValueError(f"LoRA rank must be in 1..64, got {r}.")
+        if lora_dropout != 0.0:
+            raise ValueError("Fast GGUF MoE LoRA currently requires lora_dropout=0.")
+        self.base_layer = base_layer
+        e, h, i = base_layer.num_experts, base_layer.hidden_dim, base_layer.intermediate_dim
+        dev, dt = base_layer.gate_proj.device, base_layer.compute_dtype
+
+        def factor(shape):
+            return torch.nn.Parameter(torch.empty(shape, device=dev, dtype=dt))
+
+        self.lora_A = torch.nn.ParameterDict({adapter_name: factor((e, r, h))})
+        self.lora_B = torch.nn.ParameterDict({adapter_name: factor((e, 2 * i, r))})
+        self.lora_A_down = torch.nn.ParameterDict({adapter_name: factor((e, r, i))})
+        self.lora_B_down = torch.nn.ParameterDict({adapter_name: factor((e, h, r))})
+        self.scaling = {adapter_name: lora_alpha / (math.sqrt(r) if use_rslora else r)}
+        self.active_adapter = adapter_name
+        self.disable_adapters = False
+        if init_lora_weights is True:
+            torch.nn.init.kaiming_uniform_(self.lora_A[adapter_name], a=math.sqrt(5))
+            torch.nn.init.kaiming_uniform_(self.lora_A_down[adapter_name], a=math.sqrt(5))
+        elif init_lora_weights == "gaussian":
+            torch.nn.init.normal_(self.lora_A[adapter_name], std=1 / r)
+            torch.nn.init.normal_(self.lora_A_down[adapter_name], std=1 / r)
+        elif init_lora_weights is not False:
+            raise ValueError(f"Fast GGUF MoE LoRA does not support init_lora_weights={init_lora_weights!r}.")
+        if init_lora_weights is not False:
+            torch.nn.init.zeros_(self.lora_B[adapter_name])
+            torch.nn.init.zeros_(self.lora_B_down[adapter_name])
+
+    def _active_lora_weights(self) -> _ExpertLoraWeights | None:
+        if self.disable_adapters:
+            return None
+        n = self.active_adapter
+        return _ExpertLoraWeights(self.lora_A[n], self.lora_B[n], self.lora_A_down[n], self.lora_B_down[n], float(self.scaling[n]))
+
+    def forward(self, hidden_states: torch.Tensor, top_k_index: torch.Tensor, top_k_weights: torch.Tensor) -> torch.Tensor:
+        return self.base_layer(hidden_states, top_k_index, top_k_weights, self._active_lora_weights())
+
+    def merge(self, *args: Any, **kwargs: Any) -> None:
+        raise RuntimeError("GGUF expert LoRA adapters cannot be merged into packed base weights.")
+
+    def unmerge(self) -> None:
+        raise RuntimeError("GGUF expert LoRA adapters cannot be unmerged because merging is unsupported.")
+
+    def get_delta_weight(self, *args: Any, **kwargs: Any) -> torch.Tensor:
+        raise RuntimeError("GGUF expert LoRA does not materialize a full expert delta weight.")
