@@ -32,6 +32,14 @@ extern "C" {
 
 const char* ggq_last_error(void);
 
+/* Kernel timing aid (the reference profiles with Kineto module ranges, deepseek_v4_profiler.py:39-74):
+ * between begin and end every launch of the packed-weight tile kernel is bracketed by HIP events on
+ * its stream.  ggq_profile_end synchronises on them and fills host arrays (milliseconds, GGML type id,
+ * mode 0 = forward / 1 = grad-input, epilogue id) for up to `capacity` launches; returns the number
+ * written or a negative error.  Not thread safe; at most 8192 launches are recorded. */
+int ggq_profile_begin(void);
+int ggq_profile_end(float* ms, int* qt, int* mode, int* epilogue, int capacity);
+
 /* fast_lora.py:24-31 (_NATIVE_MMQ_QUANT_TYPES / supports_native_mmq): 1 if this library has kernels
  * for the GGML type id. */
 int ggq_supports_quant_type(int qt);

@@ -21,6 +21,8 @@ _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
 # name -> (restype, argtypes); must list every symbol include/ggml_mmq_gfx950.h declares.
 SIGNATURES: dict[str, tuple] = {
     "ggq_last_error": (c_char_p, []),
+    "ggq_profile_begin": (_I, []),
+    "ggq_profile_end": (_I, [_P, _P, _P, _P, _I]),
     "ggq_supports_quant_type": (_I, [_I]),
     "ggq_row_bytes": (_L, [_I, _L]),
     "ggq_dequantize": (_I, [_I, _P, _L, _L, _P, _I, _P]),

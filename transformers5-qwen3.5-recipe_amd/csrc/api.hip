@@ -45,6 +45,13 @@ extern "C" {
 
 const char* ggq_last_error(void) { return last_error(); }
 
+int ggq_profile_begin(void) { return profile_begin(); }
+
+int ggq_profile_end(float* ms, int* qt, int* mode, int* epilogue, int capacity) {
+    if (!ms || !qt || !mode || !epilogue) return set_error(GGQ_ERR_NULL, "profile_end: null pointer");
+    return profile_end(ms, qt, mode, epilogue, capacity);
+}
+
 int ggq_supports_quant_type(int qt) { return packed_row_bytes(qt, 256) > 0 ? 1 : 0; }
 
 int64_t ggq_row_bytes(int qt, int64_t k) { return block_multiple(qt, k) ? packed_row_bytes(qt, k) : -1; }

@@ -80,6 +80,36 @@ int build_row_tiles(const int64_t* expert_ids, const int32_t* end_offsets, int g
 }
 
 // ------------------------------------------------------------------------------------------------
+// Optional per-launch timing of the tile kernel with HIP events on the launch stream (off by default).
+struct TimedLaunch {
+    hipEvent_t start, stop;
+    int qt, mode, epi;
+};
+static TimedLaunch g_timed[kMaxTimedLaunches];
+static int g_timed_count = 0;
+static bool g_timing = false;
+
+int profile_begin() {
+    g_timed_count = 0;
+    g_timing = true;
+    return GGQ_OK;
+}
+
+int profile_end(float* ms, int* qt, int* mode, int* epi, int capacity) {
+    g_timing = false;
+    int n = 0;
+    for (int i = 0; i < g_timed_count; i++) {
+        float t = 0.f;
+        if (hipEventSynchronize(g_timed[i].stop) != hipSuccess || hipEventElapsedTime(&t, g_timed[i].start, g_timed[i].stop) != hipSuccess)
+            return set_error(GGQ_ERR_RUNTIME, "profile_end: event query failed");
+        if (n < capacity) ms[n] = t, qt[n] = g_timed[i].qt, mode[n] = g_timed[i].mode, epi[n] = g_timed[i].epi, n++;
+        (void)hipEventDestroy(g_timed[i].start);
+        (void)hipEventDestroy(g_timed[i].stop);
+    }
+    g_timed_count = 0;
+    return n;
+}
+
 template <int QT, int MODE, int EPI>
 static int launch_one(const MmqParams& p, hipStream_t s) {
     const int col_tiles = (MODE == kModeNT ? p.nseg : 1) * p.col_tiles_per_seg;
@@ -87,7 +117,16 @@ static int launch_one(const MmqParams& p, hipStream_t s) {
     if (total <= 0) return GGQ_OK;
     const int64_t grid = (total + 7) / 8 * 8;  // the XCD remap inside the kernel needs a multiple of 8
     if (grid > 0x7FFFFFF0) return set_error(GGQ_ERR_SHAPE, "mmq: too many tiles for one launch");
+    TimedLaunch* t = nullptr;
+    if (g_timing && g_timed_count < kMaxTimedLaunches) {
+        t = &g_timed[g_timed_count];
+        if (hipEventCreate(&t->start) != hipSuccess || hipEventCreate(&t->stop) != hipSuccess) return set_error(GGQ_ERR_RUNTIME, "mmq: event creation failed");
+        t->qt = QT, t->mode = MODE, t->epi = EPI;
+        g_timed_count++;
+        (void)hipEventRecord(t->start, s);
+    }
     hipLaunchKernelGGL((mmq_tile_kernel<QT, MODE, EPI>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+    if (t) (void)hipEventRecord(t->stop, s);
     return check_launch("mmq_tile_kernel");
 }
 

@@ -78,6 +78,9 @@ struct MmqParams {
     int64_t ignore_index;
 };
 
+constexpr int kMaxTimedLaunches = 8192;
+int profile_begin();
+int profile_end(float* ms, int* qt, int* mode, int* epi, int capacity);
 const char* last_error();
 int launch_mmq(int qt, int mode, int epi, const MmqParams& p, hipStream_t s);
 int init_params(MmqParams& p, int qt, int mode, int m, int n, int k, int nseg);
