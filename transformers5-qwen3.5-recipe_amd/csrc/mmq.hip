@@ -125,7 +125,14 @@ static int launch_one(const MmqParams& p, hipStream_t s) {
         g_timed_count++;
         (void)hipEventRecord(t->start, s);
     }
-    hipLaunchKernelGGL((mmq_tile_kernel<QT, MODE, EPI>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+    constexpr int kSmemBytes = 2 * (kBM + kBN) * kLdsStride * 2 + (QT == kIQ2_XXS ? 2048 : 0);
+    static bool attr_set = false;  // per instantiation; the attribute is a property of the function
+    if (!attr_set) {
+        if (hipFuncSetAttribute((const void*)mmq_tile_kernel<QT, MODE, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess)
+            return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", kSmemBytes);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((mmq_tile_kernel<QT, MODE, EPI>), dim3((unsigned)grid), dim3(kThreads), kSmemBytes, s, p);
     if (t) (void)hipEventRecord(t->stop, s);
     return check_launch("mmq_tile_kernel");
 }

@@ -34,9 +34,9 @@ struct FactorGradParams {
     float scale;
 };
 
-constexpr int kBM = 128, kBN = 256, kBK = 64;
+constexpr int kBM = 256, kBN = 128, kBK = 64;
 constexpr int kLdsStride = kBK + 8;  // bf16 elements per LDS row: 144 bytes keeps 128-bit reads conflict-free
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;  // waves 0..3 run the MFMAs, waves 4..7 load and decode
 
 enum : int { kModeNT = 0, kModeNN = 1 };
 enum : int {
