@@ -125,7 +125,7 @@ static int launch_one(const MmqParams& p, hipStream_t s) {
         g_timed_count++;
         (void)hipEventRecord(t->start, s);
     }
-    constexpr int kSmemBytes = 2 * (kBM + kBN) * kLdsStride * 2 + (QT == kIQ2_XXS ? 2048 : 0);
+    constexpr int kSmemBytes = kTileLdsBytes + (QT == kIQ2_XXS ? 2048 : 0);
     static bool attr_set = false;  // per instantiation; the attribute is a property of the function
     if (!attr_set) {
         if (hipFuncSetAttribute((const void*)mmq_tile_kernel<QT, MODE, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess)

@@ -10,16 +10,18 @@
 // One workgroup = 512 lanes (8 waves) computes a 256 x 128 tile of C: tall, because every decoded
 // weight is reused by all rows of the tile and an expert's rows (about 128 on average in the MoE
 // shapes this is built for) should fit one tile.  The waves are specialised; per contraction step of 64
-//   * producer waves 4..7 move the A tile (up to 256 x 64 bf16) global -> registers -> LDS with 128-bit
-//     accesses (32-row slabs past the end of the group are skipped), and each producer lane loads the
-//     packed bytes of one 32-element run of one W row, unpacks scales/mins/codebook in registers
-//     (blocks.h) and writes bf16 into the LDS W tile laid out [output column][contraction]; in NN mode
-//     that write is the transposition (2-byte stores, the 64 lanes of a wave = 64 consecutive
-//     contraction rows).  Global loads run one step ahead of the LDS fill;
 //   * consumer waves 0..3 (2 x 2) each own four 32-row blocks (interleaved: block 2*i + wave_m, so
-//     short groups load both wave rows evenly) x two 32-column blocks of MFMA 32x32x16 accumulators
-//     and run the MFMAs of the previous step out of the other LDS buffer; the whole consumer path is
-//     instantiated per number of live row blocks, so ragged groups issue no MFMA on empty blocks.
+//     short groups load both wave rows evenly) x two 32-column blocks of MFMA 32x32x16 accumulators;
+//     the whole consumer path is instantiated per number of live row blocks, so ragged groups issue no
+//     MFMA on empty blocks.  They also move the A tile: global -> LDS directly (no registers), 1 KB =
+//     8 rows x 128 bytes per wave instruction, two steps ahead of the MFMAs through a ring of three
+//     LDS stages; 8-row groups past the end of the expert group are skipped.  A rows sit unpadded in
+//     LDS with their 16-byte slots XOR-swizzled so that both the 1 KB writes and the MFMA operand
+//     reads are bank-conflict free;
+//   * producer waves 4..7 own the weights: packed bytes global -> registers (each cache line fetched
+//     once: for Q4_K forward a lane keeps its share of a whole 256-wide block in registers for four
+//     steps), scales / mins / codebook unpacked in registers (blocks.h), bf16 written into the LDS W
+//     tile laid out [output column][contraction]; in NN mode that write is the transposition.
 // One barrier per step hands the buffers over; decode VALU work and MFMA work overlap on every SIMD.
 #pragma once
 #include "blocks.h"
@@ -32,21 +34,44 @@ namespace ggq {
 
 static __device__ const uint64_t d_iq2xxs_grid_mm[256] = GGQ_IQ2XXS_GRID_INIT;
 
-constexpr int kRowBlocks = kBM / 64;  // 32-row MFMA blocks per consumer wave (4)
-constexpr int kColBlocks = kBN / 64;  // 32-column MFMA blocks per consumer wave (2)
-constexpr int kASlabs = kBM / 32;     // A-tile load slabs of 32 rows (one uint4 per producer lane each)
-constexpr int kATile = kBM * kLdsStride, kBTile = kBN * kLdsStride;  // bf16 elements per LDS buffer
-constexpr int kLoadDepth = 3;         // steps of global loads a producer lane keeps in flight
+constexpr int kRowBlocks = kBM / 64;            // 32-row MFMA blocks per consumer wave (4)
+constexpr int kColBlocks = kBN / 64;            // 32-column MFMA blocks per consumer wave (2)
+constexpr int kAStages = 3;                     // LDS ring of A tiles
+constexpr int kARowBytes = kBK * 2;             // A rows are unpadded: 128 bytes = eight 16-byte slots
+constexpr int kAStageBytes = kBM * kARowBytes;  // 32 KB
+constexpr int kAGroups = kBM / 8;               // 8-row groups (one direct-to-LDS instruction each)
+constexpr int kBTile = kBN * kLdsStride;        // bf16 elements per W buffer (rows padded to 144 bytes)
+constexpr int kTileLdsBytes = kAStages * kAStageBytes + 2 * kBTile * 2;
+constexpr int kLoadDepth = 3;                   // steps of W loads a producer lane keeps in flight
+
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));  // native vector: loads/stores stay typed
 
 __device__ __forceinline__ uint4 zero4() { return make_uint4(0, 0, 0, 0); }
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every outstanding
-// global load (s_waitcnt vmcnt(0)), which would serialise the producers' register-ring prefetch behind
-// each step; here only LDS operations are waited for, and the compiler still places its own vmcnt
-// waits in front of the first use of a loaded register.
+// global load (s_waitcnt vmcnt(0)), which would serialise the prefetches behind each step.
 __device__ __forceinline__ void lds_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
+
+// Wait until at most n of this wave's global loads are outstanding (loads return in issue order).
+__device__ __forceinline__ void wait_loads_at_most(int n) {
+    switch (n) {
+        case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+        case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
+        case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+        case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
+        case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+        case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+        case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+        case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
+        default: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+    }
+}
+
+// 16-byte slot that holds contraction chunk kc (0..7) of A-tile row r.  Sixteen consecutive rows at one
+// kc cover all sixteen 16-byte bank groups exactly once.
+__device__ __forceinline__ int a_slot(int r, int kc) { return kc ^ ((r >> 1) & 7); }
 
 // 8 consecutive bf16 from a row, zero-filled past `valid` elements (element-wise path for rows that
 // are not 16-byte aligned or that end inside the run).
@@ -63,37 +88,103 @@ __device__ __forceinline__ uint4 load8_slow(const bf16_t* p, int valid) {
 struct TileCtx {  // wave-uniform description of the tile this workgroup computes
     int row_begin, rows_valid, col0, col_tile, seg_c, out_cols, contraction, total_steps, base;
     int64_t expert;
-    bf16_t* as;  // [2][kATile]
-    bf16_t* bs;  // [2][kBTile]
+    uint8_t* as;      // [kAStages][kAStageBytes]
+    bf16_t* bs;       // [2][kBTile]
+    uint32_t as_lds;  // LDS byte address of `as`
+    bool a_fast;      // A rows can be moved with aligned 16-byte accesses and every step is whole
     const uint2* grid;
 };
 
-// ---- producer waves: global -> registers one step ahead, registers -> LDS (with decode) per step.
-#define GGQ_FOR_SLABS(X) X(0) X(1) X(2) X(3) X(4) X(5) X(6) X(7)
-static_assert(kASlabs == 8, "GGQ_FOR_SLABS enumerates eight A slabs");
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));  // native vector: loads/stores stay typed
-struct ARegs {  // 16 bytes per 32-row slab of the A tile, held in registers between load and LDS store
-    u32x4_t r0, r1, r2, r3, r4, r5, r6, r7;
+// (segment, first contraction index) of a step; at most two segments.
+template <int MODE>
+__device__ __forceinline__ void step_origin(const MmqParams& p, int step, int& seg_k, int& kc0) {
+    seg_k = (MODE == kModeNN && step >= p.steps_per_seg) ? 1 : 0;
+    kc0 = (step - seg_k * p.steps_per_seg) * kBK;
+}
+
+// ---- A tile, fast path: each of the four consumer waves (or idle waves of the consumer quartet)
+// moves the 8-row groups g = 4*j + cw with one direct-to-LDS instruction per group.
+struct ALoader {
+    uint32_t voff[8];  // byte offset of this lane's 16 bytes inside the tile's rows, per group j
+    uint32_t lds0;     // LDS byte address of stage 0, group cw
+    int n;             // groups this wave moves per step (0 when the fast path is off)
 };
 
-struct ProducerLane {  // per-lane constants of a producer
-    int ptid, pw, lane, a_row, a_ch, a_slabs, last_row, w_ksub_nn, w_row_nt;
-    bool a_fast;
+__device__ __forceinline__ void a_loader_init(ALoader& a, const MmqParams& p, const TileCtx& c, int lane, int cw) {
+    const int sub = 8 * cw + (lane >> 3);         // row inside a 32-row slab
+    const int kc = (lane & 7) ^ ((sub >> 1) & 7);  // the chunk that belongs in this lane's LDS slot
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        // rows past the end of the group are clamped to its last row: they only feed output rows that
+        // are never stored
+        const int row = min(32 * j + sub, c.rows_valid - 1);
+        a.voff[j] = ((uint32_t)row * (uint32_t)p.lda + (uint32_t)kc * 8u) * 2u;
+    }
+    a.lds0 = c.as_lds + cw * 1024;
+    const int groups = (c.rows_valid + 7) >> 3;
+    a.n = c.a_fast ? max(0, (groups - cw + 3) >> 2) : 0;
+}
+
+template <int MODE>
+__device__ __forceinline__ void a_issue(const ALoader& a, const MmqParams& p, const TileCtx& c, int step, int stage) {
+    int seg_k, kc0;
+    step_origin<MODE>(p, step, seg_k, kc0);
+    const bf16_t* sbase = p.a[MODE == kModeNN ? seg_k : 0] + (int64_t)c.row_begin * p.lda + kc0;
+    const uint32_t lds = a.lds0 + stage * kAStageBytes;
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+        if (j < a.n)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                         :
+                         : "s"(lds + j * 4096), "v"(a.voff[j]), "s"(sbase)
+                         : "memory", "m0");
+}
+
+// Issue schedule shared by all waves of the consumer quartet: steps 0 and 1 before the first barrier,
+// step t + 2 at the top of main phase t (into the stage the MFMAs of step t - 1 have just released).
+struct AIssuer {
+    ALoader ld;
+    int next_step, next_stage;
 };
+template <int MODE>
+__device__ __forceinline__ void a_issue_next(AIssuer& s, const MmqParams& p, const TileCtx& c) {
+    if (s.next_step < c.total_steps) a_issue<MODE>(s.ld, p, c, s.next_step, s.next_stage);
+    s.next_step++;
+    s.next_stage = s.next_stage == kAStages - 1 ? 0 : s.next_stage + 1;
+}
+// Before the barrier that ends the phase of step t - 1 (t = 0: the first barrier): step t has landed
+// when only the loads of step t + 1 may still be in flight.
+__device__ __forceinline__ void a_wait_step(const AIssuer& s, const TileCtx& c, int t) {
+    wait_loads_at_most(t + 1 < c.total_steps ? s.ld.n : 0);
+}
+
+// ---- producer waves: packed weights global -> registers -> (decode) -> LDS W tile.
+struct ProducerLane {  // per-lane constants of a producer
+    int ptid, pw, lane, w_ksub_nn, w_row_nt;
+};
+
+// Element-wise A tile for shapes the fast path cannot take (unaligned rows, a contraction that ends
+// inside the step): producers write the same swizzled layout, zero-filled past the contraction.
+template <int MODE>
+__device__ __forceinline__ void fill_a_slow(const MmqParams& p, const TileCtx& c, const ProducerLane& l, int step, int stage) {
+    int seg_k, kc0;
+    step_origin<MODE>(p, step, seg_k, kc0);
+    uint8_t* at = c.as + stage * kAStageBytes;
+    for (int id = l.ptid; id < kBM * 8; id += 256) {
+        const int r = id >> 3, ch = id & 7;
+        if (r >= c.rows_valid) break;
+        const bf16_t* src = p.a[MODE == kModeNN ? seg_k : 0] + (int64_t)(c.row_begin + r) * p.lda + kc0 + ch * 8;
+        *(uint4*)(at + r * kARowBytes + a_slot(r, ch) * 16) = load8_slow(src, c.contraction - (kc0 + ch * 8));
+    }
+}
 
 template <int QT, int MODE>
-__device__ __forceinline__ void producer_issue_loads(const MmqParams& p, const TileCtx& c, const ProducerLane& l, int step,
-                                                     ARegs& a_reg, typename Fmt<QT>::Raw& w_reg) {
-    const int seg_k = MODE == kModeNN ? step / p.steps_per_seg : 0;
-    const int kc0 = (step - seg_k * p.steps_per_seg) * kBK;
-    if (l.a_fast) {
-        // rows past the end of the group are clamped to its last row: they only feed output rows that
-        // are never stored (and the repeated row stays in cache)
-        const bf16_t* abase = p.a[MODE == kModeNN ? seg_k : 0] + kc0 + l.a_ch * 8;
-#define GGQ_LOAD_SLAB(i) a_reg.r##i = *(const u32x4_t*)(abase + (int64_t)(c.row_begin + min(32 * i + l.a_row, l.last_row)) * p.lda);
-        GGQ_FOR_SLABS(GGQ_LOAD_SLAB)
-#undef GGQ_LOAD_SLAB
-    }
+__device__ __forceinline__ void w_issue_run(const MmqParams& p, const TileCtx& c, const ProducerLane& l, int step,
+                                            typename Fmt<QT>::Raw& w_reg) {
+    int seg_k, kc0;
+    step_origin<MODE>(p, step, seg_k, kc0);
+    // Rows / runs past the end are clamped to the last valid one: what they produce is either never
+    // stored (output columns) or multiplied by the zero-filled tail of the A tile (contraction rows).
     const int wrow = MODE == kModeNT ? l.w_row_nt : min(kc0 + l.lane, p.n - 1);
     const int ksub = MODE == kModeNT ? 2 * step + (l.ptid & 1) : l.w_ksub_nn;
     const int seg = MODE == kModeNT ? c.seg_c : seg_k;
@@ -101,24 +192,8 @@ __device__ __forceinline__ void producer_issue_loads(const MmqParams& p, const T
 }
 
 template <int QT, int MODE>
-__device__ __forceinline__ void producer_fill(const MmqParams& p, const TileCtx& c, const ProducerLane& l, int step, int buf,
-                                              const ARegs& a_reg, const typename Fmt<QT>::Raw& w_reg) {
-    bf16_t* at = c.as + buf * kATile;
+__device__ __forceinline__ void w_fill_run(const TileCtx& c, const ProducerLane& l, int step, int buf, const typename Fmt<QT>::Raw& w_reg) {
     bf16_t* bt = c.bs + buf * kBTile;
-    if (l.a_fast) {
-#define GGQ_STORE_SLAB(i) if (i < l.a_slabs) *(u32x4_t*)&at[(32 * i + l.a_row) * kLdsStride + l.a_ch * 8] = a_reg.r##i;
-        GGQ_FOR_SLABS(GGQ_STORE_SLAB)
-#undef GGQ_STORE_SLAB
-    } else {
-        // unaligned rows or a contraction that ends inside the step: element-wise, zero-filled
-        const int seg_k = MODE == kModeNN ? step / p.steps_per_seg : 0;
-        const int kc0 = (step - seg_k * p.steps_per_seg) * kBK;
-        const bf16_t* abase = p.a[MODE == kModeNN ? seg_k : 0] + kc0 + l.a_ch * 8;
-        const int a_valid = c.contraction - (kc0 + l.a_ch * 8);
-        for (int i = 0; i < l.a_slabs; i++)
-            *(uint4*)&at[(32 * i + l.a_row) * kLdsStride + l.a_ch * 8] =
-                load8_slow(abase + (int64_t)(c.row_begin + min(32 * i + l.a_row, l.last_row)) * p.lda, a_valid);
-    }
     uint32_t wv[16];
     Fmt<QT>::decode(w_reg, MODE == kModeNT ? 2 * step + (l.ptid & 1) : l.w_ksub_nn, wv, c.grid);
     if (MODE == kModeNT) {
@@ -135,56 +210,127 @@ __device__ __forceinline__ void producer_fill(const MmqParams& p, const TileCtx&
     }
 }
 
+// Q4_K forward: lane (output column n = ptid / 2, half h = ptid % 2) keeps, for a whole 256-wide block,
+// the block header and bytes 16h .. 16h+15 of each 32-byte quant group.  Group S feeds step S of the
+// block: its low nibbles are elements 16h .. 16h+15 of sub-block 2S, its high nibbles the same
+// elements of sub-block 2S+1.  Every cache line of the packed row is requested in one burst and used
+// once, instead of being fetched again on each of the four steps it spans.
+struct Q4KChunk {
+    u32x4_t hdr, q0, q1, q2, q3;
+};
+__device__ __forceinline__ void q4k_chunk_load(Q4KChunk& ch, const uint8_t* row, int block, int h) {
+    const uint8_t* blk = row + (int64_t)block * 144;
+    ch.hdr = *(const u32x4_t*)blk;
+    const uint8_t* q = blk + 16 + 16 * h;
+    ch.q0 = *(const u32x4_t*)q;
+    ch.q1 = *(const u32x4_t*)(q + 32);
+    ch.q2 = *(const u32x4_t*)(q + 64);
+    ch.q3 = *(const u32x4_t*)(q + 96);
+}
+template <int J>  // 6-bit (scale, min) of sub-block J
+__device__ __forceinline__ void q4k_scale_min(const u32x4_t& hdr, uint32_t& sc, uint32_t& m) {
+    const uint32_t s0 = hdr.y, s1 = hdr.z, s2 = hdr.w;
+    if (J < 4) {
+        sc = (s0 >> (8 * J)) & 63u;
+        m = (s1 >> (8 * J)) & 63u;
+    } else {
+        constexpr int sh = 8 * (J - 4);
+        sc = ((s2 >> sh) & 0xFu) | (((s0 >> (sh + 6)) & 3u) << 4);
+        m = ((s2 >> (sh + 4)) & 0xFu) | (((s1 >> (sh + 6)) & 3u) << 4);
+    }
+}
+template <int S>
+__device__ __forceinline__ void q4k_chunk_fill(const TileCtx& c, const ProducerLane& l, int buf, const Q4KChunk& ch) {
+    const float d = half_bits_to_f32(ch.hdr.x & 0xFFFFu), dmin = half_bits_to_f32(ch.hdr.x >> 16);
+    uint32_t sc0, m0, sc1, m1;
+    q4k_scale_min<2 * S>(ch.hdr, sc0, m0);
+    q4k_scale_min<2 * S + 1>(ch.hdr, sc1, m1);
+    const float dl0 = d * (float)sc0, nm0 = -(dmin * (float)m0);
+    const float dl1 = d * (float)sc1, nm1 = -(dmin * (float)m1);
+    const u32x4_t q = S == 0 ? ch.q0 : S == 1 ? ch.q1 : S == 2 ? ch.q2 : ch.q3;
+    uint32_t lo[8], hi[8];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t a = opaque(q[i] & 0x0F0F0F0Fu), b = opaque((q[i] >> 4) & 0x0F0F0F0Fu);
+        lo[2 * i] = pack_bf16(fmaf(dl0, ubyte0(a), nm0), fmaf(dl0, ubyte1(a), nm0));
+        lo[2 * i + 1] = pack_bf16(fmaf(dl0, ubyte2(a), nm0), fmaf(dl0, ubyte3(a), nm0));
+        hi[2 * i] = pack_bf16(fmaf(dl1, ubyte0(b), nm1), fmaf(dl1, ubyte1(b), nm1));
+        hi[2 * i + 1] = pack_bf16(fmaf(dl1, ubyte2(b), nm1), fmaf(dl1, ubyte3(b), nm1));
+    }
+    bf16_t* dst = c.bs + buf * kBTile + (l.ptid >> 1) * kLdsStride + (l.ptid & 1) * 16;
+    *(uint4*)(dst) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+    *(uint4*)(dst + 8) = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+    *(uint4*)(dst + 32) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+    *(uint4*)(dst + 40) = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+}
+
 template <int QT, int MODE>
 __device__ __forceinline__ void produce(const MmqParams& p, const TileCtx& c, int ptid, int pw) {
     ProducerLane l;
     l.ptid = ptid, l.pw = pw, l.lane = ptid & 63;
-    // fast A path: every run of 8 is 16-byte aligned and every step is entirely inside the contraction
-    l.a_fast = ((p.lda & 7) == 0) && ((c.contraction & 63) == 0) &&
-               ((((uintptr_t)p.a[0]) | ((uintptr_t)p.a[MODE == kModeNN && p.nseg > 1 ? 1 : 0])) & 15) == 0;
-    l.a_slabs = (c.rows_valid + 31) >> 5;     // 32-row slabs of the A tile that hold a valid row
-    l.a_row = ptid >> 3, l.a_ch = ptid & 7;   // lane's (row within a 32-row slab, 16-byte chunk)
-    l.last_row = c.rows_valid - 1;
     // W run owned by this lane: NT -> (output column n = col0 + ptid/2, run 2*step + ptid%2);
     //                           NN -> (contraction row n = kc0 + lane, run col0/32 + producer wave).
-    // Rows / runs past the end are clamped to the last valid one: what they produce is either never
-    // stored (output columns) or multiplied by the zero-filled tail of the A tile (contraction rows).
     l.w_ksub_nn = min((c.col0 >> 5) + pw, (p.k >> 5) - 1);
     l.w_row_nt = min(c.col0 + (ptid >> 1), p.n - 1);
-    // Register ring: global loads run kLoadDepth steps ahead of the LDS fill, which itself runs one
-    // step ahead of the MFMAs.  Memory latency is several MFMA phases long at these tile sizes.
-    ARegs a_ring[kLoadDepth];
-    typename Fmt<QT>::Raw w_ring[kLoadDepth];
-#pragma unroll
-    for (int j = 0; j < kLoadDepth; j++)
-        if (j < c.total_steps) producer_issue_loads<QT, MODE>(p, c, l, j, a_ring[j], w_ring[j]);
-
-    // phase for main step s (ring slot J = s % kLoadDepth): fill it into buffer (s + base) & 1, reuse the
-    // slot for step s + kLoadDepth, then meet the consumers at the barrier.  s == total_steps is the
-    // drain phase (barrier only).
-    auto phase = [&](auto slot_c, int s) __attribute__((always_inline)) {
-        constexpr int J = decltype(slot_c)::value;
-        if (s < c.total_steps) {
-            producer_fill<QT, MODE>(p, c, l, s, (s + c.base) & 1, a_ring[J], w_ring[J]);
-            if (s + kLoadDepth < c.total_steps) producer_issue_loads<QT, MODE>(p, c, l, s + kLoadDepth, a_ring[J], w_ring[J]);
-        }
+    const int steps = c.total_steps;
+    // Phase u fills step u (W tile into buffer (u + base) & 1, and the A tile when the direct path is
+    // off) and ends at a barrier; the MFMAs of step u run during phase u + 1.  A last barrier-only
+    // phase keeps the count equal to the consumers' (steps + 1).
+    int stage = c.base, buf = c.base;
+    auto close_phase = [&]() __attribute__((always_inline)) {
         lds_barrier();
+        stage = stage == kAStages - 1 ? 0 : stage + 1;
+        buf ^= 1;
     };
-    // without a LoRA phase the consumers' first phase already needs step 0: fill it before their first
-    // barrier; with one, step 0 is filled while they run the LoRA sub-steps
-    const int s_first = 1 - c.base;
-    if (c.base == 0) phase(std::integral_constant<int, 0>{}, 0);
-    static_assert(kLoadDepth == 3, "the phase loop below is unrolled for a ring of three");
-    for (int s3 = 0; s3 <= c.total_steps; s3 += 3) {
-        if (s3 >= s_first && s3 <= c.total_steps) phase(std::integral_constant<int, 0>{}, s3);
-        if (s3 + 1 >= s_first && s3 + 1 <= c.total_steps) phase(std::integral_constant<int, 1>{}, s3 + 1);
-        if (s3 + 2 >= s_first && s3 + 2 <= c.total_steps) phase(std::integral_constant<int, 2>{}, s3 + 2);
+    if (QT == kQ4_K && MODE == kModeNT) {
+        const uint8_t* wrow = p.w[c.seg_c] + c.expert * p.w_expert_bytes + (int64_t)l.w_row_nt * p.w_row_bytes;
+        const int h = ptid & 1, blocks = steps >> 2;  // K is a whole number of 256-wide blocks
+        Q4KChunk cur, nxt;
+        q4k_chunk_load(cur, wrow, 0, h);
+        if (blocks > 1) q4k_chunk_load(nxt, wrow, 1, h);
+        for (int b = 0; b < blocks; b++) {
+            if (!c.a_fast) fill_a_slow<MODE>(p, c, l, 4 * b, stage);
+            q4k_chunk_fill<0>(c, l, buf, cur);
+            close_phase();
+            if (!c.a_fast) fill_a_slow<MODE>(p, c, l, 4 * b + 1, stage);
+            q4k_chunk_fill<1>(c, l, buf, cur);
+            close_phase();
+            if (!c.a_fast) fill_a_slow<MODE>(p, c, l, 4 * b + 2, stage);
+            q4k_chunk_fill<2>(c, l, buf, cur);
+            close_phase();
+            if (!c.a_fast) fill_a_slow<MODE>(p, c, l, 4 * b + 3, stage);
+            q4k_chunk_fill<3>(c, l, buf, cur);
+            cur = nxt;
+            if (b + 2 < blocks) q4k_chunk_load(nxt, wrow, b + 2, h);
+            close_phase();
+        }
+    } else {
+        // Register ring: the loads of step u + kLoadDepth are issued as soon as step u is decoded.
+        typename Fmt<QT>::Raw w_ring[kLoadDepth];
+#pragma unroll
+        for (int j = 0; j < kLoadDepth; j++)
+            if (j < steps) w_issue_run<QT, MODE>(p, c, l, j, w_ring[j]);
+        auto phase = [&](auto slot_c, int u) __attribute__((always_inline)) {
+            constexpr int J = decltype(slot_c)::value;
+            if (!c.a_fast) fill_a_slow<MODE>(p, c, l, u, stage);
+            w_fill_run<QT, MODE>(c, l, u, buf, w_ring[J]);
+            if (u + kLoadDepth < steps) w_issue_run<QT, MODE>(p, c, l, u + kLoadDepth, w_ring[J]);
+            close_phase();
+        };
+        static_assert(kLoadDepth == 3, "the phase loop below is unrolled for a ring of three");
+        for (int u = 0; u < steps; u += 3) {
+            phase(std::integral_constant<int, 0>{}, u);
+            if (u + 1 < steps) phase(std::integral_constant<int, 1>{}, u + 1);
+            if (u + 2 < steps) phase(std::integral_constant<int, 2>{}, u + 2);
+        }
     }
+    lds_barrier();
 }
 
 // ---- consumer waves, instantiated per number of live 32-row blocks.
 template <int QT, int MODE, int EPI, int LIVE>
-__device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, int lane, int wave_m, int wave_n) {
+__device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, int lane, int cw) {
+    const int wave_m = cw >> 1, wave_n = cw & 1;
     const int lane_c = lane & 31, lane_h = lane >> 5;
     f32x16_t acc[LIVE][kColBlocks];
 #pragma unroll
@@ -193,20 +339,24 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
         for (int j = 0; j < kColBlocks; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
-    const int a_off = (32 * wave_m + lane_c) * kLdsStride + lane_h * 8;
+    // this lane's A row inside a 64-row pair of blocks, and the swizzled slot of each sub-step's chunk
+    const uint8_t* a_row = c.as + (32 * wave_m + lane_c) * kARowBytes;
+    int a_koff[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) a_koff[kk] = a_slot(lane_c, 2 * kk + lane_h) * 16;
     const int b_off = (wave_n * 64 + lane_c) * kLdsStride + lane_h * 8;
 
     // Operands of one sub-step (16 of the contraction): LIVE row-block runs of A, two column-block runs of W.
     struct Operands {
         bf16x8_t a[LIVE], b[kColBlocks];
     };
-    auto load_operands = [&](Operands& o, int buf, int kk) __attribute__((always_inline)) {
-        const bf16_t* a_lds = c.as + buf * kATile + a_off + kk * 16;
+    auto load_operands = [&](Operands& o, int stage, int buf, int kk) __attribute__((always_inline)) {
+        const uint8_t* a_lds = a_row + stage * kAStageBytes + a_koff[kk];
         const bf16_t* b_lds = c.bs + buf * kBTile + b_off + kk * 16;
 #pragma unroll
         for (int cb = 0; cb < kColBlocks; cb++) o.b[cb] = *(const bf16x8_t*)(b_lds + cb * 32 * kLdsStride);
 #pragma unroll
-        for (int rb = 0; rb < LIVE; rb++) o.a[rb] = *(const bf16x8_t*)(a_lds + rb * 64 * kLdsStride);
+        for (int rb = 0; rb < LIVE; rb++) o.a[rb] = *(const bf16x8_t*)(a_lds + rb * 64 * kARowBytes);
     };
     auto mfma_operands = [&](const Operands& o) __attribute__((always_inline)) {
 #pragma unroll
@@ -216,15 +366,18 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
                 acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.a[rb], o.b[cb], acc[rb][cb], 0, 0, 0);
     };
 
-    if (c.base == 0) lds_barrier();
-    int t = 0;
-    if (c.base == 1) {  // LoRA tiles sit in buffer 0: acc = s * LA . LB^T, r_pad / 16 sub-steps
+    AIssuer ai;
+    a_loader_init(ai.ld, p, c, lane, cw);
+    ai.next_step = 0, ai.next_stage = c.base;
+    a_issue_next<MODE>(ai, p, c);
+    a_issue_next<MODE>(ai, p, c);
+    if (c.base == 1) {  // LoRA tiles sit in stage 0 / buffer 0: acc = s * LA . LB^T, r_pad / 16 sub-steps
         const int n = p.r_pad >> 4;
 #pragma unroll
         for (int kk = 0; kk < 4; kk++)
             if (kk < n) {
                 Operands o;
-                load_operands(o, 0, kk);
+                load_operands(o, 0, 0, kk);
                 mfma_operands(o);
             }
         const float s = p.lora_scale;
@@ -234,34 +387,45 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
             for (int j = 0; j < kColBlocks; j++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc[i][j][e] *= s;
-        lds_barrier();
-        t = 1;
     }
+    a_wait_step(ai, c, 0);
+    lds_barrier();
     // Main steps, software pipelined inside the wave: the operands of sub-step k+1 are read from LDS
-    // while the MFMAs of sub-step k run, and the barrier that releases the buffer sits between the last
+    // while the MFMAs of sub-step k run, and the barrier that releases the buffers sits between the last
     // LDS read of a step and its last MFMAs, so the first read of the next step hides behind them.
-    // Main step t - base lives in buffer t & 1.
-    const int phases = c.total_steps + c.base;
-    if (t < phases) {
+    // Step t lives in A stage (t + base) % 3 and W buffer (t + base) & 1.
+    // The scheduler would otherwise sink the reads to the end of the stage (they reuse the registers of
+    // the running MFMAs' operands): pin "all LDS reads of the stage, then its MFMAs".
+#define GGQ_READS_THEN_MFMAS()                                          \
+    __builtin_amdgcn_sched_group_barrier(0x100, LIVE + kColBlocks, 0);  \
+    __builtin_amdgcn_sched_group_barrier(0x008, LIVE * kColBlocks, 0);  \
+    __builtin_amdgcn_sched_barrier(0)
+    {
+        const int steps = c.total_steps;
+        int stage = c.base, buf = c.base;
         Operands x, y;
-        load_operands(x, t & 1, 0);
-        for (; t < phases; t++) {
-            const int buf = t & 1;
-            load_operands(y, buf, 1);
+        load_operands(x, stage, buf, 0);
+        for (int t = 0; t < steps; t++) {
+            a_issue_next<MODE>(ai, p, c);  // step t + 2
+            load_operands(y, stage, buf, 1);
             mfma_operands(x);
-            __builtin_amdgcn_sched_barrier(0);
-            load_operands(x, buf, 2);
+            GGQ_READS_THEN_MFMAS();
+            load_operands(x, stage, buf, 2);
             mfma_operands(y);
-            __builtin_amdgcn_sched_barrier(0);
-            load_operands(y, buf, 3);
+            GGQ_READS_THEN_MFMAS();
+            load_operands(y, stage, buf, 3);
             mfma_operands(x);
-            __builtin_amdgcn_sched_barrier(0);
-            lds_barrier();  // every LDS read of this step has landed; the producers may refill the buffer
-            if (t + 1 < phases) load_operands(x, buf ^ 1, 0);
+            GGQ_READS_THEN_MFMAS();
+            a_wait_step(ai, c, t + 1);
+            lds_barrier();  // every LDS read of this step has landed; its stage and buffer may be refilled
+            stage = stage == kAStages - 1 ? 0 : stage + 1;
+            buf ^= 1;
+            if (t + 1 < steps) load_operands(x, stage, buf, 0);
             mfma_operands(y);
-            __builtin_amdgcn_sched_barrier(0);
+            GGQ_READS_THEN_MFMAS();
         }
     }
+#undef GGQ_READS_THEN_MFMAS
 
     // ---- epilogue.  acc[rb][cb][i]: tile row = 32*(2*rb + wave_m) + 8*(i/4) + 4*lane_h + (i%4),
     //                                 tile col = 64*wave_n + 32*cb + lane_c
@@ -332,19 +496,32 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
     }
 }
 
-// A consumer wave without a live row block only keeps the barriers company.
-__device__ __forceinline__ void consume_idle(const TileCtx& c) {
-    if (c.base == 0) lds_barrier();
-    for (int t = 0; t < c.total_steps + c.base; t++) lds_barrier();
+// A wave of the consumer quartet without a live row block still moves its share of the A tile and
+// keeps the barriers company.
+template <int MODE>
+__device__ __forceinline__ void consume_idle(const MmqParams& p, const TileCtx& c, int lane, int cw) {
+    AIssuer ai;
+    a_loader_init(ai.ld, p, c, lane, cw);
+    ai.next_step = 0, ai.next_stage = c.base;
+    a_issue_next<MODE>(ai, p, c);
+    a_issue_next<MODE>(ai, p, c);
+    a_wait_step(ai, c, 0);
+    lds_barrier();
+    for (int t = 0; t < c.total_steps; t++) {
+        a_issue_next<MODE>(ai, p, c);
+        a_wait_step(ai, c, t + 1);
+        lds_barrier();
+    }
 }
 
 template <int QT, int MODE, int EPI>
 __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(2, 2))) void mmq_tile_kernel(const MmqParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_raw[];
     TileCtx c;
-    c.as = (bf16_t*)smem_raw;
-    c.bs = c.as + 2 * kATile;
-    uint2* grid_lds = (uint2*)(c.bs + 2 * kBTile);  // [256], IQ2_XXS only
+    c.as = smem_raw;
+    c.as_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem_raw;
+    c.bs = (bf16_t*)(smem_raw + kAStages * kAStageBytes);
+    uint2* grid_lds = (uint2*)(smem_raw + kTileLdsBytes);  // [256], IQ2_XXS only
     c.grid = grid_lds;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -377,19 +554,21 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(2, 
     c.contraction = MODE == kModeNT ? p.k : p.n;  // contraction length per segment
     c.total_steps = (MODE == kModeNN ? p.nseg : 1) * p.steps_per_seg;
     c.base = p.r_pad > 0 ? 1 : 0;
+    c.a_fast = ((p.lda & 7) == 0) && ((c.contraction & 63) == 0) &&
+               ((((uintptr_t)p.a[0]) | ((uintptr_t)p.a[MODE == kModeNN && p.nseg > 1 ? 1 : 0])) & 15) == 0;
 
     if (QT == kIQ2_XXS && tid < 256) {
         const uint64_t g = d_iq2xxs_grid_mm[tid];
         grid_lds[tid] = make_uint2((uint32_t)g, (uint32_t)(g >> 32));
     }
-    // ---- LoRA tiles go to buffer 0 (all lanes load): LA[rows, :r] and LB[cols, :r]
+    // ---- LoRA tiles go to A stage 0 / W buffer 0 (all lanes load): LA[rows, :r] and LB[cols, :r]
     if (p.r_pad > 0) {
         const int chunks = p.r_pad >> 3;  // 16-byte chunks per row (r_pad % 16 == 0)
         for (int id = tid; id < kBM * 8; id += kThreads) {
             const int r = id >> 3, ch = id & 7;
             uint4 v = zero4();
             if (r < c.rows_valid && ch < chunks) v = *(const uint4*)(p.la + (int64_t)(c.row_begin + r) * p.r_pad + ch * 8);
-            *(uint4*)&c.as[r * kLdsStride + ch * 8] = v;
+            *(uint4*)(c.as + r * kARowBytes + a_slot(r, ch) * 16) = v;
         }
         const bf16_t* lb = p.lb + c.expert * p.lb_expert_elems + (int64_t)(c.seg_c * c.out_cols + c.col0) * p.r_pad;
         for (int id = tid; id < kBN * 8; id += kThreads) {
@@ -404,15 +583,15 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(2, 
     if (wave >= 4) {
         produce<QT, MODE>(p, c, tid & 255, cw);
     } else {
-        const int wave_m = cw >> 1, wave_n = cw & 1;
+        const int wave_m = cw >> 1;
         // this wave's row block i covers tile rows 32*(2*i + wave_m) .. +31; blocks fill up from row 0
         const int live = c.rows_valid > 32 * wave_m ? min(kRowBlocks, (c.rows_valid - 32 * wave_m + 63) >> 6) : 0;
         switch (live) {
-            case 0: consume_idle(c); break;
-            case 1: consume<QT, MODE, EPI, 1>(p, c, lane, wave_m, wave_n); break;
-            case 2: consume<QT, MODE, EPI, 2>(p, c, lane, wave_m, wave_n); break;
-            case 3: consume<QT, MODE, EPI, 3>(p, c, lane, wave_m, wave_n); break;
-            default: consume<QT, MODE, EPI, 4>(p, c, lane, wave_m, wave_n); break;
+            case 0: consume_idle<MODE>(p, c, lane, cw); break;
+            case 1: consume<QT, MODE, EPI, 1>(p, c, lane, cw); break;
+            case 2: consume<QT, MODE, EPI, 2>(p, c, lane, cw); break;
+            case 3: consume<QT, MODE, EPI, 3>(p, c, lane, cw); break;
+            default: consume<QT, MODE, EPI, 4>(p, c, lane, cw); break;
         }
     }
 }
