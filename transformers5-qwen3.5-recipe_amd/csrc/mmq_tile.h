@@ -125,14 +125,14 @@ __device__ __forceinline__ void a_loader_init(ALoader& a, const MmqParams& p, co
     a.n = c.a_fast ? max(0, (groups - cw + 3) >> 2) : 0;
 }
 
-template <int MODE>
+template <int MODE, int J0, int J1>
 __device__ __forceinline__ void a_issue(const ALoader& a, const MmqParams& p, const TileCtx& c, int step, int stage) {
     int seg_k, kc0;
     step_origin<MODE>(p, step, seg_k, kc0);
     const bf16_t* sbase = p.a[MODE == kModeNN ? seg_k : 0] + (int64_t)c.row_begin * p.lda + kc0;
     const uint32_t lds = a.lds0 + stage * kAStageBytes;
 #pragma unroll
-    for (int j = 0; j < 8; j++)
+    for (int j = J0; j < J1; j++)
         if (j < a.n)
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                          :
@@ -141,16 +141,24 @@ __device__ __forceinline__ void a_issue(const ALoader& a, const MmqParams& p, co
 }
 
 // Issue schedule shared by all waves of the consumer quartet: steps 0 and 1 before the first barrier,
-// step t + 2 at the top of main phase t (into the stage the MFMAs of step t - 1 have just released).
+// step t + 2 during main phase t (into the stage the MFMAs of step t - 1 have just released), two
+// groups at a time between the MFMAs so that a full memory queue never holds up the matrix pipe.
 struct AIssuer {
     ALoader ld;
     int next_step, next_stage;
 };
-template <int MODE>
-__device__ __forceinline__ void a_issue_next(AIssuer& s, const MmqParams& p, const TileCtx& c) {
-    if (s.next_step < c.total_steps) a_issue<MODE>(s.ld, p, c, s.next_step, s.next_stage);
+template <int MODE, int J0, int J1>
+__device__ __forceinline__ void a_issue_part(const AIssuer& s, const MmqParams& p, const TileCtx& c) {
+    if (s.next_step < c.total_steps) a_issue<MODE, J0, J1>(s.ld, p, c, s.next_step, s.next_stage);
+}
+__device__ __forceinline__ void a_issue_advance(AIssuer& s) {
     s.next_step++;
     s.next_stage = s.next_stage == kAStages - 1 ? 0 : s.next_stage + 1;
+}
+template <int MODE>
+__device__ __forceinline__ void a_issue_next(AIssuer& s, const MmqParams& p, const TileCtx& c) {
+    a_issue_part<MODE, 0, 8>(s, p, c);
+    a_issue_advance(s);
 }
 // Before the barrier that ends the phase of step t - 1 (t = 0: the first barrier): step t has landed
 // when only the loads of step t + 1 may still be in flight.
@@ -285,24 +293,29 @@ __device__ __forceinline__ void produce(const MmqParams& p, const TileCtx& c, in
     if (QT == kQ4_K && MODE == kModeNT) {
         const uint8_t* wrow = p.w[c.seg_c] + c.expert * p.w_expert_bytes + (int64_t)l.w_row_nt * p.w_row_bytes;
         const int h = ptid & 1, blocks = steps >> 2;  // K is a whole number of 256-wide blocks
-        Q4KChunk cur, nxt;
-        q4k_chunk_load(cur, wrow, 0, h);
-        if (blocks > 1) q4k_chunk_load(nxt, wrow, 1, h);
-        for (int b = 0; b < blocks; b++) {
+        // Two register sets, used by even and odd blocks: a set is reloaded (block + 2) right after its
+        // last use, four steps before its next one.
+        Q4KChunk even, odd;
+        q4k_chunk_load(even, wrow, 0, h);
+        if (blocks > 1) q4k_chunk_load(odd, wrow, 1, h);
+        auto block_phases = [&](Q4KChunk& ch, int b) __attribute__((always_inline)) {
             if (!c.a_fast) fill_a_slow<MODE>(p, c, l, 4 * b, stage);
-            q4k_chunk_fill<0>(c, l, buf, cur);
+            q4k_chunk_fill<0>(c, l, buf, ch);
             close_phase();
             if (!c.a_fast) fill_a_slow<MODE>(p, c, l, 4 * b + 1, stage);
-            q4k_chunk_fill<1>(c, l, buf, cur);
+            q4k_chunk_fill<1>(c, l, buf, ch);
             close_phase();
             if (!c.a_fast) fill_a_slow<MODE>(p, c, l, 4 * b + 2, stage);
-            q4k_chunk_fill<2>(c, l, buf, cur);
+            q4k_chunk_fill<2>(c, l, buf, ch);
             close_phase();
             if (!c.a_fast) fill_a_slow<MODE>(p, c, l, 4 * b + 3, stage);
-            q4k_chunk_fill<3>(c, l, buf, cur);
-            cur = nxt;
-            if (b + 2 < blocks) q4k_chunk_load(nxt, wrow, b + 2, h);
+            q4k_chunk_fill<3>(c, l, buf, ch);
+            if (b + 2 < blocks) q4k_chunk_load(ch, wrow, b + 2, h);
             close_phase();
+        };
+        for (int b = 0; b < blocks; b += 2) {
+            block_phases(even, b);
+            if (b + 1 < blocks) block_phases(odd, b + 1);
         }
     } else {
         // Register ring: the loads of step u + kLoadDepth are issued as soon as step u is decoded.
@@ -358,6 +371,17 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
 #pragma unroll
         for (int rb = 0; rb < LIVE; rb++) o.a[rb] = *(const bf16x8_t*)(a_lds + rb * 64 * kARowBytes);
     };
+    auto mfma_rows = [&](const Operands& o, int rb0, int rb1) __attribute__((always_inline)) {
+#pragma unroll
+        for (int rb = 0; rb < LIVE; rb++)
+            if (rb >= rb0 && rb < rb1)
+#pragma unroll
+                for (int cb = 0; cb < kColBlocks; cb++)
+                    acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.a[rb], o.b[cb], acc[rb][cb], 0, 0, 0);
+    };
+    auto mfma_one = [&](const Operands& o, int rb, int cb) __attribute__((always_inline)) {
+        acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.a[rb], o.b[cb], acc[rb][cb], 0, 0, 0);
+    };
     auto mfma_operands = [&](const Operands& o) __attribute__((always_inline)) {
 #pragma unroll
         for (int rb = 0; rb < LIVE; rb++)
@@ -366,6 +390,9 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
                 acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.a[rb], o.b[cb], acc[rb][cb], 0, 0, 0);
     };
 
+    // The MFMA stream must win issue arbitration against the producer wave on the same SIMD: a matrix
+    // instruction only needs an issue slot every 32 cycles, the decoder's VALU stream fills the rest.
+    __builtin_amdgcn_s_setprio(3);
     AIssuer ai;
     a_loader_init(ai.ld, p, c, lane, cw);
     ai.next_step = 0, ai.next_stage = c.base;
@@ -396,36 +423,51 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
     // Step t lives in A stage (t + base) % 3 and W buffer (t + base) & 1.
     // The scheduler would otherwise sink the reads to the end of the stage (they reuse the registers of
     // the running MFMAs' operands): pin "all LDS reads of the stage, then its MFMAs".
-#define GGQ_READS_THEN_MFMAS()                                          \
-    __builtin_amdgcn_sched_group_barrier(0x100, LIVE + kColBlocks, 0);  \
-    __builtin_amdgcn_sched_group_barrier(0x008, LIVE * kColBlocks, 0);  \
+    // A wave gets one 16-byte-per-lane LDS read through roughly every 32 cycles, the same cadence as its
+    // MFMAs, and a read that cannot issue holds up the MFMAs queued behind it: reads and MFMAs alternate
+    // one by one.  The last row block's two MFMAs frame the two A-tile loads of the stage.
+#define GGQ_MFMA_READ_PAIRS()                                                                              \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); \
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                                                     \
+    __builtin_amdgcn_sched_barrier(0)
+#define GGQ_STAGE(NEXT, CUR, KK, J0)                          \
+    load_operands(NEXT, stage, buf, KK);                      \
+    mfma_rows(CUR, 0, LIVE - 1);                              \
+    GGQ_MFMA_READ_PAIRS();                                    \
+    a_issue_part<MODE, J0, J0 + 1>(ai, p, c);                 \
+    mfma_one(CUR, LIVE - 1, 0);                               \
+    __builtin_amdgcn_sched_barrier(0);                        \
+    a_issue_part<MODE, J0 + 1, J0 + 2>(ai, p, c);             \
+    mfma_one(CUR, LIVE - 1, 1);                               \
     __builtin_amdgcn_sched_barrier(0)
     {
         const int steps = c.total_steps;
         int stage = c.base, buf = c.base;
         Operands x, y;
         load_operands(x, stage, buf, 0);
-        for (int t = 0; t < steps; t++) {
-            a_issue_next<MODE>(ai, p, c);  // step t + 2
-            load_operands(y, stage, buf, 1);
-            mfma_operands(x);
-            GGQ_READS_THEN_MFMAS();
-            load_operands(x, stage, buf, 2);
-            mfma_operands(y);
-            GGQ_READS_THEN_MFMAS();
-            load_operands(y, stage, buf, 3);
-            mfma_operands(x);
-            GGQ_READS_THEN_MFMAS();
+        for (int t = 0; t < steps; t++) {  // the A loads issued in here are those of step t + 2
+            GGQ_STAGE(y, x, 1, 0);
+            GGQ_STAGE(x, y, 2, 2);
+            GGQ_STAGE(y, x, 3, 4);
+            a_issue_part<MODE, 6, 8>(ai, p, c);
+            a_issue_advance(ai);
             a_wait_step(ai, c, t + 1);
             lds_barrier();  // every LDS read of this step has landed; its stage and buffer may be refilled
             stage = stage == kAStages - 1 ? 0 : stage + 1;
             buf ^= 1;
             if (t + 1 < steps) load_operands(x, stage, buf, 0);
-            mfma_operands(y);
-            GGQ_READS_THEN_MFMAS();
+            mfma_rows(y, 0, LIVE);
+            GGQ_MFMA_READ_PAIRS();
         }
     }
-#undef GGQ_READS_THEN_MFMAS
+#undef GGQ_MFMA_READ_PAIRS
+#undef GGQ_STAGE
+    __builtin_amdgcn_s_setprio(0);
 
     // ---- epilogue.  acc[rb][cb][i]: tile row = 32*(2*rb + wave_m) + 8*(i/4) + 4*lane_h + (i%4),
     //                                 tile col = 64*wave_n + 32*cb + lane_c
