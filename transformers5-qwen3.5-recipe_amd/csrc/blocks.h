@@ -17,6 +17,16 @@ namespace ggq {
 template <int QT>
 struct Fmt;
 
+// pin(): a compiler-level fence on the registers of a Raw: every later use stays behind this point in
+// program order (nothing is emitted).  The matmul kernel puts it behind a barrier so that the wait for
+// a prefetched run is not pulled in front of that barrier.
+#if defined(__HIP_DEVICE_COMPILE__)
+#define GGQ_PIN1(a) asm volatile("" : "+v"(a))
+#else
+#define GGQ_PIN1(a) (void)(a)
+#endif
+#define GGQ_PIN4(q) GGQ_PIN1((q).x); GGQ_PIN1((q).y); GGQ_PIN1((q).z); GGQ_PIN1((q).w)
+
 // ------------------------------------------------------------------------------------------------
 // Q8_0: 34-byte block = f16 d; i8 q[32]; one block per run.  Blocks are 2-byte aligned.
 template <>
@@ -26,6 +36,7 @@ struct Fmt<kQ8_0> {
         uint4 q0, q1;
         uint32_t d16;
     };
+    static GGQ_HD void pin(Raw& r) { GGQ_PIN4(r.q0); GGQ_PIN4(r.q1); GGQ_PIN1(r.d16); }
     static GGQ_HD void load(Raw& r, const uint8_t* row, int ksub) {
         const uint8_t* p = row + (int64_t)ksub * 34;
         r.d16 = ld_u16(p);
@@ -55,6 +66,7 @@ struct Fmt<kQ4_K> {
     struct Raw {
         uint4 hdr, q0, q1;
     };
+    static GGQ_HD void pin(Raw& r) { GGQ_PIN4(r.hdr); GGQ_PIN4(r.q0); GGQ_PIN4(r.q1); }
     static GGQ_HD void load(Raw& r, const uint8_t* row, int ksub) {
         const uint8_t* blk = row + (int64_t)(ksub >> 3) * 144;
         r.hdr = *(const uint4*)blk;
@@ -101,6 +113,7 @@ struct Fmt<kQ6_K> {
         uint4 qh[2];
         uint32_t sc2, d16;
     };
+    static GGQ_HD void pin(Raw& r) { GGQ_PIN4(r.ql[0]); GGQ_PIN4(r.ql[1]); GGQ_PIN4(r.qh[0]); GGQ_PIN4(r.qh[1]); GGQ_PIN1(r.sc2); GGQ_PIN1(r.d16); }
     static GGQ_HD void load(Raw& r, const uint8_t* row, int ksub) {
         const uint8_t* blk = row + (int64_t)(ksub >> 3) * 210;
         const int u = ksub & 7, h = u >> 2, p = u & 3;
@@ -141,6 +154,7 @@ struct Fmt<kIQ2_XXS> {
     struct Raw {
         uint32_t idx4, aux, d16;
     };
+    static GGQ_HD void pin(Raw& r) { GGQ_PIN1(r.idx4); GGQ_PIN1(r.aux); GGQ_PIN1(r.d16); }
     static GGQ_HD void load(Raw& r, const uint8_t* row, int ksub) {
         const uint8_t* blk = row + (int64_t)(ksub >> 3) * 66;
         r.d16 = ld_u16(blk);

@@ -36,7 +36,7 @@ struct FactorGradParams {
 
 constexpr int kBM = 256, kBN = 128, kBK = 64;
 constexpr int kLdsStride = kBK + 8;  // bf16 elements per LDS row: 144 bytes keeps 128-bit reads conflict-free
-constexpr int kThreads = 512;  // waves 0..3 run the MFMAs, waves 4..7 load and decode
+constexpr int kThreads = 1024;  // waves 0..7 run the MFMAs, waves 8..15 load and decode
 
 enum : int { kModeNT = 0, kModeNN = 1 };
 enum : int {

@@ -7,21 +7,25 @@
 // expert groups (row ranges of A/C that use different experts' W), and an optional rank-r LoRA term
 // s * LA[m, :] . LB[col, :] folded in as extra contraction steps ahead of the main loop.
 //
-// One workgroup = 512 lanes (8 waves) computes a 256 x 128 tile of C: tall, because every decoded
-// weight is reused by all rows of the tile and an expert's rows (about 128 on average in the MoE
-// shapes this is built for) should fit one tile.  The waves are specialised; per contraction step of 64
-//   * consumer waves 0..3 (2 x 2) each own four 32-row blocks (interleaved: block 2*i + wave_m, so
-//     short groups load both wave rows evenly) x two 32-column blocks of MFMA 32x32x16 accumulators;
-//     the whole consumer path is instantiated per number of live row blocks, so ragged groups issue no
-//     MFMA on empty blocks.  They also move the A tile: global -> LDS directly (no registers), 1 KB =
-//     8 rows x 128 bytes per wave instruction, two steps ahead of the MFMAs through a ring of three
-//     LDS stages; 8-row groups past the end of the expert group are skipped.  A rows sit unpadded in
-//     LDS with their 16-byte slots XOR-swizzled so that both the 1 KB writes and the MFMA operand
-//     reads are bank-conflict free;
-//   * producer waves 4..7 own the weights: packed bytes global -> registers (each cache line fetched
-//     once: for Q4_K forward a lane keeps its share of a whole 256-wide block in registers for four
-//     steps), scales / mins / codebook unpacked in registers (blocks.h), bf16 written into the LDS W
-//     tile laid out [output column][contraction]; in NN mode that write is the transposition.
+// One workgroup = 1024 lanes (16 waves, four per SIMD, 128 VGPRs each) computes a 256 x 128 tile of C:
+// tall, because every decoded weight is reused by all rows of the tile and an expert's rows (about 128
+// on average in the MoE shapes this is built for) should fit one tile.  The waves are specialised; per
+// contraction step of 64
+//   * consumer waves 0..7 (4 x 2) each own two 32-row blocks (blocks wave_m and wave_m + 4, so short
+//     groups still spread over all eight waves) x two 32-column blocks of MFMA 32x32x16 accumulators.
+//     Two MFMA-issuing waves share each SIMD: whenever one waits (LDS read cadence, memory queue,
+//     barrier skew) the other keeps the matrix pipe busy.  The consumer path is instantiated per number
+//     of live row blocks, so ragged groups issue no MFMA on empty blocks.  Consumers also move the A
+//     tile: global -> LDS directly (no registers), 1 KB = 8 rows x 128 bytes per wave instruction, two
+//     steps ahead of the MFMAs through a ring of three LDS stages; 8-row groups past the end of the
+//     expert group are skipped.  A rows sit unpadded in LDS with their 16-byte slots XOR-swizzled so
+//     that both the 1 KB writes and the MFMA operand reads are bank-conflict free;
+//   * producer waves 8..15 own the weights, as two quartets that take alternate steps: a quartet
+//     decodes its step into registers during one phase (packed bytes global -> registers, scales / mins
+//     / codebook unpacked in registers, blocks.h) and stores the bf16 W tile, laid out [output
+//     column][contraction], during the next, while the other quartet decodes; in NN mode that store is
+//     the transposition.  For Q4_K forward a lane loads its share of a 256-wide block once and keeps it
+//     for the block's steps, so every cache line of the packed row is requested in one burst.
 // One barrier per step hands the buffers over; decode VALU work and MFMA work overlap on every SIMD.
 #pragma once
 #include "blocks.h"
@@ -34,7 +38,7 @@ namespace ggq {
 
 static __device__ const uint64_t d_iq2xxs_grid_mm[256] = GGQ_IQ2XXS_GRID_INIT;
 
-constexpr int kRowBlocks = kBM / 64;            // 32-row MFMA blocks per consumer wave (4)
+constexpr int kRowBlocks = kBM / 128;           // 32-row MFMA blocks per consumer wave (2): wave_m, wave_m + 4
 constexpr int kColBlocks = kBN / 64;            // 32-column MFMA blocks per consumer wave (2)
 constexpr int kAStages = 3;                     // LDS ring of A tiles
 constexpr int kARowBytes = kBK * 2;             // A rows are unpadded: 128 bytes = eight 16-byte slots
@@ -42,7 +46,7 @@ constexpr int kAStageBytes = kBM * kARowBytes;  // 32 KB
 constexpr int kAGroups = kBM / 8;               // 8-row groups (one direct-to-LDS instruction each)
 constexpr int kBTile = kBN * kLdsStride;        // bf16 elements per W buffer (rows padded to 144 bytes)
 constexpr int kTileLdsBytes = kAStages * kAStageBytes + 2 * kBTile * 2;
-constexpr int kLoadDepth = 3;                   // steps of W loads a producer lane keeps in flight
+constexpr int kGroupsPerWave = kAGroups / 8;    // A-tile groups one consumer wave moves per step (4)
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));  // native vector: loads/stores stay typed
 
@@ -102,27 +106,27 @@ __device__ __forceinline__ void step_origin(const MmqParams& p, int step, int& s
     kc0 = (step - seg_k * p.steps_per_seg) * kBK;
 }
 
-// ---- A tile, fast path: each of the four consumer waves (or idle waves of the consumer quartet)
-// moves the 8-row groups g = 4*j + cw with one direct-to-LDS instruction per group.
+// ---- A tile, fast path: each of the eight waves of the consumer octet moves the 8-row groups
+// g = 8*j + cw (j = 0..3) with one direct-to-LDS instruction per group.
 struct ALoader {
-    uint32_t voff[8];  // byte offset of this lane's 16 bytes inside the tile's rows, per group j
-    uint32_t lds0;     // LDS byte address of stage 0, group cw
-    int n;             // groups this wave moves per step (0 when the fast path is off)
+    uint32_t voff[kGroupsPerWave];  // byte offset of this lane's 16 bytes inside the tile's rows, per group j
+    uint32_t lds0;                  // LDS byte address of stage 0, group cw
+    int n;                          // groups this wave moves per step (0 when the fast path is off)
 };
 
 __device__ __forceinline__ void a_loader_init(ALoader& a, const MmqParams& p, const TileCtx& c, int lane, int cw) {
-    const int sub = 8 * cw + (lane >> 3);         // row inside a 32-row slab
+    const int sub = 8 * cw + (lane >> 3);         // row inside a 64-row slab
     const int kc = (lane & 7) ^ ((sub >> 1) & 7);  // the chunk that belongs in this lane's LDS slot
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
+    for (int j = 0; j < kGroupsPerWave; j++) {
         // rows past the end of the group are clamped to its last row: they only feed output rows that
         // are never stored
-        const int row = min(32 * j + sub, c.rows_valid - 1);
+        const int row = min(64 * j + sub, c.rows_valid - 1);
         a.voff[j] = ((uint32_t)row * (uint32_t)p.lda + (uint32_t)kc * 8u) * 2u;
     }
     a.lds0 = c.as_lds + cw * 1024;
     const int groups = (c.rows_valid + 7) >> 3;
-    a.n = c.a_fast ? max(0, (groups - cw + 3) >> 2) : 0;
+    a.n = c.a_fast ? max(0, (groups - cw + 7) >> 3) : 0;
 }
 
 template <int MODE, int J0, int J1>
@@ -136,13 +140,13 @@ __device__ __forceinline__ void a_issue(const ALoader& a, const MmqParams& p, co
         if (j < a.n)
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                          :
-                         : "s"(lds + j * 4096), "v"(a.voff[j]), "s"(sbase)
+                         : "s"(lds + j * 8192), "v"(a.voff[j]), "s"(sbase)
                          : "memory", "m0");
 }
 
-// Issue schedule shared by all waves of the consumer quartet: steps 0 and 1 before the first barrier,
-// step t + 2 during main phase t (into the stage the MFMAs of step t - 1 have just released), two
-// groups at a time between the MFMAs so that a full memory queue never holds up the matrix pipe.
+// Issue schedule shared by all waves of the consumer octet: steps 0 and 1 before the first barrier,
+// step t + 2 during main phase t (into the stage the MFMAs of step t - 1 have just released), one
+// group per sub-step between the MFMAs.
 struct AIssuer {
     ALoader ld;
     int next_step, next_stage;
@@ -157,7 +161,7 @@ __device__ __forceinline__ void a_issue_advance(AIssuer& s) {
 }
 template <int MODE>
 __device__ __forceinline__ void a_issue_next(AIssuer& s, const MmqParams& p, const TileCtx& c) {
-    a_issue_part<MODE, 0, 8>(s, p, c);
+    a_issue_part<MODE, 0, kGroupsPerWave>(s, p, c);
     a_issue_advance(s);
 }
 // Before the barrier that ends the phase of step t - 1 (t = 0: the first barrier): step t has landed
@@ -199,11 +203,10 @@ __device__ __forceinline__ void w_issue_run(const MmqParams& p, const TileCtx& c
     Fmt<QT>::load(w_reg, p.w[seg] + c.expert * p.w_expert_bytes + (int64_t)wrow * p.w_row_bytes, ksub);
 }
 
-template <int QT, int MODE>
-__device__ __forceinline__ void w_fill_run(const TileCtx& c, const ProducerLane& l, int step, int buf, const typename Fmt<QT>::Raw& w_reg) {
+// The 32 decoded weights of a run (16 packed bf16 pairs) -> LDS W tile.
+template <int MODE>
+__device__ __forceinline__ void w_store_run(const TileCtx& c, const ProducerLane& l, int buf, const uint32_t* wv) {
     bf16_t* bt = c.bs + buf * kBTile;
-    uint32_t wv[16];
-    Fmt<QT>::decode(w_reg, MODE == kModeNT ? 2 * step + (l.ptid & 1) : l.w_ksub_nn, wv, c.grid);
     if (MODE == kModeNT) {
         bf16_t* dst = &bt[(l.ptid >> 1) * kLdsStride + (l.ptid & 1) * 32];
 #pragma unroll
@@ -218,22 +221,24 @@ __device__ __forceinline__ void w_fill_run(const TileCtx& c, const ProducerLane&
     }
 }
 
-// Q4_K forward: lane (output column n = ptid / 2, half h = ptid % 2) keeps, for a whole 256-wide block,
-// the block header and bytes 16h .. 16h+15 of each 32-byte quant group.  Group S feeds step S of the
-// block: its low nibbles are elements 16h .. 16h+15 of sub-block 2S, its high nibbles the same
-// elements of sub-block 2S+1.  Every cache line of the packed row is requested in one burst and used
-// once, instead of being fetched again on each of the four steps it spans.
+// Q4_K forward: lane (output column n = ptid / 2, half h = ptid % 2) keeps, for a 256-wide block, the
+// block header and bytes 16h .. 16h+15 of the two 32-byte quant groups its quartet decodes (groups
+// q and q + 2 for quartet q).  Group S feeds step S of the block: its low nibbles are elements
+// 16h .. 16h+15 of sub-block 2S, its high nibbles the same elements of sub-block 2S+1.
 struct Q4KChunk {
-    u32x4_t hdr, q0, q1, q2, q3;
+    u32x4_t hdr, qa, qb;
 };
-__device__ __forceinline__ void q4k_chunk_load(Q4KChunk& ch, const uint8_t* row, int block, int h) {
+__device__ __forceinline__ void q4k_chunk_load(Q4KChunk& ch, const uint8_t* row, int block, int h, int quartet) {
     const uint8_t* blk = row + (int64_t)block * 144;
     ch.hdr = *(const u32x4_t*)blk;
-    const uint8_t* q = blk + 16 + 16 * h;
-    ch.q0 = *(const u32x4_t*)q;
-    ch.q1 = *(const u32x4_t*)(q + 32);
-    ch.q2 = *(const u32x4_t*)(q + 64);
-    ch.q3 = *(const u32x4_t*)(q + 96);
+    const uint8_t* q = blk + 16 + 16 * h + 32 * quartet;
+    ch.qa = *(const u32x4_t*)q;
+    ch.qb = *(const u32x4_t*)(q + 64);
+}
+// Keeps every use of the block registers after this point in program order (in particular after the
+// barrier in front of it), so that no wait for a freshly issued reload is pulled forward.
+__device__ __forceinline__ void q4k_chunk_pin(Q4KChunk& ch) {
+    asm volatile("" : "+v"(ch.hdr), "+v"(ch.qa), "+v"(ch.qb));
 }
 template <int J>  // 6-bit (scale, min) of sub-block J
 __device__ __forceinline__ void q4k_scale_min(const u32x4_t& hdr, uint32_t& sc, uint32_t& m) {
@@ -247,94 +252,163 @@ __device__ __forceinline__ void q4k_scale_min(const u32x4_t& hdr, uint32_t& sc, 
         m = ((s2 >> (sh + 4)) & 0xFu) | (((s1 >> (sh + 6)) & 3u) << 4);
     }
 }
+// wv[0..7]: elements 16h .. 16h+15 of sub-block 2S; wv[8..15]: the same elements of sub-block 2S+1.
 template <int S>
-__device__ __forceinline__ void q4k_chunk_fill(const TileCtx& c, const ProducerLane& l, int buf, const Q4KChunk& ch) {
-    const float d = half_bits_to_f32(ch.hdr.x & 0xFFFFu), dmin = half_bits_to_f32(ch.hdr.x >> 16);
+__device__ __forceinline__ void q4k_chunk_decode(const u32x4_t& hdr, const u32x4_t& q, uint32_t* wv) {
+    const float d = half_bits_to_f32(hdr.x & 0xFFFFu), dmin = half_bits_to_f32(hdr.x >> 16);
     uint32_t sc0, m0, sc1, m1;
-    q4k_scale_min<2 * S>(ch.hdr, sc0, m0);
-    q4k_scale_min<2 * S + 1>(ch.hdr, sc1, m1);
+    q4k_scale_min<2 * S>(hdr, sc0, m0);
+    q4k_scale_min<2 * S + 1>(hdr, sc1, m1);
     const float dl0 = d * (float)sc0, nm0 = -(dmin * (float)m0);
     const float dl1 = d * (float)sc1, nm1 = -(dmin * (float)m1);
-    const u32x4_t q = S == 0 ? ch.q0 : S == 1 ? ch.q1 : S == 2 ? ch.q2 : ch.q3;
-    uint32_t lo[8], hi[8];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const uint32_t a = opaque(q[i] & 0x0F0F0F0Fu), b = opaque((q[i] >> 4) & 0x0F0F0F0Fu);
-        lo[2 * i] = pack_bf16(fmaf(dl0, ubyte0(a), nm0), fmaf(dl0, ubyte1(a), nm0));
-        lo[2 * i + 1] = pack_bf16(fmaf(dl0, ubyte2(a), nm0), fmaf(dl0, ubyte3(a), nm0));
-        hi[2 * i] = pack_bf16(fmaf(dl1, ubyte0(b), nm1), fmaf(dl1, ubyte1(b), nm1));
-        hi[2 * i + 1] = pack_bf16(fmaf(dl1, ubyte2(b), nm1), fmaf(dl1, ubyte3(b), nm1));
+        wv[2 * i] = pack_bf16(fmaf(dl0, ubyte0(a), nm0), fmaf(dl0, ubyte1(a), nm0));
+        wv[2 * i + 1] = pack_bf16(fmaf(dl0, ubyte2(a), nm0), fmaf(dl0, ubyte3(a), nm0));
+        wv[8 + 2 * i] = pack_bf16(fmaf(dl1, ubyte0(b), nm1), fmaf(dl1, ubyte1(b), nm1));
+        wv[8 + 2 * i + 1] = pack_bf16(fmaf(dl1, ubyte2(b), nm1), fmaf(dl1, ubyte3(b), nm1));
     }
+}
+__device__ __forceinline__ void q4k_chunk_store(const TileCtx& c, const ProducerLane& l, int buf, const uint32_t* wv) {
     bf16_t* dst = c.bs + buf * kBTile + (l.ptid >> 1) * kLdsStride + (l.ptid & 1) * 16;
-    *(uint4*)(dst) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-    *(uint4*)(dst + 8) = make_uint4(lo[4], lo[5], lo[6], lo[7]);
-    *(uint4*)(dst + 32) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-    *(uint4*)(dst + 40) = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+    *(uint4*)(dst) = make_uint4(wv[0], wv[1], wv[2], wv[3]);
+    *(uint4*)(dst + 8) = make_uint4(wv[4], wv[5], wv[6], wv[7]);
+    *(uint4*)(dst + 32) = make_uint4(wv[8], wv[9], wv[10], wv[11]);
+    *(uint4*)(dst + 40) = make_uint4(wv[12], wv[13], wv[14], wv[15]);
 }
 
-template <int QT, int MODE>
+// One producer quartet (256 lanes).  Barrier b closes the phase in which step b must reach LDS (A
+// stage (b + base) % 3 when the direct path is off, W buffer (b + base) & 1); the MFMAs of step b run
+// after it.  Quartet Q takes the steps of parity Q: it decodes step u into registers during phase
+// u - 1 (step 0: before the first phase) and stores them during phase u.  steps + 1 barriers in all.
+// The phase sequence is written out per period (no data-dependent branches between a load and its
+// use), so that the waits on the packed-weight loads stay exact instead of draining every load.
+template <int QT, int MODE, int Q>
 __device__ __forceinline__ void produce(const MmqParams& p, const TileCtx& c, int ptid, int pw) {
     ProducerLane l;
     l.ptid = ptid, l.pw = pw, l.lane = ptid & 63;
     // W run owned by this lane: NT -> (output column n = col0 + ptid/2, run 2*step + ptid%2);
-    //                           NN -> (contraction row n = kc0 + lane, run col0/32 + producer wave).
+    //                           NN -> (contraction row n = kc0 + lane, run col0/32 + wave of the quartet).
     l.w_ksub_nn = min((c.col0 >> 5) + pw, (p.k >> 5) - 1);
     l.w_row_nt = min(c.col0 + (ptid >> 1), p.n - 1);
     const int steps = c.total_steps;
-    // Phase u fills step u (W tile into buffer (u + base) & 1, and the A tile when the direct path is
-    // off) and ends at a barrier; the MFMAs of step u run during phase u + 1.  A last barrier-only
-    // phase keeps the count equal to the consumers' (steps + 1).
+    constexpr bool kChunked = QT == kQ4_K && MODE == kModeNT;
+    uint32_t wv[16];
     int stage = c.base, buf = c.base;
     auto close_phase = [&]() __attribute__((always_inline)) {
         lds_barrier();
         stage = stage == kAStages - 1 ? 0 : stage + 1;
         buf ^= 1;
     };
-    if (QT == kQ4_K && MODE == kModeNT) {
+    auto store = [&](int u) __attribute__((always_inline)) {
+        if (!c.a_fast) fill_a_slow<MODE>(p, c, l, u, stage);
+        if (kChunked) q4k_chunk_store(c, l, buf, wv);
+        else w_store_run<MODE>(c, l, buf, wv);
+    };
+    // Decoded values are fenced the same way: the decode belongs in front of the barrier that follows it.
+    auto pin_decoded = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) asm volatile("" : "+v"(wv[i]));
+    };
+    if (kChunked) {
+        // K is a whole number of 256-wide blocks: four steps per block, this quartet's are Q and Q + 2.
+        // Two register sets alternate between blocks; a set is loaded four phases before its first use.
         const uint8_t* wrow = p.w[c.seg_c] + c.expert * p.w_expert_bytes + (int64_t)l.w_row_nt * p.w_row_bytes;
-        const int h = ptid & 1, blocks = steps >> 2;  // K is a whole number of 256-wide blocks
-        // Two register sets, used by even and odd blocks: a set is reloaded (block + 2) right after its
-        // last use, four steps before its next one.
+        const int h = ptid & 1, blocks = steps >> 2;
         Q4KChunk even, odd;
-        q4k_chunk_load(even, wrow, 0, h);
-        if (blocks > 1) q4k_chunk_load(odd, wrow, 1, h);
-        auto block_phases = [&](Q4KChunk& ch, int b) __attribute__((always_inline)) {
-            if (!c.a_fast) fill_a_slow<MODE>(p, c, l, 4 * b, stage);
-            q4k_chunk_fill<0>(c, l, buf, ch);
-            close_phase();
-            if (!c.a_fast) fill_a_slow<MODE>(p, c, l, 4 * b + 1, stage);
-            q4k_chunk_fill<1>(c, l, buf, ch);
-            close_phase();
-            if (!c.a_fast) fill_a_slow<MODE>(p, c, l, 4 * b + 2, stage);
-            q4k_chunk_fill<2>(c, l, buf, ch);
-            close_phase();
-            if (!c.a_fast) fill_a_slow<MODE>(p, c, l, 4 * b + 3, stage);
-            q4k_chunk_fill<3>(c, l, buf, ch);
-            if (b + 2 < blocks) q4k_chunk_load(ch, wrow, b + 2, h);
-            close_phase();
+        q4k_chunk_load(even, wrow, 0, h, Q);
+        if (Q == 0) {
+            q4k_chunk_decode<0>(even.hdr, even.qa, wv);
+            pin_decoded();
+        }
+        // block k: `cur` holds its packed bytes, `nxt` receives those of block k + 1
+        auto block_phases = [&](Q4KChunk& cur, Q4KChunk& nxt, int k) __attribute__((always_inline)) {
+            const bool more = k + 1 < blocks;
+            if (Q == 0) {
+                store(4 * k);
+                if (more) q4k_chunk_load(nxt, wrow, k + 1, h, Q);
+                close_phase();
+                q4k_chunk_pin(cur);
+                q4k_chunk_decode<2>(cur.hdr, cur.qb, wv);
+                pin_decoded();
+                close_phase();
+                store(4 * k + 2);
+                close_phase();
+                if (more) {
+                    q4k_chunk_pin(nxt);
+                    q4k_chunk_decode<0>(nxt.hdr, nxt.qa, wv);
+                    pin_decoded();
+                }
+                close_phase();
+            } else {
+                q4k_chunk_pin(cur);
+                q4k_chunk_decode<1>(cur.hdr, cur.qa, wv);
+                pin_decoded();
+                if (more) q4k_chunk_load(nxt, wrow, k + 1, h, Q);
+                close_phase();
+                store(4 * k + 1);
+                close_phase();
+                q4k_chunk_pin(cur);
+                q4k_chunk_decode<3>(cur.hdr, cur.qb, wv);
+                pin_decoded();
+                close_phase();
+                store(4 * k + 3);
+                close_phase();
+            }
         };
-        for (int b = 0; b < blocks; b += 2) {
-            block_phases(even, b);
-            if (b + 1 < blocks) block_phases(odd, b + 1);
+        for (int k = 0; k < blocks; k += 2) {
+            block_phases(even, odd, k);
+            if (k + 1 < blocks) block_phases(odd, even, k + 1);
         }
     } else {
-        // Register ring: the loads of step u + kLoadDepth are issued as soon as step u is decoded.
-        typename Fmt<QT>::Raw w_ring[kLoadDepth];
-#pragma unroll
-        for (int j = 0; j < kLoadDepth; j++)
-            if (j < steps) w_issue_run<QT, MODE>(p, c, l, j, w_ring[j]);
-        auto phase = [&](auto slot_c, int u) __attribute__((always_inline)) {
-            constexpr int J = decltype(slot_c)::value;
-            if (!c.a_fast) fill_a_slow<MODE>(p, c, l, u, stage);
-            w_fill_run<QT, MODE>(c, l, u, buf, w_ring[J]);
-            if (u + kLoadDepth < steps) w_issue_run<QT, MODE>(p, c, l, u + kLoadDepth, w_ring[J]);
-            close_phase();
+        // Two register sets alternate between this quartet's steps (u = Q, Q + 2, ...): the packed run of
+        // step u + 4 is requested as soon as step u is decoded, three phases before its own decode.
+        typename Fmt<QT>::Raw raw_a, raw_b;
+        auto decode = [&](typename Fmt<QT>::Raw& raw, int u) __attribute__((always_inline)) {
+            if (u >= steps) return;
+            Fmt<QT>::pin(raw);
+            Fmt<QT>::decode(raw, MODE == kModeNT ? 2 * u + (l.ptid & 1) : l.w_ksub_nn, wv, c.grid);
+            pin_decoded();
+            if (u + 4 < steps) w_issue_run<QT, MODE>(p, c, l, u + 4, raw);
         };
-        static_assert(kLoadDepth == 3, "the phase loop below is unrolled for a ring of three");
-        for (int u = 0; u < steps; u += 3) {
-            phase(std::integral_constant<int, 0>{}, u);
-            if (u + 1 < steps) phase(std::integral_constant<int, 1>{}, u + 1);
-            if (u + 2 < steps) phase(std::integral_constant<int, 2>{}, u + 2);
+        if (Q < steps) w_issue_run<QT, MODE>(p, c, l, Q, raw_a);
+        if (Q + 2 < steps) w_issue_run<QT, MODE>(p, c, l, Q + 2, raw_b);
+        if (Q == 0) {
+            decode(raw_a, 0);
+            for (int b = 0; b < steps; b += 4) {
+                store(b);
+                close_phase();
+                if (b + 1 < steps) {
+                    decode(raw_b, b + 2);
+                    close_phase();
+                }
+                if (b + 2 < steps) {
+                    store(b + 2);
+                    close_phase();
+                }
+                if (b + 3 < steps) {
+                    decode(raw_a, b + 4);
+                    close_phase();
+                }
+            }
+        } else {
+            for (int b = 0; b < steps; b += 4) {
+                decode(raw_a, b + 1);
+                close_phase();
+                if (b + 1 < steps) {
+                    store(b + 1);
+                    close_phase();
+                }
+                if (b + 2 < steps) {
+                    decode(raw_b, b + 3);
+                    close_phase();
+                }
+                if (b + 3 < steps) {
+                    store(b + 3);
+                    close_phase();
+                }
+            }
         }
     }
     lds_barrier();
@@ -352,7 +426,7 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
         for (int j = 0; j < kColBlocks; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
-    // this lane's A row inside a 64-row pair of blocks, and the swizzled slot of each sub-step's chunk
+    // this lane's A row inside a 128-row half of the tile, and the swizzled slot of each sub-step's chunk
     const uint8_t* a_row = c.as + (32 * wave_m + lane_c) * kARowBytes;
     int a_koff[4];
 #pragma unroll
@@ -369,18 +443,7 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
 #pragma unroll
         for (int cb = 0; cb < kColBlocks; cb++) o.b[cb] = *(const bf16x8_t*)(b_lds + cb * 32 * kLdsStride);
 #pragma unroll
-        for (int rb = 0; rb < LIVE; rb++) o.a[rb] = *(const bf16x8_t*)(a_lds + rb * 64 * kARowBytes);
-    };
-    auto mfma_rows = [&](const Operands& o, int rb0, int rb1) __attribute__((always_inline)) {
-#pragma unroll
-        for (int rb = 0; rb < LIVE; rb++)
-            if (rb >= rb0 && rb < rb1)
-#pragma unroll
-                for (int cb = 0; cb < kColBlocks; cb++)
-                    acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.a[rb], o.b[cb], acc[rb][cb], 0, 0, 0);
-    };
-    auto mfma_one = [&](const Operands& o, int rb, int cb) __attribute__((always_inline)) {
-        acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.a[rb], o.b[cb], acc[rb][cb], 0, 0, 0);
+        for (int rb = 0; rb < LIVE; rb++) o.a[rb] = *(const bf16x8_t*)(a_lds + rb * 128 * kARowBytes);
     };
     auto mfma_operands = [&](const Operands& o) __attribute__((always_inline)) {
 #pragma unroll
@@ -390,9 +453,6 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
                 acc[rb][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.a[rb], o.b[cb], acc[rb][cb], 0, 0, 0);
     };
 
-    // The MFMA stream must win issue arbitration against the producer wave on the same SIMD: a matrix
-    // instruction only needs an issue slot every 32 cycles, the decoder's VALU stream fills the rest.
-    __builtin_amdgcn_s_setprio(3);
     AIssuer ai;
     a_loader_init(ai.ld, p, c, lane, cw);
     ai.next_step = 0, ai.next_stage = c.base;
@@ -420,31 +480,20 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
     // Main steps, software pipelined inside the wave: the operands of sub-step k+1 are read from LDS
     // while the MFMAs of sub-step k run, and the barrier that releases the buffers sits between the last
     // LDS read of a step and its last MFMAs, so the first read of the next step hides behind them.
-    // Step t lives in A stage (t + base) % 3 and W buffer (t + base) & 1.
-    // The scheduler would otherwise sink the reads to the end of the stage (they reuse the registers of
-    // the running MFMAs' operands): pin "all LDS reads of the stage, then its MFMAs".
-    // A wave gets one 16-byte-per-lane LDS read through roughly every 32 cycles, the same cadence as its
-    // MFMAs, and a read that cannot issue holds up the MFMAs queued behind it: reads and MFMAs alternate
-    // one by one.  The last row block's two MFMAs frame the two A-tile loads of the stage.
+    // Step t lives in A stage (t + base) % 3 and W buffer (t + base) & 1.  A wave gets one
+    // 16-byte-per-lane LDS read through roughly every 32 cycles, the same cadence as its MFMAs: reads
+    // and MFMAs alternate one by one; each sub-step also issues one group of the A tile of step t + 2.
 #define GGQ_MFMA_READ_PAIRS()                                                                              \
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); \
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); \
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); \
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); \
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); \
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); \
-    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                                                     \
     __builtin_amdgcn_sched_barrier(0)
-#define GGQ_STAGE(NEXT, CUR, KK, J0)                          \
-    load_operands(NEXT, stage, buf, KK);                      \
-    mfma_rows(CUR, 0, LIVE - 1);                              \
-    GGQ_MFMA_READ_PAIRS();                                    \
-    a_issue_part<MODE, J0, J0 + 1>(ai, p, c);                 \
-    mfma_one(CUR, LIVE - 1, 0);                               \
-    __builtin_amdgcn_sched_barrier(0);                        \
-    a_issue_part<MODE, J0 + 1, J0 + 2>(ai, p, c);             \
-    mfma_one(CUR, LIVE - 1, 1);                               \
-    __builtin_amdgcn_sched_barrier(0)
+#define GGQ_STAGE(NEXT, CUR, KK, J)            \
+    a_issue_part<MODE, J, J + 1>(ai, p, c);    \
+    load_operands(NEXT, stage, buf, KK);       \
+    mfma_operands(CUR);                        \
+    GGQ_MFMA_READ_PAIRS()
     {
         const int steps = c.total_steps;
         int stage = c.base, buf = c.base;
@@ -452,24 +501,23 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
         load_operands(x, stage, buf, 0);
         for (int t = 0; t < steps; t++) {  // the A loads issued in here are those of step t + 2
             GGQ_STAGE(y, x, 1, 0);
-            GGQ_STAGE(x, y, 2, 2);
-            GGQ_STAGE(y, x, 3, 4);
-            a_issue_part<MODE, 6, 8>(ai, p, c);
+            GGQ_STAGE(x, y, 2, 1);
+            GGQ_STAGE(y, x, 3, 2);
+            a_issue_part<MODE, 3, 4>(ai, p, c);
             a_issue_advance(ai);
             a_wait_step(ai, c, t + 1);
             lds_barrier();  // every LDS read of this step has landed; its stage and buffer may be refilled
             stage = stage == kAStages - 1 ? 0 : stage + 1;
             buf ^= 1;
             if (t + 1 < steps) load_operands(x, stage, buf, 0);
-            mfma_rows(y, 0, LIVE);
+            mfma_operands(y);
             GGQ_MFMA_READ_PAIRS();
         }
     }
 #undef GGQ_MFMA_READ_PAIRS
 #undef GGQ_STAGE
-    __builtin_amdgcn_s_setprio(0);
 
-    // ---- epilogue.  acc[rb][cb][i]: tile row = 32*(2*rb + wave_m) + 8*(i/4) + 4*lane_h + (i%4),
+    // ---- epilogue.  acc[rb][cb][i]: tile row = 32*(4*rb + wave_m) + 8*(i/4) + 4*lane_h + (i%4),
     //                                 tile col = 64*wave_n + 32*cb + lane_c
     const int col_base = c.col0 + wave_n * 64 + lane_c;
     if (EPI == kEpiStore || EPI == kEpiAccumF32 || EPI == kEpiCeGrad) {
@@ -477,7 +525,7 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
         for (int rb = 0; rb < LIVE; rb++) {
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                const int r = 32 * (2 * rb + wave_m) + (i >> 2) * 8 + lane_h * 4 + (i & 3);
+                const int r = 32 * (4 * rb + wave_m) + (i >> 2) * 8 + lane_h * 4 + (i & 3);
                 if (r >= c.rows_valid) continue;
                 const int64_t grow = c.row_begin + r;
                 float lse = 0.f, rs = 0.f;
@@ -510,7 +558,7 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
         for (int rb = 0; rb < LIVE; rb++) {
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                const int r = 32 * (2 * rb + wave_m) + (i >> 2) * 8 + lane_h * 4 + (i & 3);
+                const int r = 32 * (4 * rb + wave_m) + (i >> 2) * 8 + lane_h * 4 + (i & 3);
                 const bool row_ok = r < c.rows_valid;
                 const int64_t grow = c.row_begin + (row_ok ? r : 0);
                 const int64_t label = row_ok ? p.labels[grow] : -1;
@@ -538,8 +586,8 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
     }
 }
 
-// A wave of the consumer quartet without a live row block still moves its share of the A tile and
-// keeps the barriers company.
+// A consumer wave without a live row block still moves its share of the A tile and keeps the
+// barriers company.
 template <int MODE>
 __device__ __forceinline__ void consume_idle(const MmqParams& p, const TileCtx& c, int lane, int cw) {
     AIssuer ai;
@@ -557,7 +605,7 @@ __device__ __forceinline__ void consume_idle(const MmqParams& p, const TileCtx& 
 }
 
 template <int QT, int MODE, int EPI>
-__global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(2, 2))) void mmq_tile_kernel(const MmqParams p) {
+__global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(4, 4))) void mmq_tile_kernel(const MmqParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_raw[];
     TileCtx c;
     c.as = smem_raw;
@@ -568,7 +616,6 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(2, 
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps control flow scalar
-    const int cw = wave & 3;  // index inside the consumer / producer quartet
 
     // ---- tile assignment.  Hardware deals consecutive workgroup ids round-robin over the 8 XCDs; remap
     // so that consecutive logical tiles (which share an A tile) land on one XCD and hit its L2.
@@ -622,18 +669,18 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(2, 
     }
     __syncthreads();  // LoRA tiles and the codebook are visible
 
-    if (wave >= 4) {
-        produce<QT, MODE>(p, c, tid & 255, cw);
+    if (wave >= 8) {
+        if (wave < 12) produce<QT, MODE, 0>(p, c, tid & 255, wave & 3);
+        else produce<QT, MODE, 1>(p, c, tid & 255, wave & 3);
     } else {
-        const int wave_m = cw >> 1;
-        // this wave's row block i covers tile rows 32*(2*i + wave_m) .. +31; blocks fill up from row 0
-        const int live = c.rows_valid > 32 * wave_m ? min(kRowBlocks, (c.rows_valid - 32 * wave_m + 63) >> 6) : 0;
+        const int cw = wave, wave_m = cw >> 1;
+        // this wave's row blocks are tile rows 32*wave_m .. +31 and 32*(wave_m + 4) .. +31; blocks fill up from row 0
+        const int blocks = (c.rows_valid + 31) >> 5;
+        const int live = (blocks > wave_m ? 1 : 0) + (blocks > wave_m + 4 ? 1 : 0);
         switch (live) {
             case 0: consume_idle<MODE>(p, c, lane, cw); break;
             case 1: consume<QT, MODE, EPI, 1>(p, c, lane, cw); break;
-            case 2: consume<QT, MODE, EPI, 2>(p, c, lane, cw); break;
-            case 3: consume<QT, MODE, EPI, 3>(p, c, lane, cw); break;
-            default: consume<QT, MODE, EPI, 4>(p, c, lane, cw); break;
+            default: consume<QT, MODE, EPI, 2>(p, c, lane, cw); break;
         }
     }
 }
