@@ -494,7 +494,26 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
     load_operands(NEXT, stage, buf, KK);       \
     mfma_operands(CUR);                        \
     GGQ_MFMA_READ_PAIRS()
-    {
+    if (LIVE == 1) {
+        // One live row block: two MFMAs per sub-step are too few to hide the LDS latency of the next
+        // sub-step's reads, so all twelve reads of the step go out at once behind the barrier and the
+        // MFMAs follow them as they land.
+        const int steps = c.total_steps;
+        int stage = c.base, buf = c.base;
+        for (int t = 0; t < steps; t++) {  // the A loads issued in here are those of step t + 2
+            a_issue_part<MODE, 0, kGroupsPerWave>(ai, p, c);
+            a_issue_advance(ai);
+            Operands o[4];
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) load_operands(o[kk], stage, buf, kk);
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) mfma_operands(o[kk]);
+            a_wait_step(ai, c, t + 1);
+            lds_barrier();
+            stage = stage == kAStages - 1 ? 0 : stage + 1;
+            buf ^= 1;
+        }
+    } else {
         const int steps = c.total_steps;
         int stage = c.base, buf = c.base;
         Operands x, y;
