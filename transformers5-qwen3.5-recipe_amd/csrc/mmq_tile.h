@@ -540,34 +540,45 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
     //                                 tile col = 64*wave_n + 32*cb + lane_c
     const int col_base = c.col0 + wave_n * 64 + lane_c;
     if (EPI == kEpiStore || EPI == kEpiAccumF32 || EPI == kEpiCeGrad) {
+        // everything that does not depend on the element is read once, up front
+        const int64_t ldc = p.ldc;
+        char* const cbase = (char*)p.c[EPI == kEpiStore ? c.seg_c : 0];
+        const float* const lse_p = p.lse;
+        const float* const rs_p = p.row_scale;
+        const int64_t* const labels_p = p.labels;
+        const int64_t ce_off = p.ce_col_offset;
+        const int rows_valid = c.rows_valid;
+        const bool col_ok[kColBlocks] = {col_base < c.out_cols, col_base + 32 < c.out_cols};
 #pragma unroll
         for (int rb = 0; rb < LIVE; rb++) {
+            const int r_lane = 32 * (4 * rb + wave_m) + lane_h * 4;  // this lane's first row of the block
+            const int64_t lane_elem = (int64_t)(c.row_begin + r_lane) * ldc + col_base;
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                const int r = 32 * (4 * rb + wave_m) + (i >> 2) * 8 + lane_h * 4 + (i & 3);
-                if (r >= c.rows_valid) continue;
-                const int64_t grow = c.row_begin + r;
+                const int dr = (i >> 2) * 8 + (i & 3);  // uniform row step inside the block
+                if (r_lane + dr >= rows_valid) continue;
+                const int64_t elem = lane_elem + (int64_t)dr * ldc;
                 float lse = 0.f, rs = 0.f;
                 int64_t label = -1;
                 if (EPI == kEpiCeGrad) {
-                    lse = p.lse[grow];
-                    rs = p.row_scale[grow];
-                    label = p.labels[grow];
+                    const int64_t grow = c.row_begin + r_lane + dr;
+                    lse = lse_p[grow];
+                    rs = rs_p[grow];
+                    label = labels_p[grow];
                 }
 #pragma unroll
                 for (int cb = 0; cb < kColBlocks; cb++) {
-                    const int col = col_base + cb * 32;
-                    if (col >= c.out_cols) continue;
+                    if (!col_ok[cb]) continue;
                     const float v = acc[rb][cb][i];
                     if (EPI == kEpiStore) {
-                        ((bf16_t*)p.c[c.seg_c])[grow * p.ldc + col] = to_bf16(v);
+                        ((bf16_t*)cbase)[elem + cb * 32] = to_bf16(v);
                     } else if (EPI == kEpiAccumF32) {
-                        ((float*)p.c[0])[grow * p.ldc + col] += v;
+                        ((float*)cbase)[elem + cb * 32] += v;
                     } else {
                         const float logit = bf16_to_f32(to_bf16(v));  // the path's logits are bf16 values
                         float g = __expf(logit - lse);
-                        if ((int64_t)(col + p.ce_col_offset) == label) g -= 1.0f;
-                        ((bf16_t*)p.c[0])[grow * p.ldc + col] = to_bf16(g * rs);
+                        if ((int64_t)(col_base + cb * 32) + ce_off == label) g -= 1.0f;
+                        ((bf16_t*)cbase)[elem + cb * 32] = to_bf16(g * rs);
                     }
                 }
             }
