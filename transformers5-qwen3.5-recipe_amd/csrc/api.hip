@@ -62,6 +62,11 @@ int ggq_dequantize(int qt, const void* packed, int64_t rows, int64_t k, void* ou
 }
 
 // ---------------------------------------------------------------------------------------------------
+// Expert groups that average at most 192 rows run the Q4_K tile kernel in its wide shape.
+static int pick_shape(int qt, int64_t rows, int64_t groups) {
+    return (qt == 12 /* GGML Q4_K */ && groups > 0 && rows <= 192 * groups) ? kShapeWide : kShapeTall;
+}
+
 int64_t ggq_lora_workspace_bytes(int64_t rows, int64_t groups, int64_t experts, int64_t n_total, int64_t k, int r) {
     const int rp = rank_pad(r > 0 ? r : 1);
     if (experts < 1) experts = 1;
@@ -115,7 +120,7 @@ int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void*
     Bump bump{(char*)ws, ws_bytes, 0};
 
     MmqParams p;
-    if (int rc = init_params(p, qt, kModeNT, (int)rows, (int)n, (int)k, nseg)) return rc;
+    if (int rc = init_params(p, qt, kModeNT, (int)rows, (int)n, (int)k, nseg, pick_shape(qt, rows, groups))) return rc;
     p.a[0] = (const bf16_t*)x, p.lda = k;
     p.w[0] = (const uint8_t*)packed1, p.w[1] = (const uint8_t*)packed2;
     p.c[0] = y1, p.c[1] = y2, p.ldc = n;
@@ -124,13 +129,14 @@ int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void*
     const int* num_tiles64 = nullptr;
     int max_tiles64 = (int)((rows + 63) / 64);
     if (groups > 0) {
-        const int max128 = (int)(rows / kBM + groups);
+        const int tile_rows = p.shape == kShapeWide ? kWideBM : kBM;
+        const int max128 = (int)(rows / tile_rows + groups);
         max_tiles64 = (int)(rows / 64 + groups);
         TileDesc* t128 = (TileDesc*)bump.take((int64_t)max128 * sizeof(TileDesc));
         TileDesc* t64 = lora_a ? (TileDesc*)bump.take((int64_t)max_tiles64 * sizeof(TileDesc)) : nullptr;
         int* counts = (int*)bump.take(16);
         if (!t128 || !counts || (lora_a && !t64)) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
-        if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, kBM, t128, counts, nullptr, 0, s)) return rc;
+        if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, tile_rows, t128, counts, nullptr, 0, s)) return rc;
         if (lora_a) {
             if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, 64, t64, counts + 1, nullptr, 0, s)) return rc;
         }
@@ -180,7 +186,7 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
     Bump bump{(char*)ws, ws_bytes, 0};
 
     MmqParams p;
-    if (int rc = init_params(p, qt, kModeNN, (int)rows, (int)n, (int)k, nseg)) return rc;
+    if (int rc = init_params(p, qt, kModeNN, (int)rows, (int)n, (int)k, nseg, pick_shape(qt, rows, groups))) return rc;
     p.a[0] = (const bf16_t*)dy1, p.a[1] = (const bf16_t*)dy2, p.lda = n;
     p.w[0] = (const uint8_t*)packed1, p.w[1] = (const uint8_t*)packed2;
     p.c[0] = dx, p.ldc = k;
@@ -190,14 +196,15 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
     const int* ranges = nullptr;
     int max_tiles64 = (int)((rows + 63) / 64);
     if (groups > 0) {
-        const int max128 = (int)(rows / kBM + groups);
+        const int tile_rows = p.shape == kShapeWide ? kWideBM : kBM;
+        const int max128 = (int)(rows / tile_rows + groups);
         max_tiles64 = (int)(rows / 64 + groups);
         TileDesc* t128 = (TileDesc*)bump.take((int64_t)max128 * sizeof(TileDesc));
         TileDesc* t64 = lora_a ? (TileDesc*)bump.take((int64_t)max_tiles64 * sizeof(TileDesc)) : nullptr;
         int* counts = (int*)bump.take(16);
         int* rg = lora_a ? (int*)bump.take(experts * 2 * 4) : nullptr;
         if (!t128 || !counts || (lora_a && (!t64 || !rg))) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
-        if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, kBM, t128, counts, rg, (int)experts, s)) return rc;
+        if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, tile_rows, t128, counts, rg, (int)experts, s)) return rc;
         if (lora_a) {
             if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, 64, t64, counts + 1, nullptr, 0, s)) return rc;
         }

@@ -110,7 +110,7 @@ int profile_end(float* ms, int* qt, int* mode, int* epi, int capacity) {
     return n;
 }
 
-template <int QT, int MODE, int EPI>
+template <int QT, int MODE, int EPI, int SH>
 static int launch_one(const MmqParams& p, hipStream_t s) {
     const int col_tiles = (MODE == kModeNT ? p.nseg : 1) * p.col_tiles_per_seg;
     const int64_t total = (int64_t)p.max_row_tiles * col_tiles;
@@ -125,14 +125,14 @@ static int launch_one(const MmqParams& p, hipStream_t s) {
         g_timed_count++;
         (void)hipEventRecord(t->start, s);
     }
-    constexpr int kSmemBytes = kTileLdsBytes + (QT == kIQ2_XXS ? 2048 : 0);
+    constexpr int kSmemBytes = Tile<SH>::kTileLdsBytes + (QT == kIQ2_XXS ? 2048 : 0);
     static bool attr_set = false;  // per instantiation; the attribute is a property of the function
     if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)mmq_tile_kernel<QT, MODE, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess)
+        if (hipFuncSetAttribute((const void*)mmq_tile_kernel<QT, MODE, EPI, SH>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess)
             return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", kSmemBytes);
         attr_set = true;
     }
-    hipLaunchKernelGGL((mmq_tile_kernel<QT, MODE, EPI>), dim3((unsigned)grid), dim3(kThreads), kSmemBytes, s, p);
+    hipLaunchKernelGGL((mmq_tile_kernel<QT, MODE, EPI, SH>), dim3((unsigned)grid), dim3(kThreads), kSmemBytes, s, p);
     if (t) (void)hipEventRecord(t->stop, s);
     return check_launch("mmq_tile_kernel");
 }
@@ -141,14 +141,18 @@ template <int QT>
 static int launch_qt(int mode, int epi, const MmqParams& p, hipStream_t s) {
     if (mode == kModeNT) {
         switch (epi) {
-            case kEpiStore: return launch_one<QT, kModeNT, kEpiStore>(p, s);
-            case kEpiCeStats: return launch_one<QT, kModeNT, kEpiCeStats>(p, s);
-            case kEpiCeGrad: return launch_one<QT, kModeNT, kEpiCeGrad>(p, s);
+            case kEpiStore:
+                if (QT == kQ4_K && p.shape == kShapeWide) return launch_one<kQ4_K, kModeNT, kEpiStore, 1>(p, s);
+                return launch_one<QT, kModeNT, kEpiStore, 0>(p, s);
+            case kEpiCeStats: return launch_one<QT, kModeNT, kEpiCeStats, 0>(p, s);
+            case kEpiCeGrad: return launch_one<QT, kModeNT, kEpiCeGrad, 0>(p, s);
         }
     } else {
         switch (epi) {
-            case kEpiStore: return launch_one<QT, kModeNN, kEpiStore>(p, s);
-            case kEpiAccumF32: return launch_one<QT, kModeNN, kEpiAccumF32>(p, s);
+            case kEpiStore:
+                if (QT == kQ4_K && p.shape == kShapeWide) return launch_one<kQ4_K, kModeNN, kEpiStore, 1>(p, s);
+                return launch_one<QT, kModeNN, kEpiStore, 0>(p, s);
+            case kEpiAccumF32: return launch_one<QT, kModeNN, kEpiAccumF32, 0>(p, s);
         }
     }
     return set_error(GGQ_ERR_SHAPE, "mmq: unsupported mode/epilogue combination");
@@ -165,7 +169,7 @@ int launch_mmq(int qt, int mode, int epi, const MmqParams& p, hipStream_t s) {
 }
 
 // Fills the shape-derived fields of a parameter block.  n, k describe one weight segment [n, k].
-int init_params(MmqParams& p, int qt, int mode, int m, int n, int k, int nseg) {
+int init_params(MmqParams& p, int qt, int mode, int m, int n, int k, int nseg, int shape) {
     if (m < 0 || n <= 0 || k <= 0) return set_error(GGQ_ERR_SHAPE, "mmq: bad shape m=%d n=%d k=%d", m, n, k);
     if (packed_row_bytes(qt, k) < 0) return set_error(GGQ_ERR_QTYPE, "unsupported GGML type id %d", qt);
     if (!block_multiple(qt, k)) return set_error(GGQ_ERR_SHAPE, "mmq: K=%d is not a multiple of the block size of type %d", k, qt);
@@ -174,14 +178,17 @@ int init_params(MmqParams& p, int qt, int mode, int m, int n, int k, int nseg) {
     p.m = m, p.n = n, p.k = k, p.nseg = nseg;
     p.w_row_bytes = packed_row_bytes(qt, k);
     p.w_expert_bytes = p.w_row_bytes * n;
+    if (shape == kShapeWide && qt != kQ4_K) shape = kShapeTall;  // the wide instantiation exists for Q4_K only
+    const int bm = shape == kShapeWide ? kWideBM : kBM, bn = shape == kShapeWide ? kWideBN : kBN;
+    p.shape = shape;
     if (mode == kModeNT) {
-        p.col_tiles_per_seg = (n + kBN - 1) / kBN;
+        p.col_tiles_per_seg = (n + bn - 1) / bn;
         p.steps_per_seg = k / kBK;
     } else {
-        p.col_tiles_per_seg = (k + kBN - 1) / kBN;
+        p.col_tiles_per_seg = (k + bn - 1) / bn;
         p.steps_per_seg = (n + kBK - 1) / kBK;
     }
-    p.max_row_tiles = (m + kBM - 1) / kBM;
+    p.max_row_tiles = (m + bm - 1) / bm;
     return GGQ_OK;
 }
 

@@ -34,7 +34,9 @@ struct FactorGradParams {
     float scale;
 };
 
-constexpr int kBM = 256, kBN = 128, kBK = 64;
+constexpr int kBM = 256, kBN = 128, kBK = 64;  // the tall tile shape (dense launches, large expert groups)
+constexpr int kWideBM = 128, kWideBN = 256;    // the wide tile shape (Q4_K expert groups of about a hundred rows)
+constexpr int kShapeTall = 0, kShapeWide = 1;
 constexpr int kLdsStride = kBK + 8;  // bf16 elements per LDS row: 144 bytes keeps 128-bit reads conflict-free
 constexpr int kThreads = 1024;  // waves 0..7 run the MFMAs, waves 8..15 load and decode
 
@@ -62,6 +64,7 @@ struct MmqParams {
     const TileDesc* tiles;
     const int* num_tiles;
     int max_row_tiles;
+    int shape;  // kShapeTall / kShapeWide: which instantiation of the tile kernel the sizes above are for
     // LoRA
     const bf16_t* la;     // [rows, r_pad]  (x A^T in NT, dY B in NN)
     const bf16_t* lb;     // per expert [cols_total, r_pad] (B rows in NT, A^T rows in NN)
@@ -83,7 +86,7 @@ int profile_begin();
 int profile_end(float* ms, int* qt, int* mode, int* epi, int capacity);
 const char* last_error();
 int launch_mmq(int qt, int mode, int epi, const MmqParams& p, hipStream_t s);
-int init_params(MmqParams& p, int qt, int mode, int m, int n, int k, int nseg);
+int init_params(MmqParams& p, int qt, int mode, int m, int n, int k, int nseg, int shape = kShapeTall);
 
 int pad_factor(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int r, int r_pad, bool transpose, hipStream_t s);
 int transpose_factor(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int r, hipStream_t s);

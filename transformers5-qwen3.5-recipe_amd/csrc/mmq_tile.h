@@ -38,17 +38,13 @@ namespace ggq {
 
 static __device__ const uint64_t d_iq2xxs_grid_mm[256] = GGQ_IQ2XXS_GRID_INIT;
 
-constexpr int kRowBlocks = kBM / 128;           // 32-row MFMA blocks per consumer wave (2): wave_m, wave_m + 4
-constexpr int kColBlocks = kBN / 64;            // 32-column MFMA blocks per consumer wave (2)
+constexpr int kColBlocks = 2;                   // 32-column MFMA blocks per consumer wave
 constexpr int kAStages = 3;                     // LDS ring of A tiles
 constexpr int kARowBytes = kBK * 2;             // A rows are unpadded: 128 bytes = eight 16-byte slots
-constexpr int kAStageBytes = kBM * kARowBytes;  // 32 KB
-constexpr int kAGroups = kBM / 8;               // 8-row groups (one direct-to-LDS instruction each)
-constexpr int kBTile = kBN * kLdsStride;        // bf16 elements per W buffer (rows padded to 144 bytes)
-constexpr int kTileLdsBytes = kAStages * kAStageBytes + 2 * kBTile * 2;
-constexpr int kGroupsPerWave = kAGroups / 8;    // A-tile groups one consumer wave moves per step (4)
 
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));  // native vector: loads/stores stay typed
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef short v4i16_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4i16_t* lds_v4i16_ptr;  // native vector: loads/stores stay typed
 
 __device__ __forceinline__ uint4 zero4() { return make_uint4(0, 0, 0, 0); }
 
@@ -92,8 +88,8 @@ __device__ __forceinline__ uint4 load8_slow(const bf16_t* p, int valid) {
 struct TileCtx {  // wave-uniform description of the tile this workgroup computes
     int row_begin, rows_valid, col0, col_tile, seg_c, out_cols, contraction, total_steps, base;
     int64_t expert;
-    uint8_t* as;      // [kAStages][kAStageBytes]
-    bf16_t* bs;       // [2][kBTile]
+    uint8_t* as;      // [kAStages][A stage bytes]
+    bf16_t* bs;       // [2][W tile elements]
     uint32_t as_lds;  // LDS byte address of `as`
     bool a_fast;      // A rows can be moved with aligned 16-byte accesses and every step is whole
     const uint2* grid;
@@ -106,6 +102,23 @@ __device__ __forceinline__ void step_origin(const MmqParams& p, int step, int& s
     kc0 = (step - seg_k * p.steps_per_seg) * kBK;
 }
 
+// Everything below depends on the tile shape.  SH = 0: 256 x 128 ("tall": dense launches and expert
+// groups with many rows); SH = 1: 128 x 256 ("wide": expert groups of about a hundred rows, where two row
+// blocks per wave keep the LDS operand traffic at one read per MFMA and one decode of the weights serves
+// 256 output columns).  The eight consumer waves form a kWavesM x kWavesN grid; wave (wave_m, wave_n) owns
+// row blocks wave_m and wave_m + kWavesM and the 64 columns at 64 * wave_n.
+template <int SH>
+struct Tile {
+static constexpr int kTM = SH == 0 ? 256 : 128, kTN = SH == 0 ? 128 : 256;
+static constexpr int kWavesM = kTM / 64, kWavesN = kTN / 64;
+static constexpr int kAStageBytes = kTM * kARowBytes;   // 32 KB / 16 KB
+static constexpr int kAGroups = kTM / 8;                // 8-row groups (one direct-to-LDS instruction each)
+static constexpr int kGroupsPerWave = kAGroups / 8;     // groups one consumer wave moves per step (4 / 2)
+static constexpr int kBTile = kTN * kLdsStride;         // bf16 elements per W buffer
+static constexpr int kTileLdsBytes = kAStages * kAStageBytes + 2 * kBTile * 2;
+// grad-input W tile of the wide shape: [contraction row][output column], rows padded by 32 elements
+static constexpr int kNnPitch = kTN + 32;
+
 // ---- A tile, fast path: each of the eight waves of the consumer octet moves the 8-row groups
 // g = 8*j + cw (j = 0..3) with one direct-to-LDS instruction per group.
 struct ALoader {
@@ -114,7 +127,7 @@ struct ALoader {
     int n;                          // groups this wave moves per step (0 when the fast path is off)
 };
 
-__device__ __forceinline__ void a_loader_init(ALoader& a, const MmqParams& p, const TileCtx& c, int lane, int cw) {
+static __device__ __forceinline__ void a_loader_init(ALoader& a, const MmqParams& p, const TileCtx& c, int lane, int cw) {
     const int sub = 8 * cw + (lane >> 3);         // row inside a 64-row slab
     const int kc = (lane & 7) ^ ((sub >> 1) & 7);  // the chunk that belongs in this lane's LDS slot
 #pragma unroll
@@ -130,13 +143,13 @@ __device__ __forceinline__ void a_loader_init(ALoader& a, const MmqParams& p, co
 }
 
 template <int MODE, int J0, int J1>
-__device__ __forceinline__ void a_issue(const ALoader& a, const MmqParams& p, const TileCtx& c, int step, int stage) {
+static __device__ __forceinline__ void a_issue(const ALoader& a, const MmqParams& p, const TileCtx& c, int step, int stage) {
     int seg_k, kc0;
     step_origin<MODE>(p, step, seg_k, kc0);
     const bf16_t* sbase = p.a[MODE == kModeNN ? seg_k : 0] + (int64_t)c.row_begin * p.lda + kc0;
     const uint32_t lds = a.lds0 + stage * kAStageBytes;
 #pragma unroll
-    for (int j = J0; j < J1; j++)
+    for (int j = J0; j < J1 && j < kGroupsPerWave; j++)
         if (j < a.n)
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                          :
@@ -152,21 +165,21 @@ struct AIssuer {
     int next_step, next_stage;
 };
 template <int MODE, int J0, int J1>
-__device__ __forceinline__ void a_issue_part(const AIssuer& s, const MmqParams& p, const TileCtx& c) {
+static __device__ __forceinline__ void a_issue_part(const AIssuer& s, const MmqParams& p, const TileCtx& c) {
     if (s.next_step < c.total_steps) a_issue<MODE, J0, J1>(s.ld, p, c, s.next_step, s.next_stage);
 }
-__device__ __forceinline__ void a_issue_advance(AIssuer& s) {
+static __device__ __forceinline__ void a_issue_advance(AIssuer& s) {
     s.next_step++;
     s.next_stage = s.next_stage == kAStages - 1 ? 0 : s.next_stage + 1;
 }
 template <int MODE>
-__device__ __forceinline__ void a_issue_next(AIssuer& s, const MmqParams& p, const TileCtx& c) {
+static __device__ __forceinline__ void a_issue_next(AIssuer& s, const MmqParams& p, const TileCtx& c) {
     a_issue_part<MODE, 0, kGroupsPerWave>(s, p, c);
     a_issue_advance(s);
 }
 // Before the barrier that ends the phase of step t - 1 (t = 0: the first barrier): step t has landed
 // when only the loads of step t + 1 may still be in flight.
-__device__ __forceinline__ void a_wait_step(const AIssuer& s, const TileCtx& c, int t) {
+static __device__ __forceinline__ void a_wait_step(const AIssuer& s, const TileCtx& c, int t) {
     wait_loads_at_most(t + 1 < c.total_steps ? s.ld.n : 0);
 }
 
@@ -178,11 +191,11 @@ struct ProducerLane {  // per-lane constants of a producer
 // Element-wise A tile for shapes the fast path cannot take (unaligned rows, a contraction that ends
 // inside the step): producers write the same swizzled layout, zero-filled past the contraction.
 template <int MODE>
-__device__ __forceinline__ void fill_a_slow(const MmqParams& p, const TileCtx& c, const ProducerLane& l, int step, int stage) {
+static __device__ __forceinline__ void fill_a_slow(const MmqParams& p, const TileCtx& c, const ProducerLane& l, int step, int stage) {
     int seg_k, kc0;
     step_origin<MODE>(p, step, seg_k, kc0);
     uint8_t* at = c.as + stage * kAStageBytes;
-    for (int id = l.ptid; id < kBM * 8; id += 256) {
+    for (int id = l.ptid; id < kTM * 8; id += 256) {
         const int r = id >> 3, ch = id & 7;
         if (r >= c.rows_valid) break;
         const bf16_t* src = p.a[MODE == kModeNN ? seg_k : 0] + (int64_t)(c.row_begin + r) * p.lda + kc0 + ch * 8;
@@ -191,7 +204,7 @@ __device__ __forceinline__ void fill_a_slow(const MmqParams& p, const TileCtx& c
 }
 
 template <int QT, int MODE>
-__device__ __forceinline__ void w_issue_run(const MmqParams& p, const TileCtx& c, const ProducerLane& l, int step,
+static __device__ __forceinline__ void w_issue_run(const MmqParams& p, const TileCtx& c, const ProducerLane& l, int step,
                                             typename Fmt<QT>::Raw& w_reg) {
     int seg_k, kc0;
     step_origin<MODE>(p, step, seg_k, kc0);
@@ -205,7 +218,7 @@ __device__ __forceinline__ void w_issue_run(const MmqParams& p, const TileCtx& c
 
 // The 32 decoded weights of a run (16 packed bf16 pairs) -> LDS W tile.
 template <int MODE>
-__device__ __forceinline__ void w_store_run(const TileCtx& c, const ProducerLane& l, int buf, const uint32_t* wv) {
+static __device__ __forceinline__ void w_store_run(const TileCtx& c, const ProducerLane& l, int buf, const uint32_t* wv) {
     bf16_t* bt = c.bs + buf * kBTile;
     if (MODE == kModeNT) {
         bf16_t* dst = &bt[(l.ptid >> 1) * kLdsStride + (l.ptid & 1) * 32];
@@ -221,27 +234,29 @@ __device__ __forceinline__ void w_store_run(const TileCtx& c, const ProducerLane
     }
 }
 
-// Q4_K forward: lane (output column n = ptid / 2, half h = ptid % 2) keeps, for a 256-wide block, the
-// block header and bytes 16h .. 16h+15 of the two 32-byte quant groups its quartet decodes (groups
-// q and q + 2 for quartet q).  Group S feeds step S of the block: its low nibbles are elements
-// 16h .. 16h+15 of sub-block 2S, its high nibbles the same elements of sub-block 2S+1.
+// Q4_K forward, wide shape: lane (output column n = ptid / 2, half h = ptid % 2) keeps, for a 256-wide
+// block, the block header and bytes 16h .. 16h+15 of each of the four 32-byte quant groups.  Group S
+// feeds step S of the block: its low nibbles are elements 16h .. 16h+15 of sub-block 2S, its high
+// nibbles the same elements of sub-block 2S+1.
 struct Q4KChunk {
-    u32x4_t hdr, qa, qb;
+    u32x4_t hdr, g0, g1, g2, g3;
 };
-__device__ __forceinline__ void q4k_chunk_load(Q4KChunk& ch, const uint8_t* row, int block, int h, int quartet) {
+static __device__ __forceinline__ void q4k_chunk_load(Q4KChunk& ch, const uint8_t* row, int block, int h) {
     const uint8_t* blk = row + (int64_t)block * 144;
     ch.hdr = *(const u32x4_t*)blk;
-    const uint8_t* q = blk + 16 + 16 * h + 32 * quartet;
-    ch.qa = *(const u32x4_t*)q;
-    ch.qb = *(const u32x4_t*)(q + 64);
+    const uint8_t* q = blk + 16 + 16 * h;
+    ch.g0 = *(const u32x4_t*)q;
+    ch.g1 = *(const u32x4_t*)(q + 32);
+    ch.g2 = *(const u32x4_t*)(q + 64);
+    ch.g3 = *(const u32x4_t*)(q + 96);
 }
 // Keeps every use of the block registers after this point in program order (in particular after the
 // barrier in front of it), so that no wait for a freshly issued reload is pulled forward.
-__device__ __forceinline__ void q4k_chunk_pin(Q4KChunk& ch) {
-    asm volatile("" : "+v"(ch.hdr), "+v"(ch.qa), "+v"(ch.qb));
+static __device__ __forceinline__ void q4k_chunk_pin(Q4KChunk& ch) {
+    asm volatile("" : "+v"(ch.hdr), "+v"(ch.g0), "+v"(ch.g1), "+v"(ch.g2), "+v"(ch.g3));
 }
 template <int J>  // 6-bit (scale, min) of sub-block J
-__device__ __forceinline__ void q4k_scale_min(const u32x4_t& hdr, uint32_t& sc, uint32_t& m) {
+static __device__ __forceinline__ void q4k_scale_min(const u32x4_t& hdr, uint32_t& sc, uint32_t& m) {
     const uint32_t s0 = hdr.y, s1 = hdr.z, s2 = hdr.w;
     if (J < 4) {
         sc = (s0 >> (8 * J)) & 63u;
@@ -254,7 +269,7 @@ __device__ __forceinline__ void q4k_scale_min(const u32x4_t& hdr, uint32_t& sc, 
 }
 // wv[0..7]: elements 16h .. 16h+15 of sub-block 2S; wv[8..15]: the same elements of sub-block 2S+1.
 template <int S>
-__device__ __forceinline__ void q4k_chunk_decode(const u32x4_t& hdr, const u32x4_t& q, uint32_t* wv) {
+static __device__ __forceinline__ void q4k_chunk_decode(const u32x4_t& hdr, const u32x4_t& q, uint32_t* wv) {
     const float d = half_bits_to_f32(hdr.x & 0xFFFFu), dmin = half_bits_to_f32(hdr.x >> 16);
     uint32_t sc0, m0, sc1, m1;
     q4k_scale_min<2 * S>(hdr, sc0, m0);
@@ -270,7 +285,7 @@ __device__ __forceinline__ void q4k_chunk_decode(const u32x4_t& hdr, const u32x4
         wv[8 + 2 * i + 1] = pack_bf16(fmaf(dl1, ubyte2(b), nm1), fmaf(dl1, ubyte3(b), nm1));
     }
 }
-__device__ __forceinline__ void q4k_chunk_store(const TileCtx& c, const ProducerLane& l, int buf, const uint32_t* wv) {
+static __device__ __forceinline__ void q4k_chunk_store(const TileCtx& c, const ProducerLane& l, int buf, const uint32_t* wv) {
     bf16_t* dst = c.bs + buf * kBTile + (l.ptid >> 1) * kLdsStride + (l.ptid & 1) * 16;
     *(uint4*)(dst) = make_uint4(wv[0], wv[1], wv[2], wv[3]);
     *(uint4*)(dst + 8) = make_uint4(wv[4], wv[5], wv[6], wv[7]);
@@ -285,7 +300,7 @@ __device__ __forceinline__ void q4k_chunk_store(const TileCtx& c, const Producer
 // The phase sequence is written out per period (no data-dependent branches between a load and its
 // use), so that the waits on the packed-weight loads stay exact instead of draining every load.
 template <int QT, int MODE, int Q>
-__device__ __forceinline__ void produce(const MmqParams& p, const TileCtx& c, int ptid, int pw) {
+static __device__ __forceinline__ void produce(const MmqParams& p, const TileCtx& c, int ptid, int pw) {
     ProducerLane l;
     l.ptid = ptid, l.pw = pw, l.lane = ptid & 63;
     // W run owned by this lane: NT -> (output column n = col0 + ptid/2, run 2*step + ptid%2);
@@ -293,7 +308,6 @@ __device__ __forceinline__ void produce(const MmqParams& p, const TileCtx& c, in
     l.w_ksub_nn = min((c.col0 >> 5) + pw, (p.k >> 5) - 1);
     l.w_row_nt = min(c.col0 + (ptid >> 1), p.n - 1);
     const int steps = c.total_steps;
-    constexpr bool kChunked = QT == kQ4_K && MODE == kModeNT;
     uint32_t wv[16];
     int stage = c.base, buf = c.base;
     auto close_phase = [&]() __attribute__((always_inline)) {
@@ -303,65 +317,14 @@ __device__ __forceinline__ void produce(const MmqParams& p, const TileCtx& c, in
     };
     auto store = [&](int u) __attribute__((always_inline)) {
         if (!c.a_fast) fill_a_slow<MODE>(p, c, l, u, stage);
-        if (kChunked) q4k_chunk_store(c, l, buf, wv);
-        else w_store_run<MODE>(c, l, buf, wv);
+        w_store_run<MODE>(c, l, buf, wv);
     };
     // Decoded values are fenced the same way: the decode belongs in front of the barrier that follows it.
     auto pin_decoded = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < 16; i++) asm volatile("" : "+v"(wv[i]));
     };
-    if (kChunked) {
-        // K is a whole number of 256-wide blocks: four steps per block, this quartet's are Q and Q + 2.
-        // Two register sets alternate between blocks; a set is loaded four phases before its first use.
-        const uint8_t* wrow = p.w[c.seg_c] + c.expert * p.w_expert_bytes + (int64_t)l.w_row_nt * p.w_row_bytes;
-        const int h = ptid & 1, blocks = steps >> 2;
-        Q4KChunk even, odd;
-        q4k_chunk_load(even, wrow, 0, h, Q);
-        if (Q == 0) {
-            q4k_chunk_decode<0>(even.hdr, even.qa, wv);
-            pin_decoded();
-        }
-        // block k: `cur` holds its packed bytes, `nxt` receives those of block k + 1
-        auto block_phases = [&](Q4KChunk& cur, Q4KChunk& nxt, int k) __attribute__((always_inline)) {
-            const bool more = k + 1 < blocks;
-            if (Q == 0) {
-                store(4 * k);
-                if (more) q4k_chunk_load(nxt, wrow, k + 1, h, Q);
-                close_phase();
-                q4k_chunk_pin(cur);
-                q4k_chunk_decode<2>(cur.hdr, cur.qb, wv);
-                pin_decoded();
-                close_phase();
-                store(4 * k + 2);
-                close_phase();
-                if (more) {
-                    q4k_chunk_pin(nxt);
-                    q4k_chunk_decode<0>(nxt.hdr, nxt.qa, wv);
-                    pin_decoded();
-                }
-                close_phase();
-            } else {
-                q4k_chunk_pin(cur);
-                q4k_chunk_decode<1>(cur.hdr, cur.qa, wv);
-                pin_decoded();
-                if (more) q4k_chunk_load(nxt, wrow, k + 1, h, Q);
-                close_phase();
-                store(4 * k + 1);
-                close_phase();
-                q4k_chunk_pin(cur);
-                q4k_chunk_decode<3>(cur.hdr, cur.qb, wv);
-                pin_decoded();
-                close_phase();
-                store(4 * k + 3);
-                close_phase();
-            }
-        };
-        for (int k = 0; k < blocks; k += 2) {
-            block_phases(even, odd, k);
-            if (k + 1 < blocks) block_phases(odd, even, k + 1);
-        }
-    } else {
+    {
         // Two register sets alternate between this quartet's steps (u = Q, Q + 2, ...): the packed run of
         // step u + 4 is requested as soon as step u is decoded, three phases before its own decode.
         typename Fmt<QT>::Raw raw_a, raw_b;
@@ -414,10 +377,234 @@ __device__ __forceinline__ void produce(const MmqParams& p, const TileCtx& c, in
     lds_barrier();
 }
 
+// ---- Q4_K: both producer quartets (512 lanes) work on every step, half a run each.  The decode of a
+// step is the longest thing between two barriers when an expert group has few rows; splitting it over
+// all eight producer waves halves it.
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+// Forward: lane (output column n = ptid / 4, quarter q = ptid % 4) keeps, for a 256-wide block, the
+// block header and bytes 8q .. 8q+7 of each of the four 32-byte quant groups.  Group S feeds step S:
+// low nibbles are elements 8q .. 8q+7 of sub-block 2S, high nibbles the same elements of sub-block 2S+1.
+struct Q4KQuarter {
+    u32x4_t hdr;
+    u32x2_t g0, g1, g2, g3;
+};
+static __device__ __forceinline__ void q4k_quarter_load(Q4KQuarter& ch, const uint8_t* row, int block, int q) {
+    const uint8_t* blk = row + (int64_t)block * 144;
+    ch.hdr = *(const u32x4_t*)blk;
+    const uint8_t* g = blk + 16 + 8 * q;
+    ch.g0 = *(const u32x2_t*)g;
+    ch.g1 = *(const u32x2_t*)(g + 32);
+    ch.g2 = *(const u32x2_t*)(g + 64);
+    ch.g3 = *(const u32x2_t*)(g + 96);
+}
+static __device__ __forceinline__ void q4k_quarter_pin(Q4KQuarter& ch) {
+    asm volatile("" : "+v"(ch.hdr), "+v"(ch.g0), "+v"(ch.g1), "+v"(ch.g2), "+v"(ch.g3));
+}
+// lo[0..3]: elements 8q .. 8q+7 of sub-block 2S; hi[0..3]: the same elements of sub-block 2S+1.
+template <int S>
+static __device__ __forceinline__ void q4k_quarter_decode(const u32x4_t& hdr, const u32x2_t& g, uint32_t* lo, uint32_t* hi) {
+    const float d = half_bits_to_f32(hdr.x & 0xFFFFu), dmin = half_bits_to_f32(hdr.x >> 16);
+    uint32_t sc0, m0, sc1, m1;
+    q4k_scale_min<2 * S>(hdr, sc0, m0);
+    q4k_scale_min<2 * S + 1>(hdr, sc1, m1);
+    const float dl0 = d * (float)sc0, nm0 = -(dmin * (float)m0);
+    const float dl1 = d * (float)sc1, nm1 = -(dmin * (float)m1);
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const uint32_t a = opaque(g[i] & 0x0F0F0F0Fu), b = opaque((g[i] >> 4) & 0x0F0F0F0Fu);
+        lo[2 * i] = pack_bf16(fmaf(dl0, ubyte0(a), nm0), fmaf(dl0, ubyte1(a), nm0));
+        lo[2 * i + 1] = pack_bf16(fmaf(dl0, ubyte2(a), nm0), fmaf(dl0, ubyte3(a), nm0));
+        hi[2 * i] = pack_bf16(fmaf(dl1, ubyte0(b), nm1), fmaf(dl1, ubyte1(b), nm1));
+        hi[2 * i + 1] = pack_bf16(fmaf(dl1, ubyte2(b), nm1), fmaf(dl1, ubyte3(b), nm1));
+    }
+}
+
+// Grad-input: lane (contraction row n = kc0 + lane, run = col0/32 + wave of the quartet, half = quartet)
+// decodes 16 consecutive output columns of its row and stores them transposed.
+struct Q4KHalfRun {
+    u32x4_t hdr, q;
+};
+static __device__ __forceinline__ void q4k_half_run_pin(Q4KHalfRun& r) { asm volatile("" : "+v"(r.hdr), "+v"(r.q)); }
+static __device__ __forceinline__ void q4k_half_run_decode(const Q4KHalfRun& r, int j, uint32_t* out) {  // j: sub-block 0..7
+    const float d = half_bits_to_f32(r.hdr.x & 0xFFFFu), dmin = half_bits_to_f32(r.hdr.x >> 16);
+    const uint32_t s0 = r.hdr.y, s1 = r.hdr.z, s2 = r.hdr.w;
+    uint32_t sc, m;
+    if (j < 4) {
+        const int sh = 8 * j;
+        sc = (s0 >> sh) & 63u;
+        m = (s1 >> sh) & 63u;
+    } else {
+        const int sh = 8 * (j - 4);
+        sc = ((s2 >> sh) & 0xFu) | (((s0 >> (sh + 6)) & 3u) << 4);
+        m = ((s2 >> (sh + 4)) & 0xFu) | (((s1 >> (sh + 6)) & 3u) << 4);
+    }
+    const float dl = d * (float)sc, nm = -(dmin * (float)m);
+    const int shift = 4 * (j & 1);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t v = opaque((r.q[i] >> shift) & 0x0F0F0F0Fu);
+        out[2 * i] = pack_bf16(fmaf(dl, ubyte0(v), nm), fmaf(dl, ubyte1(v), nm));
+        out[2 * i + 1] = pack_bf16(fmaf(dl, ubyte2(v), nm), fmaf(dl, ubyte3(v), nm));
+    }
+}
+
+// Barrier b closes the phase in which step b reaches LDS; steps + 1 barriers in all (the last one
+// pairs with the consumers' final step).
+template <int MODE>
+static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const TileCtx& c, int ptid, int pw) {
+    // ptid 0..511 over both quartets; pw 0..7
+    const int steps = c.total_steps;
+    int stage = c.base, buf = c.base;
+    ProducerLane slow;  // the element-wise A path is the first quartet's job
+    slow.ptid = ptid, slow.pw = pw, slow.lane = ptid & 63, slow.w_ksub_nn = 0, slow.w_row_nt = 0;
+    auto open_phase = [&](int u) __attribute__((always_inline)) {
+        if (!c.a_fast && ptid < 256) fill_a_slow<MODE>(p, c, slow, u, stage);
+    };
+    auto close_phase = [&]() __attribute__((always_inline)) {
+        lds_barrier();
+        stage = stage == kAStages - 1 ? 0 : stage + 1;
+        buf ^= 1;
+    };
+    if (MODE == kModeNT && SH == 1) {
+        // wide: 256 output columns, lane = (column ptid / 2, half ptid % 2), 32 weights per lane and step
+        ProducerLane l = slow;
+        const int h = ptid & 1;
+        const uint8_t* wrow = p.w[c.seg_c] + c.expert * p.w_expert_bytes + (int64_t)min(c.col0 + (ptid >> 1), p.n - 1) * p.w_row_bytes;
+        const int blocks = steps >> 2;  // K is a whole number of 256-wide blocks
+        Q4KChunk even, odd;             // alternate between blocks; a set is loaded four phases before its first use
+        q4k_chunk_load(even, wrow, 0, h);
+        auto fill = [&](auto s_c, const Q4KChunk& ch, int u) __attribute__((always_inline)) {
+            constexpr int S = decltype(s_c)::value;
+            open_phase(u);
+            uint32_t wv[16];
+            q4k_chunk_decode<S>(ch.hdr, S == 0 ? ch.g0 : S == 1 ? ch.g1 : S == 2 ? ch.g2 : ch.g3, wv);
+            q4k_chunk_store(c, l, buf, wv);
+            close_phase();
+        };
+        auto block_phases = [&](Q4KChunk& cur, Q4KChunk& nxt, int k) __attribute__((always_inline)) {
+            if (k + 1 < blocks) q4k_chunk_load(nxt, wrow, k + 1, h);
+            q4k_chunk_pin(cur);
+            fill(std::integral_constant<int, 0>{}, cur, 4 * k);
+            q4k_chunk_pin(cur);
+            fill(std::integral_constant<int, 1>{}, cur, 4 * k + 1);
+            q4k_chunk_pin(cur);
+            fill(std::integral_constant<int, 2>{}, cur, 4 * k + 2);
+            q4k_chunk_pin(cur);
+            fill(std::integral_constant<int, 3>{}, cur, 4 * k + 3);
+        };
+        for (int k = 0; k < blocks; k += 2) {
+            block_phases(even, odd, k);
+            if (k + 1 < blocks) block_phases(odd, even, k + 1);
+        }
+    } else if (MODE == kModeNN && SH == 1) {
+        // wide: the 256 output columns of a step are exactly one block of each of the 64 contraction rows;
+        // lane = (row kc0 + lane, run = producer wave), stored as it is decoded: [row][column], the
+        // consumers transpose on the way out of LDS
+        const int lane = ptid & 63;
+        const int ksub = min((c.col0 >> 5) + pw, (p.k >> 5) - 1);  // runs past the end are clamped, never stored
+        typedef typename Fmt<kQ4_K>::Raw Raw;
+        auto issue = [&](Raw& r, int u) __attribute__((always_inline)) {
+            int seg_k, kc0;
+            step_origin<MODE>(p, u, seg_k, kc0);
+            const int wrow = min(kc0 + lane, p.n - 1);  // rows past the end meet the zero-filled tail of the A tile
+            Fmt<kQ4_K>::load(r, p.w[seg_k] + c.expert * p.w_expert_bytes + (int64_t)wrow * p.w_row_bytes, ksub);
+        };
+        bf16_t* const dst0 = c.bs + lane * kNnPitch + pw * 32;
+        auto fill = [&](Raw& r, int u) __attribute__((always_inline)) {
+            open_phase(u);
+            Fmt<kQ4_K>::pin(r);
+            uint32_t wv[16];
+            Fmt<kQ4_K>::decode(r, ksub, wv, nullptr);
+            if (u + 2 < steps) issue(r, u + 2);
+            bf16_t* dst = dst0 + buf * kBTile;
+#pragma unroll
+            for (int i = 0; i < 4; i++) *(uint4*)(dst + 8 * i) = make_uint4(wv[4 * i], wv[4 * i + 1], wv[4 * i + 2], wv[4 * i + 3]);
+            close_phase();
+        };
+        Raw ra, rb;  // even / odd steps, each reloaded two steps ahead
+        issue(ra, 0);
+        if (steps > 1) issue(rb, 1);
+        for (int u = 0; u < steps; u += 2) {
+            fill(ra, u);
+            if (u + 1 < steps) fill(rb, u + 1);
+        }
+    } else if (MODE == kModeNT) {
+        const int q = ptid & 3, n_local = ptid >> 2;
+        const uint8_t* wrow = p.w[c.seg_c] + c.expert * p.w_expert_bytes + (int64_t)min(c.col0 + n_local, p.n - 1) * p.w_row_bytes;
+        const int blocks = steps >> 2;  // K is a whole number of 256-wide blocks
+        bf16_t* const dst0 = c.bs + n_local * kLdsStride + q * 8;
+        Q4KQuarter even, odd;  // alternate between blocks; a set is loaded four phases before its first use
+        q4k_quarter_load(even, wrow, 0, q);
+        auto fill = [&](auto s_c, const Q4KQuarter& ch, int u) __attribute__((always_inline)) {
+            constexpr int S = decltype(s_c)::value;
+            open_phase(u);
+            uint32_t lo[4], hi[4];
+            q4k_quarter_decode<S>(ch.hdr, S == 0 ? ch.g0 : S == 1 ? ch.g1 : S == 2 ? ch.g2 : ch.g3, lo, hi);
+            bf16_t* dst = dst0 + buf * kBTile;
+            *(uint4*)dst = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+            *(uint4*)(dst + 32) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+            close_phase();
+        };
+        auto block_phases = [&](Q4KQuarter& cur, Q4KQuarter& nxt, int k) __attribute__((always_inline)) {
+            if (k + 1 < blocks) q4k_quarter_load(nxt, wrow, k + 1, q);
+            q4k_quarter_pin(cur);
+            fill(std::integral_constant<int, 0>{}, cur, 4 * k);
+            q4k_quarter_pin(cur);
+            fill(std::integral_constant<int, 1>{}, cur, 4 * k + 1);
+            q4k_quarter_pin(cur);
+            fill(std::integral_constant<int, 2>{}, cur, 4 * k + 2);
+            q4k_quarter_pin(cur);
+            fill(std::integral_constant<int, 3>{}, cur, 4 * k + 3);
+        };
+        for (int k = 0; k < blocks; k += 2) {
+            block_phases(even, odd, k);
+            if (k + 1 < blocks) block_phases(odd, even, k + 1);
+        }
+    } else {
+        const int lane = ptid & 63, run_w = pw & 3, half = pw >> 2;
+        const int ksub = min((c.col0 >> 5) + run_w, (p.k >> 5) - 1);  // runs past the end are clamped, never stored
+        const int j = ksub & 7;
+        const int64_t blk_off = (int64_t)(ksub >> 3) * 144;
+        const int q_off = 16 + 32 * (j >> 1) + 16 * half;
+        auto issue = [&](Q4KHalfRun& r, int u) __attribute__((always_inline)) {
+            int seg_k, kc0;
+            step_origin<MODE>(p, u, seg_k, kc0);
+            const int wrow = min(kc0 + lane, p.n - 1);  // rows past the end meet the zero-filled tail of the A tile
+            const uint8_t* blk = p.w[seg_k] + c.expert * p.w_expert_bytes + (int64_t)wrow * p.w_row_bytes + blk_off;
+            r.hdr = *(const u32x4_t*)blk;
+            r.q = *(const u32x4_t*)(blk + q_off);
+        };
+        bf16_t* const dst0 = c.bs + (run_w * 32 + half * 16) * kLdsStride + lane;
+        auto fill = [&](Q4KHalfRun& r, int u) __attribute__((always_inline)) {
+            open_phase(u);
+            q4k_half_run_pin(r);
+            uint32_t wv[8];
+            q4k_half_run_decode(r, j, wv);
+            if (u + 2 < steps) issue(r, u + 2);
+            bf16_t* dst = dst0 + buf * kBTile;
+#pragma unroll
+            for (int e2 = 0; e2 < 8; e2++) {
+                dst[(2 * e2) * kLdsStride] = (bf16_t)(wv[e2] & 0xFFFFu);
+                dst[(2 * e2 + 1) * kLdsStride] = (bf16_t)(wv[e2] >> 16);
+            }
+            close_phase();
+        };
+        Q4KHalfRun ra, rb;  // even / odd steps, each reloaded two steps ahead
+        issue(ra, 0);
+        if (steps > 1) issue(rb, 1);
+        for (int u = 0; u < steps; u += 2) {
+            fill(ra, u);
+            if (u + 1 < steps) fill(rb, u + 1);
+        }
+    }
+    lds_barrier();
+}
+
 // ---- consumer waves, instantiated per number of live 32-row blocks.
 template <int QT, int MODE, int EPI, int LIVE>
-__device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, int lane, int cw) {
-    const int wave_m = cw >> 1, wave_n = cw & 1;
+static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, int lane, int cw) {
+    const int wave_m = cw / kWavesN, wave_n = cw % kWavesN;
     const int lane_c = lane & 31, lane_h = lane >> 5;
     f32x16_t acc[LIVE][kColBlocks];
 #pragma unroll
@@ -432,18 +619,37 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
 #pragma unroll
     for (int kk = 0; kk < 4; kk++) a_koff[kk] = a_slot(lane_c, 2 * kk + lane_h) * 16;
     const int b_off = (wave_n * 64 + lane_c) * kLdsStride + lane_h * 8;
+    // transposing read: within a group of 16 lanes, lane L receives element L % 4 of the 8 bytes addressed
+    // by lanes L / 4 + 4 j (j = 0..3).  Source lane s = L % 16 therefore points at contraction row s / 4 and
+    // columns 4 (s % 4) .. +3 of its group's 16 columns; groups 0, 1 take columns 0..15 / 16..31 of the
+    // block, groups 2, 3 the same columns eight contraction rows further on.
+    const int tr_group = lane >> 4, tr_s = lane & 15;
+    const int tr_off = (8 * (tr_group >> 1) + (tr_s >> 2)) * kNnPitch + wave_n * 64 + 16 * (tr_group & 1) + 4 * (tr_s & 3);
 
     // Operands of one sub-step (16 of the contraction): LIVE row-block runs of A, two column-block runs of W.
     struct Operands {
         bf16x8_t a[LIVE], b[kColBlocks];
     };
-    auto load_operands = [&](Operands& o, int stage, int buf, int kk) __attribute__((always_inline)) {
+    // `lora`: the LoRA tiles ahead of the main steps always use the [column][contraction] W layout
+    auto load_operands = [&](Operands& o, int stage, int buf, int kk, bool lora = false) __attribute__((always_inline)) {
         const uint8_t* a_lds = a_row + stage * kAStageBytes + a_koff[kk];
-        const bf16_t* b_lds = c.bs + buf * kBTile + b_off + kk * 16;
+        if (MODE == kModeNN && SH == 1 && !lora) {
+            // W tile is [contraction row][output column]: each transposing 8-byte read hands this lane
+            // four consecutive contraction values of its column, two reads make the MFMA operand
+            const bf16_t* t_lds = c.bs + buf * kBTile + tr_off + kk * 16 * kNnPitch;
 #pragma unroll
-        for (int cb = 0; cb < kColBlocks; cb++) o.b[cb] = *(const bf16x8_t*)(b_lds + cb * 32 * kLdsStride);
+            for (int cb = 0; cb < kColBlocks; cb++) {
+                const v4i16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(t_lds + cb * 32));
+                const v4i16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(t_lds + cb * 32 + 4 * kNnPitch));
+                o.b[cb] = __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            }
+        } else {
+            const bf16_t* b_lds = c.bs + buf * kBTile + b_off + kk * 16;
 #pragma unroll
-        for (int rb = 0; rb < LIVE; rb++) o.a[rb] = *(const bf16x8_t*)(a_lds + rb * 128 * kARowBytes);
+            for (int cb = 0; cb < kColBlocks; cb++) o.b[cb] = *(const bf16x8_t*)(b_lds + cb * 32 * kLdsStride);
+        }
+#pragma unroll
+        for (int rb = 0; rb < LIVE; rb++) o.a[rb] = *(const bf16x8_t*)(a_lds + rb * kWavesM * 32 * kARowBytes);
     };
     auto mfma_operands = [&](const Operands& o) __attribute__((always_inline)) {
 #pragma unroll
@@ -464,7 +670,7 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
         for (int kk = 0; kk < 4; kk++)
             if (kk < n) {
                 Operands o;
-                load_operands(o, 0, 0, kk);
+                load_operands(o, 0, 0, kk, true);
                 mfma_operands(o);
             }
         const float s = p.lora_scale;
@@ -536,7 +742,7 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
 #undef GGQ_MFMA_READ_PAIRS
 #undef GGQ_STAGE
 
-    // ---- epilogue.  acc[rb][cb][i]: tile row = 32*(4*rb + wave_m) + 8*(i/4) + 4*lane_h + (i%4),
+    // ---- epilogue.  acc[rb][cb][i]: tile row = 32*(kWavesM*rb + wave_m) + 8*(i/4) + 4*lane_h + (i%4),
     //                                 tile col = 64*wave_n + 32*cb + lane_c
     const int col_base = c.col0 + wave_n * 64 + lane_c;
     if (EPI == kEpiStore || EPI == kEpiAccumF32 || EPI == kEpiCeGrad) {
@@ -551,7 +757,7 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
         const bool col_ok[kColBlocks] = {col_base < c.out_cols, col_base + 32 < c.out_cols};
 #pragma unroll
         for (int rb = 0; rb < LIVE; rb++) {
-            const int r_lane = 32 * (4 * rb + wave_m) + lane_h * 4;  // this lane's first row of the block
+            const int r_lane = 32 * (kWavesM * rb + wave_m) + lane_h * 4;  // this lane's first row of the block
             const int64_t lane_elem = (int64_t)(c.row_begin + r_lane) * ldc + col_base;
 #pragma unroll
             for (int i = 0; i < 16; i++) {
@@ -588,7 +794,7 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
         for (int rb = 0; rb < LIVE; rb++) {
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                const int r = 32 * (4 * rb + wave_m) + (i >> 2) * 8 + lane_h * 4 + (i & 3);
+                const int r = 32 * (kWavesM * rb + wave_m) + (i >> 2) * 8 + lane_h * 4 + (i & 3);
                 const bool row_ok = r < c.rows_valid;
                 const int64_t grow = c.row_begin + (row_ok ? r : 0);
                 const int64_t label = row_ok ? p.labels[grow] : -1;
@@ -619,7 +825,7 @@ __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, in
 // A consumer wave without a live row block still moves its share of the A tile and keeps the
 // barriers company.
 template <int MODE>
-__device__ __forceinline__ void consume_idle(const MmqParams& p, const TileCtx& c, int lane, int cw) {
+static __device__ __forceinline__ void consume_idle(const MmqParams& p, const TileCtx& c, int lane, int cw) {
     AIssuer ai;
     a_loader_init(ai.ld, p, c, lane, cw);
     ai.next_step = 0, ai.next_stage = c.base;
@@ -635,7 +841,7 @@ __device__ __forceinline__ void consume_idle(const MmqParams& p, const TileCtx& 
 }
 
 template <int QT, int MODE, int EPI>
-__global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(4, 4))) void mmq_tile_kernel(const MmqParams p) {
+static __device__ __forceinline__ void run(const MmqParams& p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_raw[];
     TileCtx c;
     c.as = smem_raw;
@@ -661,14 +867,14 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(4, 
         group = t.group, c.row_begin = t.row_begin, row_end = t.row_end;
     } else {
         if (row_tile >= p.max_row_tiles) return;
-        c.row_begin = row_tile * kBM;
-        row_end = min(p.m, c.row_begin + kBM);
+        c.row_begin = row_tile * kTM;
+        row_end = min(p.m, c.row_begin + kTM);
     }
-    c.rows_valid = row_end - c.row_begin;  // 1..kBM
+    c.rows_valid = row_end - c.row_begin;  // 1..kTM
     c.expert = p.expert_ids ? p.expert_ids[group] : 0;
     // column tile -> (segment, first output column inside the segment)
     c.seg_c = MODE == kModeNT ? c.col_tile / p.col_tiles_per_seg : 0;
-    c.col0 = (c.col_tile - c.seg_c * p.col_tiles_per_seg) * kBN;
+    c.col0 = (c.col_tile - c.seg_c * p.col_tiles_per_seg) * kTN;
     c.out_cols = MODE == kModeNT ? p.n : p.k;     // output columns per segment
     c.contraction = MODE == kModeNT ? p.k : p.n;  // contraction length per segment
     c.total_steps = (MODE == kModeNN ? p.nseg : 1) * p.steps_per_seg;
@@ -683,14 +889,14 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(4, 
     // ---- LoRA tiles go to A stage 0 / W buffer 0 (all lanes load): LA[rows, :r] and LB[cols, :r]
     if (p.r_pad > 0) {
         const int chunks = p.r_pad >> 3;  // 16-byte chunks per row (r_pad % 16 == 0)
-        for (int id = tid; id < kBM * 8; id += kThreads) {
+        for (int id = tid; id < kTM * 8; id += kThreads) {
             const int r = id >> 3, ch = id & 7;
             uint4 v = zero4();
             if (r < c.rows_valid && ch < chunks) v = *(const uint4*)(p.la + (int64_t)(c.row_begin + r) * p.r_pad + ch * 8);
             *(uint4*)(c.as + r * kARowBytes + a_slot(r, ch) * 16) = v;
         }
         const bf16_t* lb = p.lb + c.expert * p.lb_expert_elems + (int64_t)(c.seg_c * c.out_cols + c.col0) * p.r_pad;
-        for (int id = tid; id < kBN * 8; id += kThreads) {
+        for (int id = tid; id < kTN * 8; id += kThreads) {
             const int cidx = id >> 3, ch = id & 7;
             uint4 v = zero4();
             if (c.col0 + cidx < c.out_cols && ch < chunks) v = *(const uint4*)(lb + (int64_t)cidx * p.r_pad + ch * 8);
@@ -700,19 +906,26 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(4, 
     __syncthreads();  // LoRA tiles and the codebook are visible
 
     if (wave >= 8) {
-        if (wave < 12) produce<QT, MODE, 0>(p, c, tid & 255, wave & 3);
+        if (QT == kQ4_K) produce_q4k<MODE>(p, c, tid - 512, wave - 8);
+        else if (wave < 12) produce<QT, MODE, 0>(p, c, tid & 255, wave & 3);
         else produce<QT, MODE, 1>(p, c, tid & 255, wave & 3);
     } else {
-        const int cw = wave, wave_m = cw >> 1;
-        // this wave's row blocks are tile rows 32*wave_m .. +31 and 32*(wave_m + 4) .. +31; blocks fill up from row 0
+        const int cw = wave, wave_m = cw / kWavesN;
+        // this wave's row blocks are tile rows 32*wave_m .. +31 and 32*(wave_m + kWavesM) .. +31; blocks fill up from row 0
         const int blocks = (c.rows_valid + 31) >> 5;
-        const int live = (blocks > wave_m ? 1 : 0) + (blocks > wave_m + 4 ? 1 : 0);
+        const int live = (blocks > wave_m ? 1 : 0) + (blocks > wave_m + kWavesM ? 1 : 0);
         switch (live) {
             case 0: consume_idle<MODE>(p, c, lane, cw); break;
             case 1: consume<QT, MODE, EPI, 1>(p, c, lane, cw); break;
             default: consume<QT, MODE, EPI, 2>(p, c, lane, cw); break;
         }
     }
+}
+};  // struct Tile
+
+template <int QT, int MODE, int EPI, int SH>
+__global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(4, 4))) void mmq_tile_kernel(const MmqParams p) {
+    Tile<SH>::template run<QT, MODE, EPI>(p);
 }
 
 }  // namespace ggq
