@@ -39,7 +39,6 @@ namespace ggq {
 static __device__ const uint64_t d_iq2xxs_grid_mm[256] = GGQ_IQ2XXS_GRID_INIT;
 
 constexpr int kColBlocks = 2;                   // 32-column MFMA blocks per consumer wave
-constexpr int kAStages = 3;                     // LDS ring of A tiles
 constexpr int kARowBytes = kBK * 2;             // A rows are unpadded: 128 bytes = eight 16-byte slots
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -112,6 +111,10 @@ struct Tile {
 static constexpr int kTM = SH == 0 ? 256 : 128, kTN = SH == 0 ? 128 : 256;
 static constexpr int kWavesM = kTM / 64, kWavesN = kTN / 64;
 static constexpr int kAStageBytes = kTM * kARowBytes;   // 32 KB / 16 KB
+// LDS ring of A tiles: the loads of a step are issued kAStages - 1 steps ahead of its MFMAs.  Memory latency
+// under load is about two thousand cycles; the wide shape's short steps need the longer ring.
+static constexpr int kAStages = SH == 0 ? 3 : 5;
+static constexpr int kAhead = kAStages - 1;
 static constexpr int kAGroups = kTM / 8;                // 8-row groups (one direct-to-LDS instruction each)
 static constexpr int kGroupsPerWave = kAGroups / 8;     // groups one consumer wave moves per step (4 / 2)
 static constexpr int kBTile = kTN * kLdsStride;         // bf16 elements per W buffer
@@ -178,9 +181,10 @@ static __device__ __forceinline__ void a_issue_next(AIssuer& s, const MmqParams&
     a_issue_advance(s);
 }
 // Before the barrier that ends the phase of step t - 1 (t = 0: the first barrier): step t has landed
-// when only the loads of step t + 1 may still be in flight.
+// when only the loads of the steps issued after it may still be in flight.
 static __device__ __forceinline__ void a_wait_step(const AIssuer& s, const TileCtx& c, int t) {
-    wait_loads_at_most(t + 1 < c.total_steps ? s.ld.n : 0);
+    const int younger = max(0, min(s.next_step, c.total_steps) - (t + 1));
+    wait_loads_at_most(younger * s.ld.n);
 }
 
 // ---- producer waves: packed weights global -> registers -> (decode) -> LDS W tile.
@@ -662,8 +666,8 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
     AIssuer ai;
     a_loader_init(ai.ld, p, c, lane, cw);
     ai.next_step = 0, ai.next_stage = c.base;
-    a_issue_next<MODE>(ai, p, c);
-    a_issue_next<MODE>(ai, p, c);
+#pragma unroll
+    for (int d = 0; d < kAhead; d++) a_issue_next<MODE>(ai, p, c);
     if (c.base == 1) {  // LoRA tiles sit in stage 0 / buffer 0: acc = s * LA . LB^T, r_pad / 16 sub-steps
         const int n = p.r_pad >> 4;
 #pragma unroll
@@ -706,7 +710,7 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
         // MFMAs follow them as they land.
         const int steps = c.total_steps;
         int stage = c.base, buf = c.base;
-        for (int t = 0; t < steps; t++) {  // the A loads issued in here are those of step t + 2
+        for (int t = 0; t < steps; t++) {  // the A loads issued in here are those of step t + kAhead
             a_issue_part<MODE, 0, kGroupsPerWave>(ai, p, c);
             a_issue_advance(ai);
             Operands o[4];
@@ -724,7 +728,7 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
         int stage = c.base, buf = c.base;
         Operands x, y;
         load_operands(x, stage, buf, 0);
-        for (int t = 0; t < steps; t++) {  // the A loads issued in here are those of step t + 2
+        for (int t = 0; t < steps; t++) {  // the A loads issued in here are those of step t + kAhead
             GGQ_STAGE(y, x, 1, 0);
             GGQ_STAGE(x, y, 2, 1);
             GGQ_STAGE(y, x, 3, 2);
@@ -829,8 +833,8 @@ static __device__ __forceinline__ void consume_idle(const MmqParams& p, const Ti
     AIssuer ai;
     a_loader_init(ai.ld, p, c, lane, cw);
     ai.next_step = 0, ai.next_stage = c.base;
-    a_issue_next<MODE>(ai, p, c);
-    a_issue_next<MODE>(ai, p, c);
+#pragma unroll
+    for (int d = 0; d < kAhead; d++) a_issue_next<MODE>(ai, p, c);
     a_wait_step(ai, c, 0);
     lds_barrier();
     for (int t = 0; t < c.total_steps; t++) {
