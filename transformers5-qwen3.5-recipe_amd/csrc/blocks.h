@@ -89,14 +89,15 @@ struct Fmt<kQ4_K> {
             sc = ((s2 >> sh) & 0xFu) | (((s0 >> (sh + 6)) & 3u) << 4);
             m = ((s2 >> (sh + 4)) & 0xFu) | (((s1 >> (sh + 6)) & 3u) << 4);
         }
-        const float dl = d * (float)sc, nm = -(dmin * (float)m);
+        const float dl = d * (float)sc * kMixScale, nm = -(dmin * (float)m);
         const int shift = 4 * (j & 1);
         const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            const uint32_t v = opaque((q[i] >> shift) & 0x0F0F0F0Fu);
-            out[2 * i] = pack_bf16(fmaf(dl, ubyte0(v), nm), fmaf(dl, ubyte1(v), nm));
-            out[2 * i + 1] = pack_bf16(fmaf(dl, ubyte2(v), nm), fmaf(dl, ubyte3(v), nm));
+            // nibbles of bytes 0, 2 and of bytes 1, 3, each in its own 16-bit half
+            const uint32_t e02 = (q[i] >> shift) & 0x000F000Fu, e13 = (q[i] >> (shift + 8)) & 0x000F000Fu;
+            out[2 * i] = pack_bf16(mix_lo(e02, dl, nm), mix_lo(e13, dl, nm));
+            out[2 * i + 1] = pack_bf16(mix_hi(e02, dl, nm), mix_hi(e13, dl, nm));
         }
     }
 };

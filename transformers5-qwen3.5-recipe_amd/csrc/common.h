@@ -47,6 +47,18 @@ GGQ_HD float ubyte1(uint32_t x) { return (float)((x >> 8) & 0xFFu); }
 GGQ_HD float ubyte2(uint32_t x) { return (float)((x >> 16) & 0xFFu); }
 GGQ_HD float ubyte3(uint32_t x) { return (float)(x >> 24); }
 
+// Small unsigned integers sitting in the 16-bit halves of a register are read as half-precision
+// denormals (value = integer * 2^-24, exact), so one mixed-precision fma (v_fma_mix_f32) computes
+// fma(scale, integer, offset) without a separate integer->float conversion: pass scale * 2^24
+// (kMixScale), the product is the same real number and the single rounding is the same.
+constexpr float kMixScale = 16777216.0f;
+GGQ_HD float mix_lo(uint32_t r, float scale24, float offset) {
+    return __builtin_fmaf((float)__builtin_bit_cast(_Float16, (uint16_t)(r & 0xFFFFu)), scale24, offset);
+}
+GGQ_HD float mix_hi(uint32_t r, float scale24, float offset) {
+    return __builtin_fmaf((float)__builtin_bit_cast(_Float16, (uint16_t)(r >> 16)), scale24, offset);
+}
+
 // Unaligned (2-byte aligned) global loads: the target allows unaligned vector memory access, so
 // these stay single global_load instructions.
 GGQ_HD uint32_t ld_u32(const uint8_t* p) {

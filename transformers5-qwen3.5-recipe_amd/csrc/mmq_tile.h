@@ -278,15 +278,18 @@ static __device__ __forceinline__ void q4k_chunk_decode(const u32x4_t& hdr, cons
     uint32_t sc0, m0, sc1, m1;
     q4k_scale_min<2 * S>(hdr, sc0, m0);
     q4k_scale_min<2 * S + 1>(hdr, sc1, m1);
-    const float dl0 = d * (float)sc0, nm0 = -(dmin * (float)m0);
-    const float dl1 = d * (float)sc1, nm1 = -(dmin * (float)m1);
+    const float dl0 = d * (float)sc0 * kMixScale, nm0 = -(dmin * (float)m0);
+    const float dl1 = d * (float)sc1 * kMixScale, nm1 = -(dmin * (float)m1);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const uint32_t a = opaque(q[i] & 0x0F0F0F0Fu), b = opaque((q[i] >> 4) & 0x0F0F0F0Fu);
-        wv[2 * i] = pack_bf16(fmaf(dl0, ubyte0(a), nm0), fmaf(dl0, ubyte1(a), nm0));
-        wv[2 * i + 1] = pack_bf16(fmaf(dl0, ubyte2(a), nm0), fmaf(dl0, ubyte3(a), nm0));
-        wv[8 + 2 * i] = pack_bf16(fmaf(dl1, ubyte0(b), nm1), fmaf(dl1, ubyte1(b), nm1));
-        wv[8 + 2 * i + 1] = pack_bf16(fmaf(dl1, ubyte2(b), nm1), fmaf(dl1, ubyte3(b), nm1));
+        // byte b of the word: low nibble = element b of sub-block 2S, high nibble = element b of 2S+1;
+        // each nibble lands in its own 16-bit half (bytes 0, 2 / bytes 1, 3) for the mixed-precision fma
+        const uint32_t lo02 = q[i] & 0x000F000Fu, hi02 = (q[i] >> 4) & 0x000F000Fu;
+        const uint32_t lo13 = (q[i] >> 8) & 0x000F000Fu, hi13 = (q[i] >> 12) & 0x000F000Fu;
+        wv[2 * i] = pack_bf16(mix_lo(lo02, dl0, nm0), mix_lo(lo13, dl0, nm0));
+        wv[2 * i + 1] = pack_bf16(mix_hi(lo02, dl0, nm0), mix_hi(lo13, dl0, nm0));
+        wv[8 + 2 * i] = pack_bf16(mix_lo(hi02, dl1, nm1), mix_lo(hi13, dl1, nm1));
+        wv[8 + 2 * i + 1] = pack_bf16(mix_hi(hi02, dl1, nm1), mix_hi(hi13, dl1, nm1));
     }
 }
 static __device__ __forceinline__ void q4k_chunk_store(const TileCtx& c, const ProducerLane& l, int buf, const uint32_t* wv) {
@@ -412,15 +415,16 @@ static __device__ __forceinline__ void q4k_quarter_decode(const u32x4_t& hdr, co
     uint32_t sc0, m0, sc1, m1;
     q4k_scale_min<2 * S>(hdr, sc0, m0);
     q4k_scale_min<2 * S + 1>(hdr, sc1, m1);
-    const float dl0 = d * (float)sc0, nm0 = -(dmin * (float)m0);
-    const float dl1 = d * (float)sc1, nm1 = -(dmin * (float)m1);
+    const float dl0 = d * (float)sc0 * kMixScale, nm0 = -(dmin * (float)m0);
+    const float dl1 = d * (float)sc1 * kMixScale, nm1 = -(dmin * (float)m1);
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-        const uint32_t a = opaque(g[i] & 0x0F0F0F0Fu), b = opaque((g[i] >> 4) & 0x0F0F0F0Fu);
-        lo[2 * i] = pack_bf16(fmaf(dl0, ubyte0(a), nm0), fmaf(dl0, ubyte1(a), nm0));
-        lo[2 * i + 1] = pack_bf16(fmaf(dl0, ubyte2(a), nm0), fmaf(dl0, ubyte3(a), nm0));
-        hi[2 * i] = pack_bf16(fmaf(dl1, ubyte0(b), nm1), fmaf(dl1, ubyte1(b), nm1));
-        hi[2 * i + 1] = pack_bf16(fmaf(dl1, ubyte2(b), nm1), fmaf(dl1, ubyte3(b), nm1));
+        const uint32_t lo02 = g[i] & 0x000F000Fu, hi02 = (g[i] >> 4) & 0x000F000Fu;
+        const uint32_t lo13 = (g[i] >> 8) & 0x000F000Fu, hi13 = (g[i] >> 12) & 0x000F000Fu;
+        lo[2 * i] = pack_bf16(mix_lo(lo02, dl0, nm0), mix_lo(lo13, dl0, nm0));
+        lo[2 * i + 1] = pack_bf16(mix_hi(lo02, dl0, nm0), mix_hi(lo13, dl0, nm0));
+        hi[2 * i] = pack_bf16(mix_lo(hi02, dl1, nm1), mix_lo(hi13, dl1, nm1));
+        hi[2 * i + 1] = pack_bf16(mix_hi(hi02, dl1, nm1), mix_hi(hi13, dl1, nm1));
     }
 }
 
@@ -443,13 +447,13 @@ static __device__ __forceinline__ void q4k_half_run_decode(const Q4KHalfRun& r, 
         sc = ((s2 >> sh) & 0xFu) | (((s0 >> (sh + 6)) & 3u) << 4);
         m = ((s2 >> (sh + 4)) & 0xFu) | (((s1 >> (sh + 6)) & 3u) << 4);
     }
-    const float dl = d * (float)sc, nm = -(dmin * (float)m);
+    const float dl = d * (float)sc * kMixScale, nm = -(dmin * (float)m);
     const int shift = 4 * (j & 1);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const uint32_t v = opaque((r.q[i] >> shift) & 0x0F0F0F0Fu);
-        out[2 * i] = pack_bf16(fmaf(dl, ubyte0(v), nm), fmaf(dl, ubyte1(v), nm));
-        out[2 * i + 1] = pack_bf16(fmaf(dl, ubyte2(v), nm), fmaf(dl, ubyte3(v), nm));
+        const uint32_t e02 = (r.q[i] >> shift) & 0x000F000Fu, e13 = (r.q[i] >> (shift + 8)) & 0x000F000Fu;
+        out[2 * i] = pack_bf16(mix_lo(e02, dl, nm), mix_lo(e13, dl, nm));
+        out[2 * i + 1] = pack_bf16(mix_hi(e02, dl, nm), mix_hi(e13, dl, nm));
     }
 }
 
