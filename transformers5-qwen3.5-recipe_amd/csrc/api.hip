@@ -2,6 +2,8 @@
 // point replaces are in include/ggml_mmq_gfx950.h.  Plain device pointers and sizes only.
 #include "../../include/ggml_mmq_gfx950.h"
 
+#include <algorithm>
+
 #include "launch.h"
 #include "mmq_host.h"
 
@@ -62,6 +64,18 @@ int ggq_dequantize(int qt, const void* packed, int64_t rows, int64_t k, void* ou
 }
 
 // ---------------------------------------------------------------------------------------------------
+// Second launch of a grouped call that runs its small groups in the wide shape: the same operands, the
+// tall instantiation, the row tiles of the larger groups.
+static int launch_tall_remainder(int qt, int mode, const MmqParams& wide_p, int rows, int n, int k, int nseg,
+                                 const TileDesc* tiles, const int* num_tiles, int max_tiles, hipStream_t s) {
+    MmqParams sizes;
+    if (int rc = init_params(sizes, qt, mode, rows, n, k, nseg, kShapeTall)) return rc;
+    MmqParams t = wide_p;
+    t.shape = kShapeTall, t.col_tiles_per_seg = sizes.col_tiles_per_seg, t.steps_per_seg = sizes.steps_per_seg;
+    t.tiles = tiles, t.num_tiles = num_tiles, t.max_row_tiles = max_tiles;
+    return launch_mmq(qt, mode, kEpiStore, t, s);
+}
+
 // Expert groups that average at most 192 rows run the Q4_K tile kernel in its wide shape.
 static int pick_shape(int qt, int64_t rows, int64_t groups) {
     return (qt == 12 /* GGML Q4_K */ && groups > 0 && rows <= 192 * groups) ? kShapeWide : kShapeTall;
@@ -71,7 +85,7 @@ int64_t ggq_lora_workspace_bytes(int64_t rows, int64_t groups, int64_t experts, 
     const int rp = rank_pad(r > 0 ? r : 1);
     if (experts < 1) experts = 1;
     const int64_t tiles = rows / 64 + groups + 2;
-    return 2 * align256(tiles * (int64_t)sizeof(TileDesc)) + align256(16) + align256(experts * 2 * 4) +
+    return 3 * align256(tiles * (int64_t)sizeof(TileDesc)) + align256(16) + align256(experts * 2 * 4) +
            align256(experts * n_total * rp * 2) * 2 + align256(experts * k * rp * 2) + align256(rows * rp * 2) + 4096;
 }
 
@@ -128,15 +142,26 @@ int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void*
     const TileDesc* tiles64 = nullptr;
     const int* num_tiles64 = nullptr;
     int max_tiles64 = (int)((rows + 63) / 64);
+    TileDesc* t_tall = nullptr;
+    const int* n_tall = nullptr;
+    int max_tall = 0;
     if (groups > 0) {
-        const int tile_rows = p.shape == kShapeWide ? kWideBM : kBM;
-        const int max128 = (int)(rows / tile_rows + groups);
+        // Wide shape: groups of at most 128 rows take one wide tile each, larger groups go to a second,
+        // tall launch (a second wide tile for a few dozen leftover rows would cost a whole decode pass).
+        const bool wide = p.shape == kShapeWide;
+        const int max128 = wide ? (int)groups : (int)(rows / kBM + groups);
+        max_tall = wide ? (int)std::min<int64_t>(rows / kBM + groups, rows / (kWideBM + 1) + rows / kBM + 1) : 0;
         max_tiles64 = (int)(rows / 64 + groups);
         TileDesc* t128 = (TileDesc*)bump.take((int64_t)max128 * sizeof(TileDesc));
+        t_tall = wide ? (TileDesc*)bump.take((int64_t)max_tall * sizeof(TileDesc)) : nullptr;
         TileDesc* t64 = lora_a ? (TileDesc*)bump.take((int64_t)max_tiles64 * sizeof(TileDesc)) : nullptr;
         int* counts = (int*)bump.take(16);
-        if (!t128 || !counts || (lora_a && !t64)) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
-        if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, tile_rows, t128, counts, nullptr, 0, s)) return rc;
+        if (!t128 || !counts || (lora_a && !t64) || (wide && !t_tall)) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
+        if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, wide ? kWideBM : kBM, t128, counts, nullptr, 0, s, 0, wide ? kWideBM : 0x7FFFFFFF)) return rc;
+        if (wide) {
+            if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, kBM, t_tall, counts + 2, nullptr, 0, s, kWideBM, 0x7FFFFFFF)) return rc;
+            n_tall = counts + 2;
+        }
         if (lora_a) {
             if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, 64, t64, counts + 1, nullptr, 0, s)) return rc;
         }
@@ -160,7 +185,9 @@ int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void*
         }
         p.la = (const bf16_t*)xa_out, p.lb = lb, p.lb_expert_elems = (int64_t)nseg * n * rp, p.r_pad = rp, p.lora_scale = scale;
     }
-    return launch_mmq(qt, kModeNT, kEpiStore, p, s);
+    if (int rc = launch_mmq(qt, kModeNT, kEpiStore, p, s)) return rc;
+    if (t_tall) return launch_tall_remainder(qt, kModeNT, p, (int)rows, (int)n, (int)k, nseg, t_tall, n_tall, max_tall, s);
+    return GGQ_OK;
 }
 
 // Backward: dx = dy . W (+ LoRA term), and the factor gradients over all `experts` planes.
@@ -195,16 +222,25 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
     const int* num_tiles64 = nullptr;
     const int* ranges = nullptr;
     int max_tiles64 = (int)((rows + 63) / 64);
+    TileDesc* t_tall = nullptr;
+    const int* n_tall = nullptr;
+    int max_tall = 0;
     if (groups > 0) {
-        const int tile_rows = p.shape == kShapeWide ? kWideBM : kBM;
-        const int max128 = (int)(rows / tile_rows + groups);
+        const bool wide = p.shape == kShapeWide;  // small groups: wide tiles; larger ones: a second, tall launch
+        const int max128 = wide ? (int)groups : (int)(rows / kBM + groups);
+        max_tall = wide ? (int)std::min<int64_t>(rows / kBM + groups, rows / (kWideBM + 1) + rows / kBM + 1) : 0;
         max_tiles64 = (int)(rows / 64 + groups);
         TileDesc* t128 = (TileDesc*)bump.take((int64_t)max128 * sizeof(TileDesc));
+        t_tall = wide ? (TileDesc*)bump.take((int64_t)max_tall * sizeof(TileDesc)) : nullptr;
         TileDesc* t64 = lora_a ? (TileDesc*)bump.take((int64_t)max_tiles64 * sizeof(TileDesc)) : nullptr;
         int* counts = (int*)bump.take(16);
         int* rg = lora_a ? (int*)bump.take(experts * 2 * 4) : nullptr;
-        if (!t128 || !counts || (lora_a && (!t64 || !rg))) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
-        if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, tile_rows, t128, counts, rg, (int)experts, s)) return rc;
+        if (!t128 || !counts || (lora_a && (!t64 || !rg)) || (wide && !t_tall)) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
+        if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, wide ? kWideBM : kBM, t128, counts, rg, (int)experts, s, 0, wide ? kWideBM : 0x7FFFFFFF)) return rc;
+        if (wide) {
+            if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, kBM, t_tall, counts + 2, nullptr, 0, s, kWideBM, 0x7FFFFFFF)) return rc;
+            n_tall = counts + 2;
+        }
         if (lora_a) {
             if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, 64, t64, counts + 1, nullptr, 0, s)) return rc;
         }
@@ -245,7 +281,9 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
         }
     }
     if (rows == 0) return GGQ_OK;
-    return launch_mmq(qt, kModeNN, kEpiStore, p, s);
+    if (int rc = launch_mmq(qt, kModeNN, kEpiStore, p, s)) return rc;
+    if (t_tall) return launch_tall_remainder(qt, kModeNN, p, (int)rows, (int)n, (int)k, nseg, t_tall, n_tall, max_tall, s);
+    return GGQ_OK;
 }
 
 // ---------------------------------------------------------------------------------------------------

@@ -29,8 +29,9 @@ int check_launch(const char* what) {
 // Row-tile table.  One workgroup; groups are walked 256 at a time with an LDS prefix sum, so the table
 // is in group order and identical from run to run.
 __global__ __launch_bounds__(256) void build_row_tiles_kernel(const int64_t* expert_ids, const int32_t* end_offsets,
-                                                              int groups, int bm, TileDesc* tiles, int* num_tiles,
-                                                              int* expert_ranges, int num_experts) {
+                                                              int groups, int bm, int min_rows, int max_rows,
+                                                              TileDesc* tiles, int* num_tiles, int* expert_ranges,
+                                                              int num_experts) {
     __shared__ int scan[256];
     __shared__ int base;
     const int tid = threadIdx.x;
@@ -45,7 +46,8 @@ __global__ __launch_bounds__(256) void build_row_tiles_kernel(const int64_t* exp
         if (g < groups) {
             r0 = g == 0 ? 0 : end_offsets[g - 1];
             r1 = end_offsets[g];
-            count = r1 > r0 ? (r1 - r0 + bm - 1) / bm : 0;
+            // only groups with min_rows < rows <= max_rows get tiles in this table
+            count = (r1 - r0 > min_rows && r1 - r0 <= max_rows) ? (r1 - r0 + bm - 1) / bm : 0;
             if (expert_ranges) {
                 const int64_t e = expert_ids ? expert_ids[g] : g;
                 if (e >= 0 && e < num_experts) expert_ranges[2 * e] = r0, expert_ranges[2 * e + 1] = r1;
@@ -73,9 +75,9 @@ __global__ __launch_bounds__(256) void build_row_tiles_kernel(const int64_t* exp
 }
 
 int build_row_tiles(const int64_t* expert_ids, const int32_t* end_offsets, int groups, int bm, TileDesc* tiles,
-                    int* num_tiles, int* expert_ranges, int num_experts, hipStream_t s) {
-    hipLaunchKernelGGL(build_row_tiles_kernel, dim3(1), dim3(256), 0, s, expert_ids, end_offsets, groups, bm, tiles,
-                       num_tiles, expert_ranges, num_experts);
+                    int* num_tiles, int* expert_ranges, int num_experts, hipStream_t s, int min_rows, int max_rows) {
+    hipLaunchKernelGGL(build_row_tiles_kernel, dim3(1), dim3(256), 0, s, expert_ids, end_offsets, groups, bm, min_rows,
+                       max_rows, tiles, num_tiles, expert_ranges, num_experts);
     return check_launch("build_row_tiles");
 }
 

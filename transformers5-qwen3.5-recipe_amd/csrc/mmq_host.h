@@ -96,7 +96,7 @@ int factor_grad(const FactorGradParams& p, int r_pad, int64_t experts, hipStream
 // Builds the row-tile table of an expert-sorted layout on the device (no host sync):
 // tiles[0..*num_tiles) in group order, tile height bm; optionally per-expert row ranges.
 int build_row_tiles(const int64_t* expert_ids, const int32_t* end_offsets, int groups, int bm, TileDesc* tiles,
-                    int* num_tiles, int* expert_ranges, int num_experts, hipStream_t s);
+                    int* num_tiles, int* expert_ranges, int num_experts, hipStream_t s, int min_rows = 0, int max_rows = 0x7FFFFFFF);
 
 int64_t route_plan_workspace_bytes(int64_t routes, int num_experts);
 int route_plan(const void* topk_ids, int ids_are_int64, int64_t tokens, int top_k, int num_experts,

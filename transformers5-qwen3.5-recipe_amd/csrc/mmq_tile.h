@@ -863,18 +863,22 @@ static __device__ __forceinline__ void run(const MmqParams& p) {
 
     // ---- tile assignment.  Hardware deals consecutive workgroup ids round-robin over the 8 XCDs; remap
     // so that consecutive logical tiles (which share an A tile) land on one XCD and hit its L2.
+    // The split uses the number of tiles that exist (read from the device-built table for grouped
+    // launches), not the launch's upper bound, so all eight XCDs get an equal share of real work.
     const int col_tiles = (MODE == kModeNT ? p.nseg : 1) * p.col_tiles_per_seg;
-    const int per_xcd = (int)(gridDim.x >> 3);  // the launcher pads the grid to a multiple of 8
-    const int logical = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    const int row_tiles = p.tiles ? min(*p.num_tiles, p.max_row_tiles) : p.max_row_tiles;
+    const int total_tiles = row_tiles * col_tiles;
+    const int per_xcd = (total_tiles + 7) >> 3;
+    const int slot = (int)(blockIdx.x >> 3);
+    const int logical = (int)(blockIdx.x & 7) * per_xcd + slot;
+    if (slot >= per_xcd || logical >= total_tiles) return;
     const int row_tile = logical / col_tiles;
     c.col_tile = logical - row_tile * col_tiles;
     int group = 0, row_end;
     if (p.tiles) {
-        if (row_tile >= p.max_row_tiles || row_tile >= *p.num_tiles) return;
         const TileDesc t = p.tiles[row_tile];
         group = t.group, c.row_begin = t.row_begin, row_end = t.row_end;
     } else {
-        if (row_tile >= p.max_row_tiles) return;
         c.row_begin = row_tile * kTM;
         row_end = min(p.m, c.row_begin + kTM);
     }
