@@ -64,16 +64,14 @@ int ggq_dequantize(int qt, const void* packed, int64_t rows, int64_t k, void* ou
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Second launch of a grouped call that runs its small groups in the wide shape: the same operands, the
-// tall instantiation, the row tiles of the larger groups.
-static int launch_tall_remainder(int qt, int mode, const MmqParams& wide_p, int rows, int n, int k, int nseg,
-                                 const TileDesc* tiles, const int* num_tiles, int max_tiles, hipStream_t s) {
+// A grouped call that runs its small groups in the wide shape puts the row tiles of its larger groups in a
+// second table; one mixed launch covers both.
+static int launch_wide_and_tall(int qt, int mode, MmqParams& p, int rows, int n, int k, int nseg, const TileDesc* tall,
+                                const int* num_tall, int max_tall, hipStream_t s) {
     MmqParams sizes;
     if (int rc = init_params(sizes, qt, mode, rows, n, k, nseg, kShapeTall)) return rc;
-    MmqParams t = wide_p;
-    t.shape = kShapeTall, t.col_tiles_per_seg = sizes.col_tiles_per_seg, t.steps_per_seg = sizes.steps_per_seg;
-    t.tiles = tiles, t.num_tiles = num_tiles, t.max_row_tiles = max_tiles;
-    return launch_mmq(qt, mode, kEpiStore, t, s);
+    p.tiles2 = tall, p.num_tiles2 = num_tall, p.max_row_tiles2 = max_tall, p.col_tiles_per_seg2 = sizes.col_tiles_per_seg;
+    return launch_mmq_mixed(mode, p, s);
 }
 
 // Expert groups that average at most 192 rows run the Q4_K tile kernel in its wide shape.
@@ -185,9 +183,8 @@ int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void*
         }
         p.la = (const bf16_t*)xa_out, p.lb = lb, p.lb_expert_elems = (int64_t)nseg * n * rp, p.r_pad = rp, p.lora_scale = scale;
     }
-    if (int rc = launch_mmq(qt, kModeNT, kEpiStore, p, s)) return rc;
-    if (t_tall) return launch_tall_remainder(qt, kModeNT, p, (int)rows, (int)n, (int)k, nseg, t_tall, n_tall, max_tall, s);
-    return GGQ_OK;
+    if (t_tall) return launch_wide_and_tall(qt, kModeNT, p, (int)rows, (int)n, (int)k, nseg, t_tall, n_tall, max_tall, s);
+    return launch_mmq(qt, kModeNT, kEpiStore, p, s);
 }
 
 // Backward: dx = dy . W (+ LoRA term), and the factor gradients over all `experts` planes.
@@ -281,9 +278,8 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
         }
     }
     if (rows == 0) return GGQ_OK;
-    if (int rc = launch_mmq(qt, kModeNN, kEpiStore, p, s)) return rc;
-    if (t_tall) return launch_tall_remainder(qt, kModeNN, p, (int)rows, (int)n, (int)k, nseg, t_tall, n_tall, max_tall, s);
-    return GGQ_OK;
+    if (t_tall) return launch_wide_and_tall(qt, kModeNN, p, (int)rows, (int)n, (int)k, nseg, t_tall, n_tall, max_tall, s);
+    return launch_mmq(qt, kModeNN, kEpiStore, p, s);
 }
 
 // ---------------------------------------------------------------------------------------------------

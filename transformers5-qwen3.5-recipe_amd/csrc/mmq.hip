@@ -139,6 +139,39 @@ static int launch_one(const MmqParams& p, hipStream_t s) {
     return check_launch("mmq_tile_kernel");
 }
 
+template <int MODE>
+static int launch_mixed_mode(const MmqParams& p, hipStream_t s) {
+    const int segs = MODE == kModeNT ? p.nseg : 1;
+    // per XCD: ceil(wide units / 8) * wide column tiles + ceil(tall units / 8) * tall column tiles slots
+    const int64_t slots = (int64_t)((p.max_row_tiles + 7) / 8) * segs * p.col_tiles_per_seg +
+                          (int64_t)((p.max_row_tiles2 + 7) / 8) * segs * p.col_tiles_per_seg2;
+    if (slots <= 0) return GGQ_OK;
+    const int64_t grid = slots * 8;
+    if (grid > 0x7FFFFFF0) return set_error(GGQ_ERR_SHAPE, "mmq: too many tiles for one launch");
+    TimedLaunch* t = nullptr;
+    if (g_timing && g_timed_count < kMaxTimedLaunches) {
+        t = &g_timed[g_timed_count];
+        if (hipEventCreate(&t->start) != hipSuccess || hipEventCreate(&t->stop) != hipSuccess) return set_error(GGQ_ERR_RUNTIME, "mmq: event creation failed");
+        t->qt = kQ4_K, t->mode = MODE, t->epi = kEpiStore;
+        g_timed_count++;
+        (void)hipEventRecord(t->start, s);
+    }
+    constexpr int kSmemBytes = Tile<kShapeWide>::kTileLdsBytes > Tile<kShapeTall>::kTileLdsBytes ? Tile<kShapeWide>::kTileLdsBytes : Tile<kShapeTall>::kTileLdsBytes;
+    static bool attr_set = false;
+    if (!attr_set) {
+        if (hipFuncSetAttribute((const void*)mmq_mixed_kernel<kQ4_K, MODE, kEpiStore>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess)
+            return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", kSmemBytes);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((mmq_mixed_kernel<kQ4_K, MODE, kEpiStore>), dim3((unsigned)grid), dim3(kThreads), kSmemBytes, s, p);
+    if (t) (void)hipEventRecord(t->stop, s);
+    return check_launch("mmq_mixed_kernel");
+}
+
+int launch_mmq_mixed(int mode, const MmqParams& p, hipStream_t s) {
+    return mode == kModeNT ? launch_mixed_mode<kModeNT>(p, s) : launch_mixed_mode<kModeNN>(p, s);
+}
+
 template <int QT>
 static int launch_qt(int mode, int epi, const MmqParams& p, hipStream_t s) {
     if (mode == kModeNT) {

@@ -64,6 +64,11 @@ struct MmqParams {
     const TileDesc* tiles;
     const int* num_tiles;
     int max_row_tiles;
+    // second table of a mixed launch (tall tiles; `tiles` then holds the wide ones)
+    const TileDesc* tiles2;
+    const int* num_tiles2;
+    int max_row_tiles2;
+    int col_tiles_per_seg2;
     int shape;  // kShapeTall / kShapeWide: which instantiation of the tile kernel the sizes above are for
     // LoRA
     const bf16_t* la;     // [rows, r_pad]  (x A^T in NT, dY B in NN)
@@ -86,6 +91,7 @@ int profile_begin();
 int profile_end(float* ms, int* qt, int* mode, int* epi, int capacity);
 const char* last_error();
 int launch_mmq(int qt, int mode, int epi, const MmqParams& p, hipStream_t s);
+int launch_mmq_mixed(int mode, const MmqParams& p, hipStream_t s);  // Q4_K, store epilogue, tiles + tiles2
 int init_params(MmqParams& p, int qt, int mode, int m, int n, int k, int nseg, int shape = kShapeTall);
 
 int pad_factor(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int r, int r_pad, bool transpose, hipStream_t s);

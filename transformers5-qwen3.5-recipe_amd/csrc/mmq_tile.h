@@ -848,8 +848,26 @@ static __device__ __forceinline__ void consume_idle(const MmqParams& p, const Ti
     }
 }
 
+// Tile assignment of a single-shape launch.  Hardware deals consecutive workgroup ids round-robin over
+// the 8 XCDs; remap so that consecutive logical tiles (which share an A tile) land on one XCD and hit
+// its L2.  The split uses the number of tiles that exist (read from the device-built table for grouped
+// launches), not the launch's upper bound, so all eight XCDs get an equal share of real work.
 template <int QT, int MODE, int EPI>
 static __device__ __forceinline__ void run(const MmqParams& p) {
+    const int col_tiles = (MODE == kModeNT ? p.nseg : 1) * p.col_tiles_per_seg;
+    const int row_tiles = p.tiles ? min(*p.num_tiles, p.max_row_tiles) : p.max_row_tiles;
+    const int total_tiles = row_tiles * col_tiles;
+    const int per_xcd = (total_tiles + 7) >> 3;
+    const int slot = (int)(blockIdx.x >> 3);
+    const int logical = (int)(blockIdx.x & 7) * per_xcd + slot;
+    if (slot >= per_xcd || logical >= total_tiles) return;
+    const int row_tile = logical / col_tiles;
+    run_tile<QT, MODE, EPI>(p, p.tiles, row_tile, logical - row_tile * col_tiles, p.col_tiles_per_seg);
+}
+
+// One output tile: row tile `row_tile` of `tiles` (or of the dense row range), column tile `col_tile`.
+template <int QT, int MODE, int EPI>
+static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDesc* tiles, int row_tile, int col_tile, int col_tiles_per_seg) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_raw[];
     TileCtx c;
     c.as = smem_raw;
@@ -861,22 +879,10 @@ static __device__ __forceinline__ void run(const MmqParams& p) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps control flow scalar
 
-    // ---- tile assignment.  Hardware deals consecutive workgroup ids round-robin over the 8 XCDs; remap
-    // so that consecutive logical tiles (which share an A tile) land on one XCD and hit its L2.
-    // The split uses the number of tiles that exist (read from the device-built table for grouped
-    // launches), not the launch's upper bound, so all eight XCDs get an equal share of real work.
-    const int col_tiles = (MODE == kModeNT ? p.nseg : 1) * p.col_tiles_per_seg;
-    const int row_tiles = p.tiles ? min(*p.num_tiles, p.max_row_tiles) : p.max_row_tiles;
-    const int total_tiles = row_tiles * col_tiles;
-    const int per_xcd = (total_tiles + 7) >> 3;
-    const int slot = (int)(blockIdx.x >> 3);
-    const int logical = (int)(blockIdx.x & 7) * per_xcd + slot;
-    if (slot >= per_xcd || logical >= total_tiles) return;
-    const int row_tile = logical / col_tiles;
-    c.col_tile = logical - row_tile * col_tiles;
+    c.col_tile = col_tile;
     int group = 0, row_end;
-    if (p.tiles) {
-        const TileDesc t = p.tiles[row_tile];
+    if (tiles) {
+        const TileDesc t = tiles[row_tile];
         group = t.group, c.row_begin = t.row_begin, row_end = t.row_end;
     } else {
         c.row_begin = row_tile * kTM;
@@ -885,8 +891,8 @@ static __device__ __forceinline__ void run(const MmqParams& p) {
     c.rows_valid = row_end - c.row_begin;  // 1..kTM
     c.expert = p.expert_ids ? p.expert_ids[group] : 0;
     // column tile -> (segment, first output column inside the segment)
-    c.seg_c = MODE == kModeNT ? c.col_tile / p.col_tiles_per_seg : 0;
-    c.col0 = (c.col_tile - c.seg_c * p.col_tiles_per_seg) * kTN;
+    c.seg_c = MODE == kModeNT ? c.col_tile / col_tiles_per_seg : 0;
+    c.col0 = (c.col_tile - c.seg_c * col_tiles_per_seg) * kTN;
     c.out_cols = MODE == kModeNT ? p.n : p.k;     // output columns per segment
     c.contraction = MODE == kModeNT ? p.k : p.n;  // contraction length per segment
     c.total_steps = (MODE == kModeNN ? p.nseg : 1) * p.steps_per_seg;
@@ -938,6 +944,27 @@ static __device__ __forceinline__ void run(const MmqParams& p) {
 template <int QT, int MODE, int EPI, int SH>
 __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(4, 4))) void mmq_tile_kernel(const MmqParams p) {
     Tile<SH>::template run<QT, MODE, EPI>(p);
+}
+
+// Grouped launch with both shapes in one grid: wide tiles for the row tiles of table `tiles`, tall tiles
+// for those of `tiles2`.  A row tile with all its column tiles is the unit that must stay on one XCD (its
+// A tile is shared); units go round-robin over the XCDs, wide (heavier) units first, so that every XCD
+// gets an equal share of both kinds.
+template <int QT, int MODE, int EPI>
+__global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(4, 4))) void mmq_mixed_kernel(const MmqParams p) {
+    const int segs = MODE == kModeNT ? p.nseg : 1;
+    const int cols_w = segs * p.col_tiles_per_seg, cols_t = segs * p.col_tiles_per_seg2;
+    const int n_w = min(*p.num_tiles, p.max_row_tiles), n_t = min(*p.num_tiles2, p.max_row_tiles2);
+    const int xcd = (int)(blockIdx.x & 7), slot = (int)(blockIdx.x >> 3);
+    const int units_w = (n_w - xcd + 7) >> 3, units_t = (n_t - xcd + 7) >> 3;  // units xcd, xcd + 8, ...
+    const int slots_w = units_w * cols_w;
+    if (slot < slots_w) {
+        const int unit = slot / cols_w;
+        Tile<kShapeWide>::template run_tile<QT, MODE, EPI>(p, p.tiles, xcd + 8 * unit, slot - unit * cols_w, p.col_tiles_per_seg);
+    } else if (slot - slots_w < units_t * cols_t) {
+        const int s2 = slot - slots_w, unit = s2 / cols_t;
+        Tile<kShapeTall>::template run_tile<QT, MODE, EPI>(p, p.tiles2, xcd + 8 * unit, s2 - unit * cols_t, p.col_tiles_per_seg2);
+    }
 }
 
 }  // namespace ggq
