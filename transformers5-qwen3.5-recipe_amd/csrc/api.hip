@@ -155,14 +155,11 @@ int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void*
         TileDesc* t64 = lora_a ? (TileDesc*)bump.take((int64_t)max_tiles64 * sizeof(TileDesc)) : nullptr;
         int* counts = (int*)bump.take(16);
         if (!t128 || !counts || (lora_a && !t64) || (wide && !t_tall)) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
-        if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, wide ? kWideBM : kBM, t128, counts, nullptr, 0, s, 0, wide ? kWideBM : 0x7FFFFFFF)) return rc;
-        if (wide) {
-            if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, kBM, t_tall, counts + 2, nullptr, 0, s, kWideBM, 0x7FFFFFFF)) return rc;
-            n_tall = counts + 2;
-        }
-        if (lora_a) {
-            if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, 64, t64, counts + 1, nullptr, 0, s)) return rc;
-        }
+        RowTileTables tb{};
+        tb.add(wide ? kWideBM : kBM, 0, wide ? kWideBM : 0x7FFFFFFF, t128, counts);
+        if (wide) tb.add(kBM, kWideBM, 0x7FFFFFFF, t_tall, counts + 2), n_tall = counts + 2;
+        if (lora_a) tb.add(64, 0, 0x7FFFFFFF, t64, counts + 1);
+        if (int rc = build_row_tile_tables(expert_ids, end_offsets, (int)groups, tb, nullptr, 0, s)) return rc;
         p.expert_ids = expert_ids, p.tiles = t128, p.num_tiles = counts, p.max_row_tiles = max128;
         tiles64 = t64, num_tiles64 = counts + 1;
     }
@@ -233,14 +230,11 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
         int* counts = (int*)bump.take(16);
         int* rg = lora_a ? (int*)bump.take(experts * 2 * 4) : nullptr;
         if (!t128 || !counts || (lora_a && (!t64 || !rg)) || (wide && !t_tall)) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
-        if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, wide ? kWideBM : kBM, t128, counts, rg, (int)experts, s, 0, wide ? kWideBM : 0x7FFFFFFF)) return rc;
-        if (wide) {
-            if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, kBM, t_tall, counts + 2, nullptr, 0, s, kWideBM, 0x7FFFFFFF)) return rc;
-            n_tall = counts + 2;
-        }
-        if (lora_a) {
-            if (int rc = build_row_tiles(expert_ids, end_offsets, (int)groups, 64, t64, counts + 1, nullptr, 0, s)) return rc;
-        }
+        RowTileTables tb{};
+        tb.add(wide ? kWideBM : kBM, 0, wide ? kWideBM : 0x7FFFFFFF, t128, counts);
+        if (wide) tb.add(kBM, kWideBM, 0x7FFFFFFF, t_tall, counts + 2), n_tall = counts + 2;
+        if (lora_a) tb.add(64, 0, 0x7FFFFFFF, t64, counts + 1);
+        if (int rc = build_row_tile_tables(expert_ids, end_offsets, (int)groups, tb, rg, (int)experts, s)) return rc;
         p.expert_ids = expert_ids, p.tiles = t128, p.num_tiles = counts, p.max_row_tiles = max128;
         tiles64 = t64, num_tiles64 = counts + 1, ranges = rg;
     }

@@ -49,7 +49,30 @@ __global__ __launch_bounds__(256) void skinny_nt_kernel(SkinnyNtParams p) {
         const bf16_t* in = p.in[seg] + (int64_t)row * p.ld_in;
         const bool vec = ((p.ld_in & 7) == 0) && (((uintptr_t)p.in[seg] & 15) == 0);
         const bool fvec = ((p.ldf & 7) == 0) && ((p.c & 7) == 0) && (((uintptr_t)p.f & 15) == 0);
-        for (int c0 = 0; c0 < p.c; c0 += 32) {
+        int c0 = 0;
+        if (vec && fvec) {
+            // aligned operands: four sub-steps per trip with every load issued ahead of the MFMAs (the
+            // stream is latency-bound otherwise: one wave owns 16 rows)
+            for (; c0 + 128 <= p.c; c0 += 128) {
+                uint4 av[4], bv[JB][4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int cc = c0 + 32 * u + lq * 8;
+                    av[u] = row_ok ? *(const uint4*)(in + cc) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+                    for (int jb = 0; jb < JB; jb++) {
+                        const int j = jb * 16 + li;
+                        bv[jb][u] = j < p.r ? *(const uint4*)(f + (int64_t)j * p.ldf + seg * p.c + cc) : make_uint4(0, 0, 0, 0);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+#pragma unroll
+                    for (int jb = 0; jb < JB; jb++)
+                        acc[jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[u]), __builtin_bit_cast(bf16x8_t, bv[jb][u]), acc[jb], 0, 0, 0);
+            }
+        }
+        for (; c0 < p.c; c0 += 32) {
             const int cc = c0 + lq * 8;
             const uint4 av = load8g(in + cc, row_ok ? p.c - cc : 0, vec);
             const bf16x8_t a = __builtin_bit_cast(bf16x8_t, av);
@@ -146,28 +169,47 @@ __global__ __launch_bounds__(256) void factor_grad_kernel(FactorGradParams p) {
 
 // dst[e][c][0..r_pad) = src[e][c][0..r) zero padded   (transpose = false, src [E][C][r])
 // dst[e][c][0..r_pad) = src[e][0..r)[c] zero padded   (transpose = true,  src [E][r][C])
-__global__ void pad_factor_kernel(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int r, int r_pad, int transpose) {
-    const int64_t total = experts * c * r_pad;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
-        const int j = (int)(i % r_pad);
-        const int64_t ec = i / r_pad;
+// One lane per (e, c): its r_pad outputs are contiguous (16-byte stores); with transpose the reads of a
+// wave are 64 consecutive columns of one factor row.
+__global__ __launch_bounds__(256) void pad_factor_kernel(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int r, int r_pad, int transpose) {
+    const int64_t total = experts * c;
+    for (int64_t ec = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; ec < total; ec += (int64_t)gridDim.x * blockDim.x) {
         const int cc = (int)(ec % c);
         const int64_t e = ec / c;
-        bf16_t v = 0;
-        if (j < r) v = transpose ? src[(e * r + j) * c + cc] : src[(e * c + cc) * r + j];
-        dst[i] = v;
+        for (int j0 = 0; j0 < r_pad; j0 += 8) {
+            uint32_t v[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int j = j0 + i;
+                v[i] = j < r ? (uint32_t)(transpose ? src[(e * r + j) * c + cc] : src[ec * r + j]) : 0u;
+            }
+            *(uint4*)(dst + ec * r_pad + j0) = make_uint4(v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16));
+        }
     }
 }
 
-// dst[e][j][c] = src[e][c][j]  for j < r  (B [E][C][r] -> B^T [E][r][C])
-__global__ void transpose_factor_kernel(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int r) {
-    const int64_t total = experts * c * r;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
-        const int cc = (int)(i % c);
-        const int64_t ej = i / c;
-        const int j = (int)(ej % r);
-        const int64_t e = ej / r;
-        dst[i] = src[(e * c + cc) * r + j];
+// dst[e][j][c] = src[e][c][j]  for j < r  (B [E][C][r] -> B^T [E][r][C]).  One lane per (e, c): it reads
+// its r contiguous inputs and a wave writes 64 consecutive columns of each output row.
+__global__ __launch_bounds__(256) void transpose_factor_kernel(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int r) {
+    const int64_t total = experts * c;
+    const bool vec = (r & 7) == 0 && (((uintptr_t)src & 15) == 0);
+    for (int64_t ec = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; ec < total; ec += (int64_t)gridDim.x * blockDim.x) {
+        const int cc = (int)(ec % c);
+        const int64_t e = ec / c;
+        for (int j0 = 0; j0 < r; j0 += 8) {
+            uint32_t w[4] = {0u, 0u, 0u, 0u};
+            if (vec) {
+                const uint4 q = *(const uint4*)(src + ec * r + j0);
+                w[0] = q.x, w[1] = q.y, w[2] = q.z, w[3] = q.w;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; i++)
+                    if (j0 + i < r) w[i >> 1] |= (uint32_t)src[ec * r + j0 + i] << (16 * (i & 1));
+            }
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                if (j0 + i < r) dst[(e * r + j0 + i) * c + cc] = (bf16_t)(w[i >> 1] >> (16 * (i & 1)));
+        }
     }
 }
 
@@ -177,14 +219,14 @@ static inline unsigned grid_for(int64_t total, int block) {
 }
 
 int pad_factor(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int r, int r_pad, bool transpose, hipStream_t s) {
-    const int64_t total = experts * c * r_pad;
+    const int64_t total = experts * c;
     if (total == 0) return 0;
     hipLaunchKernelGGL(pad_factor_kernel, dim3(grid_for(total, 256)), dim3(256), 0, s, src, dst, experts, c, r, r_pad, transpose ? 1 : 0);
     return check_launch("pad_factor");
 }
 
 int transpose_factor(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int r, hipStream_t s) {
-    const int64_t total = experts * c * r;
+    const int64_t total = experts * c;
     if (total == 0) return 0;
     hipLaunchKernelGGL(transpose_factor_kernel, dim3(grid_for(total, 256)), dim3(256), 0, s, src, dst, experts, c, r);
     return check_launch("transpose_factor");

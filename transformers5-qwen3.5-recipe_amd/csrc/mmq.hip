@@ -26,16 +26,18 @@ int check_launch(const char* what) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Row-tile table.  One workgroup; groups are walked 256 at a time with an LDS prefix sum, so the table
-// is in group order and identical from run to run.
+// Row-tile tables.  One workgroup per table; groups are walked 256 at a time with an LDS prefix sum, so
+// a table is in group order and identical from run to run.  Table t keeps the groups with
+// min_rows[t] < rows <= max_rows[t] and cuts them into tiles of bm[t] rows.
 __global__ __launch_bounds__(256) void build_row_tiles_kernel(const int64_t* expert_ids, const int32_t* end_offsets,
-                                                              int groups, int bm, int min_rows, int max_rows,
-                                                              TileDesc* tiles, int* num_tiles, int* expert_ranges,
+                                                              int groups, RowTileTables tb, int* expert_ranges,
                                                               int num_experts) {
     __shared__ int scan[256];
     __shared__ int base;
-    const int tid = threadIdx.x;
-    if (expert_ranges) {
+    const int tid = threadIdx.x, t = blockIdx.x;
+    const int bm = tb.bm[t], min_rows = tb.min_rows[t], max_rows = tb.max_rows[t];
+    TileDesc* tiles = tb.tiles[t];
+    if (expert_ranges && t == 0) {
         for (int e = tid; e < num_experts; e += 256) expert_ranges[2 * e] = expert_ranges[2 * e + 1] = 0;
     }
     if (tid == 0) base = 0;
@@ -46,9 +48,8 @@ __global__ __launch_bounds__(256) void build_row_tiles_kernel(const int64_t* exp
         if (g < groups) {
             r0 = g == 0 ? 0 : end_offsets[g - 1];
             r1 = end_offsets[g];
-            // only groups with min_rows < rows <= max_rows get tiles in this table
             count = (r1 - r0 > min_rows && r1 - r0 <= max_rows) ? (r1 - r0 + bm - 1) / bm : 0;
-            if (expert_ranges) {
+            if (expert_ranges && t == 0) {
                 const int64_t e = expert_ids ? expert_ids[g] : g;
                 if (e >= 0 && e < num_experts) expert_ranges[2 * e] = r0, expert_ranges[2 * e + 1] = r1;
             }
@@ -62,23 +63,31 @@ __global__ __launch_bounds__(256) void build_row_tiles_kernel(const int64_t* exp
             __syncthreads();
         }
         const int first = base + scan[tid] - count;
-        for (int t = 0; t < count; t++) {
+        for (int i = 0; i < count; i++) {
             TileDesc d;
-            d.group = g, d.row_begin = r0 + t * bm, d.row_end = min(r1, r0 + (t + 1) * bm), d.pad = 0;
-            tiles[first + t] = d;
+            d.group = g, d.row_begin = r0 + i * bm, d.row_end = min(r1, r0 + (i + 1) * bm), d.pad = 0;
+            tiles[first + i] = d;
         }
         __syncthreads();
         if (tid == 255) base += scan[255];
         __syncthreads();
     }
-    if (tid == 0) *num_tiles = base;
+    if (tid == 0) *tb.num_tiles[t] = base;
+}
+
+int build_row_tile_tables(const int64_t* expert_ids, const int32_t* end_offsets, int groups, const RowTileTables& tb,
+                          int* expert_ranges, int num_experts, hipStream_t s) {
+    if (tb.count <= 0) return GGQ_OK;
+    hipLaunchKernelGGL(build_row_tiles_kernel, dim3(tb.count), dim3(256), 0, s, expert_ids, end_offsets, groups, tb,
+                       expert_ranges, num_experts);
+    return check_launch("build_row_tiles");
 }
 
 int build_row_tiles(const int64_t* expert_ids, const int32_t* end_offsets, int groups, int bm, TileDesc* tiles,
                     int* num_tiles, int* expert_ranges, int num_experts, hipStream_t s, int min_rows, int max_rows) {
-    hipLaunchKernelGGL(build_row_tiles_kernel, dim3(1), dim3(256), 0, s, expert_ids, end_offsets, groups, bm, min_rows,
-                       max_rows, tiles, num_tiles, expert_ranges, num_experts);
-    return check_launch("build_row_tiles");
+    RowTileTables tb{};
+    tb.add(bm, min_rows, max_rows, tiles, num_tiles);
+    return build_row_tile_tables(expert_ids, end_offsets, groups, tb, expert_ranges, num_experts, s);
 }
 
 // ------------------------------------------------------------------------------------------------

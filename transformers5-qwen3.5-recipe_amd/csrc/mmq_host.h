@@ -101,6 +101,19 @@ int factor_grad(const FactorGradParams& p, int r_pad, int64_t experts, hipStream
 
 // Builds the row-tile table of an expert-sorted layout on the device (no host sync):
 // tiles[0..*num_tiles) in group order, tile height bm; optionally per-expert row ranges.
+// Up to three row-tile tables built by one launch (one workgroup each).
+struct RowTileTables {
+    int count;
+    int bm[3], min_rows[3], max_rows[3];
+    TileDesc* tiles[3];
+    int* num_tiles[3];
+    void add(int bm_, int min_rows_, int max_rows_, TileDesc* tiles_, int* num_tiles_) {
+        bm[count] = bm_, min_rows[count] = min_rows_, max_rows[count] = max_rows_, tiles[count] = tiles_, num_tiles[count] = num_tiles_;
+        count++;
+    }
+};
+int build_row_tile_tables(const int64_t* expert_ids, const int32_t* end_offsets, int groups, const RowTileTables& tb,
+                          int* expert_ranges, int num_experts, hipStream_t s);
 int build_row_tiles(const int64_t* expert_ids, const int32_t* end_offsets, int groups, int bm, TileDesc* tiles,
                     int* num_tiles, int* expert_ranges, int num_experts, hipStream_t s, int min_rows = 0, int max_rows = 0x7FFFFFFF);
 
