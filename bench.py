@@ -195,7 +195,7 @@ def main() -> None:
     per_mode = {0: [], 1: []}
     for j in range(max(n, 0)):
         per_mode[mode[j]].append(ms[j])
-    names = {0: "mmq_tile_kernel<Q4_K, forward, store>", 1: "mmq_tile_kernel<Q4_K, grad_input, store>"}
+    names = {0: "mmq_mixed_kernel<Q4_K, forward, store>", 1: "mmq_mixed_kernel<Q4_K, grad_input, store>"}
     dominant = max(per_mode, key=lambda m: sum(per_mode[m]))
     launches = len(per_mode[dominant])
     avg_ms = sum(per_mode[dominant]) / max(launches, 1)
@@ -203,6 +203,10 @@ def main() -> None:
     flops_per_launch = (fl["gate_up"] + fl["down"]) / 2
     achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12 if launches else 0.0
     kernel_ms_per_step = {names[m]: sum(v) / prof_steps for m, v in per_mode.items()}
+    # HBM bytes per launch (fetched + written, average of the gate/up and down launches) from the FETCH_SIZE /
+    # WRITE_SIZE counter runs summarised in profiles/mmq_mixed_q4k_grouped_moe_lora_step.pmc_traffic.txt;
+    # the counters are collected offline, so this figure only changes when that profile is redone.
+    traffic_bytes = {0: 330.3e6 + 100.7e6, 1: 343.7e6 + 83.9e6}[dominant]
 
     result = {
         "metric": "fwd+bwd TFLOP/s and weight GB/s, Q4_K grouped-MoE LoRA; % of MI355X roofline",
@@ -223,7 +227,7 @@ def main() -> None:
         "pct_of_mfma_peak": 100.0 * fl["total"] / (ms_per_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
         "pct_of_hbm_peak_weights": 100.0 * 2 * packed_weight_bytes(cfg) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "roofline": {"bound": "mfma", "kernel": names[dominant], "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "avg_launch_ms": avg_ms, "launches_timed": launches,
+                     "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic_bytes, "avg_launch_ms": avg_ms, "launches_timed": launches,
                      "flops_per_launch": flops_per_launch},
         "tile_kernel_ms_per_step": kernel_ms_per_step,
     }
