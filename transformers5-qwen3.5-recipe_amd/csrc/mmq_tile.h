@@ -23,8 +23,9 @@
 //   * producer waves 8..15 own the weights, as two quartets that take alternate steps: a quartet
 //     decodes its step into registers during one phase (packed bytes global -> registers, scales / mins
 //     / codebook unpacked in registers, blocks.h) and stores the bf16 W tile, laid out [output
-//     column][contraction], during the next, while the other quartet decodes; in NN mode that store is
-//     the transposition.  For Q4_K forward a lane loads its share of a 256-wide block once and keeps it
+//     column][contraction] for forward, during the next, while the other quartet decodes; for grad-input
+//     the tile is stored as decoded, [contraction row][output column], and the consumers transpose it
+//     on the way out of LDS (ds_read_b64_tr_b16).  For Q4_K forward a lane loads its share of a 256-wide block once and keeps it
 //     for the block's steps, so every cache line of the packed row is requested in one burst.
 // One barrier per step hands the buffers over; decode VALU work and MFMA work overlap on every SIMD.
 #pragma once
@@ -117,10 +118,11 @@ static constexpr int kAStages = SH == 0 ? 3 : 5;
 static constexpr int kAhead = kAStages - 1;
 static constexpr int kAGroups = kTM / 8;                // 8-row groups (one direct-to-LDS instruction each)
 static constexpr int kGroupsPerWave = kAGroups / 8;     // groups one consumer wave moves per step (4 / 2)
-static constexpr int kBTile = kTN * kLdsStride;         // bf16 elements per W buffer
-static constexpr int kTileLdsBytes = kAStages * kAStageBytes + 2 * kBTile * 2;
-// grad-input W tile of the wide shape: [contraction row][output column], rows padded by 32 elements
+// W buffer: forward [output column][64 + 8]; grad-input [contraction row][columns + 32], as the rows are
+// decoded (the consumers transpose on the way out of LDS).  Sized for the larger of the two.
 static constexpr int kNnPitch = kTN + 32;
+static constexpr int kBTile = kTN * kLdsStride > kBK * kNnPitch ? kTN * kLdsStride : kBK * kNnPitch;  // bf16 elements
+static constexpr int kTileLdsBytes = kAStages * kAStageBytes + 2 * kBTile * 2;
 
 // ---- A tile, fast path: each of the eight waves of the consumer octet moves the 8-row groups
 // g = 8*j + cw (j = 0..3) with one direct-to-LDS instruction per group.
@@ -229,12 +231,10 @@ static __device__ __forceinline__ void w_store_run(const TileCtx& c, const Produ
 #pragma unroll
         for (int i = 0; i < 4; i++) *(uint4*)(dst + 8 * i) = make_uint4(wv[4 * i], wv[4 * i + 1], wv[4 * i + 2], wv[4 * i + 3]);
     } else {
-        // transpose: element e of this lane's row n is output column 32*pw + e, contraction index lane
+        // grad-input: this lane's contraction row, columns 32*pw .. +31, stored as decoded
+        bf16_t* dst = &bt[l.lane * kNnPitch + l.pw * 32];
 #pragma unroll
-        for (int e2 = 0; e2 < 16; e2++) {
-            bt[(l.pw * 32 + 2 * e2) * kLdsStride + l.lane] = (bf16_t)(wv[e2] & 0xFFFFu);
-            bt[(l.pw * 32 + 2 * e2 + 1) * kLdsStride + l.lane] = (bf16_t)(wv[e2] >> 16);
-        }
+        for (int i = 0; i < 4; i++) *(uint4*)(dst + 8 * i) = make_uint4(wv[4 * i], wv[4 * i + 1], wv[4 * i + 2], wv[4 * i + 3]);
     }
 }
 
@@ -429,7 +429,7 @@ static __device__ __forceinline__ void q4k_quarter_decode(const u32x4_t& hdr, co
 }
 
 // Grad-input: lane (contraction row n = kc0 + lane, run = col0/32 + wave of the quartet, half = quartet)
-// decodes 16 consecutive output columns of its row and stores them transposed.
+// decodes 16 consecutive output columns of its row.
 struct Q4KHalfRun {
     u32x4_t hdr, q;
 };
@@ -583,7 +583,7 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
             r.hdr = *(const u32x4_t*)blk;
             r.q = *(const u32x4_t*)(blk + q_off);
         };
-        bf16_t* const dst0 = c.bs + (run_w * 32 + half * 16) * kLdsStride + lane;
+        bf16_t* const dst0 = c.bs + lane * kNnPitch + run_w * 32 + half * 16;
         auto fill = [&](Q4KHalfRun& r, int u) __attribute__((always_inline)) {
             open_phase(u);
             q4k_half_run_pin(r);
@@ -591,11 +591,8 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
             q4k_half_run_decode(r, j, wv);
             if (u + 2 < steps) issue(r, u + 2);
             bf16_t* dst = dst0 + buf * kBTile;
-#pragma unroll
-            for (int e2 = 0; e2 < 8; e2++) {
-                dst[(2 * e2) * kLdsStride] = (bf16_t)(wv[e2] & 0xFFFFu);
-                dst[(2 * e2 + 1) * kLdsStride] = (bf16_t)(wv[e2] >> 16);
-            }
+            *(uint4*)dst = make_uint4(wv[0], wv[1], wv[2], wv[3]);
+            *(uint4*)(dst + 8) = make_uint4(wv[4], wv[5], wv[6], wv[7]);
             close_phase();
         };
         Q4KHalfRun ra, rb;  // even / odd steps, each reloaded two steps ahead
@@ -641,7 +638,7 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
     // `lora`: the LoRA tiles ahead of the main steps always use the [column][contraction] W layout
     auto load_operands = [&](Operands& o, int stage, int buf, int kk, bool lora = false) __attribute__((always_inline)) {
         const uint8_t* a_lds = a_row + stage * kAStageBytes + a_koff[kk];
-        if (MODE == kModeNN && SH == 1 && !lora) {
+        if (MODE == kModeNN && !lora) {
             // W tile is [contraction row][output column]: each transposing 8-byte read hands this lane
             // four consecutive contraction values of its column, two reads make the MFMA operand
             const bf16_t* t_lds = c.bs + buf * kBTile + tr_off + kk * 16 * kNnPitch;
