@@ -77,4 +77,38 @@ GGQ_HD uint32_t ld_u16(const uint8_t* p) {
     return v;
 }
 
+#if defined(__HIP_DEVICE_COMPILE__) || defined(__HIPCC__)
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every outstanding
+// global load (s_waitcnt vmcnt(0)), which would serialise the prefetches behind each step.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// Wait until at most n of this wave's global loads are outstanding (loads return in issue order).
+__device__ __forceinline__ void wait_loads_at_most(int n) {
+    switch (n) {
+        case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+        case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
+        case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+        case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
+        case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+        case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+        case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+        case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
+        default: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+    }
+}
+
+// 16-byte slot that holds contraction chunk kc (0..7) of A-tile row r.  Sixteen consecutive rows at one
+// kc cover all sixteen 16-byte bank groups exactly once.
+__device__ __forceinline__ int a_slot(int r, int kc) { return kc ^ ((r >> 1) & 7); }
+
+// One direct global -> LDS load: every lane moves the 16 bytes at sbase + voff to LDS address
+// lds + 16 * lane (lds is wave-uniform).  The data never passes through registers; the instruction
+// counts as one outstanding vector-memory load of the wave.
+__device__ __forceinline__ void load16_to_lds(uint32_t lds, uint32_t voff, const void* sbase) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(voff), "s"(sbase) : "memory", "m0");
+}
+#endif
+
 }  // namespace ggq

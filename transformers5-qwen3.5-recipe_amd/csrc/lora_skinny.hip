@@ -21,23 +21,34 @@ __device__ __forceinline__ uint4 load8g(const bf16_t* p, int valid, bool vec) {
     return v;
 }
 
-// ---- out[m, 0..r_pad) = In[m, :] . F[e][0..r, :]^T ; one wave per 16 rows, 64-row tiles per workgroup.
+// ---- out[m, 0..r_pad) = In[m, :] . F[e][0..r, :]^T.  One workgroup per 16 rows; its four waves deal the
+// contraction out in 128-wide trips (trip t to wave t % 4), so a 64-row tile keeps sixteen waves of loads
+// in flight, and add their partial sums through LDS in wave order (fixed order: deterministic).
 // In may be two column segments (pair): contraction runs over seg 0 then seg 1, F rows are [r][nseg*C].
 template <int JB>  // JB = r_pad / 16
 __global__ __launch_bounds__(256) void skinny_nt_kernel(SkinnyNtParams p) {
+    __shared__ float red[3][JB][4][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // Workgroup ids go round-robin over the eight XCDs; give every XCD a contiguous run of units, so the
+    // workgroups that share one expert's factor rows share an L2 as well.
+    const int units = 4 * (p.tiles ? *p.num_tiles : (int)(gridDim.x >> 2));
+    const int per_xcd = (units + 7) >> 3;
+    const int slot = blockIdx.x >> 3;
+    if (slot >= per_xcd) return;
+    const int unit = (blockIdx.x & 7) * per_xcd + slot;
+    if (unit >= units) return;
+    const int tile = unit >> 2, sub = unit & 3;
     int group = 0, row_begin, row_end;
     if (p.tiles) {
-        if ((int)blockIdx.x >= *p.num_tiles) return;
-        const TileDesc t = p.tiles[blockIdx.x];
+        const TileDesc t = p.tiles[tile];
         group = t.group, row_begin = t.row_begin, row_end = t.row_end;
     } else {
-        row_begin = blockIdx.x * 64;
+        row_begin = tile * 64;
         row_end = min(p.m, row_begin + 64);
     }
     const int64_t expert = p.expert_ids ? p.expert_ids[group] : 0;
-    const int m0 = row_begin + wave * 16;
-    if (m0 >= row_end) return;
+    const int m0 = row_begin + sub * 16;
+    if (m0 >= row_end) return;  // uniform over the workgroup
     const int li = lane & 15, lq = lane >> 4;
     const int row = m0 + li;
     const bool row_ok = row < row_end;
@@ -45,34 +56,37 @@ __global__ __launch_bounds__(256) void skinny_nt_kernel(SkinnyNtParams p) {
     f32x4_t acc[JB];
 #pragma unroll
     for (int jb = 0; jb < JB; jb++) acc[jb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-    for (int seg = 0; seg < p.nseg; seg++) {
+    const bool fvec = ((p.ldf & 7) == 0) && ((p.c & 7) == 0) && (((uintptr_t)p.f & 15) == 0);
+    bool vec = (p.ld_in & 7) == 0;
+    for (int seg = 0; seg < p.nseg; seg++) vec = vec && (((uintptr_t)p.in[seg] & 15) == 0);
+    // aligned operands: 128-wide trips, every load of a trip issued ahead of its MFMAs
+    const int trips_per_seg = (vec && fvec) ? p.c / 128 : 0;
+    for (int t = wave; t < trips_per_seg * p.nseg; t += 4) {
+        const int seg = t / trips_per_seg, c0 = (t - seg * trips_per_seg) * 128;
         const bf16_t* in = p.in[seg] + (int64_t)row * p.ld_in;
-        const bool vec = ((p.ld_in & 7) == 0) && (((uintptr_t)p.in[seg] & 15) == 0);
-        const bool fvec = ((p.ldf & 7) == 0) && ((p.c & 7) == 0) && (((uintptr_t)p.f & 15) == 0);
-        int c0 = 0;
-        if (vec && fvec) {
-            // aligned operands: four sub-steps per trip with every load issued ahead of the MFMAs (the
-            // stream is latency-bound otherwise: one wave owns 16 rows)
-            for (; c0 + 128 <= p.c; c0 += 128) {
-                uint4 av[4], bv[JB][4];
+        uint4 av[4], bv[JB][4];
 #pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    const int cc = c0 + 32 * u + lq * 8;
-                    av[u] = row_ok ? *(const uint4*)(in + cc) : make_uint4(0, 0, 0, 0);
+        for (int u = 0; u < 4; u++) {
+            const int cc = c0 + 32 * u + lq * 8;
+            av[u] = row_ok ? *(const uint4*)(in + cc) : make_uint4(0, 0, 0, 0);
 #pragma unroll
-                    for (int jb = 0; jb < JB; jb++) {
-                        const int j = jb * 16 + li;
-                        bv[jb][u] = j < p.r ? *(const uint4*)(f + (int64_t)j * p.ldf + seg * p.c + cc) : make_uint4(0, 0, 0, 0);
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < 4; u++)
-#pragma unroll
-                    for (int jb = 0; jb < JB; jb++)
-                        acc[jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[u]), __builtin_bit_cast(bf16x8_t, bv[jb][u]), acc[jb], 0, 0, 0);
+            for (int jb = 0; jb < JB; jb++) {
+                const int j = jb * 16 + li;
+                bv[jb][u] = j < p.r ? *(const uint4*)(f + (int64_t)j * p.ldf + seg * p.c + cc) : make_uint4(0, 0, 0, 0);
             }
         }
-        for (; c0 < p.c; c0 += 32) {
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int jb = 0; jb < JB; jb++)
+                acc[jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av[u]), __builtin_bit_cast(bf16x8_t, bv[jb][u]), acc[jb], 0, 0, 0);
+    }
+    // what the trips leave (and everything, for unaligned operands): 32-wide steps dealt the same way
+    int step = 0;
+    for (int seg = 0; seg < p.nseg; seg++) {
+        const bf16_t* in = p.in[seg] + (int64_t)row * p.ld_in;
+        for (int c0 = trips_per_seg * 128; c0 < p.c; c0 += 32, step++) {
+            if ((step & 3) != wave) continue;
             const int cc = c0 + lq * 8;
             const uint4 av = load8g(in + cc, row_ok ? p.c - cc : 0, vec);
             const bf16x8_t a = __builtin_bit_cast(bf16x8_t, av);
@@ -84,27 +98,168 @@ __global__ __launch_bounds__(256) void skinny_nt_kernel(SkinnyNtParams p) {
             }
         }
     }
+    if (wave > 0) {
+#pragma unroll
+        for (int jb = 0; jb < JB; jb++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) red[wave - 1][jb][v][lane] = acc[jb][v];
+    }
+    __syncthreads();
+    if (wave > 0) return;
     // acc[jb][v]: row = m0 + 4*lq + v, col = 16*jb + li
 #pragma unroll
     for (int jb = 0; jb < JB; jb++)
 #pragma unroll
         for (int v = 0; v < 4; v++) {
+            const float sum = ((acc[jb][v] + red[0][jb][v][lane]) + red[1][jb][v][lane]) + red[2][jb][v][lane];
             const int r = m0 + 4 * lq + v;
-            if (r < row_end) p.out[(int64_t)r * (JB * 16) + jb * 16 + li] = to_bf16(acc[jb][v]);
+            if (r < row_end) p.out[(int64_t)r * (JB * 16) + jb * 16 + li] = to_bf16(sum);
         }
+}
+
+// ---- The same product for aligned operands with a contraction that is a multiple of 64: every byte
+// goes global -> LDS directly in whole 128-byte row pieces (a lane-per-row register load of the MFMA
+// operand layout costs the vector cache one access per lane; these loads cost one per 64 bytes), and the
+// operands are read back from LDS.  One workgroup per 64-row tile; wave w owns rows 32*(w&1)..+31 and
+// every second 64-wide contraction step (parity w>>1), with a two-stage ring of its own: no workgroup
+// barrier inside the loop.  Rows keep their 16-byte chunks XOR-swizzled (a_slot) so both the 1 KB writes
+// and the operand reads are bank-conflict free.
+template <int JB>
+__global__ __launch_bounds__(256) void skinny_nt_direct_kernel(SkinnyNtParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t sk_lds[];
+    constexpr int kInBytes = 32 * 128, kFBytes = JB * 16 * 128, kStage = kInBytes + kFBytes;
+    constexpr int kLoads = 4 + 2 * JB;  // direct-to-LDS instructions per stage
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int units = p.tiles ? *p.num_tiles : (p.m + 63) / 64;
+    const int per_xcd = (units + 7) >> 3;
+    const int slot = blockIdx.x >> 3;
+    if (slot >= per_xcd) return;
+    const int unit = (blockIdx.x & 7) * per_xcd + slot;
+    if (unit >= units) return;
+    int group = 0, row_begin, row_end;
+    if (p.tiles) {
+        const TileDesc t = p.tiles[unit];
+        group = t.group, row_begin = t.row_begin, row_end = t.row_end;
+    } else {
+        row_begin = unit * 64;
+        row_end = min(p.m, row_begin + 64);
+    }
+    const int64_t expert = p.expert_ids ? p.expert_ids[group] : 0;
+    const int half = wave & 1, parity = wave >> 1;
+    const int r0 = row_begin + 32 * half;
+    const int rows_valid = row_end - r0;  // <= 0: this wave only joins the final barrier
+    const bf16_t* f = p.f + expert * p.f_expert_elems;  // [r][ldf]
+    uint8_t* my = sk_lds + wave * 2 * kStage;
+    const uint32_t my_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)my;
+    // lane's 16 bytes in each 8-row load: row lane/8 of the load, the chunk that belongs in slot lane%8
+    uint32_t in_off[4], f_off[2 * JB];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int rl = 8 * q + (lane >> 3);
+        const int row = min(rl, rows_valid - 1);  // rows past the tile are copies of its last row, never stored
+        in_off[q] = ((uint32_t)row * (uint32_t)p.ld_in + (uint32_t)(a_slot(rl, lane & 7) * 8)) * 2u;
+    }
+#pragma unroll
+    for (int q = 0; q < 2 * JB; q++) {
+        const int jl = 8 * q + (lane >> 3);
+        const int j = min(jl, p.r - 1);  // factor rows past the rank are masked when the operand is read
+        f_off[q] = ((uint32_t)j * (uint32_t)p.ldf + (uint32_t)(a_slot(jl, lane & 7) * 8)) * 2u;
+    }
+    const int steps_per_seg = p.c / 64, steps = steps_per_seg * p.nseg;
+    auto issue = [&](int step, int stage) {
+        const int seg = step / steps_per_seg, c0 = (step - seg * steps_per_seg) * 64;
+        const bf16_t* in_base = p.in[seg] + (int64_t)r0 * p.ld_in + c0;
+        const bf16_t* f_base = f + seg * p.c + c0;
+        const uint32_t lds = my_lds + stage * kStage;
+#pragma unroll
+        for (int q = 0; q < 4; q++) load16_to_lds(lds + q * 1024, in_off[q], in_base);
+#pragma unroll
+        for (int q = 0; q < 2 * JB; q++) load16_to_lds(lds + kInBytes + q * 1024, f_off[q], f_base);
+    };
+    const int li = lane & 15, lq = lane >> 4;
+    f32x4_t acc[2][JB];
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+        for (int jb = 0; jb < JB; jb++) acc[rb][jb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    if (rows_valid > 0) {
+        if (parity < steps) issue(parity, 0);
+        int stage = 0;
+        for (int step = parity; step < steps; step += 2, stage ^= 1) {
+            if (step + 2 < steps) {
+                issue(step + 2, stage ^ 1);
+                wait_loads_at_most(kLoads);
+            } else {
+                wait_loads_at_most(0);
+            }
+            const uint8_t* st = my + stage * kStage;
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++) {
+                uint4 b[JB];
+#pragma unroll
+                for (int jb = 0; jb < JB; jb++) {
+                    const int j = jb * 16 + li;
+                    b[jb] = *(const uint4*)(st + kInBytes + j * 128 + a_slot(j, kk * 4 + lq) * 16);
+                    if (j >= p.r) b[jb] = make_uint4(0, 0, 0, 0);
+                }
+#pragma unroll
+                for (int rb = 0; rb < 2; rb++) {
+                    const int rl = rb * 16 + li;
+                    const uint4 a = *(const uint4*)(st + rl * 128 + a_slot(rl, kk * 4 + lq) * 16);
+#pragma unroll
+                    for (int jb = 0; jb < JB; jb++)
+                        acc[rb][jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b[jb]), acc[rb][jb], 0, 0, 0);
+                }
+            }
+            // the next trip's loads overwrite the other stage only; this stage is rewritten one trip later,
+            // after these reads have returned (the MFMAs above waited for them)
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        }
+    }
+    // the odd-parity waves hand their sums to the even ones through the (now idle) ring
+    __syncthreads();
+    float* red = (float*)(sk_lds + (wave & 1) * 2 * kStage);  // the ring of wave (w&1): its loads are done
+    if (parity == 1) {
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+            for (int jb = 0; jb < JB; jb++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) red[((rb * JB + jb) * 4 + v) * 64 + lane] = acc[rb][jb][v];
+    }
+    __syncthreads();
+    if (parity == 1) return;
+    // acc[rb][jb][v]: row = r0 + 16*rb + 4*lq + v, col = 16*jb + li
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+        for (int jb = 0; jb < JB; jb++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const float sum = acc[rb][jb][v] + red[((rb * JB + jb) * 4 + v) * 64 + lane];
+                const int r = r0 + 16 * rb + 4 * lq + v;
+                if (r < row_end) p.out[(int64_t)r * (JB * 16) + jb * 16 + li] = to_bf16(sum);
+            }
 }
 
 // ---- G[e][c, j] = s * sum_m In[m, c] * S[m, j] over the rows of expert e.  One workgroup per
 // (expert, 64 columns); each wave owns 16 columns; rows are consumed 32 at a time through LDS so the
-// strided operands of the contraction over m become LDS gathers.  Experts without rows get zeros.
+// strided operands of the contraction over m become LDS gathers.  The loads of four 32-row slices are
+// issued together and the slices then go through two alternating LDS buffers, one barrier each.
+// Experts without rows get zeros.
 template <int JB>
 __global__ __launch_bounds__(256) void factor_grad_kernel(FactorGradParams p) {
-    __shared__ bf16_t in_t[32][64 + 2];
-    __shared__ bf16_t s_t[32][JB * 16 + 2];
+    __shared__ bf16_t in_t[2][32][64 + 2];
+    __shared__ bf16_t s_t[2][32][JB * 16 + 2];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int blocks_per_seg = (p.c + 63) / 64;
     const int col_blocks = p.nseg * blocks_per_seg;
-    const int e = blockIdx.x / col_blocks, cblk = blockIdx.x - e * col_blocks;
+    // contiguous runs of (expert, column block) units per XCD: one L2 sees whole rows of an expert
+    const int per_xcd = ((int)gridDim.x + 7) >> 3;
+    const int unit = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= per_xcd || unit >= p.units) return;
+    const int e = unit / col_blocks, cblk = unit - e * col_blocks;
     const int seg = cblk / blocks_per_seg;
     const int c0 = (cblk - seg * blocks_per_seg) * 64;
     int row_begin = 0, row_end = p.m;
@@ -118,52 +273,95 @@ __global__ __launch_bounds__(256) void factor_grad_kernel(FactorGradParams p) {
     f32x4_t acc[JB];
 #pragma unroll
     for (int jb = 0; jb < JB; jb++) acc[jb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-    const int rp = JB * 16;
-    for (int m0 = row_begin; m0 < row_end; m0 += 32) {
-        {   // In tile: 32 rows x 64 cols = 256 chunks of 8
-            const int r = threadIdx.x >> 3, ch = threadIdx.x & 7;
-            const int cc = c0 + ch * 8;
-            const uint4 v = load8g(in + (int64_t)(m0 + r) * p.ld_in + cc, m0 + r < row_end ? p.c - cc : 0, vec);
-            uint32_t* d = (uint32_t*)&in_t[r][ch * 8];
-            d[0] = v.x, d[1] = v.y, d[2] = v.z, d[3] = v.w;
-        }
-        for (int id = threadIdx.x; id < 32 * (rp / 8); id += 256) {
-            const int r = id / (rp / 8), ch = id - r * (rp / 8);
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (m0 + r < row_end) v = *(const uint4*)(p.s + (int64_t)(m0 + r) * rp + ch * 8);
-            uint32_t* d = (uint32_t*)&s_t[r][ch * 8];
-            d[0] = v.x, d[1] = v.y, d[2] = v.z, d[3] = v.w;
-        }
-        __syncthreads();
-        // A operand: row = column c (wave*16 + li), contraction m = 8*lq .. 8*lq+7
-        uint32_t aw[4];
+    constexpr int rp = JB * 16;
+    const int tr = threadIdx.x >> 3, tch = threadIdx.x & 7;           // In slice: 32 rows x 8 chunks of 8
+    const int sr = threadIdx.x / (rp / 8), sch = threadIdx.x % (rp / 8);  // S slice: 32 rows x rp/8 chunks
+    const int tcc = c0 + tch * 8;
+    int buf = 0;
+    for (int m0 = row_begin; m0 < row_end; m0 += 128) {
+        uint4 vin[4], vs[4];
 #pragma unroll
-        for (int h = 0; h < 4; h++)
-            aw[h] = (uint32_t)in_t[8 * lq + 2 * h][wave * 16 + li] | ((uint32_t)in_t[8 * lq + 2 * h + 1][wave * 16 + li] << 16);
-        const bf16x8_t a = __builtin_bit_cast(bf16x8_t, make_uint4(aw[0], aw[1], aw[2], aw[3]));
+        for (int u = 0; u < 4; u++) {
+            const int r = m0 + 32 * u + tr;
+            vin[u] = load8g(in + (int64_t)r * p.ld_in + tcc, r < row_end ? p.c - tcc : 0, vec);
+            vs[u] = make_uint4(0, 0, 0, 0);
+            if (sr < 32 && m0 + 32 * u + sr < row_end) vs[u] = *(const uint4*)(p.s + (int64_t)(m0 + 32 * u + sr) * rp + sch * 8);
+        }
 #pragma unroll
-        for (int jb = 0; jb < JB; jb++) {
-            uint32_t bw[4];
+        for (int u = 0; u < 4; u++) {
+            if (m0 + 32 * u >= row_end) break;  // uniform over the workgroup
+            uint32_t* d = (uint32_t*)&in_t[buf][tr][tch * 8];
+            d[0] = vin[u].x, d[1] = vin[u].y, d[2] = vin[u].z, d[3] = vin[u].w;
+            if (sr < 32) {
+                uint32_t* ds = (uint32_t*)&s_t[buf][sr][sch * 8];
+                ds[0] = vs[u].x, ds[1] = vs[u].y, ds[2] = vs[u].z, ds[3] = vs[u].w;
+            }
+            // one barrier per slice: the slice after the next reuses this buffer, and every wave passes the
+            // next barrier only after its reads of this one
+            __syncthreads();
+            // A operand: row = column c (wave*16 + li), contraction m = 8*lq .. 8*lq+7
+            uint32_t aw[4];
 #pragma unroll
             for (int h = 0; h < 4; h++)
-                bw[h] = (uint32_t)s_t[8 * lq + 2 * h][jb * 16 + li] | ((uint32_t)s_t[8 * lq + 2 * h + 1][jb * 16 + li] << 16);
-            acc[jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8_t, make_uint4(bw[0], bw[1], bw[2], bw[3])), acc[jb], 0, 0, 0);
+                aw[h] = (uint32_t)in_t[buf][8 * lq + 2 * h][wave * 16 + li] | ((uint32_t)in_t[buf][8 * lq + 2 * h + 1][wave * 16 + li] << 16);
+            const bf16x8_t a = __builtin_bit_cast(bf16x8_t, make_uint4(aw[0], aw[1], aw[2], aw[3]));
+#pragma unroll
+            for (int jb = 0; jb < JB; jb++) {
+                uint32_t bw[4];
+#pragma unroll
+                for (int h = 0; h < 4; h++)
+                    bw[h] = (uint32_t)s_t[buf][8 * lq + 2 * h][jb * 16 + li] | ((uint32_t)s_t[buf][8 * lq + 2 * h + 1][jb * 16 + li] << 16);
+                acc[jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8_t, make_uint4(bw[0], bw[1], bw[2], bw[3])), acc[jb], 0, 0, 0);
+            }
+            buf ^= 1;
         }
-        __syncthreads();
     }
     // acc[jb][v]: c = c0 + wave*16 + 4*lq + v, j = 16*jb + li
     bf16_t* out = p.out + (int64_t)e * p.out_expert_elems;
+    const int64_t ctot = (int64_t)p.nseg * p.c;
+    const int cw0 = c0 + wave * 16;  // first column of this wave
+    if (p.out_j_major) {
+        // [r][columns]: a lane holds four consecutive columns of factor row j: one 8-byte store
+        const bool vec4 = (ctot & 3) == 0 && (((uintptr_t)out & 7) == 0);
+#pragma unroll
+        for (int jb = 0; jb < JB; jb++) {
+            const int j = jb * 16 + li, c = cw0 + 4 * lq;
+            if (j >= p.r) continue;
+            bf16_t* dst = out + (int64_t)j * ctot + (int64_t)seg * p.c + c;
+            if (vec4 && c + 3 < p.c) {
+                *(uint2*)dst = make_uint2(pack_bf16(acc[jb][0] * p.scale, acc[jb][1] * p.scale), pack_bf16(acc[jb][2] * p.scale, acc[jb][3] * p.scale));
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; v++)
+                    if (c + v < p.c) dst[v] = to_bf16(acc[jb][v] * p.scale);
+            }
+        }
+        return;
+    }
+    // [columns][r]: the wave's 16 columns x r are one contiguous run; transpose through LDS (each wave
+    // reads back only what it wrote) and store 16 bytes per lane
+    __shared__ __attribute__((aligned(16))) bf16_t g_t[4][16][JB * 16];
+    const bool vec8 = (p.r & 7) == 0 && (((uintptr_t)out & 15) == 0);
+    if (vec8) {
+#pragma unroll
+        for (int jb = 0; jb < JB; jb++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) g_t[wave][4 * lq + v][jb * 16 + li] = to_bf16(acc[jb][v] * p.scale);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        const int chunks_per_row = p.r >> 3;
+        bf16_t* dst = out + ((int64_t)seg * p.c + cw0) * p.r;
+        for (int id = lane; id < 16 * chunks_per_row; id += 64) {
+            const int row = id / chunks_per_row, ch = id - row * chunks_per_row;
+            if (cw0 + row < p.c) *(uint4*)(dst + (int64_t)id * 8) = *(const uint4*)&g_t[wave][row][ch * 8];
+        }
+        return;
+    }
 #pragma unroll
     for (int jb = 0; jb < JB; jb++)
 #pragma unroll
         for (int v = 0; v < 4; v++) {
-            const int c = c0 + wave * 16 + 4 * lq + v, j = jb * 16 + li;
-            if (c < p.c && j < p.r) {
-                const bf16_t val = to_bf16(acc[jb][v] * p.scale);
-                const int64_t cg = (int64_t)seg * p.c + c;
-                if (p.out_j_major) out[(int64_t)j * (p.nseg * p.c) + cg] = val;
-                else out[cg * p.r + j] = val;
-            }
+            const int c = cw0 + 4 * lq + v, j = jb * 16 + li;
+            if (c < p.c && j < p.r) out[((int64_t)seg * p.c + c) * p.r + j] = to_bf16(acc[jb][v] * p.scale);
         }
 }
 
@@ -232,23 +430,51 @@ int transpose_factor(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int
     return check_launch("transpose_factor");
 }
 
+template <int JB>
+static int launch_skinny_direct(const SkinnyNtParams& p, int grid_tiles, hipStream_t s) {
+    constexpr int kSmem = 4 * 2 * (32 * 128 + JB * 16 * 128);
+    static bool attr_set = false;
+    if (!attr_set) {
+        if (hipFuncSetAttribute((const void*)skinny_nt_direct_kernel<JB>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmem) != hipSuccess)
+            return set_error(GGQ_ERR_RUNTIME, "skinny_nt: could not raise the dynamic LDS limit to %d bytes", kSmem);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(skinny_nt_direct_kernel<JB>, dim3(((unsigned)grid_tiles + 7u) & ~7u), dim3(256), kSmem, s, p);
+    return check_launch("skinny_nt_direct");
+}
+
 int skinny_nt(const SkinnyNtParams& p, int r_pad, int grid_tiles, hipStream_t s) {
     if (grid_tiles <= 0) return 0;
+    bool direct = (p.ld_in & 7) == 0 && (p.ldf & 7) == 0 && (p.c & 63) == 0 && ((uintptr_t)p.f & 15) == 0 && (p.f_expert_elems & 7) == 0 &&
+                  (uint64_t)64 * (uint64_t)p.ld_in * 2 < (1ull << 31) && (uint64_t)64 * (uint64_t)p.ldf * 2 < (1ull << 31);
+    for (int seg = 0; seg < p.nseg; seg++) direct = direct && ((uintptr_t)p.in[seg] & 15) == 0;
+    if (direct) {
+        switch (r_pad / 16) {
+            case 1: return launch_skinny_direct<1>(p, grid_tiles, s);
+            case 2: return launch_skinny_direct<2>(p, grid_tiles, s);
+            case 3: return launch_skinny_direct<3>(p, grid_tiles, s);
+            case 4: return launch_skinny_direct<4>(p, grid_tiles, s);
+            default: return set_error(GGQ_ERR_SHAPE, "LoRA rank must be between 1 and 64");
+        }
+    }
     switch (r_pad / 16) {
-        case 1: hipLaunchKernelGGL(skinny_nt_kernel<1>, dim3(grid_tiles), dim3(256), 0, s, p); break;
-        case 2: hipLaunchKernelGGL(skinny_nt_kernel<2>, dim3(grid_tiles), dim3(256), 0, s, p); break;
-        case 3: hipLaunchKernelGGL(skinny_nt_kernel<3>, dim3(grid_tiles), dim3(256), 0, s, p); break;
-        case 4: hipLaunchKernelGGL(skinny_nt_kernel<4>, dim3(grid_tiles), dim3(256), 0, s, p); break;
+        case 1: hipLaunchKernelGGL(skinny_nt_kernel<1>, dim3((4u * (unsigned)grid_tiles + 7u) & ~7u), dim3(256), 0, s, p); break;
+        case 2: hipLaunchKernelGGL(skinny_nt_kernel<2>, dim3((4u * (unsigned)grid_tiles + 7u) & ~7u), dim3(256), 0, s, p); break;
+        case 3: hipLaunchKernelGGL(skinny_nt_kernel<3>, dim3((4u * (unsigned)grid_tiles + 7u) & ~7u), dim3(256), 0, s, p); break;
+        case 4: hipLaunchKernelGGL(skinny_nt_kernel<4>, dim3((4u * (unsigned)grid_tiles + 7u) & ~7u), dim3(256), 0, s, p); break;
         default: return set_error(GGQ_ERR_SHAPE, "LoRA rank must be between 1 and 64");
     }
     return check_launch("skinny_nt");
 }
 
-int factor_grad(const FactorGradParams& p, int r_pad, int64_t experts, hipStream_t s) {
-    const int col_blocks = p.nseg * ((p.c + 63) / 64);
-    const int64_t grid = experts * col_blocks;
-    if (grid <= 0) return 0;
-    if (grid > 0x7FFFFFFF) return set_error(GGQ_ERR_SHAPE, "factor_grad: grid too large");
+int factor_grad(const FactorGradParams& p_in, int r_pad, int64_t experts, hipStream_t s) {
+    const int col_blocks = p_in.nseg * ((p_in.c + 63) / 64);
+    const int64_t units = experts * col_blocks;
+    if (units <= 0) return 0;
+    if (units > 0x7FFFFFF0) return set_error(GGQ_ERR_SHAPE, "factor_grad: grid too large");
+    const int64_t grid = (units + 7) / 8 * 8;
+    FactorGradParams p = p_in;
+    p.units = (int)units;
     switch (r_pad / 16) {
         case 1: hipLaunchKernelGGL(factor_grad_kernel<1>, dim3((unsigned)grid), dim3(256), 0, s, p); break;
         case 2: hipLaunchKernelGGL(factor_grad_kernel<2>, dim3((unsigned)grid), dim3(256), 0, s, p); break;

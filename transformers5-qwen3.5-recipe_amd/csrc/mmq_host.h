@@ -32,6 +32,7 @@ struct FactorGradParams {
     const int* ranges;    // per expert (row_begin, row_end); null: all m rows, one expert
     int m, c, r, nseg, out_j_major;
     float scale;
+    int units;            // experts * column blocks (set by factor_grad)
 };
 
 constexpr int kBM = 256, kBN = 128, kBK = 64;  // the tall tile shape (dense launches, large expert groups)

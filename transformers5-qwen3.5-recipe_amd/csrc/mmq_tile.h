@@ -48,31 +48,6 @@ typedef __attribute__((address_space(3))) v4i16_t* lds_v4i16_ptr;  // native vec
 
 __device__ __forceinline__ uint4 zero4() { return make_uint4(0, 0, 0, 0); }
 
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every outstanding
-// global load (s_waitcnt vmcnt(0)), which would serialise the prefetches behind each step.
-__device__ __forceinline__ void lds_barrier() {
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
-// Wait until at most n of this wave's global loads are outstanding (loads return in issue order).
-__device__ __forceinline__ void wait_loads_at_most(int n) {
-    switch (n) {
-        case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-        case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
-        case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
-        case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
-        case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
-        case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
-        case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
-        case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
-        default: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
-    }
-}
-
-// 16-byte slot that holds contraction chunk kc (0..7) of A-tile row r.  Sixteen consecutive rows at one
-// kc cover all sixteen 16-byte bank groups exactly once.
-__device__ __forceinline__ int a_slot(int r, int kc) { return kc ^ ((r >> 1) & 7); }
-
 // 8 consecutive bf16 from a row, zero-filled past `valid` elements (element-wise path for rows that
 // are not 16-byte aligned or that end inside the run).
 __device__ __forceinline__ uint4 load8_slow(const bf16_t* p, int valid) {
