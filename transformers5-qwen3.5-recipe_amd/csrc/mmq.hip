@@ -44,8 +44,9 @@ __global__ __launch_bounds__(256) void build_row_tiles_kernel(const int64_t* exp
     __syncthreads();
     for (int g0 = 0; g0 < groups; g0 += 256) {
         const int g = g0 + tid;
-        int r0 = 0, r1 = 0, count = 0;
+        int r0 = 0, r1 = 0, count = 0, expert = 0;
         if (g < groups) {
+            expert = expert_ids ? (int)expert_ids[g] : g;
             r0 = g == 0 ? 0 : end_offsets[g - 1];
             r1 = end_offsets[g];
             count = (r1 - r0 > min_rows && r1 - r0 <= max_rows) ? (r1 - r0 + bm - 1) / bm : 0;
@@ -65,7 +66,7 @@ __global__ __launch_bounds__(256) void build_row_tiles_kernel(const int64_t* exp
         const int first = base + scan[tid] - count;
         for (int i = 0; i < count; i++) {
             TileDesc d;
-            d.group = g, d.row_begin = r0 + i * bm, d.row_end = min(r1, r0 + (i + 1) * bm), d.pad = 0;
+            d.group = g, d.row_begin = r0 + i * bm, d.row_end = min(r1, r0 + (i + 1) * bm), d.expert = expert;
             tiles[first + i] = d;
         }
         __syncthreads();

@@ -7,8 +7,8 @@ namespace ggq {
 
 typedef uint16_t bf16_t;
 
-struct TileDesc {  // one row tile of an expert group: rows [row_begin, row_end) of group `group`
-    int group, row_begin, row_end, pad;
+struct TileDesc {  // one row tile of an expert group: rows [row_begin, row_end) of group `group`, whose weights are plane `expert`
+    int group, row_begin, row_end, expert;
 };
 
 struct SkinnyNtParams {

@@ -852,16 +852,16 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps control flow scalar
 
     c.col_tile = col_tile;
-    int group = 0, row_end;
+    int row_end;
     if (tiles) {
         const TileDesc t = tiles[row_tile];
-        group = t.group, c.row_begin = t.row_begin, row_end = t.row_end;
+        c.row_begin = t.row_begin, row_end = t.row_end, c.expert = t.expert;
     } else {
         c.row_begin = row_tile * kTM;
         row_end = min(p.m, c.row_begin + kTM);
+        c.expert = 0;
     }
     c.rows_valid = row_end - c.row_begin;  // 1..kTM
-    c.expert = p.expert_ids ? p.expert_ids[group] : 0;
     // column tile -> (segment, first output column inside the segment)
     c.seg_c = MODE == kModeNT ? c.col_tile / col_tiles_per_seg : 0;
     c.col0 = (c.col_tile - c.seg_c * col_tiles_per_seg) * kTN;

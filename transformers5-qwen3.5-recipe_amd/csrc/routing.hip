@@ -64,11 +64,17 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int* chunk_hist, int ch
         const int e = e0 + tid;
         int total = 0;
         if (e < num_experts) {
-            for (int c = 0; c < chunks; c++) {
-                int* h = &chunk_hist[(int64_t)c * num_experts + e];
-                const int v = *h;
-                *h = total;  // becomes the chunk's base inside the expert
-                total += v;
+            // sixteen chunk counts are loaded together (one dependent load per chunk would cost a memory
+            // round trip each); every count is replaced by the chunk's base inside the expert
+            for (int c0 = 0; c0 < chunks; c0 += 16) {
+                int v[16];
+#pragma unroll
+                for (int i = 0; i < 16; i++) v[i] = c0 + i < chunks ? chunk_hist[(int64_t)(c0 + i) * num_experts + e] : 0;
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    if (c0 + i < chunks) chunk_hist[(int64_t)(c0 + i) * num_experts + e] = total;
+                    total += v[i];
+                }
             }
             counts[e] = total;
         }
