@@ -46,7 +46,7 @@ def test_mmq_and_grad_input(pkg, dev, qt, m, n, k):
 
 
 @pytest.mark.parametrize("qt", ALL_TYPES, ids=[TYPE_NAMES[q] for q in ALL_TYPES])
-@pytest.mark.parametrize("m,n,k,r", [(33, 37, 2048, 4), (3 * 11, 64, 512, 16), (257, 300, 768, 24)])
+@pytest.mark.parametrize("m,n,k,r", [(33, 37, 2048, 4), (3 * 11, 64, 512, 16), (257, 300, 768, 24), (130, 256, 1024, 40), (64, 128, 512, 64)])
 def test_lora_linear_forward_backward(pkg, dev, qt, m, n, k, r):
     gen = torch.Generator().manual_seed(97531 + r)
     payload = make_payload(k + r + qt, qt, n, k)

@@ -239,23 +239,26 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
         tiles64 = t64, num_tiles64 = counts + 1, ranges = rg;
     }
     if (lora_a) {
-        // t = dy . B  (through B^T so both operands are contraction-contiguous)
-        bf16_t* bt = (bf16_t*)bump.take(experts * ntot * r * 2);
+        // t = dy . B
         bf16_t* dyb = (bf16_t*)bump.take(rows * rp * 2);
-        bf16_t* atp = (bf16_t*)bump.take(experts * k * rp * 2);
-        if (!bt || !dyb || !atp) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
-        if (int rc = transpose_factor((const bf16_t*)lora_b, bt, experts, (int)ntot, r, s)) return rc;
-        if (int rc = pad_factor((const bf16_t*)lora_a, atp, experts, (int)k, r, rp, true, s)) return rc;
+        if (!dyb) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
         if (rows > 0) {
             SkinnyNtParams sp{};
             sp.in[0] = (const bf16_t*)dy1, sp.in[1] = (const bf16_t*)dy2, sp.ld_in = n;
-            sp.f = bt, sp.ldf = ntot, sp.f_expert_elems = (int64_t)r * ntot;
+            sp.f = (const bf16_t*)lora_b, sp.ldf = r, sp.f_expert_elems = (int64_t)r * ntot, sp.f_natural = 1;
             sp.out = dyb;
             sp.m = (int)rows, sp.c = (int)n, sp.r = r, sp.nseg = nseg;
             sp.expert_ids = groups > 0 ? expert_ids : nullptr, sp.tiles = tiles64, sp.num_tiles = num_tiles64;
+            if (!skinny_nt_takes_natural_factor(sp)) {
+                // B^T, so that both operands are contraction-contiguous
+                bf16_t* bt = (bf16_t*)bump.take(experts * ntot * r * 2);
+                if (!bt) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
+                if (int rc = transpose_factor((const bf16_t*)lora_b, bt, experts, (int)ntot, r, s)) return rc;
+                sp.f = bt, sp.ldf = ntot, sp.f_natural = 0;
+            }
             if (int rc = skinny_nt(sp, rp, max_tiles64, s)) return rc;
         }
-        p.la = dyb, p.lb = atp, p.lb_expert_elems = k * rp, p.r_pad = rp, p.lora_scale = scale;
+        p.la = dyb, p.lb = (const bf16_t*)lora_a, p.lb_expert_elems = (int64_t)r * k, p.r_pad = rp, p.lora_rank = r, p.lora_scale = scale;
         if (d_lora_b) {
             FactorGradParams fp{};
             fp.in[0] = (const bf16_t*)dy1, fp.in[1] = (const bf16_t*)dy2, fp.ld_in = n;

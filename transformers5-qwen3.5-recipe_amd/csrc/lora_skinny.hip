@@ -124,11 +124,19 @@ __global__ __launch_bounds__(256) void skinny_nt_kernel(SkinnyNtParams p) {
 // every second 64-wide contraction step (parity w>>1), with a two-stage ring of its own: no workgroup
 // barrier inside the loop.  Rows keep their 16-byte chunks XOR-swizzled (a_slot) so both the 1 KB writes
 // and the operand reads are bank-conflict free.
-template <int JB>
+// FNAT: the factor is given as [contraction][r] (r a multiple of 8, the natural layout of B for dY . B): a
+// 64-wide step of it is one contiguous run, copied as it is; the operand reads transpose it on the way out
+// of LDS (ds_read_b64_tr_b16: within 16 lanes, lane L gets element L % 4 of the 8 bytes addressed by lanes
+// L / 4 + 4 t, t = 0..3, so source lane s points at contraction row s / 4, factor columns 4 (s % 4) .. +3).
+typedef short v4i16_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4i16_t* lds_v4i16_ptr;
+
+template <int JB, bool FNAT>
 __global__ __launch_bounds__(256) void skinny_nt_direct_kernel(SkinnyNtParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t sk_lds[];
     constexpr int kInBytes = 32 * 128, kFBytes = JB * 16 * 128, kStage = kInBytes + kFBytes;
-    constexpr int kLoads = 4 + 2 * JB;  // direct-to-LDS instructions per stage
+    const int f_loads = FNAT ? p.r >> 3 : 2 * JB;  // 1 KB direct-to-LDS instructions per stage of the factor
+    const int loads = 4 + f_loads;                 // ... and of the stage
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int units = p.tiles ? *p.num_tiles : (p.m + 63) / 64;
@@ -149,7 +157,7 @@ __global__ __launch_bounds__(256) void skinny_nt_direct_kernel(SkinnyNtParams p)
     const int half = wave & 1, parity = wave >> 1;
     const int r0 = row_begin + 32 * half;
     const int rows_valid = row_end - r0;  // <= 0: this wave only joins the final barrier
-    const bf16_t* f = p.f + expert * p.f_expert_elems;  // [r][ldf]
+    const bf16_t* f = p.f + expert * p.f_expert_elems;  // [r][ldf], or [nseg*C][r] (FNAT)
     uint8_t* my = sk_lds + wave * 2 * kStage;
     const uint32_t my_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)my;
     // lane's 16 bytes in each 8-row load: row lane/8 of the load, the chunk that belongs in slot lane%8
@@ -162,20 +170,25 @@ __global__ __launch_bounds__(256) void skinny_nt_direct_kernel(SkinnyNtParams p)
     }
 #pragma unroll
     for (int q = 0; q < 2 * JB; q++) {
-        const int jl = 8 * q + (lane >> 3);
-        const int j = min(jl, p.r - 1);  // factor rows past the rank are masked when the operand is read
-        f_off[q] = ((uint32_t)j * (uint32_t)p.ldf + (uint32_t)(a_slot(jl, lane & 7) * 8)) * 2u;
+        if (FNAT) {
+            f_off[q] = (uint32_t)(q * 64 + lane) * 16u;  // a straight copy
+        } else {
+            const int jl = 8 * q + (lane >> 3);
+            const int j = min(jl, p.r - 1);  // factor rows past the rank are masked when the operand is read
+            f_off[q] = ((uint32_t)j * (uint32_t)p.ldf + (uint32_t)(a_slot(jl, lane & 7) * 8)) * 2u;
+        }
     }
     const int steps_per_seg = p.c / 64, steps = steps_per_seg * p.nseg;
     auto issue = [&](int step, int stage) {
         const int seg = step / steps_per_seg, c0 = (step - seg * steps_per_seg) * 64;
         const bf16_t* in_base = p.in[seg] + (int64_t)r0 * p.ld_in + c0;
-        const bf16_t* f_base = f + seg * p.c + c0;
+        const bf16_t* f_base = FNAT ? f + ((int64_t)seg * p.c + c0) * p.r : f + seg * p.c + c0;
         const uint32_t lds = my_lds + stage * kStage;
 #pragma unroll
         for (int q = 0; q < 4; q++) load16_to_lds(lds + q * 1024, in_off[q], in_base);
 #pragma unroll
-        for (int q = 0; q < 2 * JB; q++) load16_to_lds(lds + kInBytes + q * 1024, f_off[q], f_base);
+        for (int q = 0; q < 2 * JB; q++)
+            if (q < f_loads) load16_to_lds(lds + kInBytes + q * 1024, f_off[q], f_base);
     };
     const int li = lane & 15, lq = lane >> 4;
     f32x4_t acc[2][JB];
@@ -189,7 +202,7 @@ __global__ __launch_bounds__(256) void skinny_nt_direct_kernel(SkinnyNtParams p)
         for (int step = parity; step < steps; step += 2, stage ^= 1) {
             if (step + 2 < steps) {
                 issue(step + 2, stage ^ 1);
-                wait_loads_at_most(kLoads);
+                wait_loads_at_most(loads);
             } else {
                 wait_loads_at_most(0);
             }
@@ -200,7 +213,14 @@ __global__ __launch_bounds__(256) void skinny_nt_direct_kernel(SkinnyNtParams p)
 #pragma unroll
                 for (int jb = 0; jb < JB; jb++) {
                     const int j = jb * 16 + li;
-                    b[jb] = *(const uint4*)(st + kInBytes + j * 128 + a_slot(j, kk * 4 + lq) * 16);
+                    if (FNAT) {
+                        const uint8_t* src = st + kInBytes + (kk * 32 + 8 * lq + (li >> 2)) * (p.r * 2) + jb * 32 + (li & 3) * 8;
+                        const v4i16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)src);
+                        const v4i16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(src + 4 * (p.r * 2)));
+                        b[jb] = __builtin_bit_cast(uint4, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                    } else {
+                        b[jb] = *(const uint4*)(st + kInBytes + j * 128 + a_slot(j, kk * 4 + lq) * 16);
+                    }
                     if (j >= p.r) b[jb] = make_uint4(0, 0, 0, 0);
                 }
 #pragma unroll
@@ -430,17 +450,26 @@ int transpose_factor(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int
     return check_launch("transpose_factor");
 }
 
-template <int JB>
+template <int JB, bool FNAT>
 static int launch_skinny_direct(const SkinnyNtParams& p, int grid_tiles, hipStream_t s) {
     constexpr int kSmem = 4 * 2 * (32 * 128 + JB * 16 * 128);
     static bool attr_set = false;
     if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)skinny_nt_direct_kernel<JB>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmem) != hipSuccess)
+        if (hipFuncSetAttribute((const void*)skinny_nt_direct_kernel<JB, FNAT>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmem) != hipSuccess)
             return set_error(GGQ_ERR_RUNTIME, "skinny_nt: could not raise the dynamic LDS limit to %d bytes", kSmem);
         attr_set = true;
     }
-    hipLaunchKernelGGL(skinny_nt_direct_kernel<JB>, dim3(((unsigned)grid_tiles + 7u) & ~7u), dim3(256), kSmem, s, p);
+    hipLaunchKernelGGL((skinny_nt_direct_kernel<JB, FNAT>), dim3(((unsigned)grid_tiles + 7u) & ~7u), dim3(256), kSmem, s, p);
     return check_launch("skinny_nt_direct");
+}
+
+// The factor may be handed over as [contraction][r] (f_natural) when this holds; otherwise the caller
+// passes it transposed, [r][contraction].
+bool skinny_nt_takes_natural_factor(const SkinnyNtParams& p) {
+    bool ok = (p.r & 7) == 0 && (p.ld_in & 7) == 0 && (p.c & 63) == 0 && ((uintptr_t)p.f & 15) == 0 && (p.f_expert_elems & 7) == 0 &&
+              (uint64_t)64 * (uint64_t)p.ld_in * 2 < (1ull << 31);
+    for (int seg = 0; seg < p.nseg; seg++) ok = ok && ((uintptr_t)p.in[seg] & 15) == 0;
+    return ok;
 }
 
 int skinny_nt(const SkinnyNtParams& p, int r_pad, int grid_tiles, hipStream_t s) {
@@ -448,12 +477,22 @@ int skinny_nt(const SkinnyNtParams& p, int r_pad, int grid_tiles, hipStream_t s)
     bool direct = (p.ld_in & 7) == 0 && (p.ldf & 7) == 0 && (p.c & 63) == 0 && ((uintptr_t)p.f & 15) == 0 && (p.f_expert_elems & 7) == 0 &&
                   (uint64_t)64 * (uint64_t)p.ld_in * 2 < (1ull << 31) && (uint64_t)64 * (uint64_t)p.ldf * 2 < (1ull << 31);
     for (int seg = 0; seg < p.nseg; seg++) direct = direct && ((uintptr_t)p.in[seg] & 15) == 0;
+    if (p.f_natural) {
+        if (!skinny_nt_takes_natural_factor(p)) return set_error(GGQ_ERR_SHAPE, "skinny_nt: this shape needs the factor transposed");
+        switch (r_pad / 16) {
+            case 1: return launch_skinny_direct<1, true>(p, grid_tiles, s);
+            case 2: return launch_skinny_direct<2, true>(p, grid_tiles, s);
+            case 3: return launch_skinny_direct<3, true>(p, grid_tiles, s);
+            case 4: return launch_skinny_direct<4, true>(p, grid_tiles, s);
+            default: return set_error(GGQ_ERR_SHAPE, "LoRA rank must be between 1 and 64");
+        }
+    }
     if (direct) {
         switch (r_pad / 16) {
-            case 1: return launch_skinny_direct<1>(p, grid_tiles, s);
-            case 2: return launch_skinny_direct<2>(p, grid_tiles, s);
-            case 3: return launch_skinny_direct<3>(p, grid_tiles, s);
-            case 4: return launch_skinny_direct<4>(p, grid_tiles, s);
+            case 1: return launch_skinny_direct<1, false>(p, grid_tiles, s);
+            case 2: return launch_skinny_direct<2, false>(p, grid_tiles, s);
+            case 3: return launch_skinny_direct<3, false>(p, grid_tiles, s);
+            case 4: return launch_skinny_direct<4, false>(p, grid_tiles, s);
             default: return set_error(GGQ_ERR_SHAPE, "LoRA rank must be between 1 and 64");
         }
     }

@@ -14,8 +14,9 @@ struct TileDesc {  // one row tile of an expert group: rows [row_begin, row_end)
 struct SkinnyNtParams {
     const bf16_t* in[2];  // [m, c] per segment
     int64_t ld_in;
-    const bf16_t* f;      // per expert [r][ldf], contraction contiguous
+    const bf16_t* f;      // per expert [r][ldf], contraction contiguous; or [nseg*c][r] when f_natural
     int64_t ldf, f_expert_elems;
+    int f_natural;
     bf16_t* out;          // [m, r_pad]
     int m, c, r, nseg;
     const int64_t* expert_ids;
@@ -73,9 +74,10 @@ struct MmqParams {
     int shape;  // kShapeTall / kShapeWide: which instantiation of the tile kernel the sizes above are for
     // LoRA
     const bf16_t* la;     // [rows, r_pad]  (x A^T in NT, dY B in NN)
-    const bf16_t* lb;     // per expert [cols_total, r_pad] (B rows in NT, A^T rows in NN)
+    const bf16_t* lb;     // per expert: NT [cols_total, r_pad] (rows of B); NN [lora_rank, k] (the factor A as it is)
     int64_t lb_expert_elems;
     int r_pad;            // multiple of 16, <= 64; 0 = no LoRA
+    int lora_rank;        // NN mode: rows of the factor A that exist (the tile's rows up to r_pad are zero)
     float lora_scale;
     // cross-entropy epilogues
     const int64_t* labels;     // [m]
@@ -98,6 +100,7 @@ int init_params(MmqParams& p, int qt, int mode, int m, int n, int k, int nseg, i
 int pad_factor(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int r, int r_pad, bool transpose, hipStream_t s);
 int transpose_factor(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int r, hipStream_t s);
 int skinny_nt(const SkinnyNtParams& p, int r_pad, int grid_tiles, hipStream_t s);
+bool skinny_nt_takes_natural_factor(const SkinnyNtParams& p);
 int factor_grad(const FactorGradParams& p, int r_pad, int64_t experts, hipStream_t s);
 
 // Builds the row-tile table of an expert-sorted layout on the device (no host sync):

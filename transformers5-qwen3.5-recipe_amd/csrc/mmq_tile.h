@@ -610,10 +610,10 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
     struct Operands {
         bf16x8_t a[LIVE], b[kColBlocks];
     };
-    // `lora`: the LoRA tiles ahead of the main steps always use the [column][contraction] W layout
-    auto load_operands = [&](Operands& o, int stage, int buf, int kk, bool lora = false) __attribute__((always_inline)) {
+    // (the LoRA tiles ahead of the main steps use the same two W layouts)
+    auto load_operands = [&](Operands& o, int stage, int buf, int kk) __attribute__((always_inline)) {
         const uint8_t* a_lds = a_row + stage * kAStageBytes + a_koff[kk];
-        if (MODE == kModeNN && !lora) {
+        if (MODE == kModeNN) {
             // W tile is [contraction row][output column]: each transposing 8-byte read hands this lane
             // four consecutive contraction values of its column, two reads make the MFMA operand
             const bf16_t* t_lds = c.bs + buf * kBTile + tr_off + kk * 16 * kNnPitch;
@@ -650,7 +650,7 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
         for (int kk = 0; kk < 4; kk++)
             if (kk < n) {
                 Operands o;
-                load_operands(o, 0, 0, kk, true);
+                load_operands(o, 0, 0, kk);
                 mfma_operands(o);
             }
         const float s = p.lora_scale;
@@ -885,12 +885,30 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
             if (r < c.rows_valid && ch < chunks) v = *(const uint4*)(p.la + (int64_t)(c.row_begin + r) * p.r_pad + ch * 8);
             *(uint4*)(c.as + r * kARowBytes + a_slot(r, ch) * 16) = v;
         }
-        const bf16_t* lb = p.lb + c.expert * p.lb_expert_elems + (int64_t)(c.seg_c * c.out_cols + c.col0) * p.r_pad;
-        for (int id = tid; id < kTN * 8; id += kThreads) {
-            const int cidx = id >> 3, ch = id & 7;
-            uint4 v = zero4();
-            if (c.col0 + cidx < c.out_cols && ch < chunks) v = *(const uint4*)(lb + (int64_t)cidx * p.r_pad + ch * 8);
-            *(uint4*)&c.bs[cidx * kLdsStride + ch * 8] = v;
+        if (MODE == kModeNT) {
+            // forward: the factor B is [columns][r_pad], the layout of the forward W tile
+            const bf16_t* lb = p.lb + c.expert * p.lb_expert_elems + (int64_t)(c.seg_c * c.out_cols + c.col0) * p.r_pad;
+            for (int id = tid; id < kTN * 8; id += kThreads) {
+                const int cidx = id >> 3, ch = id & 7;
+                uint4 v = zero4();
+                if (c.col0 + cidx < c.out_cols && ch < chunks) v = *(const uint4*)(lb + (int64_t)cidx * p.r_pad + ch * 8);
+                *(uint4*)&c.bs[cidx * kLdsStride + ch * 8] = v;
+            }
+        } else {
+            // grad-input: the factor A is [r][output columns], which is the layout of the grad-input W tile
+            // ([contraction row][column]); rows r .. r_pad - 1 are zero
+            const bf16_t* lb = p.lb + c.expert * p.lb_expert_elems + c.col0;
+            const bool vec = (c.out_cols & 7) == 0;
+            for (int id = tid; id < p.r_pad * (kTN / 8); id += kThreads) {
+                const int j = id / (kTN / 8), ch = id - j * (kTN / 8);
+                const int col = c.col0 + ch * 8;
+                uint4 v = zero4();
+                if (j < p.lora_rank) {
+                    const bf16_t* src = lb + (int64_t)j * c.out_cols + ch * 8;
+                    v = vec && col + 8 <= c.out_cols ? *(const uint4*)src : load8_slow(src, c.out_cols - col);
+                }
+                *(uint4*)&c.bs[j * kNnPitch + ch * 8] = v;
+            }
         }
     }
     __syncthreads();  // LoRA tiles and the codebook are visible
