@@ -403,8 +403,7 @@ static __device__ __forceinline__ void q4k_quarter_decode(const u32x4_t& hdr, co
     }
 }
 
-// Grad-input: lane (contraction row n = kc0 + lane, run = col0/32 + wave of the quartet, half = quartet)
-// decodes 16 consecutive output columns of its row.
+// Grad-input, tall shape: a lane decodes 16 consecutive output columns (half a run) of its contraction row.
 struct Q4KHalfRun {
     u32x4_t hdr, q;
 };
@@ -482,10 +481,13 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
         }
     } else if (MODE == kModeNN && SH == 1) {
         // wide: the 256 output columns of a step are exactly one block of each of the 64 contraction rows;
-        // lane = (row kc0 + lane, run = producer wave), stored as it is decoded: [row][column], the
-        // consumers transpose on the way out of LDS
-        const int lane = ptid & 63;
-        const int ksub = min((c.col0 >> 5) + pw, (p.k >> 5) - 1);  // runs past the end are clamped, never stored
+        // producer wave w takes rows 8w .. 8w+7, lane = (row, run of 32 columns), so that the eight lanes of
+        // a row ask for one header and four adjacent 32-byte groups (a lane-per-row split costs the vector
+        // cache one access per lane and load).  Stored as decoded: [row][column]; the consumers transpose
+        // on the way out of LDS.
+        const int lane = 8 * pw + ((ptid & 63) >> 3);  // contraction row inside the step
+        const int run = ptid & 7;
+        const int ksub = min((c.col0 >> 5) + run, (p.k >> 5) - 1);  // runs past the end are clamped, never stored
         typedef typename Fmt<kQ4_K>::Raw Raw;
         auto issue = [&](Raw& r, int u) __attribute__((always_inline)) {
             int seg_k, kc0;
@@ -493,7 +495,7 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
             const int wrow = min(kc0 + lane, p.n - 1);  // rows past the end meet the zero-filled tail of the A tile
             Fmt<kQ4_K>::load(r, p.w[seg_k] + c.expert * p.w_expert_bytes + (int64_t)wrow * p.w_row_bytes, ksub);
         };
-        bf16_t* const dst0 = c.bs + lane * kNnPitch + pw * 32;
+        bf16_t* const dst0 = c.bs + lane * kNnPitch + run * 32;
         auto fill = [&](Raw& r, int u) __attribute__((always_inline)) {
             open_phase(u);
             Fmt<kQ4_K>::pin(r);
@@ -545,7 +547,10 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
             if (k + 1 < blocks) block_phases(odd, even, k + 1);
         }
     } else {
-        const int lane = ptid & 63, run_w = pw & 3, half = pw >> 2;
+        // tall: 128 output columns = four runs per row; producer wave w takes rows 8w .. 8w+7,
+        // lane = (row, run, half of the run): the eight lanes of a row ask for one header and 64 adjacent bytes
+        const int lane = 8 * pw + ((ptid & 63) >> 3);  // contraction row inside the step
+        const int run_w = (ptid & 7) >> 1, half = ptid & 1;
         const int ksub = min((c.col0 >> 5) + run_w, (p.k >> 5) - 1);  // runs past the end are clamped, never stored
         const int j = ksub & 7;
         const int64_t blk_off = (int64_t)(ksub >> 3) * 144;
