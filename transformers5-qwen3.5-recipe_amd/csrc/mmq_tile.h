@@ -281,8 +281,10 @@ static __device__ __forceinline__ void q4k_chunk_store(const TileCtx& c, const P
 // u - 1 (step 0: before the first phase) and stores them during phase u.  steps + 1 barriers in all.
 // The phase sequence is written out per period (no data-dependent branches between a load and its
 // use), so that the waits on the packed-weight loads stay exact instead of draining every load.
-template <int QT, int MODE, int Q>
-static __device__ __forceinline__ void produce(const MmqParams& p, const TileCtx& c, int ptid, int pw) {
+// `after_issue` runs once the first packed-weight loads are on their way: the LoRA tiles are fetched
+// there by all waves, and the workgroup meets at the barrier that makes them visible.
+template <int QT, int MODE, int Q, class AfterIssue>
+static __device__ __forceinline__ void produce(const MmqParams& p, const TileCtx& c, int ptid, int pw, AfterIssue&& after_issue) {
     ProducerLane l;
     l.ptid = ptid, l.pw = pw, l.lane = ptid & 63;
     // W run owned by this lane: NT -> (output column n = col0 + ptid/2, run 2*step + ptid%2);
@@ -319,6 +321,7 @@ static __device__ __forceinline__ void produce(const MmqParams& p, const TileCtx
         };
         if (Q < steps) w_issue_run<QT, MODE>(p, c, l, Q, raw_a);
         if (Q + 2 < steps) w_issue_run<QT, MODE>(p, c, l, Q + 2, raw_b);
+        after_issue();
         if (Q == 0) {
             decode(raw_a, 0);
             for (int b = 0; b < steps; b += 4) {
@@ -433,8 +436,8 @@ static __device__ __forceinline__ void q4k_half_run_decode(const Q4KHalfRun& r, 
 
 // Barrier b closes the phase in which step b reaches LDS; steps + 1 barriers in all (the last one
 // pairs with the consumers' final step).
-template <int MODE>
-static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const TileCtx& c, int ptid, int pw) {
+template <int MODE, class AfterIssue>
+static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const TileCtx& c, int ptid, int pw, AfterIssue&& after_issue) {
     // ptid 0..511 over both quartets; pw 0..7
     const int steps = c.total_steps;
     int stage = c.base, buf = c.base;
@@ -456,6 +459,7 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
         const int blocks = steps >> 2;  // K is a whole number of 256-wide blocks
         Q4KChunk even, odd;             // alternate between blocks; a set is loaded four phases before its first use
         q4k_chunk_load(even, wrow, 0, h);
+        after_issue();
         auto fill = [&](auto s_c, const Q4KChunk& ch, int u) __attribute__((always_inline)) {
             constexpr int S = decltype(s_c)::value;
             open_phase(u);
@@ -510,6 +514,7 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
         Raw ra, rb;  // even / odd steps, each reloaded two steps ahead
         issue(ra, 0);
         if (steps > 1) issue(rb, 1);
+        after_issue();
         for (int u = 0; u < steps; u += 2) {
             fill(ra, u);
             if (u + 1 < steps) fill(rb, u + 1);
@@ -521,6 +526,7 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
         bf16_t* const dst0 = c.bs + n_local * kLdsStride + q * 8;
         Q4KQuarter even, odd;  // alternate between blocks; a set is loaded four phases before its first use
         q4k_quarter_load(even, wrow, 0, q);
+        after_issue();
         auto fill = [&](auto s_c, const Q4KQuarter& ch, int u) __attribute__((always_inline)) {
             constexpr int S = decltype(s_c)::value;
             open_phase(u);
@@ -578,6 +584,7 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
         Q4KHalfRun ra, rb;  // even / odd steps, each reloaded two steps ahead
         issue(ra, 0);
         if (steps > 1) issue(rb, 1);
+        after_issue();
         for (int u = 0; u < steps; u += 2) {
             fill(ra, u);
             if (u + 1 < steps) fill(rb, u + 1);
@@ -587,8 +594,8 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
 }
 
 // ---- consumer waves, instantiated per number of live 32-row blocks.
-template <int QT, int MODE, int EPI, int LIVE>
-static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, int lane, int cw) {
+template <int QT, int MODE, int EPI, int LIVE, class AfterIssue>
+static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx& c, int lane, int cw, AfterIssue&& after_issue) {
     const int wave_m = cw / kWavesN, wave_n = cw % kWavesN;
     const int lane_c = lane & 31, lane_h = lane >> 5;
     f32x16_t acc[LIVE][kColBlocks];
@@ -649,6 +656,7 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
     ai.next_step = 0, ai.next_stage = c.base;
 #pragma unroll
     for (int d = 0; d < kAhead; d++) a_issue_next<MODE>(ai, p, c);
+    after_issue();
     if (c.base == 1) {  // LoRA tiles sit in stage 0 / buffer 0: acc = s * LA . LB^T, r_pad / 16 sub-steps
         const int n = p.r_pad >> 4;
 #pragma unroll
@@ -809,13 +817,14 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
 
 // A consumer wave without a live row block still moves its share of the A tile and keeps the
 // barriers company.
-template <int MODE>
-static __device__ __forceinline__ void consume_idle(const MmqParams& p, const TileCtx& c, int lane, int cw) {
+template <int MODE, class AfterIssue>
+static __device__ __forceinline__ void consume_idle(const MmqParams& p, const TileCtx& c, int lane, int cw, AfterIssue&& after_issue) {
     AIssuer ai;
     a_loader_init(ai.ld, p, c, lane, cw);
     ai.next_step = 0, ai.next_stage = c.base;
 #pragma unroll
     for (int d = 0; d < kAhead; d++) a_issue_next<MODE>(ai, p, c);
+    after_issue();
     a_wait_step(ai, c, 0);
     lds_barrier();
     for (int t = 0; t < c.total_steps; t++) {
@@ -881,56 +890,60 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
         const uint64_t g = d_iq2xxs_grid_mm[tid];
         grid_lds[tid] = make_uint2((uint32_t)g, (uint32_t)(g >> 32));
     }
-    // ---- LoRA tiles go to A stage 0 / W buffer 0 (all lanes load): LA[rows, :r] and LB[cols, :r]
-    if (p.r_pad > 0) {
-        const int chunks = p.r_pad >> 3;  // 16-byte chunks per row (r_pad % 16 == 0)
-        for (int id = tid; id < kTM * 8; id += kThreads) {
-            const int r = id >> 3, ch = id & 7;
-            uint4 v = zero4();
-            if (r < c.rows_valid && ch < chunks) v = *(const uint4*)(p.la + (int64_t)(c.row_begin + r) * p.r_pad + ch * 8);
-            *(uint4*)(c.as + r * kARowBytes + a_slot(r, ch) * 16) = v;
-        }
-        if (MODE == kModeNT) {
-            // forward: the factor B is [columns][r_pad], the layout of the forward W tile
-            const bf16_t* lb = p.lb + c.expert * p.lb_expert_elems + (int64_t)(c.seg_c * c.out_cols + c.col0) * p.r_pad;
-            for (int id = tid; id < kTN * 8; id += kThreads) {
-                const int cidx = id >> 3, ch = id & 7;
+    // ---- LoRA tiles go to A stage 0 / W buffer 0 (all lanes load): LA[rows, :r] and LB.  Every wave runs
+    // this once, right after it has issued its first loads of the tile proper (A tile / packed weights),
+    // so that the two memory round trips overlap.
+    auto lora_tiles = [&]() __attribute__((always_inline)) {
+        if (p.r_pad > 0) {
+            const int chunks = p.r_pad >> 3;  // 16-byte chunks per row (r_pad % 16 == 0)
+            for (int id = tid; id < kTM * 8; id += kThreads) {
+                const int r = id >> 3, ch = id & 7;
                 uint4 v = zero4();
-                if (c.col0 + cidx < c.out_cols && ch < chunks) v = *(const uint4*)(lb + (int64_t)cidx * p.r_pad + ch * 8);
-                *(uint4*)&c.bs[cidx * kLdsStride + ch * 8] = v;
+                if (r < c.rows_valid && ch < chunks) v = *(const uint4*)(p.la + (int64_t)(c.row_begin + r) * p.r_pad + ch * 8);
+                *(uint4*)(c.as + r * kARowBytes + a_slot(r, ch) * 16) = v;
             }
-        } else {
-            // grad-input: the factor A is [r][output columns], which is the layout of the grad-input W tile
-            // ([contraction row][column]); rows r .. r_pad - 1 are zero
-            const bf16_t* lb = p.lb + c.expert * p.lb_expert_elems + c.col0;
-            const bool vec = (c.out_cols & 7) == 0;
-            for (int id = tid; id < p.r_pad * (kTN / 8); id += kThreads) {
-                const int j = id / (kTN / 8), ch = id - j * (kTN / 8);
-                const int col = c.col0 + ch * 8;
-                uint4 v = zero4();
-                if (j < p.lora_rank) {
-                    const bf16_t* src = lb + (int64_t)j * c.out_cols + ch * 8;
-                    v = vec && col + 8 <= c.out_cols ? *(const uint4*)src : load8_slow(src, c.out_cols - col);
+            if (MODE == kModeNT) {
+                // forward: the factor B is [columns][r_pad], the layout of the forward W tile
+                const bf16_t* lb = p.lb + c.expert * p.lb_expert_elems + (int64_t)(c.seg_c * c.out_cols + c.col0) * p.r_pad;
+                for (int id = tid; id < kTN * 8; id += kThreads) {
+                    const int cidx = id >> 3, ch = id & 7;
+                    uint4 v = zero4();
+                    if (c.col0 + cidx < c.out_cols && ch < chunks) v = *(const uint4*)(lb + (int64_t)cidx * p.r_pad + ch * 8);
+                    *(uint4*)&c.bs[cidx * kLdsStride + ch * 8] = v;
                 }
-                *(uint4*)&c.bs[j * kNnPitch + ch * 8] = v;
+            } else {
+                // grad-input: the factor A is [r][output columns], which is the layout of the grad-input W tile
+                // ([contraction row][column]); rows r .. r_pad - 1 are zero
+                const bf16_t* lb = p.lb + c.expert * p.lb_expert_elems + c.col0;
+                const bool vec = (c.out_cols & 7) == 0;
+                for (int id = tid; id < p.r_pad * (kTN / 8); id += kThreads) {
+                    const int j = id / (kTN / 8), ch = id - j * (kTN / 8);
+                    const int col = c.col0 + ch * 8;
+                    uint4 v = zero4();
+                    if (j < p.lora_rank) {
+                        const bf16_t* src = lb + (int64_t)j * c.out_cols + ch * 8;
+                        v = vec && col + 8 <= c.out_cols ? *(const uint4*)src : load8_slow(src, c.out_cols - col);
+                    }
+                    *(uint4*)&c.bs[j * kNnPitch + ch * 8] = v;
+                }
             }
         }
-    }
-    __syncthreads();  // LoRA tiles and the codebook are visible
+        __syncthreads();  // LoRA tiles and the codebook are visible
+    };
 
     if (wave >= 8) {
-        if (QT == kQ4_K) produce_q4k<MODE>(p, c, tid - 512, wave - 8);
-        else if (wave < 12) produce<QT, MODE, 0>(p, c, tid & 255, wave & 3);
-        else produce<QT, MODE, 1>(p, c, tid & 255, wave & 3);
+        if (QT == kQ4_K) produce_q4k<MODE>(p, c, tid - 512, wave - 8, lora_tiles);
+        else if (wave < 12) produce<QT, MODE, 0>(p, c, tid & 255, wave & 3, lora_tiles);
+        else produce<QT, MODE, 1>(p, c, tid & 255, wave & 3, lora_tiles);
     } else {
         const int cw = wave, wave_m = cw / kWavesN;
         // this wave's row blocks are tile rows 32*wave_m .. +31 and 32*(wave_m + kWavesM) .. +31; blocks fill up from row 0
         const int blocks = (c.rows_valid + 31) >> 5;
         const int live = (blocks > wave_m ? 1 : 0) + (blocks > wave_m + kWavesM ? 1 : 0);
         switch (live) {
-            case 0: consume_idle<MODE>(p, c, lane, cw); break;
-            case 1: consume<QT, MODE, EPI, 1>(p, c, lane, cw); break;
-            default: consume<QT, MODE, EPI, 2>(p, c, lane, cw); break;
+            case 0: consume_idle<MODE>(p, c, lane, cw, lora_tiles); break;
+            case 1: consume<QT, MODE, EPI, 1>(p, c, lane, cw, lora_tiles); break;
+            default: consume<QT, MODE, EPI, 2>(p, c, lane, cw, lora_tiles); break;
         }
     }
 }
