@@ -3,6 +3,7 @@
 #include "../../include/ggml_mmq_gfx950.h"
 
 #include <algorithm>
+#include <stdlib.h>
 
 #include "launch.h"
 #include "mmq_host.h"
@@ -76,7 +77,12 @@ static int launch_wide_and_tall(int qt, int mode, MmqParams& p, int rows, int n,
 
 // Expert groups that average at most 192 rows run the Q4_K tile kernel in its wide shape.
 static int pick_shape(int qt, int64_t rows, int64_t groups) {
-    return (qt == 12 /* GGML Q4_K */ && groups > 0 && rows <= 192 * groups) ? kShapeWide : kShapeTall;
+    if (!(qt == 12 /* GGML Q4_K */ && groups > 0 && rows <= 192 * groups)) return kShapeTall;
+    static const int forced = [] {
+        const char* e = getenv("GGQ_GROUPED_SHAPE");  // tuning aid: 1 = wide + tall mixed launch, 2 = half tiles
+        return e ? atoi(e) : -1;
+    }();
+    return forced == kShapeHalf ? kShapeHalf : kShapeWide;
 }
 
 int64_t ggq_lora_workspace_bytes(int64_t rows, int64_t groups, int64_t experts, int64_t n_total, int64_t k, int r) {
@@ -147,7 +153,8 @@ int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void*
         // Wide shape: groups of at most 128 rows take one wide tile each, larger groups go to a second,
         // tall launch (a second wide tile for a few dozen leftover rows would cost a whole decode pass).
         const bool wide = p.shape == kShapeWide;
-        const int max128 = wide ? (int)groups : (int)(rows / kBM + groups);
+        const int bm_main = p.shape == kShapeTall ? kBM : kWideBM;
+        const int max128 = wide ? (int)groups : (int)(rows / bm_main + groups);
         max_tall = wide ? (int)std::min<int64_t>(rows / kBM + groups, rows / (kWideBM + 1) + rows / kBM + 1) : 0;
         max_tiles64 = (int)(rows / 64 + groups);
         TileDesc* t128 = (TileDesc*)bump.take((int64_t)max128 * sizeof(TileDesc));
@@ -156,7 +163,7 @@ int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void*
         int* counts = (int*)bump.take(16);
         if (!t128 || !counts || (lora_a && !t64) || (wide && !t_tall)) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
         RowTileTables tb{};
-        tb.add(wide ? kWideBM : kBM, 0, wide ? kWideBM : 0x7FFFFFFF, t128, counts);
+        tb.add(bm_main, 0, wide ? kWideBM : 0x7FFFFFFF, t128, counts);
         if (wide) tb.add(kBM, kWideBM, 0x7FFFFFFF, t_tall, counts + 2), n_tall = counts + 2;
         if (lora_a) tb.add(64, 0, 0x7FFFFFFF, t64, counts + 1);
         if (int rc = build_row_tile_tables(expert_ids, end_offsets, (int)groups, tb, nullptr, 0, s)) return rc;
@@ -221,7 +228,8 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
     int max_tall = 0;
     if (groups > 0) {
         const bool wide = p.shape == kShapeWide;  // small groups: wide tiles; larger ones: a second, tall launch
-        const int max128 = wide ? (int)groups : (int)(rows / kBM + groups);
+        const int bm_main = p.shape == kShapeTall ? kBM : kWideBM;
+        const int max128 = wide ? (int)groups : (int)(rows / bm_main + groups);
         max_tall = wide ? (int)std::min<int64_t>(rows / kBM + groups, rows / (kWideBM + 1) + rows / kBM + 1) : 0;
         max_tiles64 = (int)(rows / 64 + groups);
         TileDesc* t128 = (TileDesc*)bump.take((int64_t)max128 * sizeof(TileDesc));
@@ -231,7 +239,7 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
         int* rg = lora_a ? (int*)bump.take(experts * 2 * 4) : nullptr;
         if (!t128 || !counts || (lora_a && (!t64 || !rg)) || (wide && !t_tall)) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
         RowTileTables tb{};
-        tb.add(wide ? kWideBM : kBM, 0, wide ? kWideBM : 0x7FFFFFFF, t128, counts);
+        tb.add(bm_main, 0, wide ? kWideBM : 0x7FFFFFFF, t128, counts);
         if (wide) tb.add(kBM, kWideBM, 0x7FFFFFFF, t_tall, counts + 2), n_tall = counts + 2;
         if (lora_a) tb.add(64, 0, 0x7FFFFFFF, t64, counts + 1);
         if (int rc = build_row_tile_tables(expert_ids, end_offsets, (int)groups, tb, rg, (int)experts, s)) return rc;

@@ -140,11 +140,14 @@ static int launch_one(const MmqParams& p, hipStream_t s) {
     constexpr int kSmemBytes = Tile<SH>::kTileLdsBytes + (QT == kIQ2_XXS ? 2048 : 0);
     static bool attr_set = false;  // per instantiation; the attribute is a property of the function
     if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)mmq_tile_kernel<QT, MODE, EPI, SH>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess)
-            return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", kSmemBytes);
+        hipError_t e;
+        if constexpr (SH == kShapeHalf) e = hipFuncSetAttribute((const void*)mmq_half_kernel<QT, MODE, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
+        else e = hipFuncSetAttribute((const void*)mmq_tile_kernel<QT, MODE, EPI, SH>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
+        if (e != hipSuccess) return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", kSmemBytes);
         attr_set = true;
     }
-    hipLaunchKernelGGL((mmq_tile_kernel<QT, MODE, EPI, SH>), dim3((unsigned)grid), dim3(kThreads), kSmemBytes, s, p);
+    if constexpr (SH == kShapeHalf) hipLaunchKernelGGL((mmq_half_kernel<QT, MODE, EPI>), dim3((unsigned)grid), dim3(Tile<kShapeHalf>::kThreadsWG), kSmemBytes, s, p);
+    else hipLaunchKernelGGL((mmq_tile_kernel<QT, MODE, EPI, SH>), dim3((unsigned)grid), dim3(kThreads), kSmemBytes, s, p);
     if (t) (void)hipEventRecord(t->stop, s);
     return check_launch("mmq_tile_kernel");
 }
@@ -188,6 +191,7 @@ static int launch_qt(int mode, int epi, const MmqParams& p, hipStream_t s) {
         switch (epi) {
             case kEpiStore:
                 if (QT == kQ4_K && p.shape == kShapeWide) return launch_one<kQ4_K, kModeNT, kEpiStore, 1>(p, s);
+                if (QT == kQ4_K && p.shape == kShapeHalf) return launch_one<kQ4_K, kModeNT, kEpiStore, 2>(p, s);
                 return launch_one<QT, kModeNT, kEpiStore, 0>(p, s);
             case kEpiCeStats: return launch_one<QT, kModeNT, kEpiCeStats, 0>(p, s);
             case kEpiCeGrad: return launch_one<QT, kModeNT, kEpiCeGrad, 0>(p, s);
@@ -196,6 +200,7 @@ static int launch_qt(int mode, int epi, const MmqParams& p, hipStream_t s) {
         switch (epi) {
             case kEpiStore:
                 if (QT == kQ4_K && p.shape == kShapeWide) return launch_one<kQ4_K, kModeNN, kEpiStore, 1>(p, s);
+                if (QT == kQ4_K && p.shape == kShapeHalf) return launch_one<kQ4_K, kModeNN, kEpiStore, 2>(p, s);
                 return launch_one<QT, kModeNN, kEpiStore, 0>(p, s);
             case kEpiAccumF32: return launch_one<QT, kModeNN, kEpiAccumF32, 0>(p, s);
         }
@@ -223,8 +228,8 @@ int init_params(MmqParams& p, int qt, int mode, int m, int n, int k, int nseg, i
     p.m = m, p.n = n, p.k = k, p.nseg = nseg;
     p.w_row_bytes = packed_row_bytes(qt, k);
     p.w_expert_bytes = p.w_row_bytes * n;
-    if (shape == kShapeWide && qt != kQ4_K) shape = kShapeTall;  // the wide instantiation exists for Q4_K only
-    const int bm = shape == kShapeWide ? kWideBM : kBM, bn = shape == kShapeWide ? kWideBN : kBN;
+    if (shape != kShapeTall && qt != kQ4_K) shape = kShapeTall;  // the wide and half instantiations exist for Q4_K only
+    const int bm = shape == kShapeTall ? kBM : kWideBM, bn = shape == kShapeWide ? kWideBN : kBN;
     p.shape = shape;
     if (mode == kModeNT) {
         p.col_tiles_per_seg = (n + bn - 1) / bn;

@@ -38,7 +38,7 @@ struct FactorGradParams {
 
 constexpr int kBM = 256, kBN = 128, kBK = 64;  // the tall tile shape (dense launches, large expert groups)
 constexpr int kWideBM = 128, kWideBN = 256;    // the wide tile shape (Q4_K expert groups of about a hundred rows)
-constexpr int kShapeTall = 0, kShapeWide = 1;
+constexpr int kShapeTall = 0, kShapeWide = 1, kShapeHalf = 2;
 constexpr int kLdsStride = kBK + 8;  // bf16 elements per LDS row: 144 bytes keeps 128-bit reads conflict-free
 constexpr int kThreads = 1024;  // waves 0..7 run the MFMAs, waves 8..15 load and decode
 

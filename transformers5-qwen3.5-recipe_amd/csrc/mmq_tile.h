@@ -48,6 +48,16 @@ typedef __attribute__((address_space(3))) v4i16_t* lds_v4i16_ptr;  // native vec
 
 __device__ __forceinline__ uint4 zero4() { return make_uint4(0, 0, 0, 0); }
 
+// A 16-byte global load that the compiler does not see as a load.  Its own wait-count pass drains every
+// outstanding load in front of a register set that was requested before a loop back-edge or a join, which
+// puts a full memory round trip into each step of a two-steps-ahead prefetch.  With this form the caller
+// waits itself (wait_loads_at_most, loads return in issue order) and fences the registers
+// (asm volatile "+v") between that wait and their first use; nothing may touch them before.
+__device__ __forceinline__ void load16_untracked(u32x4_t& dst, const void* ptr) {
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(ptr) : "memory");
+}
+__device__ __forceinline__ uint4 as_uint4(const u32x4_t& v) { return make_uint4(v.x, v.y, v.z, v.w); }
+
 // 8 consecutive bf16 from a row, zero-filled past `valid` elements (element-wise path for rows that
 // are not 16-byte aligned or that end inside the run).
 __device__ __forceinline__ uint4 load8_slow(const bf16_t* p, int valid) {
@@ -84,15 +94,21 @@ __device__ __forceinline__ void step_origin(const MmqParams& p, int step, int& s
 // row blocks wave_m and wave_m + kWavesM and the 64 columns at 64 * wave_n.
 template <int SH>
 struct Tile {
-static constexpr int kTM = SH == 0 ? 256 : 128, kTN = SH == 0 ? 128 : 256;
+static constexpr int kTM = SH == 0 ? 256 : 128, kTN = SH == 1 ? 256 : 128;
 static constexpr int kWavesM = kTM / 64, kWavesN = kTN / 64;
+// SH = 2: 128 x 128 ("half"): four consumer and four producer waves, half the registers and less than half
+// the LDS of a compute unit, so two workgroups share one: each has its own barrier, and one's waits, set-up
+// and stores run under the other's steps.
+static constexpr int kCW = kWavesM * kWavesN;       // consumer waves (8, 8, 4), as many producer waves
+static constexpr int kProducerLanes = 64 * kCW;
+static constexpr int kThreadsWG = 128 * kCW;
 static constexpr int kAStageBytes = kTM * kARowBytes;   // 32 KB / 16 KB
 // LDS ring of A tiles: the loads of a step are issued kAStages - 1 steps ahead of its MFMAs.  Memory latency
 // under load is about two thousand cycles; the wide shape's short steps need the longer ring.
-static constexpr int kAStages = SH == 0 ? 3 : 5;
+static constexpr int kAStages = SH == 0 ? 3 : SH == 1 ? 5 : 2;
 static constexpr int kAhead = kAStages - 1;
 static constexpr int kAGroups = kTM / 8;                // 8-row groups (one direct-to-LDS instruction each)
-static constexpr int kGroupsPerWave = kAGroups / 8;     // groups one consumer wave moves per step (4 / 2)
+static constexpr int kGroupsPerWave = kAGroups / kCW;   // groups one consumer wave moves per step (4 / 2 / 4)
 // W buffer: forward [output column][64 + 8]; grad-input [contraction row][columns + 32], as the rows are
 // decoded (the consumers transpose on the way out of LDS).  Sized for the larger of the two.
 static constexpr int kNnPitch = kTN + 32;
@@ -108,18 +124,18 @@ struct ALoader {
 };
 
 static __device__ __forceinline__ void a_loader_init(ALoader& a, const MmqParams& p, const TileCtx& c, int lane, int cw) {
-    const int sub = 8 * cw + (lane >> 3);         // row inside a 64-row slab
+    const int sub = 8 * cw + (lane >> 3);         // row inside a slab of 8 rows per consumer wave
     const int kc = (lane & 7) ^ ((sub >> 1) & 7);  // the chunk that belongs in this lane's LDS slot
 #pragma unroll
     for (int j = 0; j < kGroupsPerWave; j++) {
         // rows past the end of the group are clamped to its last row: they only feed output rows that
         // are never stored
-        const int row = min(64 * j + sub, c.rows_valid - 1);
+        const int row = min(8 * kCW * j + sub, c.rows_valid - 1);
         a.voff[j] = ((uint32_t)row * (uint32_t)p.lda + (uint32_t)kc * 8u) * 2u;
     }
     a.lds0 = c.as_lds + cw * 1024;
     const int groups = (c.rows_valid + 7) >> 3;
-    a.n = c.a_fast ? max(0, (groups - cw + 7) >> 3) : 0;
+    a.n = c.a_fast ? max(0, (groups - cw + kCW - 1) / kCW) : 0;
 }
 
 template <int MODE, int J0, int J1>
@@ -133,7 +149,7 @@ static __device__ __forceinline__ void a_issue(const ALoader& a, const MmqParams
         if (j < a.n)
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                          :
-                         : "s"(lds + j * 8192), "v"(a.voff[j]), "s"(sbase)
+                         : "s"(lds + j * (kCW * 1024)), "v"(a.voff[j]), "s"(sbase)
                          : "memory", "m0");
 }
 
@@ -451,8 +467,8 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
         stage = stage == kAStages - 1 ? 0 : stage + 1;
         buf ^= 1;
     };
-    if (MODE == kModeNT && SH == 1) {
-        // wide: 256 output columns, lane = (column ptid / 2, half ptid % 2), 32 weights per lane and step
+    if (MODE == kModeNT && SH != 0) {
+        // wide / half: lane = (column ptid / 2, half ptid % 2), 32 weights per lane and step
         ProducerLane l = slow;
         const int h = ptid & 1;
         const uint8_t* wrow = p.w[c.seg_c] + c.expert * p.w_expert_bytes + (int64_t)min(c.col0 + (ptid >> 1), p.n - 1) * p.w_row_bytes;
@@ -469,7 +485,9 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
             close_phase();
         };
         auto block_phases = [&](Q4KChunk& cur, Q4KChunk& nxt, int k) __attribute__((always_inline)) {
-            if (k + 1 < blocks) q4k_chunk_load(nxt, wrow, k + 1, h);
+            // (unconditional, the last block simply loads itself again: a load under a branch makes the
+            // compiler drain every outstanding load at the join, right after this one was issued)
+            q4k_chunk_load(nxt, wrow, min(k + 1, blocks - 1), h);
             q4k_chunk_pin(cur);
             fill(std::integral_constant<int, 0>{}, cur, 4 * k);
             q4k_chunk_pin(cur);
@@ -483,29 +501,40 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
             block_phases(even, odd, k);
             if (k + 1 < blocks) block_phases(odd, even, k + 1);
         }
-    } else if (MODE == kModeNN && SH == 1) {
+    } else if (MODE == kModeNN && SH != 0) {
         // wide: the 256 output columns of a step are exactly one block of each of the 64 contraction rows;
         // producer wave w takes rows 8w .. 8w+7, lane = (row, run of 32 columns), so that the eight lanes of
         // a row ask for one header and four adjacent 32-byte groups (a lane-per-row split costs the vector
         // cache one access per lane and load).  Stored as decoded: [row][column]; the consumers transpose
         // on the way out of LDS.
-        const int lane = 8 * pw + ((ptid & 63) >> 3);  // contraction row inside the step
-        const int run = ptid & 7;
+        constexpr int kRuns = kTN / 32;                             // lanes per contraction row (8 wide, 4 half)
+        const int lane = (64 / kRuns) * pw + (ptid & 63) / kRuns;  // contraction row inside the step
+        const int run = ptid % kRuns;
         const int ksub = min((c.col0 >> 5) + run, (p.k >> 5) - 1);  // runs past the end are clamped, never stored
-        typedef typename Fmt<kQ4_K>::Raw Raw;
+        struct Raw {  // header and the 32-byte quant group of the run: three untracked loads
+            u32x4_t hdr, q0, q1;
+        };
+        const int64_t blk_off = (int64_t)(ksub >> 3) * 144;
+        const int q_off = 16 + 32 * ((ksub & 7) >> 1);
         auto issue = [&](Raw& r, int u) __attribute__((always_inline)) {
             int seg_k, kc0;
             step_origin<MODE>(p, u, seg_k, kc0);
             const int wrow = min(kc0 + lane, p.n - 1);  // rows past the end meet the zero-filled tail of the A tile
-            Fmt<kQ4_K>::load(r, p.w[seg_k] + c.expert * p.w_expert_bytes + (int64_t)wrow * p.w_row_bytes, ksub);
+            const uint8_t* blk = p.w[seg_k] + c.expert * p.w_expert_bytes + (int64_t)wrow * p.w_row_bytes + blk_off;
+            load16_untracked(r.hdr, blk);
+            load16_untracked(r.q0, blk + q_off);
+            load16_untracked(r.q1, blk + q_off + 16);
         };
         bf16_t* const dst0 = c.bs + lane * kNnPitch + run * 32;
         auto fill = [&](Raw& r, int u) __attribute__((always_inline)) {
             open_phase(u);
-            Fmt<kQ4_K>::pin(r);
+            wait_loads_at_most(3);  // the other set's three loads may still be on their way
+            asm volatile("" : "+v"(r.hdr), "+v"(r.q0), "+v"(r.q1));
+            typename Fmt<kQ4_K>::Raw rr;
+            rr.hdr = as_uint4(r.hdr), rr.q0 = as_uint4(r.q0), rr.q1 = as_uint4(r.q1);
             uint32_t wv[16];
-            Fmt<kQ4_K>::decode(r, ksub, wv, nullptr);
-            if (u + 2 < steps) issue(r, u + 2);
+            Fmt<kQ4_K>::decode(rr, ksub, wv, nullptr);
+            issue(r, min(u + 2, steps - 1));  // always three loads: the count above stays exact
             bf16_t* dst = dst0 + buf * kBTile;
 #pragma unroll
             for (int i = 0; i < 4; i++) *(uint4*)(dst + 8 * i) = make_uint4(wv[4 * i], wv[4 * i + 1], wv[4 * i + 2], wv[4 * i + 3]);
@@ -513,7 +542,7 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
         };
         Raw ra, rb;  // even / odd steps, each reloaded two steps ahead
         issue(ra, 0);
-        if (steps > 1) issue(rb, 1);
+        issue(rb, min(1, steps - 1));
         after_issue();
         for (int u = 0; u < steps; u += 2) {
             fill(ra, u);
@@ -538,7 +567,7 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
             close_phase();
         };
         auto block_phases = [&](Q4KQuarter& cur, Q4KQuarter& nxt, int k) __attribute__((always_inline)) {
-            if (k + 1 < blocks) q4k_quarter_load(nxt, wrow, k + 1, q);
+            q4k_quarter_load(nxt, wrow, min(k + 1, blocks - 1), q);  // unconditional: see the wide path
             q4k_quarter_pin(cur);
             fill(std::integral_constant<int, 0>{}, cur, 4 * k);
             q4k_quarter_pin(cur);
@@ -566,16 +595,17 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
             step_origin<MODE>(p, u, seg_k, kc0);
             const int wrow = min(kc0 + lane, p.n - 1);  // rows past the end meet the zero-filled tail of the A tile
             const uint8_t* blk = p.w[seg_k] + c.expert * p.w_expert_bytes + (int64_t)wrow * p.w_row_bytes + blk_off;
-            r.hdr = *(const u32x4_t*)blk;
-            r.q = *(const u32x4_t*)(blk + q_off);
+            load16_untracked(r.hdr, blk);
+            load16_untracked(r.q, blk + q_off);
         };
         bf16_t* const dst0 = c.bs + lane * kNnPitch + run_w * 32 + half * 16;
         auto fill = [&](Q4KHalfRun& r, int u) __attribute__((always_inline)) {
             open_phase(u);
+            wait_loads_at_most(2);  // the other set's two loads may still be on their way
             q4k_half_run_pin(r);
             uint32_t wv[8];
             q4k_half_run_decode(r, j, wv);
-            if (u + 2 < steps) issue(r, u + 2);
+            issue(r, min(u + 2, steps - 1));  // always two loads: the count above stays exact
             bf16_t* dst = dst0 + buf * kBTile;
             *(uint4*)dst = make_uint4(wv[0], wv[1], wv[2], wv[3]);
             *(uint4*)(dst + 8) = make_uint4(wv[4], wv[5], wv[6], wv[7]);
@@ -583,7 +613,7 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
         };
         Q4KHalfRun ra, rb;  // even / odd steps, each reloaded two steps ahead
         issue(ra, 0);
-        if (steps > 1) issue(rb, 1);
+        issue(rb, min(1, steps - 1));
         after_issue();
         for (int u = 0; u < steps; u += 2) {
             fill(ra, u);
@@ -718,10 +748,17 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
         Operands x, y;
         load_operands(x, stage, buf, 0);
         for (int t = 0; t < steps; t++) {  // the A loads issued in here are those of step t + kAhead
+            // (a ring of two stages has one step of lead: all of the next step's groups go out at once)
+            if (kAhead == 1) a_issue_part<MODE, 1, kGroupsPerWave>(ai, p, c);
             GGQ_STAGE(y, x, 1, 0);
-            GGQ_STAGE(x, y, 2, 1);
-            GGQ_STAGE(y, x, 3, 2);
-            a_issue_part<MODE, 3, 4>(ai, p, c);
+            if (kAhead > 1) {
+                GGQ_STAGE(x, y, 2, 1);
+                GGQ_STAGE(y, x, 3, 2);
+                a_issue_part<MODE, 3, 4>(ai, p, c);
+            } else {
+                GGQ_STAGE(x, y, 2, kGroupsPerWave);
+                GGQ_STAGE(y, x, 3, kGroupsPerWave);
+            }
             a_issue_advance(ai);
             a_wait_step(ai, c, t + 1);
             lds_barrier();  // every LDS read of this step has landed; its stage and buffer may be refilled
@@ -896,7 +933,7 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
     auto lora_tiles = [&]() __attribute__((always_inline)) {
         if (p.r_pad > 0) {
             const int chunks = p.r_pad >> 3;  // 16-byte chunks per row (r_pad % 16 == 0)
-            for (int id = tid; id < kTM * 8; id += kThreads) {
+            for (int id = tid; id < kTM * 8; id += kThreadsWG) {
                 const int r = id >> 3, ch = id & 7;
                 uint4 v = zero4();
                 if (r < c.rows_valid && ch < chunks) v = *(const uint4*)(p.la + (int64_t)(c.row_begin + r) * p.r_pad + ch * 8);
@@ -905,7 +942,7 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
             if (MODE == kModeNT) {
                 // forward: the factor B is [columns][r_pad], the layout of the forward W tile
                 const bf16_t* lb = p.lb + c.expert * p.lb_expert_elems + (int64_t)(c.seg_c * c.out_cols + c.col0) * p.r_pad;
-                for (int id = tid; id < kTN * 8; id += kThreads) {
+                for (int id = tid; id < kTN * 8; id += kThreadsWG) {
                     const int cidx = id >> 3, ch = id & 7;
                     uint4 v = zero4();
                     if (c.col0 + cidx < c.out_cols && ch < chunks) v = *(const uint4*)(lb + (int64_t)cidx * p.r_pad + ch * 8);
@@ -916,7 +953,7 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
                 // ([contraction row][column]); rows r .. r_pad - 1 are zero
                 const bf16_t* lb = p.lb + c.expert * p.lb_expert_elems + c.col0;
                 const bool vec = (c.out_cols & 7) == 0;
-                for (int id = tid; id < p.r_pad * (kTN / 8); id += kThreads) {
+                for (int id = tid; id < p.r_pad * (kTN / 8); id += kThreadsWG) {
                     const int j = id / (kTN / 8), ch = id - j * (kTN / 8);
                     const int col = c.col0 + ch * 8;
                     uint4 v = zero4();
@@ -931,8 +968,8 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
         __syncthreads();  // LoRA tiles and the codebook are visible
     };
 
-    if (wave >= 8) {
-        if (QT == kQ4_K) produce_q4k<MODE>(p, c, tid - 512, wave - 8, lora_tiles);
+    if (wave >= kCW) {
+        if (QT == kQ4_K) produce_q4k<MODE>(p, c, tid - kProducerLanes, wave - kCW, lora_tiles);
         else if (wave < 12) produce<QT, MODE, 0>(p, c, tid & 255, wave & 3, lora_tiles);
         else produce<QT, MODE, 1>(p, c, tid & 255, wave & 3, lora_tiles);
     } else {
@@ -952,6 +989,12 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
 template <int QT, int MODE, int EPI, int SH>
 __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(4, 4))) void mmq_tile_kernel(const MmqParams p) {
     Tile<SH>::template run<QT, MODE, EPI>(p);
+}
+
+// The half shape: eight waves, two workgroups to a compute unit.
+template <int QT, int MODE, int EPI>
+__global__ __launch_bounds__(512, 2) __attribute__((amdgpu_waves_per_eu(4, 4))) void mmq_half_kernel(const MmqParams p) {
+    Tile<kShapeHalf>::template run<QT, MODE, EPI>(p);
 }
 
 // Grouped launch with both shapes in one grid: wide tiles for the row tiles of table `tiles`, tall tiles
