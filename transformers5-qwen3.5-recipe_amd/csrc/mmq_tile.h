@@ -112,6 +112,14 @@ static constexpr int kGroupsPerWave = kAGroups / kCW;   // groups one consumer w
 // W buffer: forward [output column][64 + 8]; grad-input [contraction row][columns + 32], as the rows are
 // decoded (the consumers transpose on the way out of LDS).  Sized for the larger of the two.
 static constexpr int kNnPitch = kTN + 32;
+// Position of 16-byte chunk q of contraction row `row` in the grad-input W tile: the two low bits of q are
+// XOR-ed with a row-dependent value so that the lanes of one 16-byte store instruction (which differ in
+// row and run, and would otherwise meet four deep on the same banks) hit distinct banks, while the four
+// rows of a transposing read keep their 32-byte pieces on distinct banks.
+static __device__ __forceinline__ int nn_chunk(int row, int q) {
+    const int sw = SH == 0 ? (((row >> 2) & 3) ^ (row & 1)) : SH == 1 ? ((row & 1) ^ (((q >> 4) & 1) << 1)) : (row & 3);
+    return q ^ sw;
+}
 static constexpr int kBTile = kTN * kLdsStride > kBK * kNnPitch ? kTN * kLdsStride : kBK * kNnPitch;  // bf16 elements
 static constexpr int kTileLdsBytes = kAStages * kAStageBytes + 2 * kBTile * 2;
 
@@ -223,9 +231,9 @@ static __device__ __forceinline__ void w_store_run(const TileCtx& c, const Produ
         for (int i = 0; i < 4; i++) *(uint4*)(dst + 8 * i) = make_uint4(wv[4 * i], wv[4 * i + 1], wv[4 * i + 2], wv[4 * i + 3]);
     } else {
         // grad-input: this lane's contraction row, columns 32*pw .. +31, stored as decoded
-        bf16_t* dst = &bt[l.lane * kNnPitch + l.pw * 32];
+        bf16_t* dst = &bt[l.lane * kNnPitch];
 #pragma unroll
-        for (int i = 0; i < 4; i++) *(uint4*)(dst + 8 * i) = make_uint4(wv[4 * i], wv[4 * i + 1], wv[4 * i + 2], wv[4 * i + 3]);
+        for (int i = 0; i < 4; i++) *(uint4*)(dst + 8 * nn_chunk(l.lane, l.pw * 4 + i)) = make_uint4(wv[4 * i], wv[4 * i + 1], wv[4 * i + 2], wv[4 * i + 3]);
     }
 }
 
@@ -333,7 +341,7 @@ static __device__ __forceinline__ void produce(const MmqParams& p, const TileCtx
             Fmt<QT>::pin(raw);
             Fmt<QT>::decode(raw, MODE == kModeNT ? 2 * u + (l.ptid & 1) : l.w_ksub_nn, wv, c.grid);
             pin_decoded();
-            if (u + 4 < steps) w_issue_run<QT, MODE>(p, c, l, u + 4, raw);
+            w_issue_run<QT, MODE>(p, c, l, u + 4 < steps ? u + 4 : u, raw);  // unconditional (a load under a branch is drained at the join)
         };
         if (Q < steps) w_issue_run<QT, MODE>(p, c, l, Q, raw_a);
         if (Q + 2 < steps) w_issue_run<QT, MODE>(p, c, l, Q + 2, raw_b);
@@ -525,7 +533,7 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
             load16_untracked(r.q0, blk + q_off);
             load16_untracked(r.q1, blk + q_off + 16);
         };
-        bf16_t* const dst0 = c.bs + lane * kNnPitch + run * 32;
+        bf16_t* const dst0 = c.bs + lane * kNnPitch;
         auto fill = [&](Raw& r, int u) __attribute__((always_inline)) {
             open_phase(u);
             wait_loads_at_most(3);  // the other set's three loads may still be on their way
@@ -537,7 +545,7 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
             issue(r, min(u + 2, steps - 1));  // always three loads: the count above stays exact
             bf16_t* dst = dst0 + buf * kBTile;
 #pragma unroll
-            for (int i = 0; i < 4; i++) *(uint4*)(dst + 8 * i) = make_uint4(wv[4 * i], wv[4 * i + 1], wv[4 * i + 2], wv[4 * i + 3]);
+            for (int i = 0; i < 4; i++) *(uint4*)(dst + 8 * nn_chunk(lane, run * 4 + i)) = make_uint4(wv[4 * i], wv[4 * i + 1], wv[4 * i + 2], wv[4 * i + 3]);
             close_phase();
         };
         Raw ra, rb;  // even / odd steps, each reloaded two steps ahead
@@ -598,7 +606,7 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
             load16_untracked(r.hdr, blk);
             load16_untracked(r.q, blk + q_off);
         };
-        bf16_t* const dst0 = c.bs + lane * kNnPitch + run_w * 32 + half * 16;
+        bf16_t* const dst0 = c.bs + lane * kNnPitch;
         auto fill = [&](Q4KHalfRun& r, int u) __attribute__((always_inline)) {
             open_phase(u);
             wait_loads_at_most(2);  // the other set's two loads may still be on their way
@@ -607,8 +615,8 @@ static __device__ __forceinline__ void produce_q4k(const MmqParams& p, const Til
             q4k_half_run_decode(r, j, wv);
             issue(r, min(u + 2, steps - 1));  // always two loads: the count above stays exact
             bf16_t* dst = dst0 + buf * kBTile;
-            *(uint4*)dst = make_uint4(wv[0], wv[1], wv[2], wv[3]);
-            *(uint4*)(dst + 8) = make_uint4(wv[4], wv[5], wv[6], wv[7]);
+            *(uint4*)(dst + 8 * nn_chunk(lane, run_w * 4 + half * 2)) = make_uint4(wv[0], wv[1], wv[2], wv[3]);
+            *(uint4*)(dst + 8 * nn_chunk(lane, run_w * 4 + half * 2 + 1)) = make_uint4(wv[4], wv[5], wv[6], wv[7]);
             close_phase();
         };
         Q4KHalfRun ra, rb;  // even / odd steps, each reloaded two steps ahead
@@ -646,7 +654,16 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
     // columns 4 (s % 4) .. +3 of its group's 16 columns; groups 0, 1 take columns 0..15 / 16..31 of the
     // block, groups 2, 3 the same columns eight contraction rows further on.
     const int tr_group = lane >> 4, tr_s = lane & 15;
-    const int tr_off = (8 * (tr_group >> 1) + (tr_s >> 2)) * kNnPitch + wave_n * 64 + 16 * (tr_group & 1) + 4 * (tr_s & 3);
+    // (the 16-byte chunk that holds them sits at its swizzled position, nn_chunk; the row's low bits do not
+    // depend on the sub-step, 16 rows on)
+    const int tr_row = 8 * (tr_group >> 1) + (tr_s >> 2);
+    int tr_lo[kColBlocks], tr_hi[kColBlocks];
+#pragma unroll
+    for (int cb = 0; cb < kColBlocks; cb++) {
+        const int col = wave_n * 64 + cb * 32 + 16 * (tr_group & 1) + 4 * (tr_s & 3);
+        tr_lo[cb] = tr_row * kNnPitch + nn_chunk(tr_row, col >> 3) * 8 + (col & 7);
+        tr_hi[cb] = (tr_row + 4) * kNnPitch + nn_chunk(tr_row + 4, col >> 3) * 8 + (col & 7);
+    }
 
     // Operands of one sub-step (16 of the contraction): LIVE row-block runs of A, two column-block runs of W.
     struct Operands {
@@ -658,11 +675,11 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
         if (MODE == kModeNN) {
             // W tile is [contraction row][output column]: each transposing 8-byte read hands this lane
             // four consecutive contraction values of its column, two reads make the MFMA operand
-            const bf16_t* t_lds = c.bs + buf * kBTile + tr_off + kk * 16 * kNnPitch;
+            const bf16_t* t_lds = c.bs + buf * kBTile + kk * 16 * kNnPitch;
 #pragma unroll
             for (int cb = 0; cb < kColBlocks; cb++) {
-                const v4i16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(t_lds + cb * 32));
-                const v4i16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(t_lds + cb * 32 + 4 * kNnPitch));
+                const v4i16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(t_lds + tr_lo[cb]));
+                const v4i16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(t_lds + tr_hi[cb]));
                 o.b[cb] = __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
             }
         } else {
@@ -961,7 +978,7 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
                         const bf16_t* src = lb + (int64_t)j * c.out_cols + ch * 8;
                         v = vec && col + 8 <= c.out_cols ? *(const uint4*)src : load8_slow(src, c.out_cols - col);
                     }
-                    *(uint4*)&c.bs[j * kNnPitch + ch * 8] = v;
+                    *(uint4*)&c.bs[j * kNnPitch + nn_chunk(j, ch) * 8] = v;
                 }
             }
         }
