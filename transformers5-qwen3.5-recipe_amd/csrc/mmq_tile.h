@@ -310,10 +310,14 @@ static __device__ __forceinline__ void q4k_chunk_store(const TileCtx& c, const P
 template <int QT, int MODE, int Q, class AfterIssue>
 static __device__ __forceinline__ void produce(const MmqParams& p, const TileCtx& c, int ptid, int pw, AfterIssue&& after_issue) {
     ProducerLane l;
-    l.ptid = ptid, l.pw = pw, l.lane = ptid & 63;
+    l.ptid = ptid;
     // W run owned by this lane: NT -> (output column n = col0 + ptid/2, run 2*step + ptid%2);
-    //                           NN -> (contraction row n = kc0 + lane, run col0/32 + wave of the quartet).
-    l.w_ksub_nn = min((c.col0 >> 5) + pw, (p.k >> 5) - 1);
+    //                           NN -> (contraction row n = kc0 + l.lane, run col0/32 + l.pw): a quartet wave takes
+    //                           16 rows, the four lanes of a row the four runs, so that they read adjacent bytes
+    //                           of the row's block (a lane-per-row split costs one cache access per lane).
+    l.lane = MODE == kModeNN ? 16 * pw + ((ptid & 63) >> 2) : (ptid & 63);
+    l.pw = MODE == kModeNN ? (ptid & 3) : pw;
+    l.w_ksub_nn = min((c.col0 >> 5) + l.pw, (p.k >> 5) - 1);
     l.w_row_nt = min(c.col0 + (ptid >> 1), p.n - 1);
     const int steps = c.total_steps;
     uint32_t wv[16];
