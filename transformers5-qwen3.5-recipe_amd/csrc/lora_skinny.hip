@@ -270,8 +270,11 @@ __global__ __launch_bounds__(256) void skinny_nt_direct_kernel(SkinnyNtParams p)
 // Experts without rows get zeros.
 template <int JB>
 __global__ __launch_bounds__(256) void factor_grad_kernel(FactorGradParams p) {
-    __shared__ bf16_t in_t[2][32][64 + 2];
-    __shared__ bf16_t s_t[2][32][JB * 16 + 2];
+    // rows are contraction rows m; the operands are read with transposing 8-byte LDS reads (lane L of a
+    // 16-lane group gets element L % 4 of the 8 bytes addressed by lanes L / 4 + 4 t), so the tiles stay as
+    // loaded; the row pitches keep four consecutive rows' 32-byte pieces on distinct banks
+    __shared__ __attribute__((aligned(16))) bf16_t in_t[2][32][64 + 32];
+    __shared__ __attribute__((aligned(16))) bf16_t s_t[2][32][JB * 16 + 8];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int blocks_per_seg = (p.c + 63) / 64;
     const int col_blocks = p.nseg * blocks_per_seg;
@@ -310,28 +313,23 @@ __global__ __launch_bounds__(256) void factor_grad_kernel(FactorGradParams p) {
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             if (m0 + 32 * u >= row_end) break;  // uniform over the workgroup
-            uint32_t* d = (uint32_t*)&in_t[buf][tr][tch * 8];
-            d[0] = vin[u].x, d[1] = vin[u].y, d[2] = vin[u].z, d[3] = vin[u].w;
-            if (sr < 32) {
-                uint32_t* ds = (uint32_t*)&s_t[buf][sr][sch * 8];
-                ds[0] = vs[u].x, ds[1] = vs[u].y, ds[2] = vs[u].z, ds[3] = vs[u].w;
-            }
+            *(uint4*)&in_t[buf][tr][tch * 8] = vin[u];
+            if (sr < 32) *(uint4*)&s_t[buf][sr][sch * 8] = vs[u];
             // one barrier per slice: the slice after the next reuses this buffer, and every wave passes the
             // next barrier only after its reads of this one
             __syncthreads();
-            // A operand: row = column c (wave*16 + li), contraction m = 8*lq .. 8*lq+7
-            uint32_t aw[4];
-#pragma unroll
-            for (int h = 0; h < 4; h++)
-                aw[h] = (uint32_t)in_t[buf][8 * lq + 2 * h][wave * 16 + li] | ((uint32_t)in_t[buf][8 * lq + 2 * h + 1][wave * 16 + li] << 16);
-            const bf16x8_t a = __builtin_bit_cast(bf16x8_t, make_uint4(aw[0], aw[1], aw[2], aw[3]));
+            // A operand: row = column c (wave*16 + li), contraction m = 8*lq .. 8*lq+7; source lane s = li
+            // points at contraction row 8*lq + s/4 (+4 for the second read), columns 4*(s%4) .. +3 of the wave's 16
+            const bf16_t* a_src = &in_t[buf][8 * lq + (li >> 2)][wave * 16 + (li & 3) * 4];
+            const v4i16_t a_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)a_src);
+            const v4i16_t a_hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(a_src + 4 * (64 + 32)));
+            const bf16x8_t a = __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7));
 #pragma unroll
             for (int jb = 0; jb < JB; jb++) {
-                uint32_t bw[4];
-#pragma unroll
-                for (int h = 0; h < 4; h++)
-                    bw[h] = (uint32_t)s_t[buf][8 * lq + 2 * h][jb * 16 + li] | ((uint32_t)s_t[buf][8 * lq + 2 * h + 1][jb * 16 + li] << 16);
-                acc[jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8_t, make_uint4(bw[0], bw[1], bw[2], bw[3])), acc[jb], 0, 0, 0);
+                const bf16_t* b_src = &s_t[buf][8 * lq + (li >> 2)][jb * 16 + (li & 3) * 4];
+                const v4i16_t b_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)b_src);
+                const v4i16_t b_hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(b_src + 4 * (JB * 16 + 8)));
+                acc[jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7)), acc[jb], 0, 0, 0);
             }
             buf ^= 1;
         }
