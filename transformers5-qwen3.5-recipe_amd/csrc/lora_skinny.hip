@@ -264,19 +264,21 @@ __global__ __launch_bounds__(256) void skinny_nt_direct_kernel(SkinnyNtParams p)
 }
 
 // ---- G[e][c, j] = s * sum_m In[m, c] * S[m, j] over the rows of expert e.  One workgroup per
-// (expert, 64 columns); each wave owns 16 columns; rows are consumed 32 at a time through LDS so the
-// strided operands of the contraction over m become LDS gathers.  The loads of four 32-row slices are
-// issued together and the slices then go through two alternating LDS buffers, one barrier each.
-// Experts without rows get zeros.
-template <int JB>
+// (expert, 64 * CB columns); each wave owns CB blocks of 16 columns; rows are consumed 32 at a time
+// through LDS, where the operands of the contraction over m are read with transposing loads.  The loads
+// of four 32-row slices are issued together and the slices then go through two alternating LDS buffers,
+// one barrier each.  Experts without rows get zeros.
+template <int JB, int CB>
 __global__ __launch_bounds__(256) void factor_grad_kernel(FactorGradParams p) {
     // rows are contraction rows m; the operands are read with transposing 8-byte LDS reads (lane L of a
     // 16-lane group gets element L % 4 of the 8 bytes addressed by lanes L / 4 + 4 t), so the tiles stay as
     // loaded; the row pitches keep four consecutive rows' 32-byte pieces on distinct banks
-    __shared__ __attribute__((aligned(16))) bf16_t in_t[2][32][64 + 32];
-    __shared__ __attribute__((aligned(16))) bf16_t s_t[2][32][JB * 16 + 8];
+    constexpr int kCols = 64 * CB, kPitch = kCols + 32, kSPitch = JB * 16 + 8;
+    __shared__ __attribute__((aligned(16))) bf16_t in_t[2][32][kPitch];
+    __shared__ __attribute__((aligned(16))) bf16_t s_t[2][32][kSPitch];
+    __shared__ __attribute__((aligned(16))) bf16_t g_t[4][16][JB * 16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int blocks_per_seg = (p.c + 63) / 64;
+    const int blocks_per_seg = (p.c + kCols - 1) / kCols;
     const int col_blocks = p.nseg * blocks_per_seg;
     // contiguous runs of (expert, column block) units per XCD: one L2 sees whole rows of an expert
     const int per_xcd = ((int)gridDim.x + 7) >> 3;
@@ -284,7 +286,7 @@ __global__ __launch_bounds__(256) void factor_grad_kernel(FactorGradParams p) {
     if ((int)(blockIdx.x >> 3) >= per_xcd || unit >= p.units) return;
     const int e = unit / col_blocks, cblk = unit - e * col_blocks;
     const int seg = cblk / blocks_per_seg;
-    const int c0 = (cblk - seg * blocks_per_seg) * 64;
+    const int c0 = (cblk - seg * blocks_per_seg) * kCols;
     int row_begin = 0, row_end = p.m;
     if (p.ranges) {
         row_begin = p.ranges[2 * e];
@@ -293,94 +295,107 @@ __global__ __launch_bounds__(256) void factor_grad_kernel(FactorGradParams p) {
     const bf16_t* in = p.in[seg];
     const bool vec = ((p.ld_in & 7) == 0) && (((uintptr_t)in & 15) == 0);
     const int li = lane & 15, lq = lane >> 4;
-    f32x4_t acc[JB];
+    f32x4_t acc[CB][JB];
 #pragma unroll
-    for (int jb = 0; jb < JB; jb++) acc[jb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+        for (int jb = 0; jb < JB; jb++) acc[cb][jb] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     constexpr int rp = JB * 16;
-    const int tr = threadIdx.x >> 3, tch = threadIdx.x & 7;           // In slice: 32 rows x 8 chunks of 8
+    const int tr = threadIdx.x >> 3, tch = threadIdx.x & 7;           // In slice: 32 rows x CB x 8 chunks of 8
     const int sr = threadIdx.x / (rp / 8), sch = threadIdx.x % (rp / 8);  // S slice: 32 rows x rp/8 chunks
-    const int tcc = c0 + tch * 8;
     int buf = 0;
     for (int m0 = row_begin; m0 < row_end; m0 += 128) {
-        uint4 vin[4], vs[4];
+        uint4 vin[4][CB], vs[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             const int r = m0 + 32 * u + tr;
-            vin[u] = load8g(in + (int64_t)r * p.ld_in + tcc, r < row_end ? p.c - tcc : 0, vec);
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++) {
+                const int tcc = c0 + cb * 64 + tch * 8;
+                vin[u][cb] = load8g(in + (int64_t)r * p.ld_in + tcc, r < row_end ? p.c - tcc : 0, vec);
+            }
             vs[u] = make_uint4(0, 0, 0, 0);
             if (sr < 32 && m0 + 32 * u + sr < row_end) vs[u] = *(const uint4*)(p.s + (int64_t)(m0 + 32 * u + sr) * rp + sch * 8);
         }
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             if (m0 + 32 * u >= row_end) break;  // uniform over the workgroup
-            *(uint4*)&in_t[buf][tr][tch * 8] = vin[u];
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++) *(uint4*)&in_t[buf][tr][cb * 64 + tch * 8] = vin[u][cb];
             if (sr < 32) *(uint4*)&s_t[buf][sr][sch * 8] = vs[u];
             // one barrier per slice: the slice after the next reuses this buffer, and every wave passes the
             // next barrier only after its reads of this one
             __syncthreads();
-            // A operand: row = column c (wave*16 + li), contraction m = 8*lq .. 8*lq+7; source lane s = li
-            // points at contraction row 8*lq + s/4 (+4 for the second read), columns 4*(s%4) .. +3 of the wave's 16
-            const bf16_t* a_src = &in_t[buf][8 * lq + (li >> 2)][wave * 16 + (li & 3) * 4];
-            const v4i16_t a_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)a_src);
-            const v4i16_t a_hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(a_src + 4 * (64 + 32)));
-            const bf16x8_t a = __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            // B operand (n = factor column j, contraction m): source lane s = li points at contraction row
+            // 8*lq + s/4 (+4 for the second read), factor columns 4*(s%4) .. +3 of the block's 16
+            bf16x8_t b[JB];
 #pragma unroll
             for (int jb = 0; jb < JB; jb++) {
                 const bf16_t* b_src = &s_t[buf][8 * lq + (li >> 2)][jb * 16 + (li & 3) * 4];
                 const v4i16_t b_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)b_src);
-                const v4i16_t b_hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(b_src + 4 * (JB * 16 + 8)));
-                acc[jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7)), acc[jb], 0, 0, 0);
+                const v4i16_t b_hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(b_src + 4 * kSPitch));
+                b[jb] = __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            }
+            // A operand (row = column c, contraction m): the same pattern over the wave's 16 columns of block cb
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++) {
+                const bf16_t* a_src = &in_t[buf][8 * lq + (li >> 2)][cb * 64 + wave * 16 + (li & 3) * 4];
+                const v4i16_t a_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)a_src);
+                const v4i16_t a_hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(a_src + 4 * kPitch));
+                const bf16x8_t a = __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7));
+#pragma unroll
+                for (int jb = 0; jb < JB; jb++) acc[cb][jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[jb], acc[cb][jb], 0, 0, 0);
             }
             buf ^= 1;
         }
     }
-    // acc[jb][v]: c = c0 + wave*16 + 4*lq + v, j = 16*jb + li
+    // acc[cb][jb][v]: c = c0 + 64*cb + wave*16 + 4*lq + v, j = 16*jb + li
     bf16_t* out = p.out + (int64_t)e * p.out_expert_elems;
     const int64_t ctot = (int64_t)p.nseg * p.c;
-    const int cw0 = c0 + wave * 16;  // first column of this wave
-    if (p.out_j_major) {
-        // [r][columns]: a lane holds four consecutive columns of factor row j: one 8-byte store
-        const bool vec4 = (ctot & 3) == 0 && (((uintptr_t)out & 7) == 0);
-#pragma unroll
-        for (int jb = 0; jb < JB; jb++) {
-            const int j = jb * 16 + li, c = cw0 + 4 * lq;
-            if (j >= p.r) continue;
-            bf16_t* dst = out + (int64_t)j * ctot + (int64_t)seg * p.c + c;
-            if (vec4 && c + 3 < p.c) {
-                *(uint2*)dst = make_uint2(pack_bf16(acc[jb][0] * p.scale, acc[jb][1] * p.scale), pack_bf16(acc[jb][2] * p.scale, acc[jb][3] * p.scale));
-            } else {
-#pragma unroll
-                for (int v = 0; v < 4; v++)
-                    if (c + v < p.c) dst[v] = to_bf16(acc[jb][v] * p.scale);
-            }
-        }
-        return;
-    }
-    // [columns][r]: the wave's 16 columns x r are one contiguous run; transpose through LDS (each wave
-    // reads back only what it wrote) and store 16 bytes per lane
-    __shared__ __attribute__((aligned(16))) bf16_t g_t[4][16][JB * 16];
+    const bool vec4 = (ctot & 3) == 0 && (((uintptr_t)out & 7) == 0);
     const bool vec8 = (p.r & 7) == 0 && (((uintptr_t)out & 15) == 0);
-    if (vec8) {
 #pragma unroll
-        for (int jb = 0; jb < JB; jb++)
+    for (int cb = 0; cb < CB; cb++) {
+        const int cw0 = c0 + 64 * cb + wave * 16;  // first column of this wave's block
+        if (p.out_j_major) {
+            // [r][columns]: a lane holds four consecutive columns of factor row j: one 8-byte store
 #pragma unroll
-            for (int v = 0; v < 4; v++) g_t[wave][4 * lq + v][jb * 16 + li] = to_bf16(acc[jb][v] * p.scale);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        const int chunks_per_row = p.r >> 3;
-        bf16_t* dst = out + ((int64_t)seg * p.c + cw0) * p.r;
-        for (int id = lane; id < 16 * chunks_per_row; id += 64) {
-            const int row = id / chunks_per_row, ch = id - row * chunks_per_row;
-            if (cw0 + row < p.c) *(uint4*)(dst + (int64_t)id * 8) = *(const uint4*)&g_t[wave][row][ch * 8];
+            for (int jb = 0; jb < JB; jb++) {
+                const int j = jb * 16 + li, c = cw0 + 4 * lq;
+                if (j >= p.r) continue;
+                bf16_t* dst = out + (int64_t)j * ctot + (int64_t)seg * p.c + c;
+                if (vec4 && c + 3 < p.c) {
+                    *(uint2*)dst = make_uint2(pack_bf16(acc[cb][jb][0] * p.scale, acc[cb][jb][1] * p.scale), pack_bf16(acc[cb][jb][2] * p.scale, acc[cb][jb][3] * p.scale));
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                        if (c + v < p.c) dst[v] = to_bf16(acc[cb][jb][v] * p.scale);
+                }
+            }
+        } else if (vec8) {
+            // [columns][r]: the wave's 16 columns x r are one contiguous run; transpose through LDS (each wave
+            // reads back only what it wrote; LDS serves a wave in order) and store 16 bytes per lane
+#pragma unroll
+            for (int jb = 0; jb < JB; jb++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) g_t[wave][4 * lq + v][jb * 16 + li] = to_bf16(acc[cb][jb][v] * p.scale);
+            const int chunks_per_row = p.r >> 3;
+            bf16_t* dst = out + ((int64_t)seg * p.c + cw0) * p.r;
+            for (int id = lane; id < 16 * chunks_per_row; id += 64) {
+                const int row = id / chunks_per_row, ch = id - row * chunks_per_row;
+                const uint4 piece = *(const uint4*)&g_t[wave][row][ch * 8];
+                if (cw0 + row < p.c) *(uint4*)(dst + (int64_t)id * 8) = piece;
+            }
+        } else {
+#pragma unroll
+            for (int jb = 0; jb < JB; jb++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const int c = cw0 + 4 * lq + v, j = jb * 16 + li;
+                    if (c < p.c && j < p.r) out[((int64_t)seg * p.c + c) * p.r + j] = to_bf16(acc[cb][jb][v] * p.scale);
+                }
         }
-        return;
     }
-#pragma unroll
-    for (int jb = 0; jb < JB; jb++)
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-            const int c = cw0 + 4 * lq + v, j = jb * 16 + li;
-            if (c < p.c && j < p.r) out[((int64_t)seg * p.c + c) * p.r + j] = to_bf16(acc[jb][v] * p.scale);
-        }
 }
 
 // dst[e][c][0..r_pad) = src[e][c][0..r) zero padded   (transpose = false, src [E][C][r])
@@ -504,8 +519,9 @@ int skinny_nt(const SkinnyNtParams& p, int r_pad, int grid_tiles, hipStream_t s)
     return check_launch("skinny_nt");
 }
 
-int factor_grad(const FactorGradParams& p_in, int r_pad, int64_t experts, hipStream_t s) {
-    const int col_blocks = p_in.nseg * ((p_in.c + 63) / 64);
+template <int CB>
+static int launch_factor_grad(const FactorGradParams& p_in, int r_pad, int64_t experts, hipStream_t s) {
+    const int col_blocks = p_in.nseg * ((p_in.c + 64 * CB - 1) / (64 * CB));
     const int64_t units = experts * col_blocks;
     if (units <= 0) return 0;
     if (units > 0x7FFFFFF0) return set_error(GGQ_ERR_SHAPE, "factor_grad: grid too large");
@@ -513,13 +529,18 @@ int factor_grad(const FactorGradParams& p_in, int r_pad, int64_t experts, hipStr
     FactorGradParams p = p_in;
     p.units = (int)units;
     switch (r_pad / 16) {
-        case 1: hipLaunchKernelGGL(factor_grad_kernel<1>, dim3((unsigned)grid), dim3(256), 0, s, p); break;
-        case 2: hipLaunchKernelGGL(factor_grad_kernel<2>, dim3((unsigned)grid), dim3(256), 0, s, p); break;
-        case 3: hipLaunchKernelGGL(factor_grad_kernel<3>, dim3((unsigned)grid), dim3(256), 0, s, p); break;
-        case 4: hipLaunchKernelGGL(factor_grad_kernel<4>, dim3((unsigned)grid), dim3(256), 0, s, p); break;
+        case 1: hipLaunchKernelGGL((factor_grad_kernel<1, CB>), dim3((unsigned)grid), dim3(256), 0, s, p); break;
+        case 2: hipLaunchKernelGGL((factor_grad_kernel<2, CB>), dim3((unsigned)grid), dim3(256), 0, s, p); break;
+        case 3: hipLaunchKernelGGL((factor_grad_kernel<3, CB>), dim3((unsigned)grid), dim3(256), 0, s, p); break;
+        case 4: hipLaunchKernelGGL((factor_grad_kernel<4, CB>), dim3((unsigned)grid), dim3(256), 0, s, p); break;
         default: return set_error(GGQ_ERR_SHAPE, "LoRA rank must be between 1 and 64");
     }
     return check_launch("factor_grad");
+}
+
+int factor_grad(const FactorGradParams& p, int r_pad, int64_t experts, hipStream_t s) {
+    // wide column blocks (256 contiguous bytes per row and workgroup) when they divide the segment
+    return p.c % 128 == 0 ? launch_factor_grad<2>(p, r_pad, experts, s) : launch_factor_grad<1>(p, r_pad, experts, s);
 }
 
 }  // namespace ggq
