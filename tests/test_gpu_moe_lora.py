@@ -79,9 +79,12 @@ def test_constant_byte_iq2_xxs_experts(pkg, dev):
     torch.testing.assert_close(h.grad.double().cpu(), want["dx"], rtol=1e-2, atol=1e-2)
 
 
-@pytest.mark.parametrize("qt,r", [(gb.Q4_K, 16), (gb.Q8_0, 4), (gb.Q6_K, 8), (gb.IQ2_XXS, 16)])
-def test_grouped_lora_projection_all_gradients(pkg, dev, qt, r):
-    # ragged groups including empty experts, a group larger than one 128-row tile, and inactive planes
+@pytest.mark.parametrize("qt,r,shape", [(gb.Q4_K, 16, ""), (gb.Q4_K, 16, "2"), (gb.Q8_0, 4, ""), (gb.Q6_K, 8, ""), (gb.IQ2_XXS, 16, "")])
+def test_grouped_lora_projection_all_gradients(pkg, dev, qt, r, shape, monkeypatch):
+    # ragged groups including empty experts, a group larger than one 128-row tile, and inactive planes;
+    # shape "2": the same through the library's alternative 128 x 128 tiles (two workgroups per compute unit)
+    if shape:
+        monkeypatch.setenv("GGQ_GROUPED_SHAPE", shape)
     ml = pkg.fast_moe_lora
     e_total, n, k = 8, 192, 512
     sizes = [0, 150, 3, 0, 129, 1, 64, 0]

@@ -78,11 +78,8 @@ static int launch_wide_and_tall(int qt, int mode, MmqParams& p, int rows, int n,
 // Expert groups that average at most 192 rows run the Q4_K tile kernel in its wide shape.
 static int pick_shape(int qt, int64_t rows, int64_t groups) {
     if (!(qt == 12 /* GGML Q4_K */ && groups > 0 && rows <= 192 * groups)) return kShapeTall;
-    static const int forced = [] {
-        const char* e = getenv("GGQ_GROUPED_SHAPE");  // tuning aid: 1 = wide + tall mixed launch, 2 = half tiles
-        return e ? atoi(e) : -1;
-    }();
-    return forced == kShapeHalf ? kShapeHalf : kShapeWide;
+    const char* e = getenv("GGQ_GROUPED_SHAPE");  // tuning aid, read per call: 2 = half tiles, otherwise the mixed launch
+    return e && atoi(e) == kShapeHalf ? kShapeHalf : kShapeWide;
 }
 
 int64_t ggq_lora_workspace_bytes(int64_t rows, int64_t groups, int64_t experts, int64_t n_total, int64_t k, int r) {
