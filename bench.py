@@ -131,7 +131,7 @@ def main() -> None:
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (every box here has one MI355X); run with --gpus 1")
     if not torch.cuda.is_available():
-        sys.exit("bench.py needs a GPU (run it through gpurun)")
+        sys.exit("bench.py needs a GPU")
     pkg = __graft_entry__.import_package()
     lib = pkg._lib.load()
     dev = torch.device("cuda:0")
