@@ -75,11 +75,17 @@ static int launch_wide_and_tall(int qt, int mode, MmqParams& p, int rows, int n,
     return launch_mmq_mixed(mode, p, s);
 }
 
-// Expert groups that average at most 192 rows run the Q4_K tile kernel in its wide shape.
-static int pick_shape(int qt, int64_t rows, int64_t groups) {
-    if (!(qt == 12 /* GGML Q4_K */ && groups > 0 && rows <= 192 * groups)) return kShapeTall;
-    const char* e = getenv("GGQ_GROUPED_SHAPE");  // tuning aid, read per call: 2 = half tiles, otherwise the mixed launch
-    return e && atoi(e) == kShapeHalf ? kShapeHalf : kShapeWide;
+// Q4_K forward over expert groups that average at most 256 rows runs the direct kernel when `direct_ok`;
+// otherwise groups that average at most 192 rows run the Q4_K tile kernel in its wide shape, mixed with tall
+// tiles for their larger groups.  GGQ_GROUPED_SHAPE is a tuning aid, read per call: 0 = tall tiles, 1 = the
+// wide / tall mix, 2 = half tiles, 3 = the direct kernel (forward) whatever the group sizes.
+static int pick_shape(int qt, int64_t rows, int64_t groups, bool direct_ok) {
+    if (qt != 12 /* GGML Q4_K */) return kShapeTall;
+    const char* e = getenv("GGQ_GROUPED_SHAPE");
+    const int forced = e && *e ? atoi(e) : -1;
+    if (direct_ok && (forced == kShapeDirect || (forced < 0 && groups > 0 && rows <= 256 * groups))) return kShapeDirect;
+    if (forced == kShapeTall || !(groups > 0 && rows <= 192 * groups)) return kShapeTall;
+    return forced == kShapeHalf ? kShapeHalf : kShapeWide;
 }
 
 int64_t ggq_lora_workspace_bytes(int64_t rows, int64_t groups, int64_t experts, int64_t n_total, int64_t k, int r) {
@@ -135,10 +141,21 @@ int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void*
     Bump bump{(char*)ws, ws_bytes, 0};
 
     MmqParams p;
-    if (int rc = init_params(p, qt, kModeNT, (int)rows, (int)n, (int)k, nseg, pick_shape(qt, rows, groups))) return rc;
+    // the direct kernel moves A, LA and LB rows with aligned 16-byte accesses
+    const bool direct_ok = aligned16(x) && k < (1 << 22) && (!lora_a || (aligned16(xa_out) && (rp != r || aligned16(lora_b))));
+    if (int rc = init_params(p, qt, kModeNT, (int)rows, (int)n, (int)k, nseg, pick_shape(qt, rows, groups, direct_ok))) return rc;
     p.a[0] = (const bf16_t*)x, p.lda = k;
     p.w[0] = (const uint8_t*)packed1, p.w[1] = (const uint8_t*)packed2;
     p.c[0] = y1, p.c[1] = y2, p.ldc = n;
+    if (p.shape == kShapeDirect) {
+        // a workgroup walks up to four column tiles of its row tile, fewer while that leaves compute units without work
+        const int64_t row_tiles = groups > 0 ? std::max<int64_t>(groups, rows / kDirectBM) : (rows + kDirectBM - 1) / kDirectBM;
+        const int col_tiles = nseg * p.col_tiles_per_seg;
+        int per_wg = 4;
+        while (per_wg > 1 && row_tiles * ((col_tiles + per_wg - 1) / per_wg) < 256) per_wg >>= 1;
+        const char* e = getenv("GGQ_DIRECT_TILES_PER_WG");  // tuning aid, read per call
+        p.col_tiles_per_wg = e && atoi(e) > 0 ? atoi(e) : per_wg;
+    }
 
     const TileDesc* tiles64 = nullptr;
     const int* num_tiles64 = nullptr;
@@ -150,7 +167,7 @@ int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void*
         // Wide shape: groups of at most 128 rows take one wide tile each, larger groups go to a second,
         // tall launch (a second wide tile for a few dozen leftover rows would cost a whole decode pass).
         const bool wide = p.shape == kShapeWide;
-        const int bm_main = p.shape == kShapeTall ? kBM : kWideBM;
+        const int bm_main = p.shape == kShapeDirect ? kDirectBM : p.shape == kShapeTall ? kBM : kWideBM;
         const int max128 = wide ? (int)groups : (int)(rows / bm_main + groups);
         max_tall = wide ? (int)std::min<int64_t>(rows / kBM + groups, rows / (kWideBM + 1) + rows / kBM + 1) : 0;
         max_tiles64 = (int)(rows / 64 + groups);
@@ -211,7 +228,7 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
     Bump bump{(char*)ws, ws_bytes, 0};
 
     MmqParams p;
-    if (int rc = init_params(p, qt, kModeNN, (int)rows, (int)n, (int)k, nseg, pick_shape(qt, rows, groups))) return rc;
+    if (int rc = init_params(p, qt, kModeNN, (int)rows, (int)n, (int)k, nseg, pick_shape(qt, rows, groups, false))) return rc;
     p.a[0] = (const bf16_t*)dy1, p.a[1] = (const bf16_t*)dy2, p.lda = n;
     p.w[0] = (const uint8_t*)packed1, p.w[1] = (const uint8_t*)packed2;
     p.c[0] = dx, p.ldc = k;

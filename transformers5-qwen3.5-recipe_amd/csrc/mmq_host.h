@@ -38,7 +38,8 @@ struct FactorGradParams {
 
 constexpr int kBM = 256, kBN = 128, kBK = 64;  // the tall tile shape (dense launches, large expert groups)
 constexpr int kWideBM = 128, kWideBN = 256;    // the wide tile shape (Q4_K expert groups of about a hundred rows)
-constexpr int kShapeTall = 0, kShapeWide = 1, kShapeHalf = 2;
+constexpr int kDirectBM = 192, kDirectBN = 256;  // the direct shape (Q4_K forward: the MFMA waves decode the weights themselves)
+constexpr int kShapeTall = 0, kShapeWide = 1, kShapeHalf = 2, kShapeDirect = 3;
 constexpr int kLdsStride = kBK + 8;  // bf16 elements per LDS row: 144 bytes keeps 128-bit reads conflict-free
 constexpr int kThreads = 1024;  // waves 0..7 run the MFMAs, waves 8..15 load and decode
 
@@ -71,7 +72,8 @@ struct MmqParams {
     const int* num_tiles2;
     int max_row_tiles2;
     int col_tiles_per_seg2;
-    int shape;  // kShapeTall / kShapeWide: which instantiation of the tile kernel the sizes above are for
+    int col_tiles_per_wg;   // direct shape: column tiles one workgroup walks through (>= 1)
+    int shape;  // kShapeTall / kShapeWide / kShapeHalf / kShapeDirect: which kernel the sizes above are for
     // LoRA
     const bf16_t* la;     // [rows, r_pad]  (x A^T in NT, dY B in NN)
     const bf16_t* lb;     // per expert: NT [cols_total, r_pad] (rows of B); NN [lora_rank, k] (the factor A as it is)
