@@ -24,11 +24,20 @@
 
 namespace ggq {
 
+#ifdef GGQ_X_STAMP
+__device__ unsigned long long g_dbg[4096 * 16];
+#define GGQ_STAMP(i) do { if (threadIdx.x == 0 && blockIdx.x < 4096) g_dbg[blockIdx.x * 16 + (i)] = __builtin_readcyclecounter(); } while (0)
+#else
+#define GGQ_STAMP(i) do { } while (0)
+#endif
+
 struct Direct {
     static constexpr int kTM = kDirectBM, kTN = kDirectBN;
     static constexpr int kStages = 4;
     static constexpr int kThreadsWG = 256;
-    static constexpr int kLdsBytes = kStages * kTM * kARowBytes;  // 96 KB
+    static constexpr int kOutPitch = 144;                              // bytes per row of a wave's output staging block (32 rows x 64 columns)
+    static constexpr int kRingBytes = kStages * kTM * kARowBytes;      // 96 KB
+    static constexpr int kLdsBytes = kRingBytes + 4 * 32 * kOutPitch;  // + 18 KB
 
     struct Scales {  // sub-block scale * 2^24, -min; dl1 is divided by 16: high nibbles are read at bits 4..7 of a half
         float dl0, nm0, dl1, nm1;
@@ -48,14 +57,19 @@ struct Direct {
     // nibbles of word 2I + J; I >= 2: the high nibbles of word 2(I-2) + J.  Writes out[2J], out[2J+1].
     template <int I, int J>
     static __device__ __forceinline__ void decode_half(const u32x4_t& q, const Scales& s, uint32_t* out) {
+#ifdef GGQ_X_NODECODE
+        out[2 * J] = q[J], out[2 * J + 1] = q[J + 2];
+        return;
+#endif
         const float dl = I < 2 ? s.dl0 : s.dl1, nm = I < 2 ? s.nm0 : s.nm1;
-        uint32_t w = q[2 * (I & 1) + J];
-        asm volatile("" : "+v"(w));  // pins this arithmetic to where the caller placed it (between two MFMAs)
+        const uint32_t w = q[2 * (I & 1) + J];
         constexpr uint32_t kMask = I < 2 ? 0x000F000Fu : 0x00F000F0u;  // a nibble in each 16-bit half: a half-precision denormal
         const uint32_t e02 = w & kMask, e13 = (w >> 8) & kMask;
         out[2 * J] = pack_bf16(mix_lo(e02, dl, nm), mix_lo(e13, dl, nm));
         out[2 * J + 1] = pack_bf16(mix_hi(e02, dl, nm), mix_hi(e13, dl, nm));
-        asm volatile("" : "+v"(out[2 * J]), "+v"(out[2 * J + 1]));  // (and keeps the results from being sunk to their use)
+        // a use of the results right here: keeps the arithmetic where the caller placed it (between two MFMAs)
+        // instead of being sunk to the MFMA that reads them
+        asm volatile("" ::"v"(out[2 * J]), "v"(out[2 * J + 1]));
     }
     static __device__ __forceinline__ bf16x8_t as_operand(const uint32_t* r) {
         const u32x4_t v = {r[0], r[1], r[2], r[3]};
@@ -80,6 +94,10 @@ struct Direct {
         const int out_cols = p.n;
         const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem_raw;
 
+        GGQ_STAMP(0);
+#ifdef GGQ_X_STAMP
+        if (threadIdx.x == 0 && blockIdx.x < 4096) g_dbg[blockIdx.x * 16 + 15] = ((unsigned long long)LIVE << 32) | (unsigned)(ct1 - ct0);
+#endif
         // A tile loads: instruction i fills slots 256 i + tid: tile row 32 i + tid / 8, slot tid % 8.  Rows past the
         // group's end repeat its last row (their results are never stored).
         const bf16_t* a_base = p.a[0] + (int64_t)c.row_begin * p.lda;
@@ -142,6 +160,7 @@ struct Direct {
         issue_group(std::integral_constant<int, 0>{}, qr[0], hc);
         issue_group(std::integral_constant<int, 1>{}, qr[1], hc);
         issue_group(std::integral_constant<int, 2>{}, qr[2], hc);
+        GGQ_STAMP(1);
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (LIVE + 2)) : "memory");  // the first step's group has landed
         asm volatile("" : "+v"(hc[0]), "+v"(hc[1]), "+v"(qr[0][0]), "+v"(qr[0][1]));
         __builtin_amdgcn_s_barrier();
@@ -167,7 +186,9 @@ struct Direct {
             for (int rb = 0; rb < LIVE; rb++) {
                 acc[rb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b0, ao[rb], acc[rb][0], 0, 0, 0);
                 acc[rb][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b1, ao[rb], acc[rb][1], 0, 0, 0);
+#ifndef GGQ_X_NOAREAD
                 ao[rb] = *(const bf16x8_t*)(src + rb * 32 * kARowBytes);
+#endif
                 if (0 * LIVE / 4 == rb) piece(std::integral_constant<int, 0>{});
                 if (1 * LIVE / 4 == rb) piece(std::integral_constant<int, 1>{});
                 if (2 * LIVE / 4 == rb) piece(std::integral_constant<int, 2>{});
@@ -176,6 +197,11 @@ struct Direct {
             }
         };
 
+        GGQ_STAMP(2);
+#ifdef GGQ_X_STAMP
+        long long wait_sum = 0, bar_sum = 0;
+#endif
+        bool stores_behind = false;  // the tile before this one went out through the staged store path
         for (int ct = ct0; ct < ct1; ct++) {
 #pragma unroll
             for (int i = 0; i < LIVE; i++)
@@ -191,12 +217,27 @@ struct Direct {
                     // next block's header when that step opens it, and this wave's part of the next A stage.
                     // Behind the barrier every wave's part has, and every wave is done with the stage of the
                     // step before this one, which the group requested now overwrites.
+                    // (behind a tile's stores - at least 4 per full row block and one for the last, issued after the groups that are in flight - the first
+                    // two steps allow that many more outstanding operations instead of waiting for the stores too)
+#ifdef GGQ_X_STAMP
+                    const long long w0 = __builtin_readcyclecounter();
+#endif
                     if (S == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LIVE + 4) : "memory");
+                    else if (S < 2 && kb == 0 && stores_behind) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(5 * LIVE - 1) : "memory");
                     else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LIVE + 2) : "memory");
                     u32x4_t* qn = qr[(S + 1) & 3];
                     asm volatile("" : "+v"(qn[0]), "+v"(qn[1]));
                     if (S == 3) asm volatile("" : "+v"(hn[0]), "+v"(hn[1]));
+#ifdef GGQ_X_STAMP
+                    const long long w1 = __builtin_readcyclecounter();
+#endif
+#ifndef GGQ_X_NOBAR
                     lds_barrier();
+#endif
+#ifdef GGQ_X_STAMP
+                    const long long w2 = __builtin_readcyclecounter();
+                    wait_sum += w1 - w0, bar_sum += w2 - w1;
+#endif
                     issue_group(std::integral_constant<int, (S + 3) & 3>{}, qr[(S + 3) & 3], hn);
                     u32x4_t* qc = qr[S];
                     __builtin_amdgcn_sched_barrier(0);
@@ -217,9 +258,7 @@ struct Direct {
                     sub_step(by, (S + 1) & 3, 0, [&](auto k_c) __attribute__((always_inline)) {
                         constexpr int K = decltype(k_c)::value;
                         if ((K & 1) == 0) {
-                            u32x4_t h = S == 3 ? hn[K >> 1] : hc[K >> 1];
-                            asm volatile("" : "+v"(h));  // (pinned here, like the decode)
-                            sc[K >> 1] = chunk_scales<(S + 1) & 3>(h);
+                            sc[K >> 1] = chunk_scales<(S + 1) & 3>(S == 3 ? hn[K >> 1] : hc[K >> 1]);
                         }
                         decode_half<0, K & 1>(qn[K >> 1], sc[K >> 1], bx[K >> 1]);
                     });
@@ -231,9 +270,10 @@ struct Direct {
                 hc[0] = hn[0], hc[1] = hn[1];
             }
 
+            if (ct - ct0 < 4) GGQ_STAMP(3 + 2 * (ct - ct0));
             // ---- LoRA term and store.  A lane holds four consecutive columns of one row: acc[rb][cb][i] is tile
             // row 32 rb + lane_c, column 64 wave + 32 cb + 8 (i / 4) + 4 h + (i % 4): a row block goes out as
-            // 8-byte stores.
+            // whole rows.
             // (own, opaque copies of the lane coordinates: none of this part's address arithmetic may be hoisted in
             // front of the tile loop, where it would sit in registers through every main loop)
             int lane_e = lane;
@@ -245,7 +285,8 @@ struct Direct {
             bf16_t* const cbase = (bf16_t*)(seg ? p.c[1] : p.c[0]);
             const int rows_valid = c.rows_valid;
             const int col_quad = col0 + 64 * wave + 4 * lane_he;  // first column of this lane's quad at cb = 0, i / 4 = 0
-            const bool vec = ((ldc & 3) == 0) && ((((uintptr_t)cbase) & 7) == 0) && col0 + kTN <= out_cols;
+            const bool vec = ((ldc & 7) == 0) && ((((uintptr_t)cbase) & 15) == 0) && col0 + kTN <= out_cols;
+            stores_behind = vec;
             const int nl = p.r_pad >> 4;  // LoRA sub-steps (0: no LoRA)
             const float ls = nl > 0 ? p.lora_scale : 0.0f;
             const bf16_t* lb_lane[2];  // this lane's rows of the factor B (its two columns), 8 h elements in
@@ -270,22 +311,27 @@ struct Direct {
                             t[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)(lb_lane[cb] + kk * 16), lao, t[cb], 0, 0, 0);
                     }
                 }
-                const bool row_ok = rb < LIVE - 1 || row < rows_valid;  // only the last live block can be partial
-                bf16_t* const crow = cbase + (int64_t)(c.row_begin + row) * ldc;
                 if (vec) {
-                    if (row_ok) {
+                    // through this wave's staging block: 8-byte pieces in, whole 128-byte rows out (LDS accesses of
+                    // one wave execute in order, so no wait is needed between the two)
+                    uint8_t* const stage = smem_raw + kRingBytes + wave * (32 * kOutPitch);
 #pragma unroll
-                        for (int cb = 0; cb < 2; cb++)
+                    for (int cb = 0; cb < 2; cb++)
 #pragma unroll
-                            for (int g = 0; g < 4; g++) {
-                                float o[4];
+                        for (int g = 0; g < 4; g++) {
+                            float o[4];
 #pragma unroll
-                                for (int j = 0; j < 4; j++) o[j] = __builtin_fmaf(ls, t[cb][4 * g + j], acc[rb][cb][4 * g + j]);
-                                const uint2 v = make_uint2(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]));
-                                *(uint2*)(crow + col_quad + 32 * cb + 8 * g) = v;
-                            }
+                            for (int j = 0; j < 4; j++) o[j] = __builtin_fmaf(ls, t[cb][4 * g + j], acc[rb][cb][4 * g + j]);
+                            *(uint2*)(stage + lane_ce * kOutPitch + (32 * cb + 8 * g + 4 * lane_he) * 2) = make_uint2(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]));
+                        }
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int r = 8 * i + (lane_e >> 3), ch = lane_e & 7;
+                        const uint4 v = *(const uint4*)(stage + r * kOutPitch + ch * 16);
+                        if (32 * rb + r < rows_valid) *(uint4*)(cbase + (int64_t)(c.row_begin + 32 * rb + r) * ldc + col0 + 64 * wave + ch * 8) = v;
                     }
-                } else if (row_ok) {
+                } else if (rb < LIVE - 1 || row < rows_valid) {  // only the last live block can be partial
+                    bf16_t* const crow = cbase + (int64_t)(c.row_begin + row) * ldc;
 #pragma unroll
                     for (int cb = 0; cb < 2; cb++)
 #pragma unroll
@@ -296,7 +342,11 @@ struct Direct {
                 }
                 __builtin_amdgcn_sched_barrier(0);  // one row block at a time: keeps the register need of this part small
             }
+            if (ct - ct0 < 4) GGQ_STAMP(4 + 2 * (ct - ct0));
         }
+#ifdef GGQ_X_STAMP
+        if (threadIdx.x == 0 && blockIdx.x < 4096) g_dbg[blockIdx.x * 16 + 13] = wait_sum, g_dbg[blockIdx.x * 16 + 14] = bar_sum;
+#endif
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may land in LDS after the workgroup has gone
     }
 
