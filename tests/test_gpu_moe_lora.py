@@ -79,14 +79,18 @@ def test_constant_byte_iq2_xxs_experts(pkg, dev):
     torch.testing.assert_close(h.grad.double().cpu(), want["dx"], rtol=1e-2, atol=1e-2)
 
 
-@pytest.mark.parametrize("qt,r,shape", [(gb.Q4_K, 16, ""), (gb.Q4_K, 16, "2"), (gb.Q8_0, 4, ""), (gb.Q6_K, 8, ""), (gb.IQ2_XXS, 16, "")])
-def test_grouped_lora_projection_all_gradients(pkg, dev, qt, r, shape, monkeypatch):
-    # ragged groups including empty experts, a group larger than one 128-row tile, and inactive planes;
-    # shape "2": the same through the library's alternative 128 x 128 tiles (two workgroups per compute unit)
+@pytest.mark.parametrize("qt,r,shape,n", [(gb.Q4_K, 16, "", 192), (gb.Q4_K, 16, "", 256), (gb.Q4_K, 16, "1", 256), (gb.Q4_K, 16, "2", 192),
+                                          (gb.Q8_0, 4, "", 192), (gb.Q6_K, 8, "", 192), (gb.IQ2_XXS, 16, "", 192)])
+def test_grouped_lora_projection_all_gradients(pkg, dev, qt, r, shape, n, monkeypatch):
+    # ragged groups including empty experts, a group larger than one 128-row tile, and inactive planes.
+    # Q4_K with n = 256 runs forward and grad-input in the kernels whose MFMA waves decode the weights themselves
+    # (n = 192: forward only, the grad-input kernel takes contraction lengths in whole groups of four 64-row steps);
+    # shape "1": the same through the wide / tall tile mix, "2": through the 128 x 128 tiles (two workgroups per
+    # compute unit)
     if shape:
         monkeypatch.setenv("GGQ_GROUPED_SHAPE", shape)
     ml = pkg.fast_moe_lora
-    e_total, n, k = 8, 192, 512
+    e_total, k = 8, 512
     sizes = [0, 150, 3, 0, 129, 1, 64, 0]
     rows = sum(sizes)
     all_ids = torch.arange(e_total, dtype=torch.int64)

@@ -88,6 +88,16 @@ static int pick_shape(int qt, int64_t rows, int64_t groups, bool direct_ok) {
     return forced == kShapeHalf ? kShapeHalf : kShapeWide;
 }
 
+// Direct shape: a workgroup walks up to four column tiles of its row tile, fewer while that leaves compute units
+// without work.  GGQ_DIRECT_TILES_PER_WG is a tuning aid, read per call.
+static int direct_tiles_per_wg(int64_t rows, int64_t groups, int col_tiles) {
+    const int64_t row_tiles = groups > 0 ? std::max<int64_t>(groups, rows / kDirectBM) : (rows + kDirectBM - 1) / kDirectBM;
+    int per_wg = 4;
+    while (per_wg > 1 && row_tiles * ((col_tiles + per_wg - 1) / per_wg) < 256) per_wg >>= 1;
+    const char* e = getenv("GGQ_DIRECT_TILES_PER_WG");
+    return e && atoi(e) > 0 ? atoi(e) : per_wg;
+}
+
 int64_t ggq_lora_workspace_bytes(int64_t rows, int64_t groups, int64_t experts, int64_t n_total, int64_t k, int r) {
     const int rp = rank_pad(r > 0 ? r : 1);
     if (experts < 1) experts = 1;
@@ -147,15 +157,7 @@ int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void*
     p.a[0] = (const bf16_t*)x, p.lda = k;
     p.w[0] = (const uint8_t*)packed1, p.w[1] = (const uint8_t*)packed2;
     p.c[0] = y1, p.c[1] = y2, p.ldc = n;
-    if (p.shape == kShapeDirect) {
-        // a workgroup walks up to four column tiles of its row tile, fewer while that leaves compute units without work
-        const int64_t row_tiles = groups > 0 ? std::max<int64_t>(groups, rows / kDirectBM) : (rows + kDirectBM - 1) / kDirectBM;
-        const int col_tiles = nseg * p.col_tiles_per_seg;
-        int per_wg = 4;
-        while (per_wg > 1 && row_tiles * ((col_tiles + per_wg - 1) / per_wg) < 256) per_wg >>= 1;
-        const char* e = getenv("GGQ_DIRECT_TILES_PER_WG");  // tuning aid, read per call
-        p.col_tiles_per_wg = e && atoi(e) > 0 ? atoi(e) : per_wg;
-    }
+    if (p.shape == kShapeDirect) p.col_tiles_per_wg = direct_tiles_per_wg(rows, groups, nseg * p.col_tiles_per_seg);
 
     const TileDesc* tiles64 = nullptr;
     const int* num_tiles64 = nullptr;
@@ -228,10 +230,13 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
     Bump bump{(char*)ws, ws_bytes, 0};
 
     MmqParams p;
-    if (int rc = init_params(p, qt, kModeNN, (int)rows, (int)n, (int)k, nseg, pick_shape(qt, rows, groups, false))) return rc;
+    // the direct kernel moves the cotangents with aligned 16-byte accesses and takes whole groups of four 64-row steps
+    const bool direct_ok = aligned16(dy1) && (!dy2 || aligned16(dy2)) && n % 64 == 0 && (nseg * (n / 64)) % 4 == 0 && n < (1 << 22);
+    if (int rc = init_params(p, qt, kModeNN, (int)rows, (int)n, (int)k, nseg, pick_shape(qt, rows, groups, direct_ok))) return rc;
     p.a[0] = (const bf16_t*)dy1, p.a[1] = (const bf16_t*)dy2, p.lda = n;
     p.w[0] = (const uint8_t*)packed1, p.w[1] = (const uint8_t*)packed2;
     p.c[0] = dx, p.ldc = k;
+    if (p.shape == kShapeDirect) p.col_tiles_per_wg = direct_tiles_per_wg(rows, groups, p.col_tiles_per_seg);
 
     const TileDesc* tiles64 = nullptr;
     const int* num_tiles64 = nullptr;
@@ -242,7 +247,7 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
     int max_tall = 0;
     if (groups > 0) {
         const bool wide = p.shape == kShapeWide;  // small groups: wide tiles; larger ones: a second, tall launch
-        const int bm_main = p.shape == kShapeTall ? kBM : kWideBM;
+        const int bm_main = p.shape == kShapeDirect ? kDirectBM : p.shape == kShapeTall ? kBM : kWideBM;
         const int max128 = wide ? (int)groups : (int)(rows / bm_main + groups);
         max_tall = wide ? (int)std::min<int64_t>(rows / kBM + groups, rows / (kWideBM + 1) + rows / kBM + 1) : 0;
         max_tiles64 = (int)(rows / 64 + groups);

@@ -1,6 +1,7 @@
 // Host launchers for the packed-weight tile kernel, the expert row-tile table and the error state.
 #include "mmq_tile.h"
 #include "mmq_direct.h"
+#include "mmq_direct_nn.h"
 #include "launch.h"
 
 #include <stdarg.h>
@@ -153,31 +154,37 @@ static int launch_one(const MmqParams& p, hipStream_t s) {
     return check_launch("mmq_tile_kernel");
 }
 
-// Q4_K forward, store epilogue, direct shape.
+// Q4_K, store epilogue, direct shape: forward or grad-input.
+template <int MODE>
 static int launch_direct(const MmqParams& p, hipStream_t s) {
-    const int col_tiles = p.nseg * p.col_tiles_per_seg;
+    const int col_tiles = (MODE == kModeNT ? p.nseg : 1) * p.col_tiles_per_seg;
     if (p.col_tiles_per_wg < 1) return set_error(GGQ_ERR_SHAPE, "mmq: column tiles per workgroup must be at least 1");
     const int64_t total = (int64_t)p.max_row_tiles * ((col_tiles + p.col_tiles_per_wg - 1) / p.col_tiles_per_wg);
     if (total <= 0) return GGQ_OK;
     const int64_t grid = (total + 7) / 8 * 8;
     if (grid > 0x7FFFFFF0) return set_error(GGQ_ERR_SHAPE, "mmq: too many tiles for one launch");
+    if (MODE == kModeNN && ((p.n & 63) || ((p.nseg * p.steps_per_seg) & 3)))
+        return set_error(GGQ_ERR_SHAPE, "mmq: the direct grad-input kernel needs whole groups of four 64-row steps");
     TimedLaunch* t = nullptr;
     if (g_timing && g_timed_count < kMaxTimedLaunches) {
         t = &g_timed[g_timed_count];
         if (hipEventCreate(&t->start) != hipSuccess || hipEventCreate(&t->stop) != hipSuccess) return set_error(GGQ_ERR_RUNTIME, "mmq: event creation failed");
-        t->qt = kQ4_K, t->mode = kModeNT, t->epi = kEpiStore;
+        t->qt = kQ4_K, t->mode = MODE, t->epi = kEpiStore;
         g_timed_count++;
         (void)hipEventRecord(t->start, s);
     }
-    static bool attr_set = false;
+    constexpr int kSmemBytes = MODE == kModeNT ? Direct::kLdsBytes : DirectNN::kLdsBytes;
+    const void* fn = MODE == kModeNT ? (const void*)mmq_direct_q4k_kernel : (const void*)mmq_direct_nn_q4k_kernel;
+    static bool attr_set = false;  // per instantiation
     if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)mmq_direct_q4k_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, Direct::kLdsBytes) != hipSuccess)
-            return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", Direct::kLdsBytes);
+        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess)
+            return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", kSmemBytes);
         attr_set = true;
     }
-    hipLaunchKernelGGL(mmq_direct_q4k_kernel, dim3((unsigned)grid), dim3(Direct::kThreadsWG), Direct::kLdsBytes, s, p);
+    if (MODE == kModeNT) hipLaunchKernelGGL(mmq_direct_q4k_kernel, dim3((unsigned)grid), dim3(Direct::kThreadsWG), kSmemBytes, s, p);
+    else hipLaunchKernelGGL(mmq_direct_nn_q4k_kernel, dim3((unsigned)grid), dim3(DirectNN::kThreadsWG), kSmemBytes, s, p);
     if (t) (void)hipEventRecord(t->stop, s);
-    return check_launch("mmq_direct_q4k_kernel");
+    return check_launch(MODE == kModeNT ? "mmq_direct_q4k_kernel" : "mmq_direct_nn_q4k_kernel");
 }
 
 template <int MODE>
@@ -218,7 +225,7 @@ static int launch_qt(int mode, int epi, const MmqParams& p, hipStream_t s) {
     if (mode == kModeNT) {
         switch (epi) {
             case kEpiStore:
-                if (QT == kQ4_K && p.shape == kShapeDirect) return launch_direct(p, s);
+                if (QT == kQ4_K && p.shape == kShapeDirect) return launch_direct<kModeNT>(p, s);
                 if (QT == kQ4_K && p.shape == kShapeWide) return launch_one<kQ4_K, kModeNT, kEpiStore, 1>(p, s);
                 if (QT == kQ4_K && p.shape == kShapeHalf) return launch_one<kQ4_K, kModeNT, kEpiStore, 2>(p, s);
                 return launch_one<QT, kModeNT, kEpiStore, 0>(p, s);
@@ -228,6 +235,7 @@ static int launch_qt(int mode, int epi, const MmqParams& p, hipStream_t s) {
     } else {
         switch (epi) {
             case kEpiStore:
+                if (QT == kQ4_K && p.shape == kShapeDirect) return launch_direct<kModeNN>(p, s);
                 if (QT == kQ4_K && p.shape == kShapeWide) return launch_one<kQ4_K, kModeNN, kEpiStore, 1>(p, s);
                 if (QT == kQ4_K && p.shape == kShapeHalf) return launch_one<kQ4_K, kModeNN, kEpiStore, 2>(p, s);
                 return launch_one<QT, kModeNN, kEpiStore, 0>(p, s);
@@ -258,7 +266,6 @@ int init_params(MmqParams& p, int qt, int mode, int m, int n, int k, int nseg, i
     p.w_row_bytes = packed_row_bytes(qt, k);
     p.w_expert_bytes = p.w_row_bytes * n;
     if (shape != kShapeTall && qt != kQ4_K) shape = kShapeTall;  // the other shapes exist for Q4_K only
-    if (shape == kShapeDirect && mode != kModeNT) shape = kShapeTall;
     const int bm = shape == kShapeDirect ? kDirectBM : shape == kShapeTall ? kBM : kWideBM;
     const int bn = shape == kShapeDirect ? kDirectBN : shape == kShapeWide ? kWideBN : kBN;
     p.shape = shape;
