@@ -62,6 +62,34 @@ def test_grouped_pair_and_single_projection_jacobian(pkg, dev, qt):
     assert torch.equal(dx_op, it.grad)
 
 
+def test_q4k_grouped_grad_input_decoding_waves(pkg, dev):
+    # Q4_K, no LoRA term, contraction length 256 (pair: 2 x 256): forward and grad-input both run in the kernels
+    # whose MFMA waves decode the weights themselves; ragged groups up to more than one 192-row tile
+    ml = pkg.fast_moe_lora
+    qt, k, n = gb.Q4_K, 512, 256
+    sizes = [5, 0, 200, 33, 0, 129, 64, 1]
+    experts = torch.arange(8, dtype=torch.int64)
+    offsets = torch.tensor(np.cumsum(sizes), dtype=torch.int32)
+    rows = sum(sizes)
+    gen = torch.Generator().manual_seed(13579)
+    pg, pu = _expert_payload(610, qt, 8, n, k), _expert_payload(650, qt, 8, n, k)
+    wg, wu = ref.weights_bf16(pg, qt), ref.weights_bf16(pu, qt)
+    hidden = bf16_randn(gen, rows, k)
+    g1, g2 = bf16_randn(gen, rows, n), bf16_randn(gen, rows, n)
+    want_g = ref.grouped_lora_linear(hidden, wg, experts, offsets, dy=g1)
+    want_u = ref.grouped_lora_linear(hidden, wu, experts, offsets, dy=g2)
+    h = hidden.to(dev).requires_grad_(True)
+    e_d, o_d = _to(dev, experts, offsets)
+    pg_d, pu_d = torch.from_numpy(pg).to(dev), torch.from_numpy(pu).to(dev)
+    gate, up = ml.grouped_mmq_pair(h, pg_d, pu_d, e_d, o_d, qt, n)
+    torch.autograd.backward((gate, up), _to(dev, g1, g2))
+    assert_close_bf16(gate, want_g["y"], "gate")
+    assert_close_bf16(up, want_u["y"], "up")
+    assert_close_bf16(h.grad, want_g["dx"] + want_u["dx"], "pair dX")
+    dx_single = ml.grouped_mmq_grad_input(g1.to(dev), pg_d, e_d, o_d, qt, k)
+    assert_close_bf16(dx_single, want_g["dx"], "single dX")
+
+
 def test_constant_byte_iq2_xxs_experts(pkg, dev):
     # test_deepseek_v4_moe_lora.py:55-118: payload of all bytes 32, experts [0,1], offsets [3,7]
     ml = pkg.fast_moe_lora
@@ -79,13 +107,13 @@ def test_constant_byte_iq2_xxs_experts(pkg, dev):
     torch.testing.assert_close(h.grad.double().cpu(), want["dx"], rtol=1e-2, atol=1e-2)
 
 
-@pytest.mark.parametrize("qt,r,shape,n", [(gb.Q4_K, 16, "", 192), (gb.Q4_K, 16, "", 256), (gb.Q4_K, 16, "1", 256), (gb.Q4_K, 16, "2", 192),
+@pytest.mark.parametrize("qt,r,shape,n", [(gb.Q4_K, 16, "", 192), (gb.Q4_K, 16, "", 256), (gb.Q4_K, 16, "3", 256), (gb.Q4_K, 16, "1", 256), (gb.Q4_K, 16, "2", 192),
                                           (gb.Q8_0, 4, "", 192), (gb.Q6_K, 8, "", 192), (gb.IQ2_XXS, 16, "", 192)])
 def test_grouped_lora_projection_all_gradients(pkg, dev, qt, r, shape, n, monkeypatch):
     # ragged groups including empty experts, a group larger than one 128-row tile, and inactive planes.
-    # Q4_K with n = 256 runs forward and grad-input in the kernels whose MFMA waves decode the weights themselves
-    # (n = 192: forward only, the grad-input kernel takes contraction lengths in whole groups of four 64-row steps);
-    # shape "1": the same through the wide / tall tile mix, "2": through the 128 x 128 tiles (two workgroups per
+    # Q4_K runs forward in the kernel whose MFMA waves decode the weights themselves; shape "3" with n = 256 also the
+    # grad-input (that kernel takes contraction lengths in whole groups of four 64-row steps, and is the default only
+    # without a LoRA term); shape "1": the wide / tall tile mix, "2": the 128 x 128 tiles (two workgroups per
     # compute unit)
     if shape:
         monkeypatch.setenv("GGQ_GROUPED_SHAPE", shape)

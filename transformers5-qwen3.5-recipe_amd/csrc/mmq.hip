@@ -281,11 +281,5 @@ int init_params(MmqParams& p, int qt, int mode, int m, int n, int k, int nseg, i
     return GGQ_OK;
 }
 
-#ifdef GGQ_X_STAMP
-extern "C" int ggq_debug_read(unsigned long long* dst, int n) {
-    if (hipDeviceSynchronize() != hipSuccess) return -1;
-    return hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_dbg), (size_t)n * 8) == hipSuccess ? 0 : -1;
-}
-#endif
 
 }  // namespace ggq

@@ -3,33 +3,32 @@
 //   C[m, n] = sum_k A[m, k] * W[n, k]  (+ s * LA[m, :] . LB[n, :])
 //
 // One workgroup = 256 lanes = four waves, one per SIMD with the whole 512-register file of its lanes,
-// computes a tile of up to 192 rows x 256 columns.  Wave w owns columns 64w .. 64w+63 of every row: up to
+// computes tiles of up to 192 rows x 256 columns.  Wave w owns columns 64w .. 64w+63 of every row: up to
 // six 32-row blocks x two 32-column blocks of MFMA 32x32x16 accumulators.  Per contraction step of 64
 //   * the A tile goes global -> LDS directly (no registers), three steps ahead, through a ring of four
 //     stages; rows are unpadded with XOR-swizzled 16-byte slots (a_slot), every wave reads all of them;
 //   * a lane (column n = lane % 32 of a column block, half h = lane / 32) loads the 16 bytes 16h .. 16h+15
 //     of its row's 32-byte quant group of the step, three steps ahead, and decodes them in registers into
-//     the B operands of the step's four MFMA sub-steps: the low nibbles are elements 16h .. 16h+15 of the
+//     the operands of the step's four MFMA sub-steps: the low nibbles are elements 16h .. 16h+15 of the
 //     group's first sub-block (sub-steps 0, 1), the high nibbles the same elements of the second (2, 3).
 //     An MFMA sums over its 16 contraction slots in any order, so lane half h simply feeds contraction
 //     elements 16h .. 16h+7 (+8 for the odd sub-steps, +32 for the high nibbles) and reads the matching
 //     16-byte slot of the A row.  No decoded weight ever touches LDS, and the tile's rows share one decode.
+// The weights are the MFMA's first operand, so a lane's accumulator registers hold four consecutive columns
+// of one row; a finished row block goes through a wave-private LDS block and leaves as whole 128-byte rows.
+// The LoRA term is added there, from operands loaded straight from global memory (one burst per tile).
 // A workgroup takes a run of column tiles of its row tile and treats their steps as one stream, so the loads
 // of a tile's first steps are in flight while the tile before it finishes.
 // The kernel is instantiated per number of live 32-row blocks, so an expert group of any size up to 192
 // rows is one row tile and issues no MFMA on empty blocks.  The packed-weight loads are inline-asm loads
-// the compiler does not track; the step waits for them with an exact count (loads return in issue order).
+// the compiler does not track; the step waits for them with an exact count (vector memory operations complete
+// in issue order).  With one wave per SIMD every instruction of the step, scalar ones included, takes an issue
+// slot of that wave: the decode arithmetic is placed by hand between the MFMAs, and the addresses of the loads
+// are scalar bases plus lane offsets that never change.
 #pragma once
 #include "mmq_tile.h"
 
 namespace ggq {
-
-#ifdef GGQ_X_STAMP
-__device__ unsigned long long g_dbg[4096 * 16];
-#define GGQ_STAMP(i) do { if (threadIdx.x == 0 && blockIdx.x < 4096) g_dbg[blockIdx.x * 16 + (i)] = __builtin_readcyclecounter(); } while (0)
-#else
-#define GGQ_STAMP(i) do { } while (0)
-#endif
 
 struct Direct {
     static constexpr int kTM = kDirectBM, kTN = kDirectBN;
@@ -57,10 +56,6 @@ struct Direct {
     // nibbles of word 2I + J; I >= 2: the high nibbles of word 2(I-2) + J.  Writes out[2J], out[2J+1].
     template <int I, int J>
     static __device__ __forceinline__ void decode_half(const u32x4_t& q, const Scales& s, uint32_t* out) {
-#ifdef GGQ_X_NODECODE
-        out[2 * J] = q[J], out[2 * J + 1] = q[J + 2];
-        return;
-#endif
         const float dl = I < 2 ? s.dl0 : s.dl1, nm = I < 2 ? s.nm0 : s.nm1;
         const uint32_t w = q[2 * (I & 1) + J];
         constexpr uint32_t kMask = I < 2 ? 0x000F000Fu : 0x00F000F0u;  // a nibble in each 16-bit half: a half-precision denormal
@@ -93,11 +88,6 @@ struct Direct {
         const int steps = p.steps_per_seg, blocks = steps >> 2;
         const int out_cols = p.n;
         const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem_raw;
-
-        GGQ_STAMP(0);
-#ifdef GGQ_X_STAMP
-        if (threadIdx.x == 0 && blockIdx.x < 4096) g_dbg[blockIdx.x * 16 + 15] = ((unsigned long long)LIVE << 32) | (unsigned)(ct1 - ct0);
-#endif
         // A tile loads: instruction i fills slots 256 i + tid: tile row 32 i + tid / 8, slot tid % 8.  Rows past the
         // group's end repeat its last row (their results are never stored).
         const bf16_t* a_base = p.a[0] + (int64_t)c.row_begin * p.lda;
@@ -160,7 +150,6 @@ struct Direct {
         issue_group(std::integral_constant<int, 0>{}, qr[0], hc);
         issue_group(std::integral_constant<int, 1>{}, qr[1], hc);
         issue_group(std::integral_constant<int, 2>{}, qr[2], hc);
-        GGQ_STAMP(1);
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (LIVE + 2)) : "memory");  // the first step's group has landed
         asm volatile("" : "+v"(hc[0]), "+v"(hc[1]), "+v"(qr[0][0]), "+v"(qr[0][1]));
         __builtin_amdgcn_s_barrier();
@@ -186,9 +175,7 @@ struct Direct {
             for (int rb = 0; rb < LIVE; rb++) {
                 acc[rb][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b0, ao[rb], acc[rb][0], 0, 0, 0);
                 acc[rb][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b1, ao[rb], acc[rb][1], 0, 0, 0);
-#ifndef GGQ_X_NOAREAD
                 ao[rb] = *(const bf16x8_t*)(src + rb * 32 * kARowBytes);
-#endif
                 if (0 * LIVE / 4 == rb) piece(std::integral_constant<int, 0>{});
                 if (1 * LIVE / 4 == rb) piece(std::integral_constant<int, 1>{});
                 if (2 * LIVE / 4 == rb) piece(std::integral_constant<int, 2>{});
@@ -196,11 +183,6 @@ struct Direct {
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
-
-        GGQ_STAMP(2);
-#ifdef GGQ_X_STAMP
-        long long wait_sum = 0, bar_sum = 0;
-#endif
         bool stores_behind = false;  // the tile before this one went out through the staged store path
         for (int ct = ct0; ct < ct1; ct++) {
 #pragma unroll
@@ -219,25 +201,13 @@ struct Direct {
                     // step before this one, which the group requested now overwrites.
                     // (behind a tile's stores - at least 4 per full row block and one for the last, issued after the groups that are in flight - the first
                     // two steps allow that many more outstanding operations instead of waiting for the stores too)
-#ifdef GGQ_X_STAMP
-                    const long long w0 = __builtin_readcyclecounter();
-#endif
                     if (S == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LIVE + 4) : "memory");
                     else if (S < 2 && kb == 0 && stores_behind) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(5 * LIVE - 1) : "memory");
                     else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LIVE + 2) : "memory");
                     u32x4_t* qn = qr[(S + 1) & 3];
                     asm volatile("" : "+v"(qn[0]), "+v"(qn[1]));
                     if (S == 3) asm volatile("" : "+v"(hn[0]), "+v"(hn[1]));
-#ifdef GGQ_X_STAMP
-                    const long long w1 = __builtin_readcyclecounter();
-#endif
-#ifndef GGQ_X_NOBAR
                     lds_barrier();
-#endif
-#ifdef GGQ_X_STAMP
-                    const long long w2 = __builtin_readcyclecounter();
-                    wait_sum += w1 - w0, bar_sum += w2 - w1;
-#endif
                     issue_group(std::integral_constant<int, (S + 3) & 3>{}, qr[(S + 3) & 3], hn);
                     u32x4_t* qc = qr[S];
                     __builtin_amdgcn_sched_barrier(0);
@@ -269,8 +239,6 @@ struct Direct {
                 step(std::integral_constant<int, 3>{});
                 hc[0] = hn[0], hc[1] = hn[1];
             }
-
-            if (ct - ct0 < 4) GGQ_STAMP(3 + 2 * (ct - ct0));
             // ---- LoRA term and store.  A lane holds four consecutive columns of one row: acc[rb][cb][i] is tile
             // row 32 rb + lane_c, column 64 wave + 32 cb + 8 (i / 4) + 4 h + (i % 4): a row block goes out as
             // whole rows.
@@ -293,6 +261,16 @@ struct Direct {
 #pragma unroll
             for (int cb = 0; cb < 2; cb++)
                 lb_lane[cb] = p.lb + c.expert * p.lb_expert_elems + ((int64_t)seg * out_cols + min(col0 + 64 * wave + lane_ce + 32 * cb, out_cols - 1)) * p.r_pad + lane_he * 8;
+            // the operands of the first 16 of the rank for the whole tile in one burst (one memory round trip per
+            // tile instead of one per row block); ranks above 16 load the rest in place
+            bf16x8_t lb0[2], la0[LIVE];
+            if (nl > 0) {
+#pragma unroll
+                for (int cb = 0; cb < 2; cb++) lb0[cb] = *(const bf16x8_t*)lb_lane[cb];
+#pragma unroll
+                for (int rb = 0; rb < LIVE; rb++)
+                    la0[rb] = *(const bf16x8_t*)(p.la + (int64_t)(c.row_begin + min(32 * rb + lane_ce, rows_valid - 1)) * p.r_pad + lane_he * 8);
+            }
 #pragma unroll
             for (int rb = 0; rb < LIVE; rb++) {
                 const int row = 32 * rb + lane_ce;
@@ -302,9 +280,11 @@ struct Direct {
 #pragma unroll
                     for (int e = 0; e < 16; e++) t[cb][e] = 0.0f;
                 if (nl > 0) {
+#pragma unroll
+                    for (int cb = 0; cb < 2; cb++) t[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lb0[cb], la0[rb], t[cb], 0, 0, 0);
                     const bf16_t* la = p.la + (int64_t)(c.row_begin + min(row, rows_valid - 1)) * p.r_pad + lane_he * 8;
 #pragma nounroll
-                    for (int kk = 0; kk < nl; kk++) {
+                    for (int kk = 1; kk < nl; kk++) {
                         const bf16x8_t lao = *(const bf16x8_t*)(la + kk * 16);
 #pragma unroll
                         for (int cb = 0; cb < 2; cb++)
@@ -342,11 +322,7 @@ struct Direct {
                 }
                 __builtin_amdgcn_sched_barrier(0);  // one row block at a time: keeps the register need of this part small
             }
-            if (ct - ct0 < 4) GGQ_STAMP(4 + 2 * (ct - ct0));
         }
-#ifdef GGQ_X_STAMP
-        if (threadIdx.x == 0 && blockIdx.x < 4096) g_dbg[blockIdx.x * 16 + 13] = wait_sum, g_dbg[blockIdx.x * 16 + 14] = bar_sum;
-#endif
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may land in LDS after the workgroup has gone
     }
 

@@ -79,7 +79,6 @@ struct DirectNN {
         const int sps = p.steps_per_seg, steps = p.nseg * sps;  // contraction steps of 64 weight rows (a multiple of 4)
         const int out_cols = p.k;
         const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem_raw;
-
         // A tile loads as in the forward kernel: fixed lane offsets, the step moves the scalar base
         uint32_t a_voff[LIVE];
 #pragma unroll
@@ -160,7 +159,6 @@ struct DirectNN {
         for (int rb = 0; rb < LIVE; rb++) ao[rb] = *(const bf16x8_t*)(a_row + a_koff[0] + rb * 32 * kARowBytes);
         bf16x8_t bops[2][4][2];  // B operands of the even / odd steps
         read_b(bops[0]);
-
         bool stores_behind = false;  // the tile before this one went out through the staged store path
         int t_step = 0;              // step inside the tile
         for (int ct = ct0; ct < ct1; ct++) {
@@ -211,7 +209,6 @@ struct DirectNN {
                 step(std::integral_constant<int, 2>{});
                 step(std::integral_constant<int, 3>{});
             }
-
             // ---- LoRA term and store (accumulator layout and staging as in the forward kernel)
             int lane_e = lane;
             asm volatile("" : "+v"(lane_e));
@@ -226,6 +223,49 @@ struct DirectNN {
             const int nl = p.r_pad >> 4;  // LoRA sub-steps (0: no LoRA)
             const float ls = nl > 0 ? p.lora_scale : 0.0f;
             const bf16_t* const lb_exp = p.lb + c.expert * p.lb_expert_elems;  // the factor A of this expert, [lora_rank][k]
+            // eight factor rows (16 kk + 8 h ..) of this lane's column of block cb; rows past the rank are zero
+            auto factor_operand = [&](int kk, int cb) __attribute__((always_inline)) {
+                const int col = min(col0 + 64 * wave + lane_ce + 32 * cb, out_cols - 1);
+                uint32_t e[8];
+#pragma unroll
+                for (int i = 0; i < 8; i++) {  // (unconditional loads of a clamped row, then a select: no branch, one round trip)
+                    const int j = kk * 16 + lane_he * 8 + i;
+                    const uint32_t v = lb_exp[(int64_t)min(j, p.lora_rank - 1) * out_cols + col];
+                    e[i] = j < p.lora_rank ? v : 0u;
+                }
+                const u32x4_t v = {e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+                return __builtin_bit_cast(bf16x8_t, v);
+            };
+            // the operands of the first 16 of the rank for the whole tile in one burst (one memory round trip per
+            // tile instead of one per row block); ranks above 16 load the rest in place
+            bf16x8_t lb0[2], la0[LIVE];
+            if (nl > 0) {
+                if (col0 + kTN <= out_cols) {
+                    // rows 0..15 of the factor x this wave's 64 columns: whole 128-byte rows into the staging block
+                    // (rows past the rank as zeros), transposing reads back out - instead of sixteen 2-byte loads per lane
+                    uint8_t* const stage = smem_raw + kOutBase + wave * (32 * kOutPitch);
+#pragma unroll
+                    for (int i = 0; i < 2; i++) {
+                        const int id = lane_e + 64 * i, j = id >> 3, ch = id & 7;
+                        const uint4 v = *(const uint4*)(lb_exp + (int64_t)min(j, p.lora_rank - 1) * out_cols + col0 + 64 * wave + ch * 8);
+                        *(uint4*)(stage + j * kOutPitch + ch * 16) = j < p.lora_rank ? v : zero4();
+                    }
+                    const int g4 = lane_e >> 4, s4 = lane_e & 15;
+                    const uint8_t* src = stage + (8 * (g4 >> 1) + (s4 >> 2)) * kOutPitch + (16 * (g4 & 1) + 4 * (s4 & 3)) * 2;
+#pragma unroll
+                    for (int cb = 0; cb < 2; cb++) {
+                        const v4i16_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(src + cb * 64));
+                        const v4i16_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16_ptr)(src + cb * 64 + 4 * kOutPitch));
+                        lb0[cb] = __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                    }
+                } else {
+#pragma unroll
+                    for (int cb = 0; cb < 2; cb++) lb0[cb] = factor_operand(0, cb);
+                }
+#pragma unroll
+                for (int rb = 0; rb < LIVE; rb++)
+                    la0[rb] = *(const bf16x8_t*)(p.la + (int64_t)(c.row_begin + min(32 * rb + lane_ce, rows_valid - 1)) * p.r_pad + lane_he * 8);
+            }
 #pragma unroll
             for (int rb = 0; rb < LIVE; rb++) {
                 const int row = 32 * rb + lane_ce;
@@ -235,23 +275,14 @@ struct DirectNN {
 #pragma unroll
                     for (int e = 0; e < 16; e++) t[cb][e] = 0.0f;
                 if (nl > 0) {
+#pragma unroll
+                    for (int cb = 0; cb < 2; cb++) t[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lb0[cb], la0[rb], t[cb], 0, 0, 0);
                     const bf16_t* la = p.la + (int64_t)(c.row_begin + min(row, rows_valid - 1)) * p.r_pad + lane_he * 8;
 #pragma nounroll
-                    for (int kk = 0; kk < nl; kk++) {
+                    for (int kk = 1; kk < nl; kk++) {
                         const bf16x8_t lao = *(const bf16x8_t*)(la + kk * 16);
 #pragma unroll
-                        for (int cb = 0; cb < 2; cb++) {
-                            // eight factor rows of this lane's column (rows past the rank are zero)
-                            const int col = min(col0 + 64 * wave + lane_ce + 32 * cb, out_cols - 1);
-                            uint32_t e[8];
-#pragma unroll
-                            for (int i = 0; i < 8; i++) {
-                                const int j = kk * 16 + lane_he * 8 + i;
-                                e[i] = j < p.lora_rank ? (uint32_t)lb_exp[(int64_t)j * out_cols + col] : 0u;
-                            }
-                            const u32x4_t v = {e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
-                            t[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, v), lao, t[cb], 0, 0, 0);
-                        }
+                        for (int cb = 0; cb < 2; cb++) t[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(factor_operand(kk, cb), lao, t[cb], 0, 0, 0);
                     }
                 }
                 if (vec) {
