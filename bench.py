@@ -195,7 +195,7 @@ def main() -> None:
     per_mode = {0: [], 1: []}
     for j in range(max(n, 0)):
         per_mode[mode[j]].append(ms[j])
-    names = {0: "mmq_mixed_kernel<Q4_K, forward, store>", 1: "mmq_mixed_kernel<Q4_K, grad_input, store>"}
+    names = {0: "mmq_direct_q4k_kernel (Q4_K, forward, store)", 1: "mmq_mixed_kernel<Q4_K, grad_input, store>"}
     dominant = max(per_mode, key=lambda m: sum(per_mode[m]))
     launches = len(per_mode[dominant])
     avg_ms = sum(per_mode[dominant]) / max(launches, 1)
@@ -204,9 +204,9 @@ def main() -> None:
     achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12 if launches else 0.0
     kernel_ms_per_step = {names[m]: sum(v) / prof_steps for m, v in per_mode.items()}
     # HBM bytes per launch (fetched + written, average of the gate/up and down launches) from the FETCH_SIZE /
-    # WRITE_SIZE counter runs summarised in profiles/mmq_mixed_q4k_grouped_moe_lora_step.pmc_traffic.txt;
+    # WRITE_SIZE counter runs summarised in profiles/mmq_direct_and_mixed_q4k_grouped_moe_lora_step.pmc_traffic.txt;
     # the counters are collected offline, so this figure only changes when that profile is redone.
-    traffic_bytes = {0: 330.1e6 + 100.7e6, 1: 343.7e6 + 83.9e6}[dominant]
+    traffic_bytes = {0: 642.2e6 + 101.1e6, 1: 343.6e6 + 83.9e6}[dominant]
 
     result = {
         "metric": "fwd+bwd TFLOP/s and weight GB/s, Q4_K grouped-MoE LoRA; % of MI355X roofline",
