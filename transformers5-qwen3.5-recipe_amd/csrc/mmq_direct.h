@@ -36,7 +36,8 @@ struct Direct {
     static constexpr int kThreadsWG = 256;
     static constexpr int kOutPitch = 144;                              // bytes per row of a wave's output staging block (32 rows x 64 columns)
     static constexpr int kRingBytes = kStages * kTM * kARowBytes;      // 96 KB
-    static constexpr int kLdsBytes = kRingBytes + 4 * 32 * kOutPitch;  // + 18 KB
+    static constexpr int kLaBase = kRingBytes + 4 * 32 * kOutPitch;    // + 18 KB: the row tile's LA rows (rank <= 16), 32 bytes each
+    static constexpr int kLdsBytes = kLaBase + kTM * 32;               // + 6 KB
 
     struct Scales {  // sub-block scale * 2^24, -min; dl1 is divided by 16: high nibbles are read at bits 4..7 of a half
         float dl0, nm0, dl1, nm1;
@@ -150,9 +151,17 @@ struct Direct {
         issue_group(std::integral_constant<int, 0>{}, qr[0], hc);
         issue_group(std::integral_constant<int, 1>{}, qr[1], hc);
         issue_group(std::integral_constant<int, 2>{}, qr[2], hc);
+        // the row tile's LA rows stay in LDS for all the column tiles of this workgroup (ranks up to 16)
+        const bool la_resident = p.r_pad == 16;
+        if (la_resident) {
+            for (int id = tid; id < LIVE * 64; id += kThreadsWG) {
+                const int row = id >> 1, half = id & 1;
+                *(uint4*)(smem_raw + kLaBase + row * 32 + half * 16) = *(const uint4*)(p.la + (int64_t)(c.row_begin + min(row, c.rows_valid - 1)) * 16 + half * 8);
+            }
+        }
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (LIVE + 2)) : "memory");  // the first step's group has landed
         asm volatile("" : "+v"(hc[0]), "+v"(hc[1]), "+v"(qr[0][0]), "+v"(qr[0][1]));
-        __builtin_amdgcn_s_barrier();
+        lds_barrier();
         Scales sc[2];
         uint32_t bx[2][4], by[2][4];  // B operands of the current / next sub-step, per column block
 #pragma unroll
@@ -191,6 +200,15 @@ struct Direct {
                 for (int j = 0; j < 2; j++)
 #pragma unroll
                     for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+            // this lane's two rows of the LoRA factor B (first 16 of the rank), requested ahead of the tile's steps
+            bf16x8_t lb0[2];
+            if (p.r_pad > 0) {
+                int seg0, colz;
+                tile_origin(ct, seg0, colz);
+#pragma unroll
+                for (int cb = 0; cb < 2; cb++)
+                    lb0[cb] = *(const bf16x8_t*)(p.lb + c.expert * p.lb_expert_elems + ((int64_t)seg0 * out_cols + min(colz + 64 * wave + lane_c + 32 * cb, out_cols - 1)) * p.r_pad + lane_h * 8);
+            }
             for (int kb = 0; kb < blocks; kb++) {
                 // the four steps of a 256-wide block, written out so that the quant group index is a constant
                 auto step = [&](auto s_c) __attribute__((always_inline)) {
@@ -261,15 +279,14 @@ struct Direct {
 #pragma unroll
             for (int cb = 0; cb < 2; cb++)
                 lb_lane[cb] = p.lb + c.expert * p.lb_expert_elems + ((int64_t)seg * out_cols + min(col0 + 64 * wave + lane_ce + 32 * cb, out_cols - 1)) * p.r_pad + lane_he * 8;
-            // the operands of the first 16 of the rank for the whole tile in one burst (one memory round trip per
-            // tile instead of one per row block); ranks above 16 load the rest in place
-            bf16x8_t lb0[2], la0[LIVE];
+            // the operands of the first 16 of the rank: LA rows from LDS (or, for ranks above 16, in one burst from
+            // memory, the rest of the rank in place); the factor rows were requested ahead of the tile's steps
+            bf16x8_t la0[LIVE];
             if (nl > 0) {
 #pragma unroll
-                for (int cb = 0; cb < 2; cb++) lb0[cb] = *(const bf16x8_t*)lb_lane[cb];
-#pragma unroll
                 for (int rb = 0; rb < LIVE; rb++)
-                    la0[rb] = *(const bf16x8_t*)(p.la + (int64_t)(c.row_begin + min(32 * rb + lane_ce, rows_valid - 1)) * p.r_pad + lane_he * 8);
+                    la0[rb] = la_resident ? *(const bf16x8_t*)(smem_raw + kLaBase + (32 * rb + lane_ce) * 32 + lane_he * 16)
+                                          : *(const bf16x8_t*)(p.la + (int64_t)(c.row_begin + min(32 * rb + lane_ce, rows_valid - 1)) * p.r_pad + lane_he * 8);
             }
 #pragma unroll
             for (int rb = 0; rb < LIVE; rb++) {

@@ -26,7 +26,8 @@ struct DirectNN {
     static constexpr int kRingBytes = kStages * kTM * kARowBytes;      // 96 KB
     static constexpr int kOutPitch = Direct::kOutPitch;
     static constexpr int kWBase = kRingBytes, kOutBase = kRingBytes + 4 * kWBlock;
-    static constexpr int kLdsBytes = kOutBase + 4 * 32 * kOutPitch;    // 96 + 36 + 18 KB
+    static constexpr int kLaBase = kOutBase + 4 * 32 * kOutPitch;      // the row tile's LA rows (rank <= 16), 32 bytes each
+    static constexpr int kLdsBytes = kLaBase + kTM * 32;               // 96 + 36 + 18 + 6 KB
 
     struct RowCtx {
         int row_begin, rows_valid;
@@ -147,9 +148,17 @@ struct DirectNN {
         issue_group(std::integral_constant<int, 0>{}, raw[0]);
         issue_group(std::integral_constant<int, 1>{}, raw[1]);
         issue_group(std::integral_constant<int, 2>{}, raw[2]);
+        // the row tile's LA rows stay in LDS for all the column tiles of this workgroup (ranks up to 16)
+        const bool la_resident = p.r_pad == 16;
+        if (la_resident) {
+            for (int id = tid; id < LIVE * 64; id += kThreadsWG) {
+                const int row = id >> 1, half = id & 1;
+                *(uint4*)(smem_raw + kLaBase + row * 32 + half * 16) = *(const uint4*)(p.la + (int64_t)(c.row_begin + min(row, c.rows_valid - 1)) * 16 + half * 8);
+            }
+        }
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (LIVE + 3)) : "memory");  // the first step's group has landed
         asm volatile("" : "+v"(raw[0].hdr), "+v"(raw[0].q0), "+v"(raw[0].q1));
-        __builtin_amdgcn_s_barrier();
+        lds_barrier();
         {
             const Scales s = wave_scales(raw[0].hdr, wave);
             decode_store(raw[0].q0, 0, 0, s), decode_store(raw[0].q0, 1, 8, s);
@@ -168,6 +177,16 @@ struct DirectNN {
                 for (int j = 0; j < 2; j++)
 #pragma unroll
                     for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+            // rows 0..15 of the LoRA factor x this wave's 64 columns (two 16-byte pieces per lane), requested ahead of
+            // the tile's steps
+            uint4 lbraw[2];
+            if (p.r_pad > 0) {
+#pragma unroll
+                for (int i = 0; i < 2; i++) {
+                    const int id = lane + 64 * i, j = id >> 3, ch = id & 7;
+                    lbraw[i] = *(const uint4*)(p.lb + c.expert * p.lb_expert_elems + (int64_t)min(j, p.lora_rank - 1) * out_cols + ct * kTN + 64 * wave + ch * 8);
+                }
+            }
             for (t_step = 0; t_step < steps; t_step += 4) {
                 auto step = [&](auto s_c) __attribute__((always_inline)) {
                     constexpr int S = decltype(s_c)::value;
@@ -247,8 +266,7 @@ struct DirectNN {
 #pragma unroll
                     for (int i = 0; i < 2; i++) {
                         const int id = lane_e + 64 * i, j = id >> 3, ch = id & 7;
-                        const uint4 v = *(const uint4*)(lb_exp + (int64_t)min(j, p.lora_rank - 1) * out_cols + col0 + 64 * wave + ch * 8);
-                        *(uint4*)(stage + j * kOutPitch + ch * 16) = j < p.lora_rank ? v : zero4();
+                        *(uint4*)(stage + j * kOutPitch + ch * 16) = j < p.lora_rank ? lbraw[i] : zero4();
                     }
                     const int g4 = lane_e >> 4, s4 = lane_e & 15;
                     const uint8_t* src = stage + (8 * (g4 >> 1) + (s4 >> 2)) * kOutPitch + (16 * (g4 & 1) + 4 * (s4 & 3)) * 2;
@@ -264,7 +282,8 @@ struct DirectNN {
                 }
 #pragma unroll
                 for (int rb = 0; rb < LIVE; rb++)
-                    la0[rb] = *(const bf16x8_t*)(p.la + (int64_t)(c.row_begin + min(32 * rb + lane_ce, rows_valid - 1)) * p.r_pad + lane_he * 8);
+                    la0[rb] = la_resident ? *(const bf16x8_t*)(smem_raw + kLaBase + (32 * rb + lane_ce) * 32 + lane_he * 16)
+                                          : *(const bf16x8_t*)(p.la + (int64_t)(c.row_begin + min(32 * rb + lane_ce, rows_valid - 1)) * p.r_pad + lane_he * 8);
             }
 #pragma unroll
             for (int rb = 0; rb < LIVE; rb++) {
