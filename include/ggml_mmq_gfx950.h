@@ -127,6 +127,17 @@ int ggq_route_combine_backward(const void* expert_out, const void* weights, int 
 int ggq_swiglu_forward(const void* gate, const void* up, void* h, int64_t elems, void* stream);
 int ggq_swiglu_backward(const void* gate, const void* up, const void* dh, void* dgate, void* dup, int64_t elems, void* stream);
 
+/* router_topk_indices (fast_moe_ranking.py:197-271; Triton kernel :163-194, key order :71-80 and :119-160): per
+ * token the top_k experts of up to 256 router scores, best first, equal scores in ascending expert index.
+ *   score_function 0: the logit itself (bf16 or fp32); 1: sqrt(softplus(logit)) in fp32 plus the optional
+ *   correction_bias float[num_experts] (:88-102).  indices int64 [tokens, top_k].
+ * Optional routing weights of the selected experts (weights may be NULL / weights_mode 0):
+ *   1: softmax over the selected logits in fp32, stored in the logits' type (_qwen_router_forward, :273-284);
+ *   2: sqrt(softplus(logit)) / (sum + 1e-20) * routed_scaling as fp32 (_deepseek_topk_router_forward, :287-303).
+ * num_experts a multiple of 4, at most 256; top_k at most 8. */
+int ggq_router_topk(const void* logits, int logits_are_bf16, int64_t tokens, int num_experts, int top_k, const float* correction_bias,
+                    int score_function, int64_t* indices, void* weights, int weights_mode, float routed_scaling, void* stream);
+
 /* _packed_q8_linear_cross_entropy_forward (gguf_liger_loss.py:38-186): chunked mmq -> Liger
  * cross-entropy -> mmq_grad_input, without the [chunk, vocab] logits tensor.  labels int64 [rows];
  * loss_per_row fp32 [rows] (already divided by the number of non-ignored rows when reduction_mean);

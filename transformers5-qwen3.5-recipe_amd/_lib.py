@@ -39,6 +39,7 @@ SIGNATURES: dict[str, tuple] = {
     "ggq_route_gather_backward": (_I, [_P, _P, _P, _L, _I, _I, _P]),
     "ggq_route_combine_forward": (_I, [_P, _P, _I, _P, _P, _L, _I, _I, _P]),
     "ggq_route_combine_backward": (_I, [_P, _P, _I, _P, _P, _P, _P, _L, _I, _I, _P]),
+    "ggq_router_topk": (_I, [_P, _I, _L, _I, _I, _P, _I, _P, _P, _I, _F, _P]),
     "ggq_swiglu_forward": (_I, [_P, _P, _P, _L, _P]),
     "ggq_swiglu_backward": (_I, [_P, _P, _P, _P, _P, _L, _P]),
     "ggq_lmhead_ce_workspace_bytes": (_L, [_L, _L, _L, _L]),

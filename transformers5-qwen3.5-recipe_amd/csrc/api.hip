@@ -354,6 +354,12 @@ int ggq_swiglu_backward(const void* gate, const void* up, const void* dh, void* 
     return swiglu_bwd(gate, up, dh, dgate, dup, elems, as_stream(stream));
 }
 
+int ggq_router_topk(const void* logits, int logits_are_bf16, int64_t tokens, int num_experts, int top_k, const float* correction_bias,
+                    int score_function, int64_t* indices, void* weights, int weights_mode, float routed_scaling, void* stream) {
+    return router_topk(logits, logits_are_bf16, tokens, num_experts, top_k, correction_bias, score_function, indices, weights,
+                       weights_mode, routed_scaling, as_stream(stream));
+}
+
 // ---------------------------------------------------------------------------------------------------
 int64_t ggq_lmhead_ce_workspace_bytes(int64_t rows, int64_t vocab, int64_t hidden_dim, int64_t chunk) {
     return lmhead_ce_workspace_bytes(rows, vocab, hidden_dim, chunk);

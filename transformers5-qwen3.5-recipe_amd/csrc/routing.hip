@@ -416,4 +416,108 @@ int swiglu_bwd(const void* gate, const void* up, const void* dh, void* dgate, vo
     return check_launch("swiglu_backward");
 }
 
+// ------------------------------------------------------------------------------------------------
+// Router top-k: per token the top_k best of up to 256 expert scores, best first, equal scores in ascending
+// expert index.  One wave per token; lane l holds experts 4l .. 4l+3.  The order is that of the packed key
+// (monotone map of the fp32 score bits) << 16 | (256 - expert): the maximum of the keys is the best score and,
+// among equal scores, the smallest index.  Score functions: 0 = the logit itself (bf16 logits compare as the
+// fp32 values they are), 1 = sqrt(softplus(logit)) in fp32 plus an optional per-expert bias.
+// Optional routing weights of the selected experts: 1 = softmax over the selected logits in fp32, stored in the
+// logits' type; 2 = sqrt(softplus(logit)) (no bias) / (sum + 1e-20) * scale, stored as fp32.
+__device__ __forceinline__ uint32_t float_order_key(float v) {
+    const uint32_t b = __builtin_bit_cast(uint32_t, v);
+    return b ^ ((b & 0x80000000u) ? 0xFFFFFFFFu : 0x80000000u);
+}
+__device__ __forceinline__ float sqrt_softplus(float x) { return sqrtf(fmaxf(x, 0.0f) + logf(1.0f + expf(-fabsf(x)))); }
+
+template <bool BF16>
+__global__ __launch_bounds__(256) void router_topk_kernel(const void* logits, int64_t tokens, int experts, int top_k, const float* bias,
+                                                          int score_fn, int64_t* indices, void* weights, int weights_mode, float scale) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= tokens) return;
+    float v[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) v[j] = 0.0f;
+    const int e0 = 4 * lane;
+    if (e0 < experts) {  // experts is a multiple of 4: a lane holds four experts or none
+        if (BF16) {
+            const uint2 r = *(const uint2*)((const bf16_t*)logits + row * experts + e0);
+            v[0] = bf16_lo(r.x), v[1] = bf16_hi(r.x), v[2] = bf16_lo(r.y), v[3] = bf16_hi(r.y);
+        } else {
+            const float4 r = *(const float4*)((const float*)logits + row * experts + e0);
+            v[0] = r.x, v[1] = r.y, v[2] = r.z, v[3] = r.w;
+        }
+    }
+    uint64_t key[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float sc = v[j];
+        if (score_fn == 1) {
+            sc = sqrt_softplus(sc);
+            if (bias && e0 < experts) sc += bias[e0 + j];
+        }
+        key[j] = e0 < experts ? ((uint64_t)float_order_key(sc) << 16) | (uint64_t)(256 - (e0 + j)) : 0ull;
+    }
+    float my_logit = 0.0f;  // lane t ends up with the logit of the rank-t expert
+    for (int t = 0; t < top_k; t++) {
+        uint64_t best = key[0];
+#pragma unroll
+        for (int j = 1; j < 4; j++) best = key[j] > best ? key[j] : best;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const uint32_t lo = __shfl_xor((uint32_t)best, off), hi = __shfl_xor((uint32_t)(best >> 32), off);
+            const uint64_t other = ((uint64_t)hi << 32) | lo;
+            best = other > best ? other : best;
+        }
+        const int expert = 256 - (int)(best & 0xFFFFu);
+        float lg = 0.0f;  // the winner's logit, from the lane that holds it
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (key[j] == best && best != 0ull) lg = v[j], key[j] = 0ull;
+        // (one lane at most had the key: packed keys are distinct)
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) lg += __shfl_xor(lg, off);
+        if (lane == t) my_logit = lg;
+        if (lane == 0) indices[row * top_k + t] = expert;
+    }
+    if (weights_mode == 0 || !weights) return;
+    const bool in = lane < top_k;
+    if (weights_mode == 1) {
+        float m = in ? my_logit : -INFINITY;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+        const float ex = in ? expf(my_logit - m) : 0.0f;
+        float sum = ex;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+        const float w = ex / sum;
+        if (in) {
+            if (BF16) ((bf16_t*)weights)[row * top_k + lane] = to_bf16(w);
+            else ((float*)weights)[row * top_k + lane] = w;
+        }
+    } else {
+        const float sc = in ? sqrt_softplus(my_logit) : 0.0f;
+        float sum = sc;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+        if (in) ((float*)weights)[row * top_k + lane] = sc / (sum + 1e-20f) * scale;
+    }
+}
+
+int router_topk(const void* logits, int logits_are_bf16, int64_t tokens, int num_experts, int top_k, const float* bias, int score_fn,
+                int64_t* indices, void* weights, int weights_mode, float scale, hipStream_t s) {
+    if (!logits || !indices) return set_error(GGQ_ERR_NULL, "router_topk: null logits or indices");
+    if (tokens < 0 || num_experts <= 0 || num_experts > 256 || (num_experts & 3) || top_k <= 0 || top_k > 8 || top_k > num_experts)
+        return set_error(GGQ_ERR_SHAPE, "router_topk: supports up to 256 experts (a multiple of 4) and top_k <= 8, got experts=%d top_k=%d", num_experts, top_k);
+    if (score_fn < 0 || score_fn > 1 || weights_mode < 0 || weights_mode > 2) return set_error(GGQ_ERR_SHAPE, "router_topk: unknown score function or weights mode");
+    if (bias && score_fn != 1) return set_error(GGQ_ERR_SHAPE, "router_topk: a correction bias needs sqrt-softplus scoring");
+    if (((uintptr_t)logits & 15) != 0) return set_error(GGQ_ERR_ALIGN, "router_topk: logits must be 16-byte aligned");
+    if (tokens == 0) return GGQ_OK;
+    const unsigned grid = (unsigned)((tokens + 3) / 4);
+    if (logits_are_bf16) hipLaunchKernelGGL(router_topk_kernel<true>, dim3(grid), dim3(256), 0, s, logits, tokens, num_experts, top_k, bias, score_fn, indices, weights, weights_mode, scale);
+    else hipLaunchKernelGGL(router_topk_kernel<false>, dim3(grid), dim3(256), 0, s, logits, tokens, num_experts, top_k, bias, score_fn, indices, weights, weights_mode, scale);
+    return check_launch("router_topk");
+}
+
 }  // namespace ggq
