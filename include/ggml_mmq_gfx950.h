@@ -127,6 +127,11 @@ int ggq_route_combine_backward(const void* expert_out, const void* weights, int 
 int ggq_swiglu_forward(const void* gate, const void* up, void* h, int64_t elems, void* stream);
 int ggq_swiglu_backward(const void* gate, const void* up, const void* dh, void* dgate, void* dup, int64_t elems, void* stream);
 
+/* The DeepSeek form of the same step (config.swiglu_limit; pinned by test_deepseek_v4_moe_lora.py:184-199):
+ * h = silu(min(gate, limit)) * clamp(up, -limit, limit), and its autograd (no gradient into a clamped input). */
+int ggq_swiglu_clamped_forward(const void* gate, const void* up, void* h, int64_t elems, float limit, void* stream);
+int ggq_swiglu_clamped_backward(const void* gate, const void* up, const void* dh, void* dgate, void* dup, int64_t elems, float limit, void* stream);
+
 /* router_topk_indices (fast_moe_ranking.py:197-271; Triton kernel :163-194, key order :71-80 and :119-160): per
  * token the top_k experts of up to 256 router scores, best first, equal scores in ascending expert index.
  *   score_function 0: the logit itself (bf16 or fp32); 1: sqrt(softplus(logit)) in fp32 plus the optional

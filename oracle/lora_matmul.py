@@ -95,7 +95,11 @@ def grouped_lora_linear(x, w_all, experts, offsets, a_all=None, b_all=None, s=1.
     return res
 
 
-def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+def silu_mul(gate: torch.Tensor, up: torch.Tensor, limit: float | None = None) -> torch.Tensor:
+    """silu(gate) * up; with ``limit`` the DeepSeek form act(gate.clamp(max=limit)) * up.clamp(-limit, limit)
+    (the expression test_deepseek_v4_moe_lora.py:194-196 compares the module with)."""
+    if limit is not None:
+        gate, up = gate.clamp(max=limit), up.clamp(min=-limit, max=limit)
     return gate * torch.sigmoid(gate) * up
 
 

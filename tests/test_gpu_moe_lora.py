@@ -256,3 +256,28 @@ def test_moe_guards(pkg, dev):
     assert ml._complete_group_sizes(sizes, ids, 4).tolist() == [3, 3, 0, 0]
     with pytest.raises(ValueError):
         ml._group_sizes_from_offsets(offs.long())
+
+
+@pytest.mark.parametrize("limit", [7.0, 0.05])
+def test_clamped_swiglu_forward_and_gradients(pkg, dev, limit):
+    # DeepSeek's expert activation (config.swiglu_limit): the probe of test_deepseek_v4_moe_lora.py:184-199 (inputs four
+    # times the limit either way) and random inputs around the limit, against autograd of the clamp expression
+    ml = pkg.fast_moe_lora
+    gen = torch.Generator().manual_seed(4321)
+    probe = torch.tensor([[limit * 4, -limit * 4] * 4], dtype=torch.bfloat16)
+    gate = torch.cat([probe, bf16_randn(gen, 63, 8) * limit * 2]).to(torch.bfloat16)
+    up = torch.cat([probe, bf16_randn(gen, 63, 8) * limit * 2]).to(torch.bfloat16)
+    dh = bf16_randn(gen, 64, 8).to(torch.bfloat16)
+    g64, u64 = gate.double().requires_grad_(True), up.double().requires_grad_(True)
+    want = ref.silu_mul(g64, u64, limit)
+    want.backward(dh.double())
+    gd, ud = gate.to(dev).requires_grad_(True), up.to(dev).requires_grad_(True)
+    h = ml.swiglu(gd, ud, limit)
+    h.backward(dh.to(dev))
+    assert_close_bf16(h, want.detach(), "clamped h")
+    assert_close_bf16(gd.grad, g64.grad, "clamped dgate")
+    assert_close_bf16(ud.grad, u64.grad, "clamped dup")
+    # the clamped probe entries: h = silu(limit) * (+-limit), and no gradient reaches a clamped gate or up
+    assert float(gd.grad[0, 0]) == 0.0 and float(ud.grad[0, 0]) == 0.0 and float(ud.grad[0, 1]) == 0.0
+    with pytest.raises(ValueError):
+        ml.swiglu(gd, ud, 0.0)

@@ -42,6 +42,8 @@ SIGNATURES: dict[str, tuple] = {
     "ggq_router_topk": (_I, [_P, _I, _L, _I, _I, _P, _I, _P, _P, _I, _F, _P]),
     "ggq_swiglu_forward": (_I, [_P, _P, _P, _L, _P]),
     "ggq_swiglu_backward": (_I, [_P, _P, _P, _P, _P, _L, _P]),
+    "ggq_swiglu_clamped_forward": (_I, [_P, _P, _P, _L, _F, _P]),
+    "ggq_swiglu_clamped_backward": (_I, [_P, _P, _P, _P, _P, _L, _F, _P]),
     "ggq_lmhead_ce_workspace_bytes": (_L, [_L, _L, _L, _L]),
     "ggq_lmhead_cross_entropy": (_I, [_I, _P, _P, _P, _L, _L, _L, _L, _L, _I, _P, _P, _P, _P, _P, _L, _P]),
 }

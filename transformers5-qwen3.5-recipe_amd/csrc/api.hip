@@ -346,12 +346,24 @@ int ggq_route_combine_backward(const void* expert_out, const void* weights, int 
 
 int ggq_swiglu_forward(const void* gate, const void* up, void* h, int64_t elems, void* stream) {
     if (!gate || !up || !h) return set_error(GGQ_ERR_NULL, "swiglu_forward: null pointer");
-    return swiglu_fwd(gate, up, h, elems, as_stream(stream));
+    return swiglu_fwd(gate, up, h, elems, 0.0f, as_stream(stream));
+}
+
+int ggq_swiglu_clamped_forward(const void* gate, const void* up, void* h, int64_t elems, float limit, void* stream) {
+    if (!gate || !up || !h) return set_error(GGQ_ERR_NULL, "swiglu_clamped_forward: null pointer");
+    if (!(limit > 0.0f)) return set_error(GGQ_ERR_SHAPE, "swiglu_clamped_forward: the limit must be positive");
+    return swiglu_fwd(gate, up, h, elems, limit, as_stream(stream));
 }
 
 int ggq_swiglu_backward(const void* gate, const void* up, const void* dh, void* dgate, void* dup, int64_t elems, void* stream) {
     if (!gate || !up || !dh || !dgate || !dup) return set_error(GGQ_ERR_NULL, "swiglu_backward: null pointer");
-    return swiglu_bwd(gate, up, dh, dgate, dup, elems, as_stream(stream));
+    return swiglu_bwd(gate, up, dh, dgate, dup, elems, 0.0f, as_stream(stream));
+}
+
+int ggq_swiglu_clamped_backward(const void* gate, const void* up, const void* dh, void* dgate, void* dup, int64_t elems, float limit, void* stream) {
+    if (!gate || !up || !dh || !dgate || !dup) return set_error(GGQ_ERR_NULL, "swiglu_clamped_backward: null pointer");
+    if (!(limit > 0.0f)) return set_error(GGQ_ERR_SHAPE, "swiglu_clamped_backward: the limit must be positive");
+    return swiglu_bwd(gate, up, dh, dgate, dup, elems, limit, as_stream(stream));
 }
 
 int ggq_router_topk(const void* logits, int logits_are_bf16, int64_t tokens, int num_experts, int top_k, const float* correction_bias,

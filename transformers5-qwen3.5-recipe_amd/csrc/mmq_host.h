@@ -133,8 +133,8 @@ int route_combine_fwd(const void* expert_out, const void* weights, int w_is_bf16
 int route_combine_bwd(const void* expert_out, const void* weights, int w_is_bf16, const int64_t* permutation, const void* grad_out, void* grad_expert_out, void* grad_weights, int64_t tokens, int top_k, int hidden_dim, hipStream_t s);
 int router_topk(const void* logits, int logits_are_bf16, int64_t tokens, int num_experts, int top_k, const float* bias, int score_fn,
                 int64_t* indices, void* weights, int weights_mode, float scale, hipStream_t s);
-int swiglu_fwd(const void* gate, const void* up, void* h, int64_t elems, hipStream_t s);
-int swiglu_bwd(const void* gate, const void* up, const void* dh, void* dgate, void* dup, int64_t elems, hipStream_t s);
+int swiglu_fwd(const void* gate, const void* up, void* h, int64_t elems, float limit, hipStream_t s);
+int swiglu_bwd(const void* gate, const void* up, const void* dh, void* dgate, void* dup, int64_t elems, float limit, hipStream_t s);
 
 int64_t lmhead_ce_workspace_bytes(int64_t rows, int64_t vocab, int64_t hidden, int64_t chunk);
 int lmhead_ce(int qt, const void* hidden, const void* packed, const int64_t* labels, int64_t rows, int64_t vocab,

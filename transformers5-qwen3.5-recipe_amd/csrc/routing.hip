@@ -360,22 +360,27 @@ int route_combine_bwd(const void* expert_out, const void* weights, int w_is_bf16
 
 // ------------------------------------------------------------------------------------------------
 // SiLU-gated product of the expert FFN: h = silu(gate) * up, and its backward.
-__global__ __launch_bounds__(256) void swiglu_fwd_kernel(const uint4* gate, const uint4* up, uint4* h, int64_t chunks) {
+// limit > 0 selects the clamped form: the gate is cut off above `limit`, up is kept within [-limit, limit].
+__global__ __launch_bounds__(256) void swiglu_fwd_kernel(const uint4* gate, const uint4* up, uint4* h, int64_t chunks, float limit) {
+    const float hi = limit > 0.0f ? limit : INFINITY;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < chunks; i += (int64_t)gridDim.x * 256) {
         const uint4 g = gate[i], u = up[i];
         const uint32_t gv[4] = {g.x, g.y, g.z, g.w}, uv[4] = {u.x, u.y, u.z, u.w};
         uint32_t r[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            const float g0 = bf16_lo(gv[e]), g1 = bf16_hi(gv[e]);
+            const float g0 = fminf(bf16_lo(gv[e]), hi), g1 = fminf(bf16_hi(gv[e]), hi);
+            const float u0 = fminf(fmaxf(bf16_lo(uv[e]), -hi), hi), u1 = fminf(fmaxf(bf16_hi(uv[e]), -hi), hi);
             const float s0 = g0 / (1.0f + __expf(-g0)), s1 = g1 / (1.0f + __expf(-g1));
-            r[e] = pack_bf16(s0 * bf16_lo(uv[e]), s1 * bf16_hi(uv[e]));
+            r[e] = pack_bf16(s0 * u0, s1 * u1);
         }
         h[i] = make_uint4(r[0], r[1], r[2], r[3]);
     }
 }
 
-__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint4* gate, const uint4* up, const uint4* dh, uint4* dgate, uint4* dup, int64_t chunks) {
+// (clamped form: no gradient flows into a gate above the limit or an up outside [-limit, limit])
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint4* gate, const uint4* up, const uint4* dh, uint4* dgate, uint4* dup, int64_t chunks, float limit) {
+    const float hi = limit > 0.0f ? limit : INFINITY;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < chunks; i += (int64_t)gridDim.x * 256) {
         const uint4 g = gate[i], u = up[i], d = dh[i];
         const uint32_t gv[4] = {g.x, g.y, g.z, g.w}, uv[4] = {u.x, u.y, u.z, u.w}, dv[4] = {d.x, d.y, d.z, d.w};
@@ -385,12 +390,13 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint4* gate, cons
             float og[2], ou[2];
 #pragma unroll
             for (int hlf = 0; hlf < 2; hlf++) {
-                const float x = hlf ? bf16_hi(gv[e]) : bf16_lo(gv[e]);
-                const float uu = hlf ? bf16_hi(uv[e]) : bf16_lo(uv[e]);
+                const float xr = hlf ? bf16_hi(gv[e]) : bf16_lo(gv[e]);
+                const float ur = hlf ? bf16_hi(uv[e]) : bf16_lo(uv[e]);
                 const float dd = hlf ? bf16_hi(dv[e]) : bf16_lo(dv[e]);
+                const float x = fminf(xr, hi), uu = fminf(fmaxf(ur, -hi), hi);
                 const float sig = 1.0f / (1.0f + __expf(-x));
-                og[hlf] = dd * uu * (sig * (1.0f + x * (1.0f - sig)));
-                ou[hlf] = dd * x * sig;
+                og[hlf] = xr <= hi ? dd * uu * (sig * (1.0f + x * (1.0f - sig))) : 0.0f;
+                ou[hlf] = (ur >= -hi && ur <= hi) ? dd * x * sig : 0.0f;
             }
             rg[e] = pack_bf16(og[0], og[1]);
             ru[e] = pack_bf16(ou[0], ou[1]);
@@ -400,19 +406,19 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint4* gate, cons
     }
 }
 
-int swiglu_fwd(const void* gate, const void* up, void* h, int64_t elems, hipStream_t s) {
+int swiglu_fwd(const void* gate, const void* up, void* h, int64_t elems, float limit, hipStream_t s) {
     if (elems % 8) return set_error(GGQ_ERR_SHAPE, "swiglu: element count must be a multiple of 8");
     if (((uintptr_t)gate | (uintptr_t)up | (uintptr_t)h) & 15) return set_error(GGQ_ERR_ALIGN, "swiglu: buffers must be 16-byte aligned");
     if (elems == 0) return GGQ_OK;
-    hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(stream_grid(elems / 8)), dim3(256), 0, s, (const uint4*)gate, (const uint4*)up, (uint4*)h, elems / 8);
+    hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(stream_grid(elems / 8)), dim3(256), 0, s, (const uint4*)gate, (const uint4*)up, (uint4*)h, elems / 8, limit);
     return check_launch("swiglu_forward");
 }
 
-int swiglu_bwd(const void* gate, const void* up, const void* dh, void* dgate, void* dup, int64_t elems, hipStream_t s) {
+int swiglu_bwd(const void* gate, const void* up, const void* dh, void* dgate, void* dup, int64_t elems, float limit, hipStream_t s) {
     if (elems % 8) return set_error(GGQ_ERR_SHAPE, "swiglu: element count must be a multiple of 8");
     if (((uintptr_t)gate | (uintptr_t)up | (uintptr_t)dh | (uintptr_t)dgate | (uintptr_t)dup) & 15) return set_error(GGQ_ERR_ALIGN, "swiglu: buffers must be 16-byte aligned");
     if (elems == 0) return GGQ_OK;
-    hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(stream_grid(elems / 8)), dim3(256), 0, s, (const uint4*)gate, (const uint4*)up, (const uint4*)dh, (uint4*)dgate, (uint4*)dup, elems / 8);
+    hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(stream_grid(elems / 8)), dim3(256), 0, s, (const uint4*)gate, (const uint4*)up, (const uint4*)dh, (uint4*)dgate, (uint4*)dup, elems / 8, limit);
     return check_launch("swiglu_backward");
 }
 

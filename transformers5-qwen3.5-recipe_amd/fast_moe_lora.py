@@ -186,12 +186,17 @@ def grouped_lora_mmq_pair(hidden_states, first_payload, second_payload, expert_i
 
 class _SwiGLU(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, gate, up):
+    def forward(ctx, gate, up, limit):
         _lib.require_device_tensor(gate, "gate", torch.bfloat16)
         _lib.require_device_tensor(up, "up", torch.bfloat16)
         h = torch.empty_like(gate)
-        _lib.check(_lib.load().ggq_swiglu_forward(gate.data_ptr(), up.data_ptr(), h.data_ptr(), gate.numel(), _lib.stream_handle(gate.device)))
+        lib, stream = _lib.load(), _lib.stream_handle(gate.device)
+        if limit is None:
+            _lib.check(lib.ggq_swiglu_forward(gate.data_ptr(), up.data_ptr(), h.data_ptr(), gate.numel(), stream))
+        else:
+            _lib.check(lib.ggq_swiglu_clamped_forward(gate.data_ptr(), up.data_ptr(), h.data_ptr(), gate.numel(), float(limit), stream))
         ctx.save_for_backward(gate, up)
+        ctx.limit = limit
         return h
 
     @staticmethod
@@ -199,14 +204,22 @@ class _SwiGLU(torch.autograd.Function):
         gate, up = ctx.saved_tensors
         dh = dh.contiguous()
         dgate, dup = torch.empty_like(gate), torch.empty_like(up)
-        _lib.check(_lib.load().ggq_swiglu_backward(gate.data_ptr(), up.data_ptr(), dh.data_ptr(), dgate.data_ptr(), dup.data_ptr(),
-                                                   gate.numel(), _lib.stream_handle(gate.device)))
-        return dgate, dup
+        lib, stream = _lib.load(), _lib.stream_handle(gate.device)
+        if ctx.limit is None:
+            _lib.check(lib.ggq_swiglu_backward(gate.data_ptr(), up.data_ptr(), dh.data_ptr(), dgate.data_ptr(), dup.data_ptr(), gate.numel(), stream))
+        else:
+            _lib.check(lib.ggq_swiglu_clamped_backward(gate.data_ptr(), up.data_ptr(), dh.data_ptr(), dgate.data_ptr(), dup.data_ptr(),
+                                                       gate.numel(), float(ctx.limit), stream))
+        return dgate, dup, None
 
 
-def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
-    """silu(gate) * up (the fork's ``_apply_split_gate`` for ``hidden_act="silu"``, fast_moe_lora.py:747)."""
-    return _SwiGLU.apply(gate, up)
+def swiglu(gate: torch.Tensor, up: torch.Tensor, limit: float | None = None) -> torch.Tensor:
+    """silu(gate) * up (the fork's ``_apply_split_gate`` for ``hidden_act="silu"``, fast_moe_lora.py:747); with
+    ``limit`` the DeepSeek form silu(min(gate, limit)) * clamp(up, -limit, limit) (``config.swiglu_limit``,
+    test_deepseek_v4_moe_lora.py:184-199)."""
+    if limit is not None and not limit > 0:
+        raise ValueError(f"swiglu limit must be positive, got {limit}")
+    return _SwiGLU.apply(gate, up, limit)
 
 
 # ------------------------------------------------------------------------------------------------
@@ -249,8 +262,9 @@ class GGUFExperts(torch.nn.Module):
     has_gate = True
 
     def __init__(self, gate_proj: GGUFQuantizedTensor, up_proj: GGUFQuantizedTensor, down_proj: GGUFQuantizedTensor,
-                 compute_dtype: torch.dtype = torch.bfloat16):
+                 compute_dtype: torch.dtype = torch.bfloat16, swiglu_limit: float | None = None):
         super().__init__()
+        self.swiglu_limit = swiglu_limit  # DeepSeek's config.swiglu_limit; None: plain silu(gate) * up
         e, i, h = gate_proj.logical_shape
         if tuple(up_proj.logical_shape) != (e, i, h) or tuple(down_proj.logical_shape) != (e, h, i):
             raise ValueError("expert projections must be gate/up [E,I,H] and down [E,H,I]")
@@ -268,7 +282,7 @@ class GGUFExperts(torch.nn.Module):
         return _ExpertExecutionPlan(self._all_experts, routing_plan.expert_end_offsets, None)
 
     def _apply_split_gate(self, gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
-        return swiglu(gate, up)
+        return swiglu(gate, up, self.swiglu_limit)
 
     def forward(self, hidden_states, top_k_index, top_k_weights, lora_weights: _ExpertLoraWeights | None = None):
         return qwen3_5_moe_gguf_mmq_lora_forward(self, hidden_states, top_k_index, top_k_weights, lora_weights)
