@@ -97,6 +97,16 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
                                   const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b, void* ws,
                                   int64_t ws_bytes, void* stream);
 
+/* torch_ggml_ops.fixed_grouped_mmq (deepseek_v4_lora.py:91-124: DeepSeek's frozen eight-group output projection) and
+ * its input gradient: x [rows, groups, k] bf16, packed_groups [groups, n_group, row bytes], y [rows, groups, n_group];
+ * y[:, g, :] = x[:, g, :] . W_g^T.  Each group runs as the dense launch over its strided rows, so the results are
+ * bit-identical to ggq_mmq / ggq_mmq_grad_input on contiguous per-group copies (the relation the reference pins,
+ * test_deepseek_v4_lora.py:131-151). */
+int ggq_fixed_grouped_mmq(const void* x, const void* packed_groups, int qt, int64_t rows, int groups, int64_t n_group, int64_t k, void* y,
+                          void* stream);
+int ggq_fixed_grouped_mmq_grad_input(const void* dy, const void* packed_groups, int qt, int64_t rows, int groups, int64_t n_group, int64_t k,
+                                     void* dx, void* stream);
+
 /* prepare_expert_routing (fast_moe_routing.py:379-428: torch.sort of the flat top-k ids + inverse
  * permutation kernel :88-98) and the grouped-execution offsets of the expert module
  * (fast_moe_lora.py:709-719, 652-672).  Stable order: ties keep ascending route index.

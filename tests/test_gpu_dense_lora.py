@@ -118,3 +118,31 @@ def test_dense_guards(pkg, dev):
     y = fl.mmq(x.requires_grad_(True), p, gb.Q4_K, 8)
     (g,) = torch.autograd.grad(y.sum(), x, create_graph=False)
     assert g.shape == x.shape
+
+
+@pytest.mark.parametrize("qt,lead,groups,n_group,k", [(gb.Q8_0, (2,), 8, 128, 512), (gb.Q8_0, (3, 43), 8, 64, 256), (gb.Q4_K, (130,), 4, 128, 512)])
+def test_fixed_grouped_mmq_equals_per_group_dense_calls(pkg, dev, qt, lead, groups, n_group, k):
+    # the relation the reference pins for DeepSeek's eight-group frozen projection (test_deepseek_v4_lora.py:101-151):
+    # output and input gradient equal, bit for bit, the per-group dense op on contiguous slices; and both sit on the oracle
+    fl = pkg.fast_lora
+    gen = torch.Generator().manual_seed(4242)
+    payload = np.stack([make_payload(900 + g, qt, n_group, k) for g in range(groups)])
+    x = bf16_randn(gen, *lead, groups, k)
+    dy = bf16_randn(gen, *lead, groups, n_group)
+    pd = torch.from_numpy(payload).to(dev)
+    xd = x.to(dev).requires_grad_(True)
+    y = fl.fixed_grouped_mmq(xd, pd, qt)
+    y.backward(dy.to(dev))
+    assert y.shape == (*lead, groups, n_group)
+    xr = x.to(dev).requires_grad_(True)
+    want = torch.stack([fl.mmq(xr[..., g, :].contiguous(), pd[g].clone(), qt, n_group) for g in range(groups)], dim=-2)
+    want.backward(dy.to(dev))
+    assert torch.equal(y, want)
+    assert torch.equal(xd.grad, xr.grad)
+    w = ref.weights_bf16(payload, qt)
+    for g in (0, groups - 1):
+        res = ref.lora_linear(x[..., g, :].reshape(-1, k), w[g], dy=dy[..., g, :].reshape(-1, n_group))
+        assert_close_bf16(y[..., g, :].reshape(-1, n_group), res["y"], "fixed grouped y")
+        assert_close_bf16(xd.grad[..., g, :].reshape(-1, k), res["dx"], "fixed grouped dx")
+    with pytest.raises(ValueError):
+        fl.fixed_grouped_mmq(xd[..., :2, :].contiguous(), pd, qt)

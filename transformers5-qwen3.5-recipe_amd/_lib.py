@@ -28,6 +28,8 @@ SIGNATURES: dict[str, tuple] = {
     "ggq_dequantize": (_I, [_I, _P, _L, _L, _P, _I, _P]),
     "ggq_mmq": (_I, [_P, _P, _I, _L, _L, _L, _P, _P]),
     "ggq_mmq_grad_input": (_I, [_P, _P, _I, _L, _L, _L, _P, _P]),
+    "ggq_fixed_grouped_mmq": (_I, [_P, _P, _I, _L, _I, _L, _L, _P, _P]),
+    "ggq_fixed_grouped_mmq_grad_input": (_I, [_P, _P, _I, _L, _I, _L, _L, _P, _P]),
     "ggq_lora_workspace_bytes": (_L, [_L, _L, _L, _L, _L, _I]),
     "ggq_lora_mmq_forward": (_I, [_P, _P, _I, _L, _L, _L, _P, _P, _I, _F, _P, _P, _P, _L, _P]),
     "ggq_lora_mmq_backward": (_I, [_P, _P, _I, _L, _L, _L, _P, _P, _P, _P, _I, _F, _P, _P, _P, _P, _L, _P]),

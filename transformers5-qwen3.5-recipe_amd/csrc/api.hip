@@ -130,6 +130,40 @@ int ggq_mmq_grad_input(const void* dy, const void* packed, int qt, int64_t m, in
                                          nullptr, nullptr, 0, 0.f, dx, nullptr, nullptr, nullptr, 0, stream);
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Fixed groups: x [rows, groups, k], one packed [n_group, k] matrix per group, y [rows, groups, n_group].  Group g is
+// a dense matmul over the strided rows x[:, g, :]; it runs as that launch (same tiles, same arithmetic as ggq_mmq on a
+// contiguous copy), so the results are bit-identical to the per-group dense calls.
+static int fixed_grouped(const char* what, int mode, const void* in, const void* packed, int qt, int64_t rows, int groups, int64_t n_group,
+                         int64_t k, void* out, hipStream_t s) {
+    if (rows < 0 || groups <= 0 || n_group <= 0 || k <= 0 || rows >= (1ll << 31) || n_group >= (1ll << 30) || k >= (1ll << 30) ||
+        (int64_t)groups * std::max(n_group, k) >= (1ll << 31))
+        return set_error(GGQ_ERR_SHAPE, "%s: bad shape rows=%lld groups=%d n_group=%lld k=%lld", what, (long long)rows, groups, (long long)n_group, (long long)k);
+    if (int rc = check_weights(what, qt, packed, k)) return rc;
+    if (!in || !out) return set_error(GGQ_ERR_NULL, "%s: null activation or output pointer", what);
+    if (rows == 0) return GGQ_OK;
+    const int64_t in_cols = mode == kModeNT ? k : n_group, out_cols = mode == kModeNT ? n_group : k;
+    for (int g = 0; g < groups; g++) {
+        MmqParams p;
+        if (int rc = init_params(p, qt, mode, (int)rows, (int)n_group, (int)k, 1, kShapeTall)) return rc;
+        p.a[0] = (const bf16_t*)in + g * in_cols, p.lda = groups * in_cols;
+        p.w[0] = (const uint8_t*)packed + g * p.w_expert_bytes;
+        p.c[0] = (bf16_t*)out + g * out_cols, p.ldc = groups * out_cols;
+        if (int rc = launch_mmq(qt, mode, kEpiStore, p, s)) return rc;
+    }
+    return GGQ_OK;
+}
+
+int ggq_fixed_grouped_mmq(const void* x, const void* packed_groups, int qt, int64_t rows, int groups, int64_t n_group, int64_t k, void* y,
+                          void* stream) {
+    return fixed_grouped("fixed_grouped_mmq", kModeNT, x, packed_groups, qt, rows, groups, n_group, k, y, as_stream(stream));
+}
+
+int ggq_fixed_grouped_mmq_grad_input(const void* dy, const void* packed_groups, int qt, int64_t rows, int groups, int64_t n_group, int64_t k,
+                                     void* dx, void* stream) {
+    return fixed_grouped("fixed_grouped_mmq_grad_input", kModeNN, dy, packed_groups, qt, rows, groups, n_group, k, dx, as_stream(stream));
+}
+
 // Forward of one projection (or a gate/up pair) over expert-sorted rows, optional LoRA fused.
 // groups == 0 means dense: one group of all rows using expert 0.
 int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void* packed2, const int64_t* expert_ids,

@@ -87,6 +87,45 @@ def mmq(x: torch.Tensor, payload: torch.Tensor, quant_type: int, out_features: i
     return _Mmq.apply(x, payload, int(quant_type), int(out_features))
 
 
+class _FixedGroupedMmq(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, packed_groups, quant_type):
+        _lib.require_device_tensor(x, "fixed grouped input", torch.bfloat16)
+        _lib.require_device_tensor(packed_groups, "packed groups", torch.uint8)
+        if x.ndim < 2 or packed_groups.ndim != 3 or x.shape[-2] != packed_groups.shape[0]:
+            raise ValueError(f"fixed grouped MMQ takes [..., groups, k] and [groups, n, bytes], got {tuple(x.shape)} and {tuple(packed_groups.shape)}")
+        groups, n_group, k = packed_groups.shape[0], packed_groups.shape[1], x.shape[-1]
+        _check_packed(packed_groups[0], quant_type, n_group, k, "fixed grouped MMQ")
+        rows = x.numel() // (groups * k)
+        y = torch.empty(*x.shape[:-1], n_group, dtype=torch.bfloat16, device=x.device)
+        _lib.check(_lib.load().ggq_fixed_grouped_mmq(x.data_ptr(), packed_groups.data_ptr(), quant_type, rows, groups, n_group, k, y.data_ptr(),
+                                                     _lib.stream_handle(x.device)))
+        ctx.save_for_backward(packed_groups)
+        ctx.quant_type, ctx.k = quant_type, k
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        if torch.is_grad_enabled():
+            raise RuntimeError("packed MMQ does not support higher-order gradients")
+        if not ctx.needs_input_grad[0]:
+            return None, None, None
+        (packed_groups,) = ctx.saved_tensors
+        g = grad_output.contiguous()
+        groups, n_group = packed_groups.shape[0], packed_groups.shape[1]
+        rows = g.numel() // (groups * n_group)
+        dx = torch.empty(*g.shape[:-1], ctx.k, dtype=torch.bfloat16, device=g.device)
+        _lib.check(_lib.load().ggq_fixed_grouped_mmq_grad_input(g.data_ptr(), packed_groups.data_ptr(), ctx.quant_type, rows, groups, n_group, ctx.k,
+                                                                dx.data_ptr(), _lib.stream_handle(g.device)))
+        return dx, None, None
+
+
+def fixed_grouped_mmq(x: torch.Tensor, packed_groups: torch.Tensor, quant_type: int = 8) -> torch.Tensor:
+    """[..., groups, k] x packed [groups, n, bytes] -> [..., groups, n]: every group its own frozen packed matrix (the
+    reference's ``torch_ggml_ops.fixed_grouped_mmq``, deepseek_v4_lora.py:91-124; Q8_0 there, any supported type here)."""
+    return _FixedGroupedMmq.apply(x, packed_groups.as_subclass(torch.Tensor), int(quant_type))
+
+
 def _workspace(device, rows: int, groups: int, experts: int, n_total: int, k: int, r: int) -> torch.Tensor:
     nbytes = _lib.load().ggq_lora_workspace_bytes(rows, groups, experts, n_total, k, r)
     return torch.empty(nbytes, dtype=torch.uint8, device=device)
