@@ -6,7 +6,7 @@
  * The reference reaches these decoders through un-vendored dependencies
  * (dequantize_gguf_tensor: fast_moe_lora.py:163-165, test_fast_lora.py:110-115; packed payloads
  * handed to torch_ggml_ops: fast_lora.py:154-160).  The loops below restate the published ggml
- * algorithm (ggml-quants.c dequantize_row_q8_0 / _q4_K / _q6_K / _iq2_xxs) one scalar at a time,
+ * algorithm (ggml-quants.c dequantize_row_q8_0 / _q2_K / _q4_K / _q5_K / _q6_K / _iq2_xxs) one scalar at a time,
  * independently of the vectorised numpy restatement in gguf_blocks.py; the two are checked against
  * each other and against hand-computed blocks in tests/test_oracle_blocks.py.
  * parity unpinned: no upstream decoder output exists in the build environment; the IQ2_XXS codebook
@@ -82,6 +82,56 @@ void oracle_dequant_q4_k(const uint8_t *x, int64_t nb, float *y) {
             for (int l = 0; l < 32; l++) *y++ = d2 * (float)(q[l] >> 4) - m2;
             q += 32;
             is += 2;
+        }
+    }
+}
+
+/* y[256*nb] from nb blocks of {f16 d; f16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]} (dequantize_row_q5_K) */
+void oracle_dequant_q5_k(const uint8_t *x, int64_t nb, float *y) {
+    for (int64_t i = 0; i < nb; i++, x += 176) {
+        float d = half_to_float(rd16(x));
+        float dmin = half_to_float(rd16(x + 2));
+        const uint8_t *scales = x + 4;
+        const uint8_t *qh = x + 16;
+        const uint8_t *ql = x + 48;
+        int is = 0;
+        uint8_t u1 = 1, u2 = 2;
+        for (int j = 0; j < 256; j += 64) {
+            uint8_t sc, m;
+            scale_min_k4(is + 0, scales, &sc, &m);
+            float d1 = d * sc, m1 = dmin * m;
+            scale_min_k4(is + 1, scales, &sc, &m);
+            float d2 = d * sc, m2 = dmin * m;
+            for (int l = 0; l < 32; l++) *y++ = d1 * (float)((ql[l] & 0x0F) + ((qh[l] & u1) ? 16 : 0)) - m1;
+            for (int l = 0; l < 32; l++) *y++ = d2 * (float)((ql[l] >> 4) + ((qh[l] & u2) ? 16 : 0)) - m2;
+            ql += 32;
+            is += 2;
+            u1 <<= 2;
+            u2 <<= 2;
+        }
+    }
+}
+
+/* y[256*nb] from nb blocks of {u8 scales[16]; u8 qs[64]; f16 d; f16 dmin} (dequantize_row_q2_K) */
+void oracle_dequant_q2_k(const uint8_t *x, int64_t nb, float *y) {
+    for (int64_t i = 0; i < nb; i++, x += 84) {
+        const uint8_t *scales = x;
+        const uint8_t *q = x + 16;
+        float d = half_to_float(rd16(x + 80));
+        float dmin = half_to_float(rd16(x + 82));
+        int is = 0;
+        for (int n = 0; n < 256; n += 128) {
+            int shift = 0;
+            for (int j = 0; j < 4; j++) {
+                uint8_t sc = scales[is++];
+                float dl = d * (sc & 0xF), ml = dmin * (sc >> 4);
+                for (int l = 0; l < 16; l++) *y++ = dl * (float)((q[l] >> shift) & 3) - ml;
+                sc = scales[is++];
+                dl = d * (sc & 0xF), ml = dmin * (sc >> 4);
+                for (int l = 0; l < 16; l++) *y++ = dl * (float)((q[l + 16] >> shift) & 3) - ml;
+                shift += 2;
+            }
+            q += 32;
         }
     }
 }

@@ -11,12 +11,14 @@ decoders below restate the published ggml block layouts (ggml-common.h / ggml-qu
 
   type      id  block bytes  elements  layout
   Q8_0       8      34          32     f16 d; i8 qs[32]
+  Q2_K      10      84         256     u8 scales[16]; u8 qs[64]; f16 d; f16 dmin
   Q4_K      12     144         256     f16 d; f16 dmin; u8 scales[12]; u8 qs[128]
+  Q5_K      13     176         256     f16 d; f16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]
   Q6_K      14     210         256     u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d
   IQ2_XXS   16      66         256     f16 d; u16 qs[32]
 
-All decoders return float32 values that are *exact* products except Q4_K, whose ``d*sc*q - dmin*m``
-rounds once to float32 (d*sc, dmin*m and (d*sc)*q are exact: 11+6+4 significand bits).  The bf16
+All decoders return float32 values that are *exact* products except Q2_K, Q4_K and Q5_K, whose
+``d*sc*q - dmin*m`` rounds once to float32 (d*sc, dmin*m and (d*sc)*q are exact: 11+6+4 significand bits).  The bf16
 weights the matmul oracles use are ``round-to-nearest-even(float32 value)``.
 
 Pinned by: hand-computed known-answer blocks and format invariants in tests/test_oracle_blocks.py and
@@ -35,10 +37,10 @@ import numpy as np
 
 from .iq2xxs_grid import IQ2XXS_GRID
 
-Q8_0, Q4_K, Q6_K, IQ2_XXS = 8, 12, 14, 16
+Q8_0, Q2_K, Q4_K, Q5_K, Q6_K, IQ2_XXS = 8, 10, 12, 13, 14, 16
 # (elements per block, bytes per block); matches gguf.GGML_QUANT_SIZES used at
 # test_deepseek_v4_moe_lora.py:58.
-QUANT_SIZES = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210), IQ2_XXS: (256, 66)}
+QUANT_SIZES = {Q8_0: (32, 34), Q2_K: (256, 84), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), IQ2_XXS: (256, 66)}
 
 _GRID_BYTES = np.array(IQ2XXS_GRID, dtype=np.uint64).view(np.uint8).reshape(256, 8)  # little endian
 # ksigns_iq2xs[i] = i | (parity(i) << 7): the eighth sign makes the number of minus signs even.
@@ -67,7 +69,7 @@ def dequantize(payload: np.ndarray, qt: int) -> np.ndarray:
         raise ValueError("payload row is not a whole number of blocks")
     lead = payload.shape[:-1]
     blocks = payload.reshape(-1, nbytes)
-    out = {Q8_0: _deq_q8_0, Q4_K: _deq_q4_k, Q6_K: _deq_q6_k, IQ2_XXS: _deq_iq2_xxs}[qt](blocks)
+    out = {Q8_0: _deq_q8_0, Q2_K: _deq_q2_k, Q4_K: _deq_q4_k, Q5_K: _deq_q5_k, Q6_K: _deq_q6_k, IQ2_XXS: _deq_iq2_xxs}[qt](blocks)
     return out.reshape(*lead, payload.shape[-1] // nbytes * elems)
 
 
@@ -103,6 +105,45 @@ def _deq_q4_k(b: np.ndarray) -> np.ndarray:
     q = q.reshape(nb, 8, 32)
     y = dl[:, :, None] * q                                 # exact in float32
     y = y - ml[:, :, None]                                 # one float32 rounding
+    return y.reshape(nb, 256)
+
+
+def _deq_q5_k(b: np.ndarray) -> np.ndarray:
+    """Q4_K's layout with a fifth bit per element: bit 2c (+1 for the high nibbles) of qh[l] belongs to element l of
+    the c-th 64-element chunk (ggml dequantize_row_q5_K)."""
+    nb = b.shape[0]
+    d = _f16(b[:, 0:2])
+    dmin = _f16(b[:, 2:4])
+    sc, m = unpack_q4_k_scales(b[:, 4:16])
+    dl = d * sc.astype(np.float32)
+    ml = dmin * m.astype(np.float32)
+    qh = b[:, 16:48]                                        # [nb,32]
+    qs = b[:, 48:176].reshape(nb, 4, 32)
+    q = np.empty((nb, 4, 2, 32), dtype=np.float32)
+    for c in range(4):
+        q[:, c, 0, :] = (qs[:, c, :] & 0x0F) + (((qh >> (2 * c)) & 1) << 4)
+        q[:, c, 1, :] = (qs[:, c, :] >> 4) + (((qh >> (2 * c + 1)) & 1) << 4)
+    q = q.reshape(nb, 8, 32)
+    y = dl[:, :, None] * q                                 # exact in float32 (11 + 6 + 5 bits)
+    y = y - ml[:, :, None]                                 # one float32 rounding
+    return y.reshape(nb, 256)
+
+
+def _deq_q2_k(b: np.ndarray) -> np.ndarray:
+    """Sixteen 16-element sub-blocks, each with a 4-bit scale (low nibble) and a 4-bit min (high nibble); element
+    128 n + 32 j + l is bits 2j..2j+1 of qs[32 n + l] (ggml dequantize_row_q2_K)."""
+    nb = b.shape[0]
+    scales = b[:, 0:16]
+    qs = b[:, 16:80].reshape(nb, 2, 32)
+    d = _f16(b[:, 80:82])
+    dmin = _f16(b[:, 82:84])
+    dl = d * (scales & 0x0F).astype(np.float32)            # [nb,16] exact
+    ml = dmin * (scales >> 4).astype(np.float32)
+    q = np.empty((nb, 2, 4, 32), dtype=np.float32)
+    for j in range(4):
+        q[:, :, j, :] = (qs >> (2 * j)) & 3
+    q = q.reshape(nb, 16, 16)                              # sub-block 8 n + 2 j + (l >= 16)
+    y = dl[:, :, None] * q - ml[:, :, None]
     return y.reshape(nb, 256)
 
 
@@ -173,7 +214,7 @@ def quantize(w: np.ndarray, qt: int) -> np.ndarray:
         raise ValueError(f"last dim {w.shape[-1]} is not a multiple of {elems}")
     lead = w.shape[:-1]
     blocks = w.reshape(-1, elems)
-    out = {Q8_0: _q_q8_0, Q4_K: _q_q4_k, Q6_K: _q_q6_k, IQ2_XXS: _q_iq2_xxs}[qt](blocks)
+    out = {Q8_0: _q_q8_0, Q2_K: _q_q2_k, Q4_K: _q_q4_k, Q5_K: _q_q5_k, Q6_K: _q_q6_k, IQ2_XXS: _q_iq2_xxs}[qt](blocks)
     return out.reshape(*lead, w.shape[-1] // elems * nbytes)
 
 
@@ -219,6 +260,61 @@ def _q_q4_k(x: np.ndarray) -> np.ndarray:
     out[:, 2:4] = _f16_bytes(dmin).reshape(-1, 2)
     out[:, 4:16] = pack_q4_k_scales(sc, m)
     out[:, 16:] = (q[:, :, 0, :] | (q[:, :, 1, :] << 4)).reshape(nb, 128)
+    return out
+
+
+def _q_q5_k(x: np.ndarray) -> np.ndarray:
+    nb = x.shape[0]
+    sub = x.reshape(nb, 8, 32)
+    lo = np.minimum(sub.min(axis=2), 0)
+    hi = sub.max(axis=2)
+    scale = (hi - lo) / np.float32(31)
+    off = -lo
+    d = (scale.max(axis=1, keepdims=True) / np.float32(63)).astype(np.float16).astype(np.float32)
+    dmin = (off.max(axis=1, keepdims=True) / np.float32(63)).astype(np.float16).astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        sc = np.where(d > 0, np.clip(_roundf(scale / d), 0, 63), 0).astype(np.uint8)
+        m = np.where(dmin > 0, np.clip(_roundf(off / dmin), 0, 63), 0).astype(np.uint8)
+        dl = d * sc.astype(np.float32)
+        ml = dmin * m.astype(np.float32)
+        q = np.where(dl[:, :, None] > 0, _roundf((sub + ml[:, :, None]) / dl[:, :, None]), 0)
+    q = np.clip(q, 0, 31).astype(np.uint8).reshape(nb, 4, 2, 32)
+    out = np.empty((nb, 176), dtype=np.uint8)
+    out[:, 0:2] = _f16_bytes(d).reshape(-1, 2)
+    out[:, 2:4] = _f16_bytes(dmin).reshape(-1, 2)
+    out[:, 4:16] = pack_q4_k_scales(sc, m)
+    qh = np.zeros((nb, 32), dtype=np.uint8)
+    for c in range(4):
+        qh |= ((q[:, c, 0, :] >> 4) << (2 * c)) | ((q[:, c, 1, :] >> 4) << (2 * c + 1))
+    out[:, 16:48] = qh
+    out[:, 48:] = ((q[:, :, 0, :] & 0x0F) | ((q[:, :, 1, :] & 0x0F) << 4)).reshape(nb, 128)
+    return out
+
+
+def _q_q2_k(x: np.ndarray) -> np.ndarray:
+    nb = x.shape[0]
+    sub = x.reshape(nb, 16, 16)
+    lo = np.minimum(sub.min(axis=2), 0)
+    hi = sub.max(axis=2)
+    scale = (hi - lo) / np.float32(3)
+    off = -lo
+    d = (scale.max(axis=1, keepdims=True) / np.float32(15)).astype(np.float16).astype(np.float32)
+    dmin = (off.max(axis=1, keepdims=True) / np.float32(15)).astype(np.float16).astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        sc = np.where(d > 0, np.clip(_roundf(scale / d), 0, 15), 0).astype(np.uint8)
+        m = np.where(dmin > 0, np.clip(_roundf(off / dmin), 0, 15), 0).astype(np.uint8)
+        dl = d * sc.astype(np.float32)
+        ml = dmin * m.astype(np.float32)
+        q = np.where(dl[:, :, None] > 0, _roundf((sub + ml[:, :, None]) / dl[:, :, None]), 0)
+    q = np.clip(q, 0, 3).astype(np.uint8).reshape(nb, 2, 4, 32)   # [n, j, l]: element 128 n + 32 j + l
+    out = np.empty((nb, 84), dtype=np.uint8)
+    out[:, 0:16] = sc | (m << 4)
+    qs = np.zeros((nb, 2, 32), dtype=np.uint8)
+    for j in range(4):
+        qs |= q[:, :, j, :] << (2 * j)
+    out[:, 16:80] = qs.reshape(nb, 64)
+    out[:, 80:82] = _f16_bytes(d).reshape(-1, 2)
+    out[:, 82:84] = _f16_bytes(dmin).reshape(-1, 2)
     return out
 
 
@@ -285,12 +381,15 @@ def random_payload(rng: np.random.Generator, qt: int, rows: int, k: int, std: fl
     elems, nbytes = QUANT_SIZES[qt]
     nb = rows * (k // elems)
     b = rng.integers(0, 256, size=(nb, nbytes), dtype=np.uint8)
-    mag = {Q8_0: std / 64, Q4_K: std / 250, Q6_K: std / 1500, IQ2_XXS: std / 60}[qt]
+    mag = {Q8_0: std / 64, Q2_K: std / 25, Q4_K: std / 250, Q5_K: std / 800, Q6_K: std / 1500, IQ2_XXS: std / 60}[qt]
     d = (mag * (0.5 + rng.random(nb))).astype(np.float32)
     if qt == Q6_K:
         b[:, 208:210] = _f16_bytes(d).reshape(-1, 2)
+    elif qt == Q2_K:
+        b[:, 80:82] = _f16_bytes(d).reshape(-1, 2)
+        b[:, 82:84] = _f16_bytes(d * np.float32(0.7)).reshape(-1, 2)
     else:
         b[:, 0:2] = _f16_bytes(d).reshape(-1, 2)
-    if qt == Q4_K:
+    if qt in (Q4_K, Q5_K):
         b[:, 2:4] = _f16_bytes(d * np.float32(0.7)).reshape(-1, 2)
     return b.reshape(rows, k // elems * nbytes)

@@ -47,6 +47,40 @@ def test_q4_k_known_answer():
         assert y[e] == v, (e, y[e], v)
 
 
+def test_q5_k_known_answer():
+    # Same d, dmin and scale bytes as the Q4_K block above (sc = 1,2,3,4,33,34,35,36, m = 5..8,37..40) and
+    # the same nibbles; qh[l] = 0xA5 for even l and 0x5A for odd l.  Sub-block s takes its fifth bit from
+    # bit s of qh[l], so even l sees bits {0,2,5,7} set and odd l bits {1,3,4,6}.
+    blk = np.zeros(176, dtype=np.uint8)
+    blk[0:2] = F16[1.0]
+    blk[2:4] = F16[0.5]
+    blk[4:16] = [129, 130, 131, 132, 133, 134, 135, 136, 81, 98, 115, 132]
+    blk[16:48] = [0xA5, 0x5A] * 16
+    i = np.arange(128)
+    blk[48:] = (i % 16) | ((15 - i % 16) << 4)
+    y = both(blk[None, :], gb.Q5_K)[0]
+    want = {0: 13.5, 1: -1.5, 32: 27.0, 33: 57.0, 64: 44.5, 111: 60.0, 128: -18.5, 131: 608.5,
+            192: -19.5, 193: 575.5, 224: 1096.0, 255: -20.0}
+    for e, v in want.items():
+        assert y[e] == v, (e, y[e], v)
+
+
+def test_q2_k_known_answer():
+    # d = 0.5, dmin = 0.25; scales[k] = k | (15-k) << 4 (scale k, min 15-k); qs = 0xE4 at even bytes
+    # (bit pairs 0,1,2,3 from the bottom) and 0x1B at odd bytes (3,2,1,0).
+    blk = np.zeros(84, dtype=np.uint8)
+    k = np.arange(16)
+    blk[0:16] = k | ((15 - k) << 4)
+    blk[16:80] = [0xE4, 0x1B] * 32
+    blk[80:82] = F16[0.5]
+    blk[82:84] = F16[0.25]
+    y = both(blk[None, :], gb.Q2_K)[0]
+    want = {0: -3.75, 17: -2.0, 32: -2.25, 49: 0.0, 96: 6.75, 127: -2.0, 128: -1.75, 145: 12.0,
+            254: 22.5, 255: 0.0}
+    for e, v in want.items():
+        assert y[e] == v, (e, y[e], v)
+
+
 def test_q6_k_known_answer():
     # d = 0.25; int8 sub-scales 1,-2,3,-4,...,15,-16; ql = 0x21 for l < 32 and 0x43 for l >= 32 of each
     # 64-byte half; qh = 0xE4 (bit pairs 0,1,2,3 from the bottom).
@@ -92,7 +126,7 @@ def test_iq2xxs_grid_structure():
     assert int(((n19 == 2) & (n2b == 0)).sum()) == 28 and int(((n19 == 0) & (n2b == 1)).sum()) == 8
 
 
-@pytest.mark.parametrize("qt", [gb.Q8_0, gb.Q4_K, gb.Q6_K, gb.IQ2_XXS])
+@pytest.mark.parametrize("qt", [gb.Q8_0, gb.Q2_K, gb.Q4_K, gb.Q5_K, gb.Q6_K, gb.IQ2_XXS])
 def test_numpy_and_c_agree_on_arbitrary_bytes(qt):
     payload = gb.random_payload(np.random.default_rng(qt), qt, 23, 1024)
     y = both(payload, qt)
@@ -109,6 +143,25 @@ def test_format_invariants():
     _, m = gb.unpack_q4_k_scales(p[0, 4:16])
     dmin = p[0, 2:4].copy().view(np.float16).astype(np.float32)[0]
     assert np.array_equal(y, np.repeat((-(dmin * m.astype(np.float32)))[:, None], 32, axis=1))
+    # Q5_K: clearing qh removes exactly 16*d*sc from the values whose fifth bit was set, and a block with
+    # qh = 0 decodes like the Q4_K block made of the same header, scales and nibbles
+    p = gb.random_payload(rng, gb.Q5_K, 1, 256)
+    q4 = np.concatenate([p[:, :16], p[:, 48:]], axis=1)
+    p0 = p.copy()
+    p0[0, 16:48] = 0
+    assert np.array_equal(gb.dequantize(p0, gb.Q5_K), gb.dequantize(q4, gb.Q4_K))
+    sc, _ = gb.unpack_q4_k_scales(p[0, 4:16])
+    d = p[0, 0:2].copy().view(np.float16).astype(np.float32)[0]
+    bits = ((p[0, 16:48][None, :] >> np.arange(8)[:, None]) & 1).astype(np.float32)  # [sub-block, l]
+    step = (d * sc.astype(np.float32))[:, None] * 16.0 * bits
+    got = (gb.dequantize(p, gb.Q5_K) - gb.dequantize(p0, gb.Q5_K))[0].reshape(8, 32)
+    assert np.allclose(got, step, rtol=1e-6, atol=0)
+    # Q2_K with all-zero quants decodes to -dmin*(scales >> 4) per run of sixteen
+    p = gb.random_payload(rng, gb.Q2_K, 1, 256)
+    p[0, 16:80] = 0
+    dmin = p[0, 82:84].copy().view(np.float16).astype(np.float32)[0]
+    y = gb.dequantize(p, gb.Q2_K)[0].reshape(16, 16)
+    assert np.array_equal(y, np.repeat((-(dmin * (p[0, :16] >> 4).astype(np.float32)))[:, None], 16, axis=1))
     # negating an IQ2_XXS block scale negates every weight; Q8_0 is linear in d
     p = gb.random_payload(rng, gb.IQ2_XXS, 1, 256)
     q = p.copy()
@@ -126,7 +179,8 @@ def test_bf16_rounding_is_nearest_even():
     assert np.array_equal(gb.to_bf16_bits(x), want)
 
 
-@pytest.mark.parametrize("qt,bound", [(gb.Q8_0, 0.01), (gb.Q4_K, 0.12), (gb.Q6_K, 0.03), (gb.IQ2_XXS, 0.6)])
+@pytest.mark.parametrize("qt,bound", [(gb.Q8_0, 0.01), (gb.Q2_K, 0.35), (gb.Q4_K, 0.12), (gb.Q5_K, 0.06), (gb.Q6_K, 0.03),
+                                      (gb.IQ2_XXS, 0.6)])
 def test_quantizer_round_trip_error(qt, bound):
     rng = np.random.default_rng(11)
     w = (rng.standard_normal((16, 1024)) * 0.02).astype(np.float32)

@@ -103,6 +103,95 @@ struct Fmt<kQ4_K> {
 };
 
 // ------------------------------------------------------------------------------------------------
+// Q5_K: 176-byte block = f16 d; f16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]: Q4_K with a fifth bit per
+// element.  Sub-block j (run ksub & 7) uses qs[32*(j/2) .. +31] (low nibbles for even j, high for odd j) and bit j
+// of qh[l] for its element l, with Q4_K's 6-bit (sc, m).
+template <>
+struct Fmt<kQ5_K> {
+    static constexpr int kBlockElems = 256, kBlockBytes = 176;
+    struct Raw {
+        uint4 hdr, h0, h1, q0, q1;
+    };
+    static GGQ_HD void pin(Raw& r) { GGQ_PIN4(r.hdr); GGQ_PIN4(r.h0); GGQ_PIN4(r.h1); GGQ_PIN4(r.q0); GGQ_PIN4(r.q1); }
+    static GGQ_HD void load(Raw& r, const uint8_t* row, int ksub) {
+        const uint8_t* blk = row + (int64_t)(ksub >> 3) * 176;
+        r.hdr = *(const uint4*)blk;
+        r.h0 = *(const uint4*)(blk + 16);
+        r.h1 = *(const uint4*)(blk + 32);
+        const uint8_t* q = blk + 48 + 32 * ((ksub & 7) >> 1);
+        r.q0 = *(const uint4*)q;
+        r.q1 = *(const uint4*)(q + 16);
+    }
+    static GGQ_HD void decode(const Raw& r, int ksub, uint32_t* out, const uint2*) {
+        const int j = ksub & 7;
+        const float d = half_bits_to_f32(r.hdr.x & 0xFFFFu);
+        const float dmin = half_bits_to_f32(r.hdr.x >> 16);
+        const uint32_t s0 = r.hdr.y, s1 = r.hdr.z, s2 = r.hdr.w;
+        uint32_t sc, m;
+        if (j < 4) {
+            const int sh = 8 * j;
+            sc = (s0 >> sh) & 63u;
+            m = (s1 >> sh) & 63u;
+        } else {
+            const int sh = 8 * (j - 4);
+            sc = ((s2 >> sh) & 0xFu) | (((s0 >> (sh + 6)) & 3u) << 4);
+            m = ((s2 >> (sh + 4)) & 0xFu) | (((s1 >> (sh + 6)) & 3u) << 4);
+        }
+        const float dl = d * (float)sc * kMixScale, nm = -(dmin * (float)m);
+        const int shift = 4 * (j & 1);
+        const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+        const uint32_t h[8] = {r.h0.x, r.h0.y, r.h0.z, r.h0.w, r.h1.x, r.h1.y, r.h1.z, r.h1.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            // five-bit values of bytes 0, 2 and of bytes 1, 3, each in its own 16-bit half (a half-precision denormal)
+            const uint32_t hb = (h[i] >> j) & 0x01010101u;  // the element's fifth bit, one per byte
+            const uint32_t v = ((q[i] >> shift) & 0x0F0F0F0Fu) | (hb << 4);
+            const uint32_t e02 = v & 0x001F001Fu, e13 = (v >> 8) & 0x001F001Fu;
+            out[2 * i] = pack_bf16(mix_lo(e02, dl, nm), mix_lo(e13, dl, nm));
+            out[2 * i + 1] = pack_bf16(mix_hi(e02, dl, nm), mix_hi(e13, dl, nm));
+        }
+    }
+};
+
+// ------------------------------------------------------------------------------------------------
+// Q2_K: 84-byte block = u8 scales[16]; u8 qs[64]; f16 d; f16 dmin (4-byte aligned).  Run u = ksub & 7 lives in
+// half n = u / 4 with bit pair s = u % 4 of qs[32 n .. +31]; its elements 0..15 use scales[8 n + 2 s], elements
+// 16..31 scales[8 n + 2 s + 1] (low nibble: scale, high nibble: min).
+template <>
+struct Fmt<kQ2_K> {
+    static constexpr int kBlockElems = 256, kBlockBytes = 84;
+    struct Raw {
+        uint4 q0, q1;
+        uint32_t sc2, dd;
+    };
+    static GGQ_HD void pin(Raw& r) { GGQ_PIN4(r.q0); GGQ_PIN4(r.q1); GGQ_PIN1(r.sc2); GGQ_PIN1(r.dd); }
+    static GGQ_HD void load(Raw& r, const uint8_t* row, int ksub) {
+        const uint8_t* blk = row + (int64_t)(ksub >> 3) * 84;
+        const int u = ksub & 7, n = u >> 2, s = u & 3;
+        r.q0 = ld_u128(blk + 16 + 32 * n);
+        r.q1 = ld_u128(blk + 32 + 32 * n);
+        r.sc2 = ld_u16(blk + 8 * n + 2 * s);
+        r.dd = ld_u32(blk + 80);
+    }
+    static GGQ_HD void decode(const Raw& r, int ksub, uint32_t* out, const uint2*) {
+        const int shift = 2 * (ksub & 3);
+        const float d = half_bits_to_f32(r.dd & 0xFFFFu), dmin = half_bits_to_f32(r.dd >> 16);
+        const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const uint32_t sb = (r.sc2 >> (8 * half)) & 0xFFu;
+            const float dl = d * (float)(sb & 0xFu) * kMixScale, nm = -(dmin * (float)(sb >> 4));
+#pragma unroll
+            for (int i = 4 * half; i < 4 * half + 4; i++) {
+                const uint32_t e02 = (q[i] >> shift) & 0x00030003u, e13 = (q[i] >> (shift + 8)) & 0x00030003u;
+                out[2 * i] = pack_bf16(mix_lo(e02, dl, nm), mix_lo(e13, dl, nm));
+                out[2 * i + 1] = pack_bf16(mix_hi(e02, dl, nm), mix_hi(e13, dl, nm));
+            }
+        }
+    }
+};
+
+// ------------------------------------------------------------------------------------------------
 // Q6_K: 210-byte block = u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d.  Blocks are only 2-byte
 // aligned.  Run u = ksub & 7 lives in half h = u/4 as part p = u%4: low (p < 2) or high nibbles of
 // ql[64h + 32(p&1) .. +31], bit pair 2p of qh[32h .. +31], int8 scales[8h + 2p], [8h + 2p + 1].

@@ -40,6 +40,34 @@ __device__ __forceinline__ void decode8(const uint8_t* raw, int g, float* y) {
         const int shift = 4 * (j & 1);
 #pragma unroll
         for (int i = 0; i < 8; i++) y[i] = __fsub_rn(__fmul_rn(dl, (float)((q[i] >> shift) & 0xFu)), ml);
+    } else if constexpr (QT == kQ5_K) {
+        const uint8_t* blk = raw + (g >> 5) * 176;
+        const int e0 = 8 * (g & 31), j = e0 >> 5, l0 = e0 & 31;
+        const float d = half_bits_to_f32(lds_u16(blk)), dmin = half_bits_to_f32(lds_u16(blk + 2));
+        const uint8_t* s = blk + 4;
+        uint32_t sc, m;
+        if (j < 4) {
+            sc = s[j] & 63u;
+            m = s[j + 4] & 63u;
+        } else {
+            sc = (s[j + 4] & 0xFu) | ((uint32_t)(s[j - 4] >> 6) << 4);
+            m = (uint32_t)(s[j + 4] >> 4) | ((uint32_t)(s[j] >> 6) << 4);
+        }
+        const float dl = d * (float)sc, ml = dmin * (float)m;
+        const uint8_t* qh = blk + 16 + l0;
+        const uint8_t* q = blk + 48 + 32 * (j >> 1) + l0;
+        const int shift = 4 * (j & 1);
+#pragma unroll
+        for (int i = 0; i < 8; i++) y[i] = __fsub_rn(__fmul_rn(dl, (float)(((q[i] >> shift) & 0xFu) + (((qh[i] >> j) & 1u) << 4))), ml);
+    } else if constexpr (QT == kQ2_K) {
+        const uint8_t* blk = raw + (g >> 5) * 84;
+        const int e0 = 8 * (g & 31), n = e0 >> 7, j = (e0 & 127) >> 5, l0 = e0 & 31;
+        const float d = half_bits_to_f32(lds_u16(blk + 80)), dmin = half_bits_to_f32(lds_u16(blk + 82));
+        const uint32_t sb = blk[e0 >> 4];
+        const float dl = d * (float)(sb & 0xFu), ml = dmin * (float)(sb >> 4);
+        const uint8_t* q = blk + 16 + 32 * n + l0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) y[i] = __fsub_rn(__fmul_rn(dl, (float)((q[i] >> (2 * j)) & 3u)), ml);
     } else if constexpr (QT == kQ6_K) {
         const uint8_t* blk = raw + (g >> 5) * 210;
         const int e0 = 8 * (g & 31), h = e0 >> 7, part = (e0 & 127) >> 5, l0 = e0 & 31;
@@ -76,7 +104,7 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
                                                        void* __restrict__ out) {
     constexpr int kBE = Fmt<QT>::kBlockElems, kBB = Fmt<QT>::kBlockBytes;
     constexpr int kBlocksPerWg = kElemsPerWg / kBE;
-    constexpr int kRawBytes = kBlocksPerWg * kBB;  // a multiple of 16 for all four formats
+    constexpr int kRawBytes = kBlocksPerWg * kBB;  // a multiple of 16 for every format
     __shared__ __attribute__((aligned(16))) uint8_t raw[kRawBytes];
     const int64_t e_begin = (int64_t)blockIdx.x * kElemsPerWg;
     const int64_t e_left = total_elems - e_begin;
@@ -122,7 +150,9 @@ int dequantize(int qt, const void* payload, int64_t rows, int64_t k, void* out, 
     const int64_t total = rows * k;
     switch (qt) {
         case kQ8_0: return launch_dequant<kQ8_0>(payload, total, out, out_f32, stream);
+        case kQ2_K: return launch_dequant<kQ2_K>(payload, total, out, out_f32, stream);
         case kQ4_K: return launch_dequant<kQ4_K>(payload, total, out, out_f32, stream);
+        case kQ5_K: return launch_dequant<kQ5_K>(payload, total, out, out_f32, stream);
         case kQ6_K: return launch_dequant<kQ6_K>(payload, total, out, out_f32, stream);
         case kIQ2_XXS: return launch_dequant<kIQ2_XXS>(payload, total, out, out_f32, stream);
     }

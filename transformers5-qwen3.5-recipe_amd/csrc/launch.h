@@ -21,14 +21,16 @@ int check_launch(const char* what);
 inline bool block_multiple(int qt, int64_t k) {
     switch (qt) {
         case 8: return k % 32 == 0;
-        case 12: case 14: case 16: return k % 256 == 0;
+        case 10: case 12: case 13: case 14: case 16: return k % 256 == 0;
     }
     return true;  // unknown types are rejected by the callers' switch
 }
 inline int64_t packed_row_bytes(int qt, int64_t k) {
     switch (qt) {
         case 8: return k / 32 * 34;
+        case 10: return k / 256 * 84;
         case 12: return k / 256 * 144;
+        case 13: return k / 256 * 176;
         case 14: return k / 256 * 210;
         case 16: return k / 256 * 66;
     }
