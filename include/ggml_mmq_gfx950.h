@@ -98,6 +98,26 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
                                   const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b, void* ws,
                                   int64_t ws_bytes, void* stream);
 
+/* The two calls above over rows that are never materialised: the reference gathers the routed rows first
+ * (prepare_expert_routing, fast_moe_routing.py:379-420: _RouteGather.apply(hidden_states, permutation, ...)) and hands the
+ * copy to the grouped ops; here row i of the expert-sorted layout is read in place as row row_index[i] / index_div of
+ * x [x_rows, k] (row_index = the sorted-position -> route permutation, index_div = top_k).  Results are bit-identical to
+ * the plain calls on the gathered copy.  Only some launches can do this: ask ggq_grouped_forward_reads_indexed_rows
+ * (host-only, 1 = yes) with the same qt / rows / groups / x_rows / k first; the indexed forward returns the shape error
+ * otherwise.  dx is still per expert-sorted row, [rows, k]. */
+int ggq_grouped_forward_reads_indexed_rows(int qt, int64_t rows, int64_t groups, int64_t x_rows, int64_t k);
+int ggq_grouped_lora_mmq_forward_indexed(const void* x, int64_t x_rows, const int64_t* row_index, int index_div, const void* packed1,
+                                         const void* packed2, const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups,
+                                         int64_t experts, int qt, int64_t rows, int64_t n, int64_t k, const void* lora_a,
+                                         const void* lora_b, int r, float scale, void* xa_out, void* y1, void* y2, void* ws,
+                                         int64_t ws_bytes, void* stream);
+int ggq_grouped_lora_mmq_backward_indexed(const void* dy1, const void* dy2, const void* packed1, const void* packed2,
+                                          const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts,
+                                          int qt, int64_t rows, int64_t n, int64_t k, const void* x, int64_t x_rows,
+                                          const int64_t* row_index, int index_div, const void* xa, const void* lora_a,
+                                          const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b,
+                                          void* ws, int64_t ws_bytes, void* stream);
+
 /* torch_ggml_ops.fixed_grouped_mmq (deepseek_v4_lora.py:91-124: DeepSeek's frozen eight-group output projection) and
  * its input gradient: x [rows, groups, k] bf16, packed_groups [groups, n_group, row bytes], y [rows, groups, n_group];
  * y[:, g, :] = x[:, g, :] . W_g^T.  Each group runs as the dense launch over its strided rows, so the results are

@@ -166,11 +166,20 @@ int ggq_fixed_grouped_mmq_grad_input(const void* dy, const void* packed_groups, 
 
 // Forward of one projection (or a gate/up pair) over expert-sorted rows, optional LoRA fused.
 // groups == 0 means dense: one group of all rows using expert 0.
-int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void* packed2, const int64_t* expert_ids,
-                                 const int32_t* end_offsets, int64_t groups, int64_t experts, int qt, int64_t rows, int64_t n,
-                                 int64_t k, const void* lora_a, const void* lora_b, int r, float scale, void* xa_out, void* y1,
-                                 void* y2, void* ws, int64_t ws_bytes, void* stream) {
-    const char* what = "grouped_lora_mmq_forward";
+// The forward launch reads its rows through an index only in the direct kernel: Q4_K expert groups of at most 256 rows
+// on average, and a source matrix under 4 GiB (the lane offsets of its loads are 32-bit).
+static bool forward_reads_indexed_rows(int qt, int64_t rows, int64_t groups, int64_t x_rows, int64_t k) {
+    return x_rows > 0 && k < (1 << 22) && (uint64_t)x_rows * (uint64_t)k * 2 < (1ull << 32) && pick_shape(qt, rows, groups, true) == kShapeDirect;
+}
+
+int ggq_grouped_forward_reads_indexed_rows(int qt, int64_t rows, int64_t groups, int64_t x_rows, int64_t k) {
+    return forward_reads_indexed_rows(qt, rows, groups, x_rows, k) ? 1 : 0;
+}
+
+static int grouped_forward(const char* what, const void* x, RowIndex x_index, const void* packed1, const void* packed2, const int64_t* expert_ids,
+                           const int32_t* end_offsets, int64_t groups, int64_t experts, int qt, int64_t rows, int64_t n,
+                           int64_t k, const void* lora_a, const void* lora_b, int r, float scale, void* xa_out, void* y1,
+                           void* y2, void* ws, int64_t ws_bytes, void* stream) {
     hipStream_t s = as_stream(stream);
     if (rows < 0 || n <= 0 || k <= 0 || rows >= (1ll << 31) || n >= (1ll << 30) || k >= (1ll << 30)) return set_error(GGQ_ERR_SHAPE, "%s: bad shape rows=%lld n=%lld k=%lld", what, (long long)rows, (long long)n, (long long)k);
     if (int rc = check_weights(what, qt, packed1, k)) return rc;
@@ -188,7 +197,9 @@ int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void*
     // the direct kernel moves A, LA and LB rows with aligned 16-byte accesses
     const bool direct_ok = aligned16(x) && k < (1 << 22) && (!lora_a || (aligned16(xa_out) && (rp != r || aligned16(lora_b))));
     if (int rc = init_params(p, qt, kModeNT, (int)rows, (int)n, (int)k, nseg, pick_shape(qt, rows, groups, direct_ok))) return rc;
-    p.a[0] = (const bf16_t*)x, p.lda = k;
+    if (x_index.on() && (p.shape != kShapeDirect || !forward_reads_indexed_rows(qt, rows, groups, x_index.index_rows, k) || x_index.index_div <= 0))
+        return set_error(GGQ_ERR_SHAPE, "%s: this type, shape or alignment cannot read its rows through an index (ask ggq_grouped_forward_reads_indexed_rows first)", what);
+    p.a[0] = (const bf16_t*)x, p.lda = k, p.a_rows = x_index;
     p.w[0] = (const uint8_t*)packed1, p.w[1] = (const uint8_t*)packed2;
     p.c[0] = y1, p.c[1] = y2, p.ldc = n;
     if (p.shape == kShapeDirect) p.col_tiles_per_wg = direct_tiles_per_wg(rows, groups, nseg * p.col_tiles_per_seg);
@@ -222,7 +233,7 @@ int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void*
     }
     if (lora_a) {
         SkinnyNtParams sp{};
-        sp.in[0] = (const bf16_t*)x, sp.ld_in = k;
+        sp.in[0] = (const bf16_t*)x, sp.ld_in = k, sp.in_rows = x_index;
         sp.f = (const bf16_t*)lora_a, sp.ldf = k, sp.f_expert_elems = (int64_t)r * k;
         sp.out = (bf16_t*)xa_out;
         sp.m = (int)rows, sp.c = (int)k, sp.r = r, sp.nseg = 1;
@@ -241,13 +252,34 @@ int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void*
     return launch_mmq(qt, kModeNT, kEpiStore, p, s);
 }
 
+int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void* packed2, const int64_t* expert_ids,
+                                 const int32_t* end_offsets, int64_t groups, int64_t experts, int qt, int64_t rows, int64_t n,
+                                 int64_t k, const void* lora_a, const void* lora_b, int r, float scale, void* xa_out, void* y1,
+                                 void* y2, void* ws, int64_t ws_bytes, void* stream) {
+    return grouped_forward("grouped_lora_mmq_forward", x, RowIndex{}, packed1, packed2, expert_ids, end_offsets, groups, experts, qt, rows, n, k,
+                           lora_a, lora_b, r, scale, xa_out, y1, y2, ws, ws_bytes, stream);
+}
+
+// The same forward over rows that are not materialised: row i of the expert-sorted layout is row
+// row_index[i] / index_div of x [x_rows, k].
+int ggq_grouped_lora_mmq_forward_indexed(const void* x, int64_t x_rows, const int64_t* row_index, int index_div, const void* packed1,
+                                         const void* packed2, const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups,
+                                         int64_t experts, int qt, int64_t rows, int64_t n, int64_t k, const void* lora_a,
+                                         const void* lora_b, int r, float scale, void* xa_out, void* y1, void* y2, void* ws,
+                                         int64_t ws_bytes, void* stream) {
+    const char* what = "grouped_lora_mmq_forward_indexed";
+    if (!row_index) return set_error(GGQ_ERR_NULL, "%s: null row index", what);
+    if (x_rows <= 0 || x_rows >= (1ll << 31) || index_div <= 0) return set_error(GGQ_ERR_SHAPE, "%s: bad x_rows=%lld or index_div=%d", what, (long long)x_rows, index_div);
+    return grouped_forward(what, x, RowIndex{row_index, index_div, (int)x_rows}, packed1, packed2, expert_ids, end_offsets, groups, experts, qt,
+                           rows, n, k, lora_a, lora_b, r, scale, xa_out, y1, y2, ws, ws_bytes, stream);
+}
+
 // Backward: dx = dy . W (+ LoRA term), and the factor gradients over all `experts` planes.
-int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* packed1, const void* packed2,
-                                  const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts, int qt,
-                                  int64_t rows, int64_t n, int64_t k, const void* x, const void* xa, const void* lora_a,
-                                  const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b, void* ws,
-                                  int64_t ws_bytes, void* stream) {
-    const char* what = "grouped_lora_mmq_backward";
+static int grouped_backward(const char* what, const void* dy1, const void* dy2, const void* packed1, const void* packed2,
+                            const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts, int qt,
+                            int64_t rows, int64_t n, int64_t k, const void* x, RowIndex x_index, const void* xa, const void* lora_a,
+                            const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b, void* ws,
+                            int64_t ws_bytes, void* stream) {
     hipStream_t s = as_stream(stream);
     if (rows < 0 || n <= 0 || k <= 0 || rows >= (1ll << 31) || n >= (1ll << 30) || k >= (1ll << 30)) return set_error(GGQ_ERR_SHAPE, "%s: bad shape rows=%lld n=%lld k=%lld", what, (long long)rows, (long long)n, (long long)k);
     if (int rc = check_weights(what, qt, packed1, k)) return rc;
@@ -333,7 +365,7 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
         }
         if (d_lora_a) {
             FactorGradParams fp{};
-            fp.in[0] = (const bf16_t*)x, fp.ld_in = k;
+            fp.in[0] = (const bf16_t*)x, fp.ld_in = k, fp.in_rows = x_index;
             fp.s = dyb, fp.out = (bf16_t*)d_lora_a, fp.out_expert_elems = (int64_t)r * k;
             fp.ranges = ranges, fp.m = (int)rows, fp.c = (int)k, fp.r = r, fp.nseg = 1, fp.out_j_major = 1, fp.scale = scale;
             if (int rc = factor_grad(fp, rp, experts, s)) return rc;
@@ -342,6 +374,31 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
     if (rows == 0) return GGQ_OK;
     if (t_tall) return launch_wide_and_tall(qt, kModeNN, p, (int)rows, (int)n, (int)k, nseg, t_tall, n_tall, max_tall, s);
     return launch_mmq(qt, kModeNN, kEpiStore, p, s);
+}
+
+int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* packed1, const void* packed2,
+                                  const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts, int qt,
+                                  int64_t rows, int64_t n, int64_t k, const void* x, const void* xa, const void* lora_a,
+                                  const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b, void* ws,
+                                  int64_t ws_bytes, void* stream) {
+    return grouped_backward("grouped_lora_mmq_backward", dy1, dy2, packed1, packed2, expert_ids, end_offsets, groups, experts, qt, rows, n, k, x,
+                            RowIndex{}, xa, lora_a, lora_b, r, scale, dx, d_lora_a, d_lora_b, ws, ws_bytes, stream);
+}
+
+// The backward of the indexed forward: x is the [x_rows, k] matrix the forward read through row_index (it is only
+// read for the gradient of the factor A); dx comes out per expert-sorted row, [rows, k], as in the plain backward.
+int ggq_grouped_lora_mmq_backward_indexed(const void* dy1, const void* dy2, const void* packed1, const void* packed2,
+                                          const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts,
+                                          int qt, int64_t rows, int64_t n, int64_t k, const void* x, int64_t x_rows,
+                                          const int64_t* row_index, int index_div, const void* xa, const void* lora_a,
+                                          const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b,
+                                          void* ws, int64_t ws_bytes, void* stream) {
+    const char* what = "grouped_lora_mmq_backward_indexed";
+    if (!row_index) return set_error(GGQ_ERR_NULL, "%s: null row index", what);
+    if (x_rows <= 0 || x_rows >= (1ll << 31) || index_div <= 0) return set_error(GGQ_ERR_SHAPE, "%s: bad x_rows=%lld or index_div=%d", what, (long long)x_rows, index_div);
+    return grouped_backward(what, dy1, dy2, packed1, packed2, expert_ids, end_offsets, groups, experts, qt, rows, n, k, x,
+                            RowIndex{row_index, index_div, (int)x_rows}, xa, lora_a, lora_b, r, scale, dx, d_lora_a, d_lora_b, ws, ws_bytes,
+                            stream);
 }
 
 // ---------------------------------------------------------------------------------------------------

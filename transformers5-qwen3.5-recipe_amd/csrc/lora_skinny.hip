@@ -52,6 +52,7 @@ __global__ __launch_bounds__(256) void skinny_nt_kernel(SkinnyNtParams p) {
     const int li = lane & 15, lq = lane >> 4;
     const int row = m0 + li;
     const bool row_ok = row < row_end;
+    const int src_row = row_ok ? p.in_rows.source(row) : 0;  // stored row of segment 0 (an index comes with one segment)
     const bf16_t* f = p.f + expert * p.f_expert_elems;  // [r][ldf]
     f32x4_t acc[JB];
 #pragma unroll
@@ -63,7 +64,7 @@ __global__ __launch_bounds__(256) void skinny_nt_kernel(SkinnyNtParams p) {
     const int trips_per_seg = (vec && fvec) ? p.c / 128 : 0;
     for (int t = wave; t < trips_per_seg * p.nseg; t += 4) {
         const int seg = t / trips_per_seg, c0 = (t - seg * trips_per_seg) * 128;
-        const bf16_t* in = p.in[seg] + (int64_t)row * p.ld_in;
+        const bf16_t* in = p.in[seg] + (int64_t)src_row * p.ld_in;
         uint4 av[4], bv[JB][4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
@@ -84,7 +85,7 @@ __global__ __launch_bounds__(256) void skinny_nt_kernel(SkinnyNtParams p) {
     // what the trips leave (and everything, for unaligned operands): 32-wide steps dealt the same way
     int step = 0;
     for (int seg = 0; seg < p.nseg; seg++) {
-        const bf16_t* in = p.in[seg] + (int64_t)row * p.ld_in;
+        const bf16_t* in = p.in[seg] + (int64_t)src_row * p.ld_in;
         for (int c0 = trips_per_seg * 128; c0 < p.c; c0 += 32, step++) {
             if ((step & 3) != wave) continue;
             const int cc = c0 + lq * 8;
@@ -165,7 +166,8 @@ __global__ __launch_bounds__(256) void skinny_nt_direct_kernel(SkinnyNtParams p)
 #pragma unroll
     for (int q = 0; q < 4; q++) {
         const int rl = 8 * q + (lane >> 3);
-        const int row = min(rl, rows_valid - 1);  // rows past the tile are copies of its last row, never stored
+        int row = min(rl, rows_valid - 1);  // rows past the tile are copies of its last row, never stored
+        if (p.in_rows.on()) row = rows_valid > 0 ? p.in_rows.source(r0 + row) : 0;  // the whole stored row (matrix under 4 GiB)
         in_off[q] = ((uint32_t)row * (uint32_t)p.ld_in + (uint32_t)(a_slot(rl, lane & 7) * 8)) * 2u;
     }
 #pragma unroll
@@ -181,7 +183,7 @@ __global__ __launch_bounds__(256) void skinny_nt_direct_kernel(SkinnyNtParams p)
     const int steps_per_seg = p.c / 64, steps = steps_per_seg * p.nseg;
     auto issue = [&](int step, int stage) {
         const int seg = step / steps_per_seg, c0 = (step - seg * steps_per_seg) * 64;
-        const bf16_t* in_base = p.in[seg] + (int64_t)r0 * p.ld_in + c0;
+        const bf16_t* in_base = p.in[seg] + (p.in_rows.on() ? 0 : (int64_t)r0 * p.ld_in) + c0;
         const bf16_t* f_base = FNAT ? f + ((int64_t)seg * p.c + c0) * p.r : f + seg * p.c + c0;
         const uint32_t lds = my_lds + stage * kStage;
 #pragma unroll
@@ -309,10 +311,11 @@ __global__ __launch_bounds__(256) void factor_grad_kernel(FactorGradParams p) {
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             const int r = m0 + 32 * u + tr;
+            const int src = r < row_end ? p.in_rows.source(r) : 0;
 #pragma unroll
             for (int cb = 0; cb < CB; cb++) {
                 const int tcc = c0 + cb * 64 + tch * 8;
-                vin[u][cb] = load8g(in + (int64_t)r * p.ld_in + tcc, r < row_end ? p.c - tcc : 0, vec);
+                vin[u][cb] = load8g(in + (int64_t)src * p.ld_in + tcc, r < row_end ? p.c - tcc : 0, vec);
             }
             vs[u] = make_uint4(0, 0, 0, 0);
             if (sr < 32 && m0 + 32 * u + sr < row_end) vs[u] = *(const uint4*)(p.s + (int64_t)(m0 + 32 * u + sr) * rp + sch * 8);
@@ -490,6 +493,10 @@ int skinny_nt(const SkinnyNtParams& p, int r_pad, int grid_tiles, hipStream_t s)
     bool direct = (p.ld_in & 7) == 0 && (p.ldf & 7) == 0 && (p.c & 63) == 0 && ((uintptr_t)p.f & 15) == 0 && (p.f_expert_elems & 7) == 0 &&
                   (uint64_t)64 * (uint64_t)p.ld_in * 2 < (1ull << 31) && (uint64_t)64 * (uint64_t)p.ldf * 2 < (1ull << 31);
     for (int seg = 0; seg < p.nseg; seg++) direct = direct && ((uintptr_t)p.in[seg] & 15) == 0;
+    if (p.in_rows.on()) {
+        if (p.nseg != 1 || p.in_rows.index_div <= 0 || p.in_rows.index_rows <= 0) return set_error(GGQ_ERR_SHAPE, "skinny_nt: a row index needs one segment and a positive divisor and row count");
+        direct = direct && (uint64_t)p.in_rows.index_rows * (uint64_t)p.ld_in * 2 < (1ull << 32);
+    }
     if (p.f_natural) {
         if (!skinny_nt_takes_natural_factor(p)) return set_error(GGQ_ERR_SHAPE, "skinny_nt: this shape needs the factor transposed");
         switch (r_pad / 16) {

@@ -91,13 +91,16 @@ struct Direct {
         const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem_raw;
         // A tile loads: instruction i fills slots 256 i + tid: tile row 32 i + tid / 8, slot tid % 8.  Rows past the
         // group's end repeat its last row (their results are never stored).
-        const bf16_t* a_base = p.a[0] + (int64_t)c.row_begin * p.lda;
+        // With a row index the lane offsets carry the whole stored row (the host keeps the matrix under 4 GiB).
+        const bf16_t* a_base = p.a[0] + (p.a_rows.on() ? 0 : (int64_t)c.row_begin * p.lda);
         uint32_t a_voff[LIVE];  // (lane offsets stay fixed; the step moves the scalar base)
 #pragma unroll
         for (int i = 0; i < LIVE; i++) {
             const int r = 32 * i + (tid >> 3), s = tid & 7;
             const int kc = s ^ ((r >> 1) & 7);
-            a_voff[i] = (uint32_t)(((int64_t)min(r, c.rows_valid - 1) * p.lda + kc * 8) * 2);
+            const int rr = min(r, c.rows_valid - 1);
+            const int src = p.a_rows.on() ? p.a_rows.source(c.row_begin + rr) : rr;
+            a_voff[i] = (uint32_t)(((int64_t)src * p.lda + kc * 8) * 2);
         }
         // The load cursor: (column tile, step) of the next step to request.  A lane's two packed rows are the
         // columns 64 wave + lane_c (+ 32) of the cursor's tile (columns past the segment's end repeat its last).

@@ -11,9 +11,24 @@ struct TileDesc {  // one row tile of an expert group: rows [row_begin, row_end)
     int group, row_begin, row_end, expert;
 };
 
+// Rows read through an index: logical row i of an operand is its stored row row_index[i] / index_div (clamped to
+// index_rows - 1), so expert-sorted routes can read the token matrix in place: row_index = the sorted-position ->
+// route permutation, index_div = routes per token.  A null row_index means stored row i.
+struct RowIndex {
+    const int64_t* row_index;
+    int index_div, index_rows;
+    __host__ __device__ bool on() const { return row_index != nullptr; }
+#if defined(__HIPCC__)
+    __device__ __forceinline__ int source(int i) const {
+        return row_index ? min((int)((uint32_t)row_index[i] / (uint32_t)index_div), index_rows - 1) : i;
+    }
+#endif
+};
+
 struct SkinnyNtParams {
     const bf16_t* in[2];  // [m, c] per segment
     int64_t ld_in;
+    RowIndex in_rows;     // segment 0 only (nseg == 1 when set)
     const bf16_t* f;      // per expert [r][ldf], contraction contiguous; or [nseg*c][r] when f_natural
     int64_t ldf, f_expert_elems;
     int f_natural;
@@ -27,6 +42,7 @@ struct SkinnyNtParams {
 struct FactorGradParams {
     const bf16_t* in[2];  // [m, c] per segment
     int64_t ld_in;
+    RowIndex in_rows;     // segment 0 only (nseg == 1 when set)
     const bf16_t* s;      // [m, r_pad]
     bf16_t* out;          // per expert: [nseg*c][r] (out_j_major = 0) or [r][nseg*c] (= 1)
     int64_t out_expert_elems;
@@ -54,6 +70,7 @@ enum : int {
 struct MmqParams {
     const bf16_t* a[2];   // activations; [1] only for a pair in NN mode
     int64_t lda;
+    RowIndex a_rows;      // direct shape, NT mode only
     const uint8_t* w[2];  // packed weights; [1] only for a pair
     int64_t w_row_bytes, w_expert_bytes;
     void* c[2];           // outputs; [1] only for a pair in NT mode

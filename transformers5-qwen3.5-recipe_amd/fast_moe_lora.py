@@ -50,8 +50,10 @@ def _lora_ws(device, rows, groups, experts, n_total, k, r):
     return torch.empty(nbytes, dtype=torch.uint8, device=device)
 
 
-def _grouped_forward(x, p1, p2, expert_indices, expert_offsets, quant_type, n, lora_a, lora_b, scaling):
-    rows, k = x.shape
+def _grouped_forward(x, p1, p2, expert_indices, expert_offsets, quant_type, n, lora_a, lora_b, scaling, row_index=None, index_div=1):
+    """``row_index`` (int64, one entry per expert-sorted row) makes row i of the launch row ``row_index[i] // index_div`` of x."""
+    k = x.shape[1]
+    rows = x.shape[0] if row_index is None else row_index.numel()
     experts = p1.shape[0]
     _check_grouped(x, p1, expert_indices, expert_offsets, quant_type, n, k, "grouped_mmq")
     if p2 is not None:
@@ -72,14 +74,18 @@ def _grouped_forward(x, p1, p2, expert_indices, expert_offsets, quant_type, n, l
     y2 = torch.empty(rows, n, dtype=torch.bfloat16, device=x.device) if p2 is not None else None
     if rows:
         ws = _lora_ws(x.device, rows, expert_indices.numel(), experts, nseg * n, k, r)
-        _lib.check(_lib.load().ggq_grouped_lora_mmq_forward(
-            x.data_ptr(), p1.data_ptr(), _lib.ptr(p2), expert_indices.data_ptr(), expert_offsets.data_ptr(), expert_indices.numel(),
-            experts, quant_type, rows, n, k, _lib.ptr(lora_a), _lib.ptr(lora_b), r, float(scaling), _lib.ptr(xa), y1.data_ptr(),
-            _lib.ptr(y2), ws.data_ptr(), ws.numel(), _lib.stream_handle(x.device)))
+        tail = (p1.data_ptr(), _lib.ptr(p2), expert_indices.data_ptr(), expert_offsets.data_ptr(), expert_indices.numel(),
+                experts, quant_type, rows, n, k, _lib.ptr(lora_a), _lib.ptr(lora_b), r, float(scaling), _lib.ptr(xa), y1.data_ptr(),
+                _lib.ptr(y2), ws.data_ptr(), ws.numel(), _lib.stream_handle(x.device))
+        if row_index is None:
+            _lib.check(_lib.load().ggq_grouped_lora_mmq_forward(x.data_ptr(), *tail))
+        else:
+            _lib.check(_lib.load().ggq_grouped_lora_mmq_forward_indexed(x.data_ptr(), x.shape[0], row_index.data_ptr(), int(index_div), *tail))
     return y1, y2, xa
 
 
-def _grouped_backward(dy1, dy2, p1, p2, expert_indices, expert_offsets, quant_type, k, x, xa, lora_a, lora_b, scaling, want_da, want_db):
+def _grouped_backward(dy1, dy2, p1, p2, expert_indices, expert_offsets, quant_type, k, x, xa, lora_a, lora_b, scaling, want_da, want_db,
+                      row_index=None, index_div=1):
     rows, n = dy1.shape
     experts = p1.shape[0]
     _check_grouped(dy1, p1, expert_indices, expert_offsets, quant_type, n, k, "grouped_mmq_grad_input")
@@ -91,10 +97,14 @@ def _grouped_backward(dy1, dy2, p1, p2, expert_indices, expert_offsets, quant_ty
     da = torch.empty_like(lora_a) if (lora_a is not None and want_da) else None
     db = torch.empty_like(lora_b) if (lora_b is not None and want_db) else None
     ws = _lora_ws(dy1.device, rows, expert_indices.numel(), experts, nseg * n, k, r)
-    _lib.check(_lib.load().ggq_grouped_lora_mmq_backward(
-        dy1.data_ptr(), _lib.ptr(dy2), p1.data_ptr(), _lib.ptr(p2), expert_indices.data_ptr(), expert_offsets.data_ptr(),
-        expert_indices.numel(), experts, quant_type, rows, n, k, _lib.ptr(x), _lib.ptr(xa), _lib.ptr(lora_a), _lib.ptr(lora_b), r,
-        float(scaling), dx.data_ptr(), _lib.ptr(da), _lib.ptr(db), ws.data_ptr(), ws.numel(), _lib.stream_handle(dy1.device)))
+    head = (dy1.data_ptr(), _lib.ptr(dy2), p1.data_ptr(), _lib.ptr(p2), expert_indices.data_ptr(), expert_offsets.data_ptr(),
+            expert_indices.numel(), experts, quant_type, rows, n, k, _lib.ptr(x))
+    tail = (_lib.ptr(xa), _lib.ptr(lora_a), _lib.ptr(lora_b), r, float(scaling), dx.data_ptr(), _lib.ptr(da), _lib.ptr(db), ws.data_ptr(),
+            ws.numel(), _lib.stream_handle(dy1.device))
+    if row_index is None:
+        _lib.check(_lib.load().ggq_grouped_lora_mmq_backward(*head, *tail))
+    else:
+        _lib.check(_lib.load().ggq_grouped_lora_mmq_backward_indexed(*head, x.shape[0], row_index.data_ptr(), int(index_div), *tail))
     return dx, da, db
 
 
@@ -155,6 +165,66 @@ class _GroupedLoraProjection(torch.autograd.Function):
         dx, da, db = _grouped_backward(g1, g2, p1, p2, expert_indices, expert_offsets, quant_type, x.shape[1], x, xa, lora_a, lora_b,
                                        scaling, want_da, want_db)
         return (dx if ctx.needs_input_grad[0] else None), None, None, None, None, None, None, da, db, None
+
+
+class _RoutedGroupedLoraProjection(torch.autograd.Function):
+    """``_GroupedLoraProjection`` applied to ``hidden_states[permutation // top_k]`` without that copy: the launch reads the
+    token rows through the permutation, and the backward sums every token's routes (the backward of the reference's
+    ``_RouteGather``, fast_moe_routing.py:126-160) after the input-gradient launch.  Bit-identical to gather + projection."""
+
+    @staticmethod
+    def forward(ctx, hidden_states, permutation, inverse_permutation, top_k, p1, p2, expert_indices, expert_offsets, quant_type, n,
+                lora_a, lora_b, scaling):
+        y1, y2, xa = _grouped_forward(hidden_states, p1, p2, expert_indices, expert_offsets, quant_type, n, lora_a, lora_b, scaling,
+                                      row_index=permutation, index_div=top_k)
+        tensors = [hidden_states, permutation, inverse_permutation, expert_indices, expert_offsets, p1]
+        ctx.has_pair, ctx.has_lora = p2 is not None, lora_a is not None
+        if ctx.has_pair:
+            tensors.append(p2)
+        if ctx.has_lora:
+            tensors += [xa, lora_a, lora_b]
+        ctx.save_for_backward(*tensors)
+        ctx.meta = (quant_type, n, float(scaling), int(top_k))
+        if ctx.has_pair:
+            return y1, y2
+        return y1
+
+    @staticmethod
+    def backward(ctx, *grads):
+        if torch.is_grad_enabled():
+            raise RuntimeError("packed grouped MMQ does not support higher-order gradients")
+        saved = list(ctx.saved_tensors)
+        hidden_states, permutation, inverse_permutation, expert_indices, expert_offsets, p1 = saved[:6]
+        rest = saved[6:]
+        p2 = rest.pop(0) if ctx.has_pair else None
+        xa, lora_a, lora_b = rest if ctx.has_lora else (None, None, None)
+        quant_type, n, scaling, top_k = ctx.meta
+        g1 = grads[0]
+        g2 = grads[1] if ctx.has_pair else None
+        if ctx.has_pair and (g1 is None or g2 is None):
+            if g1 is None and g2 is None:
+                return (None,) * 13
+            like = g1 if g1 is not None else g2
+            g1 = torch.zeros_like(like) if g1 is None else g1
+            g2 = torch.zeros_like(like) if g2 is None else g2
+        g1 = g1.contiguous()
+        g2 = g2.contiguous() if g2 is not None else None
+        want_da, want_db = ctx.needs_input_grad[10], ctx.needs_input_grad[11]
+        tokens, k = hidden_states.shape
+        d_selected, da, db = _grouped_backward(g1, g2, p1, p2, expert_indices, expert_offsets, quant_type, k, hidden_states, xa, lora_a,
+                                               lora_b, scaling, want_da, want_db, row_index=permutation, index_div=top_k)
+        d_hidden = None
+        if ctx.needs_input_grad[0]:
+            d_hidden = torch.empty(tokens, k, dtype=d_selected.dtype, device=d_selected.device)
+            _lib.check(_lib.load().ggq_route_gather_backward(d_selected.data_ptr(), inverse_permutation.data_ptr(), d_hidden.data_ptr(),
+                                                             tokens, top_k, k, _lib.stream_handle(d_selected.device)))
+        return (d_hidden,) + (None,) * 9 + (da, db, None)
+
+
+def routed_projection_reads_tokens_in_place(quant_type: int, routes: int, groups: int, tokens: int, in_features: int) -> bool:
+    """Whether the first grouped launch of an expert FFN can read the token matrix through the routing permutation
+    (host-side answer of the library, no device work)."""
+    return bool(_lib.load().ggq_grouped_forward_reads_indexed_rows(int(quant_type), int(routes), int(groups), int(tokens), int(in_features)))
 
 
 def _as_payload(w):
@@ -306,7 +376,11 @@ def qwen3_5_moe_gguf_mmq_lora_forward(self: GGUFExperts, hidden_states: torch.Te
         raise RuntimeError("Paired grouped GGUF MMQ requires one quantization type.")
 
     compute_hidden_states = self._prepare_expert_hidden_states(hidden_states)
-    routing_plan = prepare_expert_routing(compute_hidden_states, top_k_index, top_k_weights, self.num_experts)
+    tokens, top_k = top_k_index.shape[0], top_k_index.shape[1]
+    # The gate/up launch reads the token rows in place where it can; the routed copy is made otherwise.
+    in_place = (compute_hidden_states.ndim == 2 and compute_hidden_states.is_contiguous() and compute_hidden_states.data_ptr() % 16 == 0
+                and routed_projection_reads_tokens_in_place(self.gate_proj.quant_type, tokens * top_k, self.num_experts, tokens, self.hidden_dim))
+    routing_plan = prepare_expert_routing(compute_hidden_states, top_k_index, top_k_weights, self.num_experts, gather=not in_place)
     execution_plan = self._prepare_expert_execution(routing_plan, "grouped_mm")
     if execution_plan.offsets is None:
         raise RuntimeError("GGUF LoRA requires grouped expert offsets.")
@@ -315,9 +389,15 @@ def qwen3_5_moe_gguf_mmq_lora_forward(self: GGUFExperts, hidden_states: torch.Te
     lw = lora_weights
     s = lw.scaling if lw is not None else 0.0
 
-    gate, up = _GroupedLoraProjection.apply(
-        selected, _as_payload(self.gate_proj), _as_payload(self.up_proj), expert_indices, expert_offsets,
-        int(self.gate_proj.quant_type), self.intermediate_dim, lw.gate_up_a if lw else None, lw.gate_up_b if lw else None, s)
+    if in_place:
+        gate, up = _RoutedGroupedLoraProjection.apply(
+            compute_hidden_states, routing_plan.permutation, routing_plan.inverse_permutation, top_k, _as_payload(self.gate_proj),
+            _as_payload(self.up_proj), expert_indices, expert_offsets, int(self.gate_proj.quant_type), self.intermediate_dim,
+            lw.gate_up_a if lw else None, lw.gate_up_b if lw else None, s)
+    else:
+        gate, up = _GroupedLoraProjection.apply(
+            selected, _as_payload(self.gate_proj), _as_payload(self.up_proj), expert_indices, expert_offsets,
+            int(self.gate_proj.quant_type), self.intermediate_dim, lw.gate_up_a if lw else None, lw.gate_up_b if lw else None, s)
     intermediate = self._apply_split_gate(gate, up)
     output = _GroupedLoraProjection.apply(
         intermediate, _as_payload(self.down_proj), None, expert_indices, expert_offsets, int(self.down_proj.quant_type),

@@ -20,7 +20,7 @@ from . import _lib
 
 @dataclass(frozen=True)
 class ExpertRoutingPlan:
-    selected_hidden_states: torch.Tensor   # [routes, hidden] bf16, expert-sorted
+    selected_hidden_states: torch.Tensor | None  # [routes, hidden] bf16, expert-sorted (None: prepared with gather=False)
     expert_indices: torch.Tensor           # [routes] int64, sorted expert id of every row
     routing_weights: torch.Tensor          # [tokens, top_k]
     permutation: torch.Tensor              # [routes] int64: sorted position -> route (token*k + rank)
@@ -136,7 +136,9 @@ def _validate_routing(hidden_states, top_k_index, top_k_weights) -> None:
 
 
 def prepare_expert_routing(hidden_states: torch.Tensor, top_k_index: torch.Tensor, top_k_weights: torch.Tensor,
-                           num_experts: int | None = None) -> ExpertRoutingPlan:
+                           num_experts: int | None = None, gather: bool = True) -> ExpertRoutingPlan:
+    """``gather=False`` leaves ``selected_hidden_states`` unset, for a caller whose first grouped launch reads the token
+    rows through ``permutation`` itself."""
     if hidden_states.ndim != 2:
         raise ValueError(f"Expert routing expects hidden states [tokens, hidden], got {hidden_states.shape}.")
     if top_k_index.ndim != 2 or top_k_weights.shape != top_k_index.shape:
@@ -149,7 +151,7 @@ def prepare_expert_routing(hidden_states: torch.Tensor, top_k_index: torch.Tenso
         # the reference's sort needs no expert count; without one, size the histogram from the data
         num_experts = int(top_k_index.max().item()) + 1
     sorted_ids, perm, inv, counts, ends, active_ids, active_ends, status = build_route_plan(top_k_index.contiguous(), num_experts)
-    selected = _RouteGather.apply(hidden_states, perm, inv)
+    selected = _RouteGather.apply(hidden_states, perm, inv) if gather else None
     return ExpertRoutingPlan(
         selected_hidden_states=selected, expert_indices=sorted_ids, routing_weights=routing_weights,
         permutation=perm, inverse_permutation=inv, num_tokens=hidden_states.shape[0], num_top_k=top_k_index.shape[1],
