@@ -206,7 +206,7 @@ def main() -> None:
     # HBM bytes per launch (fetched + written, average of the gate/up and down launches) from the FETCH_SIZE /
     # WRITE_SIZE counter runs summarised in profiles/mmq_direct_and_mixed_q4k_grouped_moe_lora_step.pmc_traffic.txt;
     # the counters are collected offline, so this figure only changes when that profile is redone.
-    traffic_bytes = {0: 642.2e6 + 101.1e6, 1: 343.6e6 + 83.9e6}[dominant]
+    traffic_bytes = {0: 572.1e6 + 100.7e6, 1: 343.6e6 + 83.9e6}[dominant]
 
     result = {
         "metric": "fwd+bwd TFLOP/s and weight GB/s, Q4_K grouped-MoE LoRA; % of MI355X roofline",
