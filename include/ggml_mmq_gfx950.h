@@ -9,8 +9,8 @@
  *   - every pointer is a device pointer unless it is a `stream` (a hipStream_t passed as void*);
  *   - matrices are row-major and contiguous; activations and LoRA factors are bf16 (uint16 storage);
  *   - packed weights are the raw GGUF blocks of a [N, K] tensor, row after row, read-only, never
- *     copied or repacked; supported GGML type ids: 8 (Q8_0), 10 (Q2_K), 12 (Q4_K), 13 (Q5_K), 14 (Q6_K),
- *     16 (IQ2_XXS);
+ *     copied or repacked; supported GGML type ids: 8 (Q8_0), 10 (Q2_K), 11 (Q3_K), 12 (Q4_K), 13 (Q5_K),
+ *     14 (Q6_K), 16 (IQ2_XXS);
  *     K must be a multiple of 64 and of the type's block size;
  *   - nothing is allocated inside: the caller passes outputs and, where stated, a workspace whose size
  *     comes from the matching *_workspace_bytes function (256-byte aligned carving inside);

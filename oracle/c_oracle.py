@@ -8,7 +8,7 @@ from pathlib import Path
 
 import numpy as np
 
-from .gguf_blocks import IQ2_XXS, Q2_K, Q4_K, Q5_K, Q6_K, Q8_0, QUANT_SIZES
+from .gguf_blocks import IQ2_XXS, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K, Q8_0, QUANT_SIZES
 from .iq2xxs_grid import IQ2XXS_GRID
 
 _HERE = Path(__file__).resolve().parent
@@ -49,6 +49,8 @@ def dequantize(payload: np.ndarray, qt: int) -> np.ndarray:
         L.oracle_dequant_q5_k(src, ctypes.c_int64(nb), dst)
     elif qt == Q2_K:
         L.oracle_dequant_q2_k(src, ctypes.c_int64(nb), dst)
+    elif qt == Q3_K:
+        L.oracle_dequant_q3_k(src, ctypes.c_int64(nb), dst)
     elif qt == IQ2_XXS:
         grid = np.array(IQ2XXS_GRID, dtype=np.uint64)
         L.oracle_dequant_iq2_xxs(src, ctypes.c_int64(nb), grid.ctypes.data_as(ctypes.c_void_p), dst)

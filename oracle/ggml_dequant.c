@@ -136,6 +136,41 @@ void oracle_dequant_q2_k(const uint8_t *x, int64_t nb, float *y) {
     }
 }
 
+/* y[256*nb] from nb blocks of {u8 hmask[32]; u8 qs[64]; u8 scales[12]; f16 d} (dequantize_row_q3_K): the twelve
+ * scale bytes unpack to sixteen 6-bit values through the word-wise mask shuffle of the format's reference code. */
+void oracle_dequant_q3_k(const uint8_t *x, int64_t nb, float *y) {
+    const uint32_t kmask1 = 0x03030303u, kmask2 = 0x0f0f0f0fu;
+    for (int64_t i = 0; i < nb; i++, x += 110) {
+        const uint8_t *hm = x;
+        const uint8_t *q = x + 32;
+        float d_all = half_to_float(rd16(x + 108));
+        uint32_t aux[4];
+        for (int w = 0; w < 3; w++)
+            aux[w] = (uint32_t)x[96 + 4 * w] | ((uint32_t)x[97 + 4 * w] << 8) | ((uint32_t)x[98 + 4 * w] << 16) | ((uint32_t)x[99 + 4 * w] << 24);
+        uint32_t tmp = aux[2];
+        aux[2] = ((aux[0] >> 4) & kmask2) | (((tmp >> 4) & kmask1) << 4);
+        aux[3] = ((aux[1] >> 4) & kmask2) | (((tmp >> 6) & kmask1) << 4);
+        aux[0] = (aux[0] & kmask2) | (((tmp >> 0) & kmask1) << 4);
+        aux[1] = (aux[1] & kmask2) | (((tmp >> 2) & kmask1) << 4);
+        int8_t scales[16];
+        for (int k = 0; k < 16; k++) scales[k] = (int8_t)((aux[k / 4] >> (8 * (k % 4))) & 0xFF);
+        int is = 0;
+        uint8_t m = 1;
+        for (int n = 0; n < 256; n += 128) {
+            int shift = 0;
+            for (int j = 0; j < 4; j++) {
+                float dl = d_all * (float)(scales[is++] - 32);
+                for (int l = 0; l < 16; l++) *y++ = dl * (float)((int)((q[l] >> shift) & 3) - ((hm[l] & m) ? 0 : 4));
+                dl = d_all * (float)(scales[is++] - 32);
+                for (int l = 0; l < 16; l++) *y++ = dl * (float)((int)((q[l + 16] >> shift) & 3) - ((hm[l + 16] & m) ? 0 : 4));
+                shift += 2;
+                m <<= 1;
+            }
+            q += 32;
+        }
+    }
+}
+
 /* y[256*nb] from nb blocks of {u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d} */
 void oracle_dequant_q6_k(const uint8_t *x, int64_t nb, float *y) {
     for (int64_t i = 0; i < nb; i++, x += 210) {

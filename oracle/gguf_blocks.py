@@ -12,12 +12,13 @@ decoders below restate the published ggml block layouts (ggml-common.h / ggml-qu
   type      id  block bytes  elements  layout
   Q8_0       8      34          32     f16 d; i8 qs[32]
   Q2_K      10      84         256     u8 scales[16]; u8 qs[64]; f16 d; f16 dmin
+  Q3_K      11     110         256     u8 hmask[32]; u8 qs[64]; u8 scales[12]; f16 d
   Q4_K      12     144         256     f16 d; f16 dmin; u8 scales[12]; u8 qs[128]
   Q5_K      13     176         256     f16 d; f16 dmin; u8 scales[12]; u8 qh[32]; u8 qs[128]
   Q6_K      14     210         256     u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d
   IQ2_XXS   16      66         256     f16 d; u16 qs[32]
 
-All decoders return float32 values that are *exact* products except Q2_K, Q4_K and Q5_K, whose
+All decoders return float32 values that are *exact* products (Q3_K included) except Q2_K, Q4_K and Q5_K, whose
 ``d*sc*q - dmin*m`` rounds once to float32 (d*sc, dmin*m and (d*sc)*q are exact: 11+6+4 significand bits).  The bf16
 weights the matmul oracles use are ``round-to-nearest-even(float32 value)``.
 
@@ -37,10 +38,10 @@ import numpy as np
 
 from .iq2xxs_grid import IQ2XXS_GRID
 
-Q8_0, Q2_K, Q4_K, Q5_K, Q6_K, IQ2_XXS = 8, 10, 12, 13, 14, 16
+Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K, IQ2_XXS = 8, 10, 11, 12, 13, 14, 16
 # (elements per block, bytes per block); matches gguf.GGML_QUANT_SIZES used at
 # test_deepseek_v4_moe_lora.py:58.
-QUANT_SIZES = {Q8_0: (32, 34), Q2_K: (256, 84), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), IQ2_XXS: (256, 66)}
+QUANT_SIZES = {Q8_0: (32, 34), Q2_K: (256, 84), Q3_K: (256, 110), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), IQ2_XXS: (256, 66)}
 
 _GRID_BYTES = np.array(IQ2XXS_GRID, dtype=np.uint64).view(np.uint8).reshape(256, 8)  # little endian
 # ksigns_iq2xs[i] = i | (parity(i) << 7): the eighth sign makes the number of minus signs even.
@@ -69,7 +70,7 @@ def dequantize(payload: np.ndarray, qt: int) -> np.ndarray:
         raise ValueError("payload row is not a whole number of blocks")
     lead = payload.shape[:-1]
     blocks = payload.reshape(-1, nbytes)
-    out = {Q8_0: _deq_q8_0, Q2_K: _deq_q2_k, Q4_K: _deq_q4_k, Q5_K: _deq_q5_k, Q6_K: _deq_q6_k, IQ2_XXS: _deq_iq2_xxs}[qt](blocks)
+    out = {Q8_0: _deq_q8_0, Q2_K: _deq_q2_k, Q3_K: _deq_q3_k, Q4_K: _deq_q4_k, Q5_K: _deq_q5_k, Q6_K: _deq_q6_k, IQ2_XXS: _deq_iq2_xxs}[qt](blocks)
     return out.reshape(*lead, payload.shape[-1] // nbytes * elems)
 
 
@@ -127,6 +128,35 @@ def _deq_q5_k(b: np.ndarray) -> np.ndarray:
     y = dl[:, :, None] * q                                 # exact in float32 (11 + 6 + 5 bits)
     y = y - ml[:, :, None]                                 # one float32 rounding
     return y.reshape(nb, 256)
+
+
+def unpack_q3_k_scales(s: np.ndarray) -> np.ndarray:
+    """12 packed bytes -> sixteen signed scales (6-bit value - 32): scale k keeps its low four bits in nibble k // 8 of
+    byte (k // 4 % 2) * 4 + k % 4 and its high two bits at position 2 (k // 4) of byte 8 + k % 4."""
+    s = s.astype(np.int32)
+    out = np.empty(s.shape[:-1] + (16,), dtype=np.int32)
+    for k in range(16):
+        low = (s[..., (k // 4 % 2) * 4 + k % 4] >> (4 * (k // 8))) & 0xF
+        high = (s[..., 8 + k % 4] >> (2 * (k // 4))) & 3
+        out[..., k] = (low | (high << 4)) - 32
+    return out
+
+
+def _deq_q3_k(b: np.ndarray) -> np.ndarray:
+    """Sixteen 16-element sub-blocks with signed 6-bit scales; element 128 n + 32 j + l is bits 2j..2j+1 of
+    qs[32 n + l], minus 4 unless bit 4 n + j of hmask[l] is set (ggml dequantize_row_q3_K)."""
+    nb = b.shape[0]
+    hm = b[:, 0:32]
+    qs = b[:, 32:96].reshape(nb, 2, 32)
+    d = _f16(b[:, 108:110])
+    dl = d * unpack_q3_k_scales(b[:, 96:108]).astype(np.float32)     # [nb,16] exact
+    q = np.empty((nb, 2, 4, 32), dtype=np.float32)
+    for n in range(2):
+        for j in range(4):
+            low = ((qs[:, n, :] >> (2 * j)) & 3).astype(np.int32)
+            high = ((hm >> (4 * n + j)) & 1).astype(np.int32)
+            q[:, n, j, :] = low - 4 * (1 - high)
+    return (dl[:, :, None] * q.reshape(nb, 16, 16)).reshape(nb, 256)
 
 
 def _deq_q2_k(b: np.ndarray) -> np.ndarray:
@@ -214,7 +244,7 @@ def quantize(w: np.ndarray, qt: int) -> np.ndarray:
         raise ValueError(f"last dim {w.shape[-1]} is not a multiple of {elems}")
     lead = w.shape[:-1]
     blocks = w.reshape(-1, elems)
-    out = {Q8_0: _q_q8_0, Q2_K: _q_q2_k, Q4_K: _q_q4_k, Q5_K: _q_q5_k, Q6_K: _q_q6_k, IQ2_XXS: _q_iq2_xxs}[qt](blocks)
+    out = {Q8_0: _q_q8_0, Q2_K: _q_q2_k, Q3_K: _q_q3_k, Q4_K: _q_q4_k, Q5_K: _q_q5_k, Q6_K: _q_q6_k, IQ2_XXS: _q_iq2_xxs}[qt](blocks)
     return out.reshape(*lead, w.shape[-1] // elems * nbytes)
 
 
@@ -318,6 +348,33 @@ def _q_q2_k(x: np.ndarray) -> np.ndarray:
     return out
 
 
+def _q_q3_k(x: np.ndarray) -> np.ndarray:
+    nb = x.shape[0]
+    sub = x.reshape(nb, 16, 16)
+    scale = np.abs(sub).max(axis=2) / np.float32(4)
+    d = (scale.max(axis=1, keepdims=True) / np.float32(31)).astype(np.float16).astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        sc = np.where(d > 0, np.clip(_roundf(scale / d), 0, 31), 0).astype(np.int32)
+        dl = d * sc.astype(np.float32)
+        q = np.where(dl[:, :, None] > 0, _roundf(sub / dl[:, :, None]), 0)
+    v = (np.clip(q, -4, 3).astype(np.int32) + 4).astype(np.uint8).reshape(nb, 2, 4, 32)   # [n, j, l]: element 128 n + 32 j + l
+    out = np.zeros((nb, 110), dtype=np.uint8)
+    hm = np.zeros((nb, 32), dtype=np.uint8)
+    qs = np.zeros((nb, 2, 32), dtype=np.uint8)
+    for n in range(2):
+        for j in range(4):
+            qs[:, n, :] |= (v[:, n, j, :] & 3) << (2 * j)
+            hm |= (v[:, n, j, :] >> 2) << (4 * n + j)
+    out[:, 0:32] = hm
+    out[:, 32:96] = qs.reshape(nb, 64)
+    s6 = (sc + 32).astype(np.uint8)
+    for k in range(16):
+        out[:, 96 + (k // 4 % 2) * 4 + k % 4] |= (s6[:, k] & 0xF) << (4 * (k // 8))
+        out[:, 104 + k % 4] |= (s6[:, k] >> 4) << (2 * (k // 4))
+    out[:, 108:110] = _f16_bytes(d).reshape(-1, 2)
+    return out
+
+
 def _q_q6_k(x: np.ndarray) -> np.ndarray:
     nb = x.shape[0]
     sub = x.reshape(nb, 16, 16)
@@ -381,10 +438,12 @@ def random_payload(rng: np.random.Generator, qt: int, rows: int, k: int, std: fl
     elems, nbytes = QUANT_SIZES[qt]
     nb = rows * (k // elems)
     b = rng.integers(0, 256, size=(nb, nbytes), dtype=np.uint8)
-    mag = {Q8_0: std / 64, Q2_K: std / 25, Q4_K: std / 250, Q5_K: std / 800, Q6_K: std / 1500, IQ2_XXS: std / 60}[qt]
+    mag = {Q8_0: std / 64, Q2_K: std / 25, Q3_K: std / 60, Q4_K: std / 250, Q5_K: std / 800, Q6_K: std / 1500, IQ2_XXS: std / 60}[qt]
     d = (mag * (0.5 + rng.random(nb))).astype(np.float32)
     if qt == Q6_K:
         b[:, 208:210] = _f16_bytes(d).reshape(-1, 2)
+    elif qt == Q3_K:
+        b[:, 108:110] = _f16_bytes(d).reshape(-1, 2)
     elif qt == Q2_K:
         b[:, 80:82] = _f16_bytes(d).reshape(-1, 2)
         b[:, 82:84] = _f16_bytes(d * np.float32(0.7)).reshape(-1, 2)

@@ -7,8 +7,8 @@ import torch
 
 from oracle import gguf_blocks as gb
 
-ALL_TYPES = (gb.Q8_0, gb.Q2_K, gb.Q4_K, gb.Q5_K, gb.Q6_K, gb.IQ2_XXS)
-TYPE_NAMES = {gb.Q8_0: "Q8_0", gb.Q2_K: "Q2_K", gb.Q4_K: "Q4_K", gb.Q5_K: "Q5_K", gb.Q6_K: "Q6_K", gb.IQ2_XXS: "IQ2_XXS"}
+ALL_TYPES = (gb.Q8_0, gb.Q2_K, gb.Q3_K, gb.Q4_K, gb.Q5_K, gb.Q6_K, gb.IQ2_XXS)
+TYPE_NAMES = {gb.Q8_0: "Q8_0", gb.Q2_K: "Q2_K", gb.Q3_K: "Q3_K", gb.Q4_K: "Q4_K", gb.Q5_K: "Q5_K", gb.Q6_K: "Q6_K", gb.IQ2_XXS: "IQ2_XXS"}
 # bf16 tolerance of the path (BASELINE: max rel err <= 2e-2)
 MAX_REL = 2e-2
 

@@ -46,7 +46,7 @@ def test_host_only_helpers(pkg):
         assert lib.ggq_row_bytes(qt, 4 * elems) == 4 * nbytes
         assert lib.ggq_row_bytes(qt, elems + 1) == -1
         assert pkg.gguf.row_bytes(qt, 2 * elems) == 2 * nbytes
-    for qt in (0, 2, 11, 99):  # F32, Q4_0, Q3_K: no kernels here
+    for qt in (0, 2, 15, 99):  # F32, Q4_0, Q8_K: no kernels here
         assert lib.ggq_supports_quant_type(qt) == 0
         assert lib.ggq_row_bytes(qt, 256) == -1
     assert isinstance(lib.ggq_last_error(), bytes)

@@ -65,6 +65,23 @@ def test_q5_k_known_answer():
         assert y[e] == v, (e, y[e], v)
 
 
+def test_q3_k_known_answer():
+    # d = 0.5; 6-bit scales 24..39 (signed -8..7), packed by hand: low nibbles 8..15 in the low halves of bytes 0..7,
+    # 0..7 in their high halves, the upper two bits (1,1,2,2 per group of four) as 0xA5 in bytes 8..11; qs as in the
+    # Q2_K block; hmask[l] = 0xA5 for even l, 0x5A for odd l (a clear bit subtracts 4).
+    blk = np.zeros(110, dtype=np.uint8)
+    blk[0:32] = [0xA5, 0x5A] * 16
+    blk[32:96] = [0xE4, 0x1B] * 32
+    blk[96:108] = [0x08, 0x19, 0x2A, 0x3B, 0x4C, 0x5D, 0x6E, 0x7F, 0xA5, 0xA5, 0xA5, 0xA5]
+    blk[108:110] = F16[0.5]
+    assert gb.unpack_q3_k_scales(blk[96:108]).tolist() == list(range(-8, 8))
+    y = both(blk[None, :], gb.Q3_K)[0]
+    want = {0: 0.0, 1: 4.0, 17: 3.5, 32: 9.0, 33: -6.0, 96: 1.0, 127: 0.0, 128: 0.0, 160: 1.0, 177: -3.0,
+            254: 10.5, 255: -14.0}
+    for e, v in want.items():
+        assert y[e] == v, (e, y[e], v)
+
+
 def test_q2_k_known_answer():
     # d = 0.5, dmin = 0.25; scales[k] = k | (15-k) << 4 (scale k, min 15-k); qs = 0xE4 at even bytes
     # (bit pairs 0,1,2,3 from the bottom) and 0x1B at odd bytes (3,2,1,0).
@@ -126,7 +143,7 @@ def test_iq2xxs_grid_structure():
     assert int(((n19 == 2) & (n2b == 0)).sum()) == 28 and int(((n19 == 0) & (n2b == 1)).sum()) == 8
 
 
-@pytest.mark.parametrize("qt", [gb.Q8_0, gb.Q2_K, gb.Q4_K, gb.Q5_K, gb.Q6_K, gb.IQ2_XXS])
+@pytest.mark.parametrize("qt", [gb.Q8_0, gb.Q2_K, gb.Q3_K, gb.Q4_K, gb.Q5_K, gb.Q6_K, gb.IQ2_XXS])
 def test_numpy_and_c_agree_on_arbitrary_bytes(qt):
     payload = gb.random_payload(np.random.default_rng(qt), qt, 23, 1024)
     y = both(payload, qt)
@@ -162,6 +179,19 @@ def test_format_invariants():
     dmin = p[0, 82:84].copy().view(np.float16).astype(np.float32)[0]
     y = gb.dequantize(p, gb.Q2_K)[0].reshape(16, 16)
     assert np.array_equal(y, np.repeat((-(dmin * (p[0, :16] >> 4).astype(np.float32)))[:, None], 16, axis=1))
+    # Q3_K: setting every hmask bit adds exactly 4*d*scale to the values whose bit was clear; negating d negates all
+    p = gb.random_payload(rng, gb.Q3_K, 1, 256)
+    p1 = p.copy()
+    p1[0, 0:32] = 0xFF
+    d = p[0, 108:110].copy().view(np.float16).astype(np.float32)[0]
+    sc = gb.unpack_q3_k_scales(p[0, 96:108]).astype(np.float32)
+    clear = 1.0 - ((p[0, 0:32][None, :] >> np.arange(8)[:, None]) & 1).astype(np.float32)     # [run u, l]
+    step = (d * sc).reshape(8, 2)[:, :, None] * 4.0 * clear.reshape(8, 2, 16)
+    got = (gb.dequantize(p1, gb.Q3_K) - gb.dequantize(p, gb.Q3_K))[0].reshape(8, 2, 16)
+    assert np.array_equal(got, step)
+    pn = p.copy()
+    pn[0, 109] ^= 0x80
+    assert np.array_equal(gb.dequantize(pn, gb.Q3_K), -gb.dequantize(p, gb.Q3_K))
     # negating an IQ2_XXS block scale negates every weight; Q8_0 is linear in d
     p = gb.random_payload(rng, gb.IQ2_XXS, 1, 256)
     q = p.copy()
@@ -179,7 +209,7 @@ def test_bf16_rounding_is_nearest_even():
     assert np.array_equal(gb.to_bf16_bits(x), want)
 
 
-@pytest.mark.parametrize("qt,bound", [(gb.Q8_0, 0.01), (gb.Q2_K, 0.35), (gb.Q4_K, 0.12), (gb.Q5_K, 0.06), (gb.Q6_K, 0.03),
+@pytest.mark.parametrize("qt,bound", [(gb.Q8_0, 0.01), (gb.Q2_K, 0.35), (gb.Q3_K, 0.25), (gb.Q4_K, 0.12), (gb.Q5_K, 0.06), (gb.Q6_K, 0.03),
                                       (gb.IQ2_XXS, 0.6)])
 def test_quantizer_round_trip_error(qt, bound):
     rng = np.random.default_rng(11)

@@ -192,6 +192,51 @@ struct Fmt<kQ2_K> {
 };
 
 // ------------------------------------------------------------------------------------------------
+// Q3_K: 110-byte block = u8 hmask[32]; u8 qs[64]; u8 scales[12]; f16 d (2-byte aligned).  Run u = ksub & 7 takes
+// bit pair u % 4 of qs[32 (u / 4) .. +31] and bit u of hmask[l] for its element l: value (pair | bit << 2) - 4 in
+// [-4, 3].  Sixteen 6-bit scales (stored + 32): scale k has its low four bits in the nibble k / 8 of byte
+// (k / 4 % 2) * 4 + k % 4 and its high two bits at position 2 (k / 4) of byte 8 + k % 4; elements 0..15 of the run use
+// scale 2 u, elements 16..31 scale 2 u + 1.
+template <>
+struct Fmt<kQ3_K> {
+    static constexpr int kBlockElems = 256, kBlockBytes = 110;
+    struct Raw {
+        uint4 h0, h1, q0, q1;
+        uint32_t sl, sh, d16;
+    };
+    static GGQ_HD void pin(Raw& r) { GGQ_PIN4(r.h0); GGQ_PIN4(r.h1); GGQ_PIN4(r.q0); GGQ_PIN4(r.q1); GGQ_PIN1(r.sl); GGQ_PIN1(r.sh); GGQ_PIN1(r.d16); }
+    static GGQ_HD void load(Raw& r, const uint8_t* row, int ksub) {
+        const uint8_t* blk = row + (int64_t)(ksub >> 3) * 110;
+        const int u = ksub & 7, n = u >> 2, g = u >> 1, b = 2 * (u & 1);
+        r.h0 = ld_u128(blk), r.h1 = ld_u128(blk + 16);
+        r.q0 = ld_u128(blk + 32 + 32 * n), r.q1 = ld_u128(blk + 48 + 32 * n);
+        r.sl = ld_u16(blk + 96 + 4 * (g & 1) + b);
+        r.sh = ld_u16(blk + 104 + b);
+        r.d16 = ld_u16(blk + 108);
+    }
+    static GGQ_HD void decode(const Raw& r, int ksub, uint32_t* out, const uint2*) {
+        const int u = ksub & 7, g = u >> 1, shift = 2 * (u & 3);
+        const float d = half_bits_to_f32(r.d16);
+        const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+        const uint32_t h[8] = {r.h0.x, r.h0.y, r.h0.z, r.h0.w, r.h1.x, r.h1.y, r.h1.z, r.h1.w};
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const uint32_t lo = (r.sl >> (8 * half)) & 0xFFu, hi = (r.sh >> (8 * half)) & 0xFFu;
+            const int sc = (int)(((lo >> (4 * (g >> 1))) & 0xFu) | (((hi >> (2 * g)) & 3u) << 4)) - 32;
+            const float ds = d * (float)sc;
+            const float dl = ds * kMixScale, nm = -4.0f * ds;
+#pragma unroll
+            for (int i = 4 * half; i < 4 * half + 4; i++) {
+                const uint32_t v = ((q[i] >> shift) & 0x03030303u) | (((h[i] >> u) & 0x01010101u) << 2);
+                const uint32_t e02 = v & 0x00070007u, e13 = (v >> 8) & 0x00070007u;
+                out[2 * i] = pack_bf16(mix_lo(e02, dl, nm), mix_lo(e13, dl, nm));
+                out[2 * i + 1] = pack_bf16(mix_hi(e02, dl, nm), mix_hi(e13, dl, nm));
+            }
+        }
+    }
+};
+
+// ------------------------------------------------------------------------------------------------
 // Q6_K: 210-byte block = u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d.  Blocks are only 2-byte
 // aligned.  Run u = ksub & 7 lives in half h = u/4 as part p = u%4: low (p < 2) or high nibbles of
 // ql[64h + 32(p&1) .. +31], bit pair 2p of qh[32h .. +31], int8 scales[8h + 2p], [8h + 2p + 1].

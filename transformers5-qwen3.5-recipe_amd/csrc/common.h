@@ -6,7 +6,7 @@
 namespace ggq {
 
 // GGML type ids of the supported block formats.
-enum : int { kQ8_0 = 8, kQ2_K = 10, kQ4_K = 12, kQ5_K = 13, kQ6_K = 14, kIQ2_XXS = 16 };
+enum : int { kQ8_0 = 8, kQ2_K = 10, kQ3_K = 11, kQ4_K = 12, kQ5_K = 13, kQ6_K = 14, kIQ2_XXS = 16 };
 
 // Decoder helpers are host+device so the bit unpacking can also be exercised in a CPU build.
 #define GGQ_HD __host__ __device__ __forceinline__

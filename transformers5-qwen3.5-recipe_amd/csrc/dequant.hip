@@ -68,6 +68,16 @@ __device__ __forceinline__ void decode8(const uint8_t* raw, int g, float* y) {
         const uint8_t* q = blk + 16 + 32 * n + l0;
 #pragma unroll
         for (int i = 0; i < 8; i++) y[i] = __fsub_rn(__fmul_rn(dl, (float)((q[i] >> (2 * j)) & 3u)), ml);
+    } else if constexpr (QT == kQ3_K) {
+        const uint8_t* blk = raw + (g >> 5) * 110;
+        const int e0 = 8 * (g & 31), n = e0 >> 7, u = e0 >> 5, l0 = e0 & 31, k = e0 >> 4, kg = k >> 2, kb = k & 3;
+        const float d = half_bits_to_f32(lds_u16(blk + 108));
+        const int sc = (int)(((blk[96 + 4 * (kg & 1) + kb] >> (4 * (kg >> 1))) & 0xFu) | (((blk[104 + kb] >> (2 * kg)) & 3u) << 4)) - 32;
+        const float dl = d * (float)sc;
+        const uint8_t* q = blk + 32 + 32 * n + l0;
+        const uint8_t* hm = blk + l0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) y[i] = dl * (float)((int)((q[i] >> (2 * (u & 3))) & 3u) - (((hm[i] >> u) & 1u) ? 0 : 4));
     } else if constexpr (QT == kQ6_K) {
         const uint8_t* blk = raw + (g >> 5) * 210;
         const int e0 = 8 * (g & 31), h = e0 >> 7, part = (e0 & 127) >> 5, l0 = e0 & 31;
@@ -151,6 +161,7 @@ int dequantize(int qt, const void* payload, int64_t rows, int64_t k, void* out, 
     switch (qt) {
         case kQ8_0: return launch_dequant<kQ8_0>(payload, total, out, out_f32, stream);
         case kQ2_K: return launch_dequant<kQ2_K>(payload, total, out, out_f32, stream);
+        case kQ3_K: return launch_dequant<kQ3_K>(payload, total, out, out_f32, stream);
         case kQ4_K: return launch_dequant<kQ4_K>(payload, total, out, out_f32, stream);
         case kQ5_K: return launch_dequant<kQ5_K>(payload, total, out, out_f32, stream);
         case kQ6_K: return launch_dequant<kQ6_K>(payload, total, out, out_f32, stream);

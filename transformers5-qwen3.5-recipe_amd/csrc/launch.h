@@ -21,7 +21,7 @@ int check_launch(const char* what);
 inline bool block_multiple(int qt, int64_t k) {
     switch (qt) {
         case 8: return k % 32 == 0;
-        case 10: case 12: case 13: case 14: case 16: return k % 256 == 0;
+        case 10: case 11: case 12: case 13: case 14: case 16: return k % 256 == 0;
     }
     return true;  // unknown types are rejected by the callers' switch
 }
@@ -29,6 +29,7 @@ inline int64_t packed_row_bytes(int qt, int64_t k) {
     switch (qt) {
         case 8: return k / 32 * 34;
         case 10: return k / 256 * 84;
+        case 11: return k / 256 * 110;
         case 12: return k / 256 * 144;
         case 13: return k / 256 * 176;
         case 14: return k / 256 * 210;

@@ -249,12 +249,13 @@ int launch_mmq(int qt, int mode, int epi, const MmqParams& p, hipStream_t s) {
     switch (qt) {
         case kQ8_0: return launch_qt<kQ8_0>(mode, epi, p, s);
         case kQ2_K: return launch_qt<kQ2_K>(mode, epi, p, s);
+        case kQ3_K: return launch_qt<kQ3_K>(mode, epi, p, s);
         case kQ4_K: return launch_qt<kQ4_K>(mode, epi, p, s);
         case kQ5_K: return launch_qt<kQ5_K>(mode, epi, p, s);
         case kQ6_K: return launch_qt<kQ6_K>(mode, epi, p, s);
         case kIQ2_XXS: return launch_qt<kIQ2_XXS>(mode, epi, p, s);
     }
-    return set_error(GGQ_ERR_QTYPE, "unsupported GGML type id %d (supported: 8 Q8_0, 10 Q2_K, 12 Q4_K, 13 Q5_K, 14 Q6_K, 16 IQ2_XXS)", qt);
+    return set_error(GGQ_ERR_QTYPE, "unsupported GGML type id %d (supported: 8 Q8_0, 10 Q2_K, 11 Q3_K, 12 Q4_K, 13 Q5_K, 14 Q6_K, 16 IQ2_XXS)", qt);
 }
 
 // Fills the shape-derived fields of a parameter block.  n, k describe one weight segment [n, k].

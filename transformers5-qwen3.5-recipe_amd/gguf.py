@@ -18,10 +18,10 @@ import torch
 
 from . import _lib
 
-Q8_0, Q2_K, Q4_K, Q5_K, Q6_K, IQ2_XXS = 8, 10, 12, 13, 14, 16
+Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K, IQ2_XXS = 8, 10, 11, 12, 13, 14, 16
 # type id -> (elements per block, bytes per block)
-GGML_QUANT_SIZES = {Q8_0: (32, 34), Q2_K: (256, 84), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), IQ2_XXS: (256, 66)}
-QUANT_NAMES = {Q8_0: "Q8_0", Q2_K: "Q2_K", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", IQ2_XXS: "IQ2_XXS"}
+GGML_QUANT_SIZES = {Q8_0: (32, 34), Q2_K: (256, 84), Q3_K: (256, 110), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), IQ2_XXS: (256, 66)}
+QUANT_NAMES = {Q8_0: "Q8_0", Q2_K: "Q2_K", Q3_K: "Q3_K", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", IQ2_XXS: "IQ2_XXS"}
 
 
 def row_bytes(quant_type: int, k: int) -> int:
