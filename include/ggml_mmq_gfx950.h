@@ -102,9 +102,9 @@ int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* 
  * (prepare_expert_routing, fast_moe_routing.py:379-420: _RouteGather.apply(hidden_states, permutation, ...)) and hands the
  * copy to the grouped ops; here row i of the expert-sorted layout is read in place as row row_index[i] / index_div of
  * x [x_rows, k] (row_index = the sorted-position -> route permutation, index_div = top_k).  Results are bit-identical to
- * the plain calls on the gathered copy.  Only some launches can do this: ask ggq_grouped_forward_reads_indexed_rows
- * (host-only, 1 = yes) with the same qt / rows / groups / x_rows / k first; the indexed forward returns the shape error
- * otherwise.  dx is still per expert-sorted row, [rows, k]. */
+ * the plain calls on the gathered copy.  x must stay under 4 GiB (the kernels address its rows with 32-bit offsets): ask
+ * ggq_grouped_forward_reads_indexed_rows (host-only, 1 = yes) with the same qt / rows / groups / x_rows / k first; the
+ * indexed forward returns the shape error otherwise.  dx is still per expert-sorted row, [rows, k]. */
 int ggq_grouped_forward_reads_indexed_rows(int qt, int64_t rows, int64_t groups, int64_t x_rows, int64_t k);
 int ggq_grouped_lora_mmq_forward_indexed(const void* x, int64_t x_rows, const int64_t* row_index, int index_div, const void* packed1,
                                          const void* packed2, const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups,

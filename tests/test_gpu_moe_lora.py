@@ -157,11 +157,16 @@ def test_grouped_lora_projection_all_gradients(pkg, dev, qt, r, shape, n, monkey
     assert_close_bf16(bd2.grad, want1["db"], "single dB")
 
 
-@pytest.mark.parametrize("top_k,rank,pair", [(8, 16, True), (3, 4, True), (1, 16, False), (8, 0, True)])
-def test_routed_projection_reads_tokens_in_place(pkg, dev, top_k, rank, pair):
+@pytest.mark.parametrize("top_k,rank,pair,qt,shape", [(8, 16, True, gb.Q4_K, ""), (3, 4, True, gb.Q4_K, ""), (1, 16, False, gb.Q4_K, ""),
+                                                      (8, 0, True, gb.Q4_K, ""), (8, 16, True, gb.Q4_K, "1"), (3, 16, True, gb.Q4_K, "0"),
+                                                      (2, 8, True, gb.Q4_K, "2"), (8, 16, True, gb.Q6_K, ""), (3, 4, False, gb.IQ2_XXS, "")])
+def test_routed_projection_reads_tokens_in_place(pkg, dev, top_k, rank, pair, qt, shape, monkeypatch):
     # The gate/up launch that reads the token matrix through the routing permutation against the same launch on the
     # gathered copy: outputs, token gradients (summed over each token's routes) and factor gradients are the same bits.
-    # Skewed routing: some experts receive no route, one receives more than a 192-row tile.
+    # Skewed routing: some experts receive no route, one receives more than a 192-row tile.  Every kernel shape of the
+    # forward launch takes the index (the decoding-wave kernel by default for Q4_K, the tile kernels otherwise).
+    if shape:
+        monkeypatch.setenv("GGQ_GROUPED_SHAPE", shape)
     ml, mr = pkg.fast_moe_lora, pkg.fast_moe_routing
     tokens, k, n, experts = 211, 512, 256, 12
     gen = torch.Generator().manual_seed(977 + top_k)
@@ -172,16 +177,16 @@ def test_routed_projection_reads_tokens_in_place(pkg, dev, top_k, rank, pair):
     scores[:, 2] += 0.9 if top_k > 1 else 0.4
     idx = scores.topk(top_k, dim=1).indices
     w = torch.full((tokens, top_k), 1.0 / top_k)
-    p1, p2 = _expert_payload(31, gb.Q4_K, experts, n, k), _expert_payload(32, gb.Q4_K, experts, n, k)
+    p1, p2 = _expert_payload(31, qt, experts, n, k), _expert_payload(32, qt, experts, n, k)
     p1d, p2d = torch.from_numpy(p1).to(dev), (torch.from_numpy(p2).to(dev) if pair else None)
     nseg = 2 if pair else 1
     a = bf16_randn(gen, experts, rank, k, std=k ** -0.5) if rank else None
     b = bf16_randn(gen, experts, nseg * n, rank, std=0.02) if rank else None
     dy = [bf16_randn(gen, tokens * top_k, n).to(dev) for _ in range(nseg)]
     routes = tokens * top_k
-    assert ml.routed_projection_reads_tokens_in_place(gb.Q4_K, routes, experts, tokens, k)
-    assert not ml.routed_projection_reads_tokens_in_place(gb.Q6_K, routes, experts, tokens, k)
-    assert not ml.routed_projection_reads_tokens_in_place(gb.Q4_K, routes, 1, tokens, k) or routes <= 256
+    assert ml.routed_projection_reads_tokens_in_place(qt, routes, experts, tokens, k)
+    assert not ml.routed_projection_reads_tokens_in_place(qt, routes, experts, 1 << 21, 1024)   # a 4 GiB token matrix
+    assert not ml.routed_projection_reads_tokens_in_place(3, routes, experts, tokens, k)        # no kernels for this type
 
     def run(in_place):
         xd = x.to(dev).requires_grad_(True)
@@ -191,9 +196,9 @@ def test_routed_projection_reads_tokens_in_place(pkg, dev, top_k, rank, pair):
         if in_place:
             assert plan.selected_hidden_states is None
             out = ml._RoutedGroupedLoraProjection.apply(xd, plan.permutation, plan.inverse_permutation, top_k, p1d, p2d, ids,
-                                                        plan.expert_end_offsets, gb.Q4_K, n, ad, bd, 2.0)
+                                                        plan.expert_end_offsets, qt, n, ad, bd, 2.0)
         else:
-            out = ml._GroupedLoraProjection.apply(plan.selected_hidden_states, p1d, p2d, ids, plan.expert_end_offsets, gb.Q4_K, n, ad, bd, 2.0)
+            out = ml._GroupedLoraProjection.apply(plan.selected_hidden_states, p1d, p2d, ids, plan.expert_end_offsets, qt, n, ad, bd, 2.0)
         out = out if pair else (out,)
         torch.autograd.backward(out, tuple(dy))
         return [*out, xd.grad] + ([ad.grad, bd.grad] if rank else [])
@@ -205,7 +210,7 @@ def test_routed_projection_reads_tokens_in_place(pkg, dev, top_k, rank, pair):
     _, perm, _ = rref.plan(idx)
     sel = rref.gather_forward(x, perm, top_k)
     ends = torch.cumsum(rref.expert_counts(idx, experts).to(torch.int64), 0).to(torch.int32)
-    wcat = torch.cat([ref.weights_bf16(p1, gb.Q4_K)] + ([ref.weights_bf16(p2, gb.Q4_K)] if pair else []), dim=1)
+    wcat = torch.cat([ref.weights_bf16(p1, qt)] + ([ref.weights_bf16(p2, qt)] if pair else []), dim=1)
     o = ref.grouped_lora_linear(sel, wcat, torch.arange(experts), ends, a, b, 2.0, torch.cat([d.cpu() for d in dy], dim=1))
     assert_close_bf16(torch.cat(got[:nseg], dim=1), o["y"], "in-place Y against the oracle")
     if rank:

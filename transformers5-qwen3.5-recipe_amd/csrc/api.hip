@@ -166,10 +166,11 @@ int ggq_fixed_grouped_mmq_grad_input(const void* dy, const void* packed_groups, 
 
 // Forward of one projection (or a gate/up pair) over expert-sorted rows, optional LoRA fused.
 // groups == 0 means dense: one group of all rows using expert 0.
-// The forward launch reads its rows through an index only in the direct kernel: Q4_K expert groups of at most 256 rows
-// on average, and a source matrix under 4 GiB (the lane offsets of its loads are 32-bit).
+// The forward launch reads its rows through an index when the source matrix stays under 4 GiB (the lane offsets of its
+// loads are 32-bit).
 static bool forward_reads_indexed_rows(int qt, int64_t rows, int64_t groups, int64_t x_rows, int64_t k) {
-    return x_rows > 0 && k < (1 << 22) && (uint64_t)x_rows * (uint64_t)k * 2 < (1ull << 32) && pick_shape(qt, rows, groups, true) == kShapeDirect;
+    (void)rows, (void)groups;
+    return packed_row_bytes(qt, 256) > 0 && x_rows > 0 && k > 0 && (uint64_t)x_rows * (uint64_t)k * 2 < (1ull << 32);
 }
 
 int ggq_grouped_forward_reads_indexed_rows(int qt, int64_t rows, int64_t groups, int64_t x_rows, int64_t k) {
@@ -197,8 +198,8 @@ static int grouped_forward(const char* what, const void* x, RowIndex x_index, co
     // the direct kernel moves A, LA and LB rows with aligned 16-byte accesses
     const bool direct_ok = aligned16(x) && k < (1 << 22) && (!lora_a || (aligned16(xa_out) && (rp != r || aligned16(lora_b))));
     if (int rc = init_params(p, qt, kModeNT, (int)rows, (int)n, (int)k, nseg, pick_shape(qt, rows, groups, direct_ok))) return rc;
-    if (x_index.on() && (p.shape != kShapeDirect || !forward_reads_indexed_rows(qt, rows, groups, x_index.index_rows, k) || x_index.index_div <= 0))
-        return set_error(GGQ_ERR_SHAPE, "%s: this type, shape or alignment cannot read its rows through an index (ask ggq_grouped_forward_reads_indexed_rows first)", what);
+    if (x_index.on() && (!forward_reads_indexed_rows(qt, rows, groups, x_index.index_rows, k) || x_index.index_div <= 0))
+        return set_error(GGQ_ERR_SHAPE, "%s: this source matrix cannot be read through a row index (ask ggq_grouped_forward_reads_indexed_rows first)", what);
     p.a[0] = (const bf16_t*)x, p.lda = k, p.a_rows = x_index;
     p.w[0] = (const uint8_t*)packed1, p.w[1] = (const uint8_t*)packed2;
     p.c[0] = y1, p.c[1] = y2, p.ldc = n;

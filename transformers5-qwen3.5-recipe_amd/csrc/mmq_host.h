@@ -70,7 +70,7 @@ enum : int {
 struct MmqParams {
     const bf16_t* a[2];   // activations; [1] only for a pair in NN mode
     int64_t lda;
-    RowIndex a_rows;      // direct shape, NT mode only
+    RowIndex a_rows;      // NT mode only (segment 0 is the only activation matrix there)
     const uint8_t* w[2];  // packed weights; [1] only for a pair
     int64_t w_row_bytes, w_expert_bytes;
     void* c[2];           // outputs; [1] only for a pair in NT mode

@@ -138,7 +138,9 @@ static __device__ __forceinline__ void a_loader_init(ALoader& a, const MmqParams
     for (int j = 0; j < kGroupsPerWave; j++) {
         // rows past the end of the group are clamped to its last row: they only feed output rows that
         // are never stored
-        const int row = min(8 * kCW * j + sub, c.rows_valid - 1);
+        int row = min(8 * kCW * j + sub, c.rows_valid - 1);
+        // with a row index the offset carries the whole stored row (the host keeps that matrix under 4 GiB)
+        if (p.a_rows.on()) row = c.rows_valid > 0 ? p.a_rows.source(c.row_begin + row) : 0;
         a.voff[j] = ((uint32_t)row * (uint32_t)p.lda + (uint32_t)kc * 8u) * 2u;
     }
     a.lds0 = c.as_lds + cw * 1024;
@@ -150,7 +152,7 @@ template <int MODE, int J0, int J1>
 static __device__ __forceinline__ void a_issue(const ALoader& a, const MmqParams& p, const TileCtx& c, int step, int stage) {
     int seg_k, kc0;
     step_origin<MODE>(p, step, seg_k, kc0);
-    const bf16_t* sbase = p.a[MODE == kModeNN ? seg_k : 0] + (int64_t)c.row_begin * p.lda + kc0;
+    const bf16_t* sbase = p.a[MODE == kModeNN ? seg_k : 0] + (p.a_rows.on() ? 0 : (int64_t)c.row_begin * p.lda) + kc0;
     const uint32_t lds = a.lds0 + stage * kAStageBytes;
 #pragma unroll
     for (int j = J0; j < J1 && j < kGroupsPerWave; j++)
@@ -203,7 +205,7 @@ static __device__ __forceinline__ void fill_a_slow(const MmqParams& p, const Til
     for (int id = l.ptid; id < kTM * 8; id += 256) {
         const int r = id >> 3, ch = id & 7;
         if (r >= c.rows_valid) break;
-        const bf16_t* src = p.a[MODE == kModeNN ? seg_k : 0] + (int64_t)(c.row_begin + r) * p.lda + kc0 + ch * 8;
+        const bf16_t* src = p.a[MODE == kModeNN ? seg_k : 0] + (int64_t)p.a_rows.source(c.row_begin + r) * p.lda + kc0 + ch * 8;
         *(uint4*)(at + r * kARowBytes + a_slot(r, ch) * 16) = load8_slow(src, c.contraction - (kc0 + ch * 8));
     }
 }

@@ -378,7 +378,7 @@ def qwen3_5_moe_gguf_mmq_lora_forward(self: GGUFExperts, hidden_states: torch.Te
     compute_hidden_states = self._prepare_expert_hidden_states(hidden_states)
     tokens, top_k = top_k_index.shape[0], top_k_index.shape[1]
     # The gate/up launch reads the token rows in place where it can; the routed copy is made otherwise.
-    in_place = (compute_hidden_states.ndim == 2 and compute_hidden_states.is_contiguous() and compute_hidden_states.data_ptr() % 16 == 0
+    in_place = (compute_hidden_states.ndim == 2 and compute_hidden_states.is_contiguous()
                 and routed_projection_reads_tokens_in_place(self.gate_proj.quant_type, tokens * top_k, self.num_experts, tokens, self.hidden_dim))
     routing_plan = prepare_expert_routing(compute_hidden_states, top_k_index, top_k_weights, self.num_experts, gather=not in_place)
     execution_plan = self._prepare_expert_execution(routing_plan, "grouped_mm")
