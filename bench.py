@@ -62,10 +62,10 @@ def build_workload(pkg, dev, cfg, seed=19260817 + 2):
     experts = pkg.fast_moe_lora.GGUFExperts(gate, up, down)
     layer = pkg.fast_moe_lora.FastGGUFMoeLora(experts, r=r, lora_alpha=cfg["alpha"])
     with torch.no_grad():
-        layer.lora_A["default"].copy_((torch.randn(e, r, h, generator=g, device=dev) * h ** -0.5).to(torch.bfloat16))
-        layer.lora_B["default"].copy_((torch.randn(e, 2 * i, r, generator=g, device=dev) * 0.01).to(torch.bfloat16))
-        layer.lora_A_down["default"].copy_((torch.randn(e, r, i, generator=g, device=dev) * i ** -0.5).to(torch.bfloat16))
-        layer.lora_B_down["default"].copy_((torch.randn(e, h, r, generator=g, device=dev) * 0.01).to(torch.bfloat16))
+        layer.lora_A["default"].weight.copy_((torch.randn(e, r, h, generator=g, device=dev) * h ** -0.5).to(torch.bfloat16))
+        layer.lora_B["default"].weight.copy_((torch.randn(e, 2 * i, r, generator=g, device=dev) * 0.01).to(torch.bfloat16))
+        layer.lora_A_down["default"].weight.copy_((torch.randn(e, r, i, generator=g, device=dev) * i ** -0.5).to(torch.bfloat16))
+        layer.lora_B_down["default"].weight.copy_((torch.randn(e, h, r, generator=g, device=dev) * 0.01).to(torch.bfloat16))
     x = torch.randn(cfg["tokens"], h, generator=g, device=dev).to(torch.bfloat16).requires_grad_(True)
     logits = torch.randn(cfg["tokens"], e, generator=g, device=dev)
     top = torch.topk(logits, cfg["top_k"], dim=-1)

@@ -263,8 +263,8 @@ def test_expert_layer_forward_backward(pkg, dev, qt, tokens, hidden, inter, expe
                          G(torch.from_numpy(pd).to(dev), qt, (experts, hidden, inter)))
     layer = ml.FastGGUFMoeLora(mod, r=r, lora_alpha=32)
     with torch.no_grad():
-        layer.lora_A["default"].copy_(a_gu.to(dev)); layer.lora_B["default"].copy_(b_gu.to(dev))
-        layer.lora_A_down["default"].copy_(a_d.to(dev)); layer.lora_B_down["default"].copy_(b_d.to(dev))
+        layer.lora_A["default"].weight.copy_(a_gu.to(dev)); layer.lora_B["default"].weight.copy_(b_gu.to(dev))
+        layer.lora_A_down["default"].weight.copy_(a_d.to(dev)); layer.lora_B_down["default"].weight.copy_(b_d.to(dev))
     xd = x.to(dev).requires_grad_(True)
     wd = w.to(dev).requires_grad_(True)
     out = layer(xd, idx.to(dev), wd)
@@ -275,7 +275,7 @@ def test_expert_layer_forward_backward(pkg, dev, qt, tokens, hidden, inter, expe
     assert_close_bf16(wd.grad, want_dw, "dRoutingWeights", ulps=6)
     for name, param, key in (("dA_gate_up", layer.lora_A, "da_gu"), ("dB_gate_up", layer.lora_B, "db_gu"),
                              ("dA_down", layer.lora_A_down, "da_d"), ("dB_down", layer.lora_B_down, "db_d")):
-        assert_close_bf16(param["default"].grad, res[key], name, ulps=6)
+        assert_close_bf16(param["default"].weight.grad, res[key], name, ulps=6)
     active = torch.unique(idx)
     inactive = torch.ones(experts, dtype=torch.bool)
     inactive[active] = False

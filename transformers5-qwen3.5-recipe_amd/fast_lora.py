@@ -263,3 +263,52 @@ class FastGGUFLoraLinear(torch.nn.Module):
 
     def unmerge(self) -> None:
         raise RuntimeError("GGUF LoRA adapters cannot be unmerged because merging is unsupported.")
+
+
+# ------------------------------------------------------------------------------------------------
+# Adapter checkpoints with PEFT's key names (what the reference saves and loads through
+# get_peft_model_state_dict / set_peft_model_state_dict, test_deepseek_v4_serialization.py:74-101): only the LoRA
+# factors, the adapter's name taken out of the keys ("...lora_A_down.default.weight" -> "...lora_A_down.weight").
+_ADAPTER_PREFIX = "lora_"
+
+
+def get_adapter_state_dict(model: torch.nn.Module, adapter_name: str = "default", prefix: str = "") -> dict[str, torch.Tensor]:
+    """The adapter's factors under checkpoint names; ``prefix`` (e.g. ``"base_model.model."``) is put in front of every
+    key for files that PEFT's own wrapper is to read."""
+    out = {}
+    for key, value in model.state_dict().items():
+        if _ADAPTER_PREFIX not in key:
+            continue
+        parts = key.split(".")
+        if adapter_name not in parts:
+            continue  # another adapter's factors
+        i = len(parts) - 1 - parts[::-1].index(adapter_name)
+        out[prefix + ".".join(parts[:i] + parts[i + 1:])] = value
+    return out
+
+
+def set_adapter_state_dict(model: torch.nn.Module, state: dict[str, torch.Tensor], adapter_name: str = "default", prefix: str = ""):
+    """Loads a checkpoint written under those names.  Returns (missing_keys, unexpected_keys): adapter parameters of the
+    model the checkpoint lacks, and checkpoint entries no parameter takes.  Shapes must match; dtypes are cast."""
+    own = {k: v for k, v in model.state_dict().items() if _ADAPTER_PREFIX in k and adapter_name in k.split(".")}
+    renamed = {}
+    for key, value in state.items():
+        k = key[len(prefix):] if prefix and key.startswith(prefix) else key
+        if _ADAPTER_PREFIX in k:
+            suffix = k.split(_ADAPTER_PREFIX)[-1]
+            if "." in suffix:  # "A_down.weight": the adapter's name goes in front of what follows the factor's name
+                rest = ".".join(suffix.split(".")[1:])
+                k = k[: len(k) - len(rest)] + f"{adapter_name}." + rest
+            else:
+                k = f"{k}.{adapter_name}"
+        renamed[k] = value
+    unexpected = [k for k in renamed if k not in own]
+    missing = [k for k in own if k not in renamed]
+    with torch.no_grad():
+        for k, target in own.items():
+            if k in renamed:
+                src = renamed[k]
+                if tuple(src.shape) != tuple(target.shape):
+                    raise ValueError(f"adapter checkpoint entry {k}: shape {tuple(src.shape)} does not fit {tuple(target.shape)}")
+                target.copy_(src.to(device=target.device, dtype=target.dtype))
+    return missing, unexpected

@@ -405,6 +405,15 @@ def qwen3_5_moe_gguf_mmq_lora_forward(self: GGUFExperts, hidden_states: torch.Te
     return finalize_expert_routing(output, hidden_states, routing_plan, execution_plan.output_mask).reshape(hidden_states.shape)
 
 
+class _ExpertFactor(torch.nn.Module):
+    """One expert factor family as a module with a ``weight`` (fast_moe_lora.py:463-470), so adapter checkpoints carry the
+    reference's key names (``...lora_A_down.<adapter>.weight``)."""
+
+    def __init__(self, shape: tuple[int, ...], *, device, dtype):
+        super().__init__()
+        self.weight = torch.nn.Parameter(torch.empty(shape, device=device, dtype=dtype))
+
+
 class FastGGUFMoeLora(torch.nn.Module):
     """LoRA wrapper owning the four factor families of one packed ``GGUFExperts`` module
     (counterpart of fast_moe_lora.py:482-646; same parameter names and shapes)."""
@@ -425,32 +434,32 @@ class FastGGUFMoeLora(torch.nn.Module):
         dev, dt = base_layer.gate_proj.device, base_layer.compute_dtype
 
         def factor(shape):
-            return torch.nn.Parameter(torch.empty(shape, device=dev, dtype=dt))
+            return _ExpertFactor(shape, device=dev, dtype=dt)
 
-        self.lora_A = torch.nn.ParameterDict({adapter_name: factor((e, r, h))})
-        self.lora_B = torch.nn.ParameterDict({adapter_name: factor((e, 2 * i, r))})
-        self.lora_A_down = torch.nn.ParameterDict({adapter_name: factor((e, r, i))})
-        self.lora_B_down = torch.nn.ParameterDict({adapter_name: factor((e, h, r))})
+        self.lora_A = torch.nn.ModuleDict({adapter_name: factor((e, r, h))})
+        self.lora_B = torch.nn.ModuleDict({adapter_name: factor((e, 2 * i, r))})
+        self.lora_A_down = torch.nn.ModuleDict({adapter_name: factor((e, r, i))})
+        self.lora_B_down = torch.nn.ModuleDict({adapter_name: factor((e, h, r))})
         self.scaling = {adapter_name: lora_alpha / (math.sqrt(r) if use_rslora else r)}
         self.active_adapter = adapter_name
         self.disable_adapters = False
         if init_lora_weights is True:
-            torch.nn.init.kaiming_uniform_(self.lora_A[adapter_name], a=math.sqrt(5))
-            torch.nn.init.kaiming_uniform_(self.lora_A_down[adapter_name], a=math.sqrt(5))
+            torch.nn.init.kaiming_uniform_(self.lora_A[adapter_name].weight, a=math.sqrt(5))
+            torch.nn.init.kaiming_uniform_(self.lora_A_down[adapter_name].weight, a=math.sqrt(5))
         elif init_lora_weights == "gaussian":
-            torch.nn.init.normal_(self.lora_A[adapter_name], std=1 / r)
-            torch.nn.init.normal_(self.lora_A_down[adapter_name], std=1 / r)
+            torch.nn.init.normal_(self.lora_A[adapter_name].weight, std=1 / r)
+            torch.nn.init.normal_(self.lora_A_down[adapter_name].weight, std=1 / r)
         elif init_lora_weights is not False:
             raise ValueError(f"Fast GGUF MoE LoRA does not support init_lora_weights={init_lora_weights!r}.")
         if init_lora_weights is not False:
-            torch.nn.init.zeros_(self.lora_B[adapter_name])
-            torch.nn.init.zeros_(self.lora_B_down[adapter_name])
+            torch.nn.init.zeros_(self.lora_B[adapter_name].weight)
+            torch.nn.init.zeros_(self.lora_B_down[adapter_name].weight)
 
     def _active_lora_weights(self) -> _ExpertLoraWeights | None:
         if self.disable_adapters:
             return None
         n = self.active_adapter
-        return _ExpertLoraWeights(self.lora_A[n], self.lora_B[n], self.lora_A_down[n], self.lora_B_down[n], float(self.scaling[n]))
+        return _ExpertLoraWeights(self.lora_A[n].weight, self.lora_B[n].weight, self.lora_A_down[n].weight, self.lora_B_down[n].weight, float(self.scaling[n]))
 
     def forward(self, hidden_states: torch.Tensor, top_k_index: torch.Tensor, top_k_weights: torch.Tensor) -> torch.Tensor:
         return self.base_layer(hidden_states, top_k_index, top_k_weights, self._active_lora_weights())
