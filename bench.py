@@ -75,7 +75,7 @@ def build_workload(pkg, dev, cfg, seed=19260817 + 2):
     return layer, x, idx, weights, dy
 
 
-def cpu_baseline(cfg, sample_experts=64, repeats=5):
+def cpu_baseline(cfg, sample_experts=64, repeats=21):
     """Dequantize-then-matmul on the host (the reference's non-native shape of the path,
     fast_moe_lora.py:230-247): oracle decoders -> bf16 weights -> torch matmul + autograd per expert,
     on `sample_experts` experts with 128 rows each (the layer's mean load)."""
