@@ -120,8 +120,104 @@ def cpu_baseline(cfg, sample_experts=64, repeats=21):
                 sample=f"{sample_experts} of {cfg['experts']} experts x {rows} rows, dequantize (numpy oracle) + torch bf16 matmul/autograd, median of {repeats}, {med:.2f} s per pass")
 
 
+def other_workload(name, pkg, lib, dev, args):
+    """The other BASELINE configurations, timed the same way (eager launches): not the headline line, but the same JSON
+    shape, so that their kernels can be traced with the same command."""
+    g = torch.Generator(device=dev).manual_seed(3)
+
+    def bf(*shape, std=1.0):
+        return (torch.randn(*shape, generator=g, device=dev) * std).to(torch.bfloat16)
+
+    if name == "dense_q4k":  # configs[1]
+        n, k, rows = 4096, 2048, 4096
+        payload = pkg.gguf.quantize_q4_k(torch.randn(n, k, generator=g, device=dev) * 0.02)
+        x, a, b = bf(rows, k).requires_grad_(True), bf(16, k, std=k ** -0.5).requires_grad_(True), bf(n, 16, std=0.01).requires_grad_(True)
+        dy = bf(rows, n)
+        flops = 2 * 2 * rows * n * k + 3 * 2 * rows * 16 * (n + k)
+        launch_flops, launches_per_step = 2 * rows * n * k, 2
+        workload = "configs[1]: dense Q4_K LoRA linear fwd+bwd, W [4096x2048], X [4096, 2048], r=16 alpha=32"
+        metric = "fwd+bwd TFLOP/s, dense Q4_K LoRA linear"
+
+        def step():
+            x.grad = a.grad = b.grad = None
+            pkg.fast_lora.lora_mmq(x, payload, 12, n, a, b, 2.0).backward(dy)
+    elif name == "lmhead_q6k":  # configs[3]
+        vocab, hidden, rows, chunk = 151936, 2048, 4096, 1024
+        payload = torch.cat([pkg.gguf.quantize_q6_k(torch.randn(min(18992, vocab - lo), hidden, generator=g, device=dev) * 0.02)
+                             for lo in range(0, vocab, 18992)], dim=0)
+        hs = bf(rows, hidden).requires_grad_(True)
+        labels = torch.randint(0, vocab, (rows,), device=dev, generator=g)
+        labels[torch.rand(rows, device=dev, generator=g) < 0.05] = -100
+        flops = 2 * 2 * rows * vocab * hidden
+        launch_flops, launches_per_step = None, None   # three kinds of launches (statistics, gradient slab, grad-input) of different sizes
+        workload = "configs[3]: chunked cross-entropy through a Q6_K lm_head [151936x2048], 4096 rows, chunks of 1024, loss + dHidden"
+        metric = "fwd+bwd TFLOP/s (two algorithmic GEMMs), chunked lm_head cross-entropy"
+
+        def step():
+            hs.grad = None
+            pkg.gguf_liger_loss.packed_linear_cross_entropy(hs, payload, labels, 14, vocab, chunk).backward()
+    elif name == "moe_iq2xxs":  # configs[4], routed experts
+        tokens, hidden, inter, e, top_k, r = 2048, 4096, 2048, 256, 8, 16
+        G = pkg.gguf.GGUFQuantizedTensor
+        gate = G(pkg.gguf.random_iq2_xxs((e, inter, hidden), g, dev), 16, (e, inter, hidden))
+        up = G(pkg.gguf.random_iq2_xxs((e, inter, hidden), g, dev), 16, (e, inter, hidden))
+        down = G(pkg.gguf.random_iq2_xxs((e, hidden, inter), g, dev), 16, (e, hidden, inter))
+        layer = pkg.fast_moe_lora.FastGGUFMoeLora(pkg.fast_moe_lora.GGUFExperts(gate, up, down), r=r, lora_alpha=32)
+        with torch.no_grad():
+            for pname, p in layer.named_parameters():
+                p.copy_(bf(*p.shape, std=p.shape[-1] ** -0.5 if "lora_A" in pname else 0.01))
+        x = bf(tokens, hidden).requires_grad_(True)
+        top = torch.topk(torch.randn(tokens, e, generator=g, device=dev), top_k, dim=-1)
+        idx, weights = top.indices, torch.softmax(top.values, dim=-1).requires_grad_(True)
+        dy = bf(tokens, hidden)
+        routes = tokens * top_k
+        flops = 2 * 2 * routes * (2 * inter * hidden + hidden * inter) + 3 * 2 * routes * r * ((hidden + 2 * inter) + (inter + hidden))
+        launch_flops, launches_per_step = 2 * routes * (2 * inter * hidden + hidden * inter) / 2, 4
+        workload = "configs[4] routed experts: grouped-MoE IQ2_XXS LoRA fwd+bwd, 2048 tokens x top-8, hidden 4096, 256 experts, gate_up [4096x4096], down [4096x2048], r=16 alpha=32"
+        metric = "fwd+bwd TFLOP/s, IQ2_XXS grouped-MoE LoRA"
+        params = list(layer.parameters())
+
+        def step():
+            for p in params:
+                p.grad = None
+            x.grad = weights.grad = None
+            layer(x, idx, weights).backward(dy)
+    else:
+        sys.exit(f"unknown workload {name!r}")
+
+    for _ in range(max(args.warmup, 1)):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    lib.ggq_profile_begin()
+    prof_steps = min(args.steps, 5)
+    for _ in range(prof_steps):
+        step()
+    torch.cuda.synchronize()
+    cap = 8192
+    ms, qt, mode, epi = (ctypes.c_float * cap)(), (ctypes.c_int * cap)(), (ctypes.c_int * cap)(), (ctypes.c_int * cap)()
+    n_l = max(lib.ggq_profile_end(ms, qt, mode, epi, cap), 0)
+    tile_ms = sum(ms[j] for j in range(n_l)) / prof_steps
+    roofline = None
+    if launch_flops is not None and n_l:
+        avg_ms = tile_ms / launches_per_step
+        achieved = launch_flops / (avg_ms * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "kernel": "packed-weight tile kernels (all launches of the step)", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
+                    "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "avg_launch_ms": avg_ms, "launches_timed": n_l}
+    print(json.dumps({
+        "metric": metric, "value": flops / (ms_per_step * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": workload, "launch": "eager"}, "roofline": roofline, "tile_kernel_ms_per_step": tile_ms, "tile_kernel_launches_per_step": n_l / prof_steps}))
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
+    ap.add_argument("--workload", default="moe_q4k", choices=["moe_q4k", "dense_q4k", "lmhead_q6k", "moe_iq2xxs"],
+                    help="moe_q4k (default) is the headline configuration; the others are timed for reference")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
@@ -135,6 +231,9 @@ def main() -> None:
     pkg = __graft_entry__.import_package()
     lib = pkg._lib.load()
     dev = torch.device("cuda:0")
+    if args.workload != "moe_q4k":
+        other_workload(args.workload, pkg, lib, dev, args)
+        return
     cfg = CFG
     layer, x, idx, weights, dy = build_workload(pkg, dev, cfg)
     params = list(layer.parameters())

@@ -98,12 +98,17 @@ static int direct_tiles_per_wg(int64_t rows, int64_t groups, int col_tiles) {
     return e && atoi(e) > 0 ? atoi(e) : per_wg;
 }
 
+// A dense layer's factor gradients deal their rows to at most this many workgroups per column block (fp32 partial sums
+// in the workspace).
+constexpr int64_t kDenseFactorSplits = 32;
+
 int64_t ggq_lora_workspace_bytes(int64_t rows, int64_t groups, int64_t experts, int64_t n_total, int64_t k, int r) {
     const int rp = rank_pad(r > 0 ? r : 1);
     if (experts < 1) experts = 1;
     const int64_t tiles = rows / 64 + groups + 2;
     return 3 * align256(tiles * (int64_t)sizeof(TileDesc)) + align256(16) + align256(experts * 2 * 4) +
-           align256(experts * n_total * rp * 2) * 2 + align256(experts * k * rp * 2) + align256(rows * rp * 2) + 4096;
+           align256(experts * n_total * rp * 2) * 2 + align256(experts * k * rp * 2) + align256(rows * rp * 2) + 4096 +
+           (groups == 0 ? align256(kDenseFactorSplits * std::max(n_total, k) * rp * 4) : 0);
 }
 
 int ggq_lora_mmq_forward(const void* x, const void* packed, int qt, int64_t m, int64_t n, int64_t k, const void* lora_a,
@@ -357,8 +362,16 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
             if (int rc = skinny_nt(sp, rp, max_tiles64, s)) return rc;
         }
         p.la = dyb, p.lb = (const bf16_t*)lora_a, p.lb_expert_elems = (int64_t)r * k, p.r_pad = rp, p.lora_rank = r, p.lora_scale = scale;
+        float* partials = nullptr;
+        int64_t partials_bytes = 0;
+        if (groups == 0 && (d_lora_a || d_lora_b)) {  // optional: without it the rows are not split
+            partials_bytes = kDenseFactorSplits * std::max<int64_t>(ntot, k) * rp * 4;
+            partials = (float*)bump.take(partials_bytes);
+            if (!partials) partials_bytes = 0;
+        }
         if (d_lora_b) {
             FactorGradParams fp{};
+            fp.partials = partials, fp.partials_bytes = partials_bytes;
             fp.in[0] = (const bf16_t*)dy1, fp.in[1] = (const bf16_t*)dy2, fp.ld_in = n;
             fp.s = (const bf16_t*)xa, fp.out = (bf16_t*)d_lora_b, fp.out_expert_elems = ntot * r;
             fp.ranges = ranges, fp.m = (int)rows, fp.c = (int)n, fp.r = r, fp.nseg = nseg, fp.out_j_major = 0, fp.scale = scale;
@@ -366,6 +379,7 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
         }
         if (d_lora_a) {
             FactorGradParams fp{};
+            fp.partials = partials, fp.partials_bytes = partials_bytes;
             fp.in[0] = (const bf16_t*)x, fp.ld_in = k, fp.in_rows = x_index;
             fp.s = dyb, fp.out = (bf16_t*)d_lora_a, fp.out_expert_elems = (int64_t)r * k;
             fp.ranges = ranges, fp.m = (int)rows, fp.c = (int)k, fp.r = r, fp.nseg = 1, fp.out_j_major = 1, fp.scale = scale;

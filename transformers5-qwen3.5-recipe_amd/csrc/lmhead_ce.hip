@@ -1,12 +1,14 @@
 // Chunked cross-entropy through a packed lm_head without ever holding [rows, vocab] logits.
 //
-// Per row chunk:  pass 1 runs the packed-weight tile kernel over the whole vocabulary with an epilogue
+// Pass 1, per row chunk: the packed-weight tile kernel runs over the whole vocabulary with an epilogue
 // that reduces every 128-column slab of a logits tile to (max, sum exp) per row and records the target
-// logit; a small kernel merges the slabs into log-sum-exp and the per-row loss.  Pass 2 walks the
-// vocabulary in blocks of kVocabBlock columns: the tile kernel recomputes that block's logits and its
-// epilogue turns them into d(loss)/d(logits) (bf16, [chunk, kVocabBlock] only); the grad-input form of
-// the tile kernel contracts the block with the same packed rows into an fp32 accumulator.  Three
-// vocabulary-sized matmuls instead of two is the price of not materialising the logits.
+// logit; a small kernel merges the slabs into log-sum-exp and the per-row loss.  Pass 2, per block of up to
+// kGradRows rows, walks the vocabulary in blocks of kVocabBlock columns: the tile kernel recomputes that
+// block's logits and its epilogue turns them into d(loss)/d(logits) (bf16, [rows of the block, kVocabBlock]
+// only); the grad-input form of the tile kernel contracts the block with the same packed rows into an fp32
+// accumulator.  Three vocabulary-sized matmuls instead of two is the price of not materialising the logits.
+#include <algorithm>
+
 #include "common.h"
 #include "launch.h"
 #include "mmq_host.h"
@@ -14,6 +16,10 @@
 namespace ggq {
 
 constexpr int kVocabBlock = 8192;
+// The gradient pass takes up to this many rows at a time, whatever the caller's chunk (which bounds the statistics pass
+// and stands for the reference's [chunk, vocab] logits): 4096 rows fill the chip with tiles of the [rows, hidden]
+// grad-input output (a 1024-row chunk makes 64 tiles for 256 compute units) and cost a 64 MiB gradient slab.
+constexpr int64_t kGradRows = 4096;
 
 // row_scale[m] = 0 for ignored rows, else 1/n_valid (mean) or 1 (sum); n_valid = 0 gives all zeros.
 __global__ __launch_bounds__(1024) void ce_row_scale_kernel(const int64_t* labels, int64_t rows, int64_t ignore_index,
@@ -76,8 +82,9 @@ static int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
 
 int64_t lmhead_ce_workspace_bytes(int64_t rows, int64_t vocab, int64_t hidden, int64_t chunk) {
     const int64_t rc = chunk < rows ? chunk : rows;
+    const int64_t gr = std::min(rows, std::max(chunk, kGradRows));
     const int64_t nparts = (vocab + kBN - 1) / kBN * 2;
-    return align256(rows * 4) * 3 + align256(rc * nparts * 8) + align256(rc * kVocabBlock * 2) + align256(rc * hidden * 4) + 1024;
+    return align256(rows * 4) * 3 + align256(rc * nparts * 8) + align256(gr * kVocabBlock * 2) + align256(gr * hidden * 4) + 1024;
 }
 
 int lmhead_ce(int qt, const void* hidden, const void* packed, const int64_t* labels, int64_t rows, int64_t vocab,
@@ -90,13 +97,14 @@ int lmhead_ce(int qt, const void* hidden, const void* packed, const int64_t* lab
     if (((uintptr_t)hidden | (uintptr_t)packed | (uintptr_t)grad_hidden | (uintptr_t)ws) & 15) return set_error(GGQ_ERR_ALIGN, "lmhead_ce: pointers must be 16-byte aligned");
     if (rows == 0) return GGQ_OK;
     const int64_t rc_max = chunk < rows ? chunk : rows;
+    const int64_t gr_max = std::min(rows, std::max(chunk, kGradRows));
     const int nparts = (int)((vocab + kBN - 1) / kBN) * 2;
     char* w = (char*)ws;
     float* row_scale = (float*)w; w += align256(rows * 4);
     float* lse = lse_out ? lse_out : (float*)w; w += align256(rows * 4);
     float* target = (float*)w; w += align256(rows * 4);
     float2* partials = (float2*)w; w += align256(rc_max * nparts * 8);
-    bf16_t* dlogits = (bf16_t*)w; w += align256(rc_max * kVocabBlock * 2);
+    bf16_t* dlogits = (bf16_t*)w; w += align256(gr_max * kVocabBlock * 2);
     float* dh32 = (float*)w;
 
     hipLaunchKernelGGL(ce_row_scale_kernel, dim3(1), dim3(1024), 0, s, labels, rows, ignore_index, reduction_mean, row_scale, n_valid_out);
@@ -112,6 +120,11 @@ int lmhead_ce(int qt, const void* hidden, const void* packed, const int64_t* lab
         p.ignore_index = ignore_index;
         if (int rcode = launch_mmq(qt, kModeNT, kEpiCeStats, p, s)) return rcode;
         hipLaunchKernelGGL(ce_finalize_kernel, dim3((rc + 3) / 4), dim3(256), 0, s, partials, nparts, nparts, target + r0, row_scale + r0, rc, lse + r0, loss_1d + r0);
+    }
+    // gradient pass: the log-sum-exp of every row is known; row blocks of up to gr_max rows
+    for (int64_t r0 = 0; r0 < rows; r0 += gr_max) {
+        const int rc = (int)std::min(rows - r0, gr_max);
+        const bf16_t* hid = (const bf16_t*)hidden + r0 * hidden_dim;
         hipLaunchKernelGGL(fill_f32_kernel, dim3(grid1d((int64_t)rc * hidden_dim)), dim3(256), 0, s, dh32, (int64_t)rc * hidden_dim, 0.f);
         for (int64_t v0 = 0; v0 < vocab; v0 += kVocabBlock) {
             const int nb = (int)((vocab - v0) < kVocabBlock ? (vocab - v0) : kVocabBlock);

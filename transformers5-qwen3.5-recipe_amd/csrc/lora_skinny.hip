@@ -4,6 +4,7 @@
 //   skinny_nt      out[m, j]  = sum_c In[m, c] * F[e][j, c]          (x A^T,  dY B via B^T)
 //   factor_grad    G[e][c, j] = s * sum_{m in group e} In[m, c] * S[m, j]   (dB, dA; fixed order, no atomics)
 //   pad / transpose helpers that lay the factors out [cols][r_pad] for the tile kernel.
+#include <algorithm>
 #include "common.h"
 #include "launch.h"
 #include "mmq_host.h"
@@ -286,13 +287,19 @@ __global__ __launch_bounds__(256) void factor_grad_kernel(FactorGradParams p) {
     const int per_xcd = ((int)gridDim.x + 7) >> 3;
     const int unit = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if ((int)(blockIdx.x >> 3) >= per_xcd || unit >= p.units) return;
-    const int e = unit / col_blocks, cblk = unit - e * col_blocks;
+    const int splits = p.row_splits > 1 ? p.row_splits : 1;
+    const int split = unit % splits, ucb = unit / splits;
+    const int e = ucb / col_blocks, cblk = ucb - e * col_blocks;
     const int seg = cblk / blocks_per_seg;
     const int c0 = (cblk - seg * blocks_per_seg) * kCols;
     int row_begin = 0, row_end = p.m;
     if (p.ranges) {
         row_begin = p.ranges[2 * e];
         row_end = p.ranges[2 * e + 1];
+    } else if (splits > 1) {  // this workgroup's share of the rows, in whole 32-row slices
+        const int share = (((p.m + splits - 1) / splits) + 31) & ~31;
+        row_begin = min(p.m, split * share);
+        row_end = min(p.m, row_begin + share);
     }
     const bf16_t* in = p.in[seg];
     const bool vec = ((p.ld_in & 7) == 0) && (((uintptr_t)in & 15) == 0);
@@ -353,8 +360,21 @@ __global__ __launch_bounds__(256) void factor_grad_kernel(FactorGradParams p) {
         }
     }
     // acc[cb][jb][v]: c = c0 + 64*cb + wave*16 + 4*lq + v, j = 16*jb + li
-    bf16_t* out = p.out + (int64_t)e * p.out_expert_elems;
     const int64_t ctot = (int64_t)p.nseg * p.c;
+    if (splits > 1) {  // unscaled fp32 partial sums [split][column][r_pad]; factor_reduce_kernel finishes
+        float* part = p.partials + (int64_t)split * ctot * rp;
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+            for (int jb = 0; jb < JB; jb++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const int c = c0 + 64 * cb + wave * 16 + 4 * lq + v;
+                    if (c < p.c) part[((int64_t)seg * p.c + c) * rp + jb * 16 + li] = acc[cb][jb][v];
+                }
+        return;
+    }
+    bf16_t* out = p.out + (int64_t)e * p.out_expert_elems;
     const bool vec4 = (ctot & 3) == 0 && (((uintptr_t)out & 7) == 0);
     const bool vec8 = (p.r & 7) == 0 && (((uintptr_t)out & 15) == 0);
 #pragma unroll
@@ -398,6 +418,21 @@ __global__ __launch_bounds__(256) void factor_grad_kernel(FactorGradParams p) {
                     if (c < p.c && j < p.r) out[((int64_t)seg * p.c + c) * p.r + j] = to_bf16(acc[cb][jb][v] * p.scale);
                 }
         }
+    }
+}
+
+// out = bf16(scale * sum over the row splits, in split order) of the partial sums of a split factor_grad launch.
+// One lane per (column, j < r_pad); lanes of a wave run along j, then columns: contiguous reads.
+__global__ __launch_bounds__(256) void factor_reduce_kernel(const float* partials, bf16_t* out, int64_t ctot, int r, int r_pad, int splits, int out_j_major,
+                                                            float scale) {
+    const int64_t total = ctot * r_pad;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int64_t c = i / r_pad;
+        const int j = (int)(i - c * r_pad);
+        if (j >= r) continue;
+        float sum = 0.f;
+        for (int sp = 0; sp < splits; sp++) sum += partials[(int64_t)sp * total + i];
+        out[out_j_major ? (int64_t)j * ctot + c : c * r + j] = to_bf16(sum * scale);
     }
 }
 
@@ -529,11 +564,19 @@ int skinny_nt(const SkinnyNtParams& p, int r_pad, int grid_tiles, hipStream_t s)
 template <int CB>
 static int launch_factor_grad(const FactorGradParams& p_in, int r_pad, int64_t experts, hipStream_t s) {
     const int col_blocks = p_in.nseg * ((p_in.c + 64 * CB - 1) / (64 * CB));
-    const int64_t units = experts * col_blocks;
+    FactorGradParams p = p_in;
+    // One row range for everything (a dense layer) leaves only the column blocks to spread over the compute units: deal
+    // the rows out as well, enough to give every unit a workgroup, in shares of at least 128 rows.
+    p.row_splits = 1;
+    if (!p.ranges && experts == 1 && p.partials && col_blocks < 256 && p.m >= 256) {
+        const int64_t want = (256 + col_blocks - 1) / col_blocks;
+        const int64_t fit = p.partials_bytes / ((int64_t)p.nseg * p.c * r_pad * 4);
+        p.row_splits = (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, p.m / 128), std::min<int64_t>(fit, 64)));
+    }
+    const int64_t units = experts * col_blocks * p.row_splits;
     if (units <= 0) return 0;
     if (units > 0x7FFFFFF0) return set_error(GGQ_ERR_SHAPE, "factor_grad: grid too large");
     const int64_t grid = (units + 7) / 8 * 8;
-    FactorGradParams p = p_in;
     p.units = (int)units;
     switch (r_pad / 16) {
         case 1: hipLaunchKernelGGL((factor_grad_kernel<1, CB>), dim3((unsigned)grid), dim3(256), 0, s, p); break;
@@ -542,7 +585,14 @@ static int launch_factor_grad(const FactorGradParams& p_in, int r_pad, int64_t e
         case 4: hipLaunchKernelGGL((factor_grad_kernel<4, CB>), dim3((unsigned)grid), dim3(256), 0, s, p); break;
         default: return set_error(GGQ_ERR_SHAPE, "LoRA rank must be between 1 and 64");
     }
-    return check_launch("factor_grad");
+    if (int rc = check_launch("factor_grad")) return rc;
+    if (p.row_splits > 1) {
+        const int64_t ctot = (int64_t)p.nseg * p.c;
+        const unsigned blocks = (unsigned)std::min<int64_t>((ctot * r_pad + 255) / 256, 4096);
+        hipLaunchKernelGGL(factor_reduce_kernel, dim3(blocks), dim3(256), 0, s, p.partials, p.out, ctot, p.r, r_pad, p.row_splits, p.out_j_major, p.scale);
+        return check_launch("factor_reduce");
+    }
+    return 0;
 }
 
 int factor_grad(const FactorGradParams& p, int r_pad, int64_t experts, hipStream_t s) {

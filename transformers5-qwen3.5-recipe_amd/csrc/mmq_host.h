@@ -49,7 +49,12 @@ struct FactorGradParams {
     const int* ranges;    // per expert (row_begin, row_end); null: all m rows, one expert
     int m, c, r, nseg, out_j_major;
     float scale;
-    int units;            // experts * column blocks (set by factor_grad)
+    int units;            // experts * column blocks * row splits (set by factor_grad)
+    // one row range for all (ranges == null) and a scratch buffer: the rows are dealt to row_splits workgroups per column
+    // block, whose fp32 partial sums [row_splits][nseg*c][r_pad] a second kernel adds in split order (set by factor_grad)
+    float* partials;      // null: no splitting
+    int64_t partials_bytes;
+    int row_splits;
 };
 
 constexpr int kBM = 256, kBN = 128, kBK = 64;  // the tall tile shape (dense launches, large expert groups)
