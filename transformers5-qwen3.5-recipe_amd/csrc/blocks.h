@@ -297,25 +297,37 @@ struct Fmt<kIQ2_XXS> {
         r.idx4 = ld_u32(g);
         r.aux = ld_u32(g + 4);
     }
-    static GGQ_HD uint32_t signed_pair(float db, float m0, float m1, uint32_t signs, int j) {
-        float v0 = db * m0, v1 = db * m1;
-        uint32_t b0 = __builtin_bit_cast(uint32_t, v0) ^ ((signs << (31 - j)) & 0x80000000u);
-        uint32_t b1 = __builtin_bit_cast(uint32_t, v1) ^ ((signs << (30 - j)) & 0x80000000u);
-        return pack_bf16(__builtin_bit_cast(float, b0), __builtin_bit_cast(float, b1));
+    // Tables the tile kernel stages in LDS once per workgroup (built by table_entry below): for every codebook entry the
+    // four byte selectors that pick its eight magnitudes, two per word, out of a 3-entry bf16 table, and for every 7-bit
+    // sign index the four words that flip the signs of the eight values (bit 15 / bit 31 of a pair; the eighth sign is
+    // the parity of the other seven).  A run then costs one selection and one exclusive-or per pair of weights.
+    static constexpr int kTableWords = 256 * 4 + 128 * 4;  // uint32 words: selectors [256][4], then sign masks [128][4]
+    // Word `i` of the tables (i < kTableWords); `grid_entry` is the codebook entry i / 4 for i < 1024.
+    static GGQ_HD uint32_t table_word(int i, uint64_t grid_entry) {
+        if (i < 1024) {
+            const int p = i & 3;  // pair of the entry: magnitudes 2p, 2p + 1; codebook bytes are 0x08, 0x19, 0x2b: index = byte >> 4
+            const uint32_t t0 = (uint32_t)(grid_entry >> (16 * p + 4)) & 3u, t1 = (uint32_t)(grid_entry >> (16 * p + 12)) & 3u;
+            return (2 * t0) | ((2 * t0 + 1) << 8) | ((2 * t1) << 16) | ((2 * t1 + 1) << 24);
+        }
+        const uint32_t s7 = (uint32_t)(i - 1024) >> 2, p = (uint32_t)i & 3u;
+        const uint32_t signs = s7 | ((__builtin_popcount(s7) & 1u) << 7);
+        return (((signs >> (2 * p)) & 1u) << 15) | (((signs >> (2 * p + 1)) & 1u) << 31);
     }
-    static GGQ_HD void decode(const Raw& r, int, uint32_t* out, const uint2* grid) {
+    static __device__ __forceinline__ void decode(const Raw& r, int, uint32_t* out, const uint2* tables) {
+        const uint4* sel = (const uint4*)tables;
+        const uint4* flip = sel + 256;
         const float d = half_bits_to_f32(r.d16);
         const float db = d * (0.5f + (float)(r.aux >> 28)) * 0.25f;
+        // the three products a weight can be, as bf16: bytes 0..5 of {hi : lo}
+        const uint32_t lo = pack_bf16(db * 8.0f, db * 25.0f), hi = pack_bf16(db * 43.0f, 0.0f);
 #pragma unroll
         for (int l = 0; l < 4; l++) {
-            const uint2 g = grid[(r.idx4 >> (8 * l)) & 0xFFu];
-            const uint32_t s7 = (r.aux >> (7 * l)) & 127u;
-            const uint32_t signs = s7 | ((__builtin_popcount(s7) & 1u) << 7);
-            const uint32_t glo = opaque(g.x), ghi = opaque(g.y);
-            out[4 * l + 0] = signed_pair(db, ubyte0(glo), ubyte1(glo), signs, 0);
-            out[4 * l + 1] = signed_pair(db, ubyte2(glo), ubyte3(glo), signs, 2);
-            out[4 * l + 2] = signed_pair(db, ubyte0(ghi), ubyte1(ghi), signs, 4);
-            out[4 * l + 3] = signed_pair(db, ubyte2(ghi), ubyte3(ghi), signs, 6);
+            const uint4 e = sel[(r.idx4 >> (8 * l)) & 0xFFu];
+            const uint4 f = flip[(r.aux >> (7 * l)) & 127u];
+            out[4 * l + 0] = __builtin_amdgcn_perm(hi, lo, e.x) ^ f.x;
+            out[4 * l + 1] = __builtin_amdgcn_perm(hi, lo, e.y) ^ f.y;
+            out[4 * l + 2] = __builtin_amdgcn_perm(hi, lo, e.z) ^ f.z;
+            out[4 * l + 3] = __builtin_amdgcn_perm(hi, lo, e.w) ^ f.w;
         }
     }
 };

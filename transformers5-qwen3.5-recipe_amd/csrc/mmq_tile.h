@@ -919,7 +919,7 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
     c.as = smem_raw;
     c.as_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem_raw;
     c.bs = (bf16_t*)(smem_raw + kAStages * kAStageBytes);
-    uint2* grid_lds = (uint2*)(smem_raw + kTileLdsBytes);  // [256], IQ2_XXS only
+    uint2* grid_lds = (uint2*)(smem_raw + kTileLdsBytes);  // the decoder's tables, IQ2_XXS only
     c.grid = grid_lds;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -946,9 +946,9 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
     c.a_fast = ((p.lda & 7) == 0) && ((c.contraction & 63) == 0) &&
                ((((uintptr_t)p.a[0]) | ((uintptr_t)p.a[MODE == kModeNN && p.nseg > 1 ? 1 : 0])) & 15) == 0;
 
-    if (QT == kIQ2_XXS && tid < 256) {
-        const uint64_t g = d_iq2xxs_grid_mm[tid];
-        grid_lds[tid] = make_uint2((uint32_t)g, (uint32_t)(g >> 32));
+    if (QT == kIQ2_XXS) {  // selector and sign tables of the decoder (6 KB)
+        uint32_t* words = (uint32_t*)grid_lds;
+        for (int i = tid; i < Fmt<kIQ2_XXS>::kTableWords; i += kThreadsWG) words[i] = Fmt<kIQ2_XXS>::table_word(i, i < 1024 ? d_iq2xxs_grid_mm[i >> 2] : 0);
     }
     // ---- LoRA tiles go to A stage 0 / W buffer 0 (all lanes load): LA[rows, :r] and LB.  Every wave runs
     // this once, right after it has issued its first loads of the tile proper (A tile / packed weights),
