@@ -61,7 +61,8 @@ int ggq_mmq(const void* x, const void* packed, int qt, int64_t m, int64_t n, int
  * test_fast_lora.py:104-105): dx[M,K] = dy[M,N] . W with W decoded to bf16, fp32 accumulation. */
 int ggq_mmq_grad_input(const void* dy, const void* packed, int qt, int64_t m, int64_t n, int64_t k, void* dx, void* stream);
 
-/* Workspace bound for the four LoRA entry points below (n_total = N, or 2N for a pair). */
+/* Workspace bound for the four LoRA entry points below (n_total = N, or 2N for a pair).  groups = 0 (the dense calls)
+ * includes the fp32 partial sums of the factor gradients, whose rows are then dealt over the whole chip. */
 int64_t ggq_lora_workspace_bytes(int64_t rows, int64_t groups, int64_t experts, int64_t n_total, int64_t k, int r);
 
 /* FastGGUFLoraLinear._base_layer_forward + _fused_lora_add (fast_lora.py:34-65, 134-163) in one call:
@@ -177,7 +178,8 @@ int ggq_router_topk(const void* logits, int logits_are_bf16, int64_t tokens, int
 /* _packed_q8_linear_cross_entropy_forward (gguf_liger_loss.py:38-186): chunked mmq -> Liger
  * cross-entropy -> mmq_grad_input, without the [chunk, vocab] logits tensor.  labels int64 [rows];
  * loss_per_row fp32 [rows] (already divided by the number of non-ignored rows when reduction_mean);
- * grad_hidden bf16 [rows, hidden]; lse_out fp32 [rows] or NULL; n_valid_out int32[1] or NULL. */
+ * grad_hidden bf16 [rows, hidden]; lse_out fp32 [rows] or NULL; n_valid_out int32[1] or NULL.  `chunk` bounds the rows of
+ * one statistics launch; the gradient pass takes up to 4096 rows at a time through a [rows, 8192] bf16 slab in the workspace. */
 int64_t ggq_lmhead_ce_workspace_bytes(int64_t rows, int64_t vocab, int64_t hidden_dim, int64_t chunk);
 int ggq_lmhead_cross_entropy(int qt, const void* hidden, const void* packed, const int64_t* labels, int64_t rows, int64_t vocab,
                              int64_t hidden_dim, int64_t chunk, int64_t ignore_index, int reduction_mean, float* loss_per_row,
