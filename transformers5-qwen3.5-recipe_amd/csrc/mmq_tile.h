@@ -78,6 +78,7 @@ struct TileCtx {  // wave-uniform description of the tile this workgroup compute
     uint32_t as_lds;  // LDS byte address of `as`
     bool a_fast;      // A rows can be moved with aligned 16-byte accesses and every step is whole
     const uint2* grid;
+    const float4* row_meta;  // cross-entropy epilogues: per tile row (lse, row scale, label as int bits, -), staged in LDS
 };
 
 // (segment, first contraction index) of a step; at most two segments.
@@ -802,9 +803,6 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
         // everything that does not depend on the element is read once, up front
         const int64_t ldc = p.ldc;
         char* const cbase = (char*)p.c[EPI == kEpiStore ? c.seg_c : 0];
-        const float* const lse_p = p.lse;
-        const float* const rs_p = p.row_scale;
-        const int64_t* const labels_p = p.labels;
         const int64_t ce_off = p.ce_col_offset;
         const int rows_valid = c.rows_valid;
         const bool col_ok[kColBlocks] = {col_base < c.out_cols, col_base + 32 < c.out_cols};
@@ -820,10 +818,8 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
                 float lse = 0.f, rs = 0.f;
                 int64_t label = -1;
                 if (EPI == kEpiCeGrad) {
-                    const int64_t grow = c.row_begin + r_lane + dr;
-                    lse = lse_p[grow];
-                    rs = rs_p[grow];
-                    label = labels_p[grow];
+                    const float4 meta = c.row_meta[r_lane + dr];
+                    lse = meta.x, rs = meta.y, label = (int64_t)__float_as_int(meta.z);
                 }
 #pragma unroll
                 for (int cb = 0; cb < kColBlocks; cb++) {
@@ -850,7 +846,7 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
                 const int r = 32 * (kWavesM * rb + wave_m) + (i >> 2) * 8 + lane_h * 4 + (i & 3);
                 const bool row_ok = r < c.rows_valid;
                 const int64_t grow = c.row_begin + (row_ok ? r : 0);
-                const int64_t label = row_ok ? p.labels[grow] : -1;
+                const int64_t label = row_ok ? (int64_t)__float_as_int(c.row_meta[r].z) : -1;
                 float v[kColBlocks];
                 float mx = -INFINITY;
 #pragma unroll
@@ -921,6 +917,10 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
     c.bs = (bf16_t*)(smem_raw + kAStages * kAStageBytes);
     uint2* grid_lds = (uint2*)(smem_raw + kTileLdsBytes);  // the decoder's tables, IQ2_XXS only
     c.grid = grid_lds;
+    // what the cross-entropy epilogues need per row, read once per tile: one dependent global load per row and lane in
+    // the epilogue costs a memory round trip each
+    float4* row_meta = (float4*)(smem_raw + kTileLdsBytes + (QT == kIQ2_XXS ? Fmt<kIQ2_XXS>::kTableWords * 4 : 0));
+    c.row_meta = row_meta;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps control flow scalar
@@ -988,7 +988,14 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
                 }
             }
         }
-        __syncthreads();  // LoRA tiles and the codebook are visible
+        if (EPI == kEpiCeStats || EPI == kEpiCeGrad) {
+            for (int r = tid; r < kTM; r += kThreadsWG) {
+                const int64_t grow = c.row_begin + min(r, c.rows_valid - 1);
+                row_meta[r] = make_float4(EPI == kEpiCeGrad ? p.lse[grow] : 0.f, EPI == kEpiCeGrad ? p.row_scale[grow] : 0.f,
+                                          __int_as_float((int)p.labels[grow]), 0.f);
+            }
+        }
+        __syncthreads();  // LoRA tiles, the codebook tables and the row values are visible
     };
 
     if (wave >= kCW) {
