@@ -70,6 +70,28 @@ __device__ __forceinline__ uint4 load8_slow(const bf16_t* p, int valid) {
     return v;
 }
 
+// All-reduce over each half of a wave (lanes 0..31, 32..63): four data-parallel-primitive steps inside the rows of 16
+// lanes (neighbour, pair of a quad, mirror of 8, mirror of 16: every lane of a row ends with the row's result) and one
+// cross-lane exchange between the two rows of a half.  Five exchanges through the LDS crossbar cost several times more.
+template <int CTRL>
+static __device__ __forceinline__ float dpp_f32(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
+}
+static __device__ __forceinline__ float half_wave_max(float x) {
+    x = fmaxf(x, dpp_f32<0xB1>(x));   // quad_perm [1,0,3,2]
+    x = fmaxf(x, dpp_f32<0x4E>(x));   // quad_perm [2,3,0,1]
+    x = fmaxf(x, dpp_f32<0x141>(x));  // row_half_mirror
+    x = fmaxf(x, dpp_f32<0x140>(x));  // row_mirror
+    return fmaxf(x, __shfl_xor(x, 16, 64));
+}
+static __device__ __forceinline__ float half_wave_sum(float x) {
+    x += dpp_f32<0xB1>(x);
+    x += dpp_f32<0x4E>(x);
+    x += dpp_f32<0x141>(x);
+    x += dpp_f32<0x140>(x);
+    return x + __shfl_xor(x, 16, 64);
+}
+
 struct TileCtx {  // wave-uniform description of the tile this workgroup computes
     int row_begin, rows_valid, col0, col_tile, seg_c, out_cols, contraction, total_steps, base;
     int64_t expert;
@@ -857,13 +879,11 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
                     if (row_ok && col < c.out_cols && (int64_t)(col + p.ce_col_offset) == label) p.ce_target_logit[grow] = v[cb];
                 }
                 // reduce over the 32 lanes that share this row (lanes with equal lane_h)
-#pragma unroll
-                for (int off = 16; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+                mx = half_wave_max(mx);
                 float sum = 0.f;
 #pragma unroll
                 for (int cb = 0; cb < kColBlocks; cb++) sum += v[cb] == -INFINITY ? 0.f : __expf(v[cb] - mx);
-#pragma unroll
-                for (int off = 16; off >= 1; off >>= 1) sum += __shfl_xor(sum, off, 64);
+                sum = half_wave_sum(sum);
                 if (row_ok && lane_c == 0)
                     p.ce_partials[grow * p.ce_partials_ld + p.ce_partial_offset + c.col_tile * 2 + wave_n] = make_float2(mx, sum);
             }
