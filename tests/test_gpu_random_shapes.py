@@ -1,0 +1,90 @@
+"""Seeded sweep over shapes of the grouped LoRA projection (block format, expert count, ragged and empty groups, output
+widths that are not whole tiles, ranks, pair or single, every kernel shape) against fp32 matmuls on the decoded weights,
+whose decoders are checked bit for bit elsewhere.  Tolerance of the path: max rel err <= 2e-2 plus the per-element bound of
+assert_close_bf16."""
+
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_close_bf16
+from oracle import gguf_blocks as gb
+
+pytestmark = pytest.mark.gpu
+
+
+def _bf16(t):
+    return t.to(torch.bfloat16).float()
+
+
+def _payload(pkg, dev, qt, e, n, k, g):
+    if qt == gb.IQ2_XXS:
+        return pkg.gguf.random_iq2_xxs((e, n, k), g, dev)
+    w = torch.randn(e, n, k, generator=g, device=dev) * 0.02
+    if qt in (gb.Q8_0, gb.Q4_K, gb.Q6_K):
+        return pkg.gguf.quantize(w, qt)
+    return torch.from_numpy(gb.quantize(w.cpu().numpy().reshape(e * n, k), qt)).reshape(e, n, -1).to(dev)
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_grouped_projection_over_random_shapes(pkg, dev, seed, monkeypatch):
+    ml = pkg.fast_moe_lora
+    rnd = random.Random(seed)
+    for case in range(40):
+        qt = rnd.choice([gb.Q8_0, gb.Q2_K, gb.Q3_K, gb.Q4_K, gb.Q4_K, gb.Q4_K, gb.Q5_K, gb.Q6_K, gb.IQ2_XXS])
+        e = rnd.choice([1, 3, 8, 17])
+        k = rnd.choice([256, 512, 768, 1024])
+        n = rnd.choice([8, 64, 72, 128, 192, 256, 320, 520])
+        r = rnd.choice([0, 0, 4, 8, 16, 16, 24, 64])
+        pair = rnd.random() < 0.5
+        shape = rnd.choice(["", "", "0", "1", "2", "3"])
+        sizes = [rnd.choice([0, 1, 5, 31, 64, 100, 128, 129, 200, 260, 400]) for _ in range(e)]
+        if sum(sizes) == 0:
+            sizes[0] = 7
+        what = f"case {case}: qt={qt} e={e} k={k} n={n} r={r} pair={pair} shape={shape!r} sizes={sizes}"
+        print(what, flush=True)
+        if shape:
+            monkeypatch.setenv("GGQ_GROUPED_SHAPE", shape)
+        else:
+            monkeypatch.delenv("GGQ_GROUPED_SHAPE", raising=False)
+        g = torch.Generator(device=dev).manual_seed(1000 * seed + case)
+        rows, nseg = sum(sizes), 2 if pair else 1
+        p1 = _payload(pkg, dev, qt, e, n, k, g)
+        p2 = _payload(pkg, dev, qt, e, n, k, g) if pair else None
+        x = torch.randn(rows, k, generator=g, device=dev).to(torch.bfloat16).requires_grad_(True)
+        a = (torch.randn(e, r, k, generator=g, device=dev) * k ** -0.5).to(torch.bfloat16).requires_grad_(True) if r else None
+        b = (torch.randn(e, nseg * n, r, generator=g, device=dev) * 0.02).to(torch.bfloat16).requires_grad_(True) if r else None
+        dy = torch.randn(rows, nseg * n, generator=g, device=dev).to(torch.bfloat16)
+        ids = torch.arange(e, dtype=torch.int64, device=dev)
+        ends = torch.tensor(np.cumsum(sizes), dtype=torch.int32, device=dev)
+        if pair:
+            y = torch.cat(ml.grouped_lora_mmq_pair(x, p1, p2, ids, ends, qt, n, a, b, 2.0) if r else ml.grouped_mmq_pair(x, p1, p2, ids, ends, qt, n), dim=1)
+        else:
+            y = ml.grouped_lora_mmq(x, p1, ids, ends, qt, n, a, b, 2.0) if r else ml.grouped_mmq(x, p1, ids, ends, qt, n)
+        y.backward(dy)
+        w = pkg.gguf.dequantize_gguf_tensor(p1, qt, torch.bfloat16).float()
+        if pair:
+            w = torch.cat([w, pkg.gguf.dequantize_gguf_tensor(p2, qt, torch.bfloat16).float()], dim=1)
+        want_y, want_dx = torch.zeros(rows, nseg * n, device=dev), torch.zeros(rows, k, device=dev)
+        want_da = torch.zeros(a.shape, device=dev) if r else None
+        want_db = torch.zeros(b.shape, device=dev) if r else None
+        r0 = 0
+        for ei, sz in enumerate(sizes):
+            r1 = r0 + sz
+            if sz:
+                xe, de = x.detach()[r0:r1].float(), dy[r0:r1].float()
+                want_y[r0:r1], want_dx[r0:r1] = xe @ w[ei].T, de @ w[ei]
+                if r:
+                    af, bfm = a.detach()[ei].float(), b.detach()[ei].float()
+                    xa, dyb = _bf16(xe @ af.T), _bf16(de @ bfm)
+                    want_y[r0:r1] += 2.0 * (xa @ bfm.T)
+                    want_dx[r0:r1] += 2.0 * (dyb @ af)
+                    want_da[ei], want_db[ei] = 2.0 * (dyb.T @ xe), 2.0 * (de.T @ xa)
+            r0 = r1
+        assert_close_bf16(y, want_y.double(), what + ": Y")
+        assert_close_bf16(x.grad, want_dx.double(), what + ": dX")
+        if r:
+            assert_close_bf16(a.grad, want_da.double(), what + ": dA")
+            assert_close_bf16(b.grad, want_db.double(), what + ": dB")
