@@ -88,3 +88,74 @@ def test_grouped_projection_over_random_shapes(pkg, dev, seed, monkeypatch):
         if r:
             assert_close_bf16(a.grad, want_da.double(), what + ": dA")
             assert_close_bf16(b.grad, want_db.double(), what + ": dB")
+
+
+def _dense_payload(pkg, dev, qt, n, k, g):
+    return _payload(pkg, dev, qt, 1, n, k, g)[0]
+
+
+def test_dense_lora_linear_over_random_shapes(pkg, dev):
+    # row counts on both sides of the sizes at which the factor gradients split their rows over workgroups
+    rnd = random.Random(21)
+    for case in range(36):
+        qt = rnd.choice([gb.Q8_0, gb.Q2_K, gb.Q3_K, gb.Q4_K, gb.Q4_K, gb.Q5_K, gb.Q6_K, gb.IQ2_XXS])
+        m = rnd.choice([1, 7, 64, 255, 256, 257, 700, 1024, 3000, 4096, 5000])
+        k = rnd.choice([256, 512, 1024, 2048])
+        n = rnd.choice([8, 72, 128, 520, 1024, 4096])
+        r = rnd.choice([4, 8, 16, 16, 24, 64])
+        what = f"case {case}: qt={qt} m={m} k={k} n={n} r={r}"
+        print(what, flush=True)
+        g = torch.Generator(device=dev).manual_seed(77 + case)
+        p = _dense_payload(pkg, dev, qt, n, k, g)
+        x = torch.randn(m, k, generator=g, device=dev).to(torch.bfloat16).requires_grad_(True)
+        a = (torch.randn(r, k, generator=g, device=dev) * k ** -0.5).to(torch.bfloat16).requires_grad_(True)
+        b = (torch.randn(n, r, generator=g, device=dev) * 0.02).to(torch.bfloat16).requires_grad_(True)
+        dy = torch.randn(m, n, generator=g, device=dev).to(torch.bfloat16)
+        y = pkg.fast_lora.lora_mmq(x, p, qt, n, a, b, 2.0)
+        y.backward(dy)
+        w = pkg.gguf.dequantize_gguf_tensor(p, qt, torch.bfloat16).float()
+        xf, af, bfm, df = x.detach().float(), a.detach().float(), b.detach().float(), dy.float()
+        xa, dyb = _bf16(xf @ af.T), _bf16(df @ bfm)
+        assert_close_bf16(y, (xf @ w.T + 2 * (xa @ bfm.T)).double(), what + ": Y")
+        assert_close_bf16(x.grad, (df @ w + 2 * (dyb @ af)).double(), what + ": dX")
+        assert_close_bf16(a.grad, (2 * (dyb.T @ xf)).double(), what + ": dA")
+        assert_close_bf16(b.grad, (2 * (df.T @ xa)).double(), what + ": dB")
+
+
+def test_lm_head_loss_over_random_shapes(pkg, dev):
+    # vocabularies around one 8192-column block, row counts around one chunk and around one 4096-row gradient block
+    from helpers import max_rel
+
+    rnd = random.Random(31)
+    for case in range(14):
+        qt = rnd.choice([gb.Q8_0, gb.Q4_K, gb.Q6_K, gb.Q6_K])
+        rows = rnd.choice([1, 33, 256, 257, 1000, 4097, 6000])
+        hidden = rnd.choice([256, 512, 2048])
+        vocab = rnd.choice([37, 1000, 8192, 8193, 20000, 50000])
+        chunk = rnd.choice([32, 256, 1024, 5000])
+        red = rnd.choice(["mean", "sum"])
+        what = f"case {case}: qt={qt} rows={rows} hidden={hidden} vocab={vocab} chunk={chunk} {red}"
+        print(what, flush=True)
+        g = torch.Generator(device=dev).manual_seed(177 + case)
+        p = _dense_payload(pkg, dev, qt, vocab, hidden, g)
+        hid = torch.randn(rows, hidden, generator=g, device=dev).to(torch.bfloat16)
+        labels = torch.randint(0, vocab, (rows,), generator=g, device=dev)
+        labels[torch.rand(rows, generator=g, device=dev) < 0.1] = -100
+        h = hid.clone().requires_grad_(True)
+        loss = pkg.gguf_liger_loss.packed_linear_cross_entropy(h, p, labels, qt, vocab, chunk, -100, red)
+        loss.backward()
+        w = pkg.gguf.dequantize_gguf_tensor(p, qt, torch.bfloat16).float()
+        valid = labels != -100
+        n_valid = max(int(valid.sum()), 1)
+        scale = 1.0 / n_valid if red == "mean" else 1.0
+        logits = _bf16(hid.float() @ w.T)
+        lse = torch.logsumexp(logits, 1)
+        tgt = logits.gather(1, labels.clamp(min=0)[:, None])[:, 0]
+        want = float(((lse - tgt) * valid).double().sum() * scale)
+        d = torch.softmax(logits, 1)
+        d[torch.arange(rows, device=dev), labels.clamp(min=0)] -= 1.0
+        want_dh = _bf16(d * (valid[:, None] * scale)) @ w
+        assert abs(float(loss) - want) * (1.0 if red == "mean" else 1.0 / n_valid) <= 1e-3, (what, float(loss), want)
+        if bool(valid.any()):
+            assert max_rel(h.grad, want_dh) <= 2e-2, what
+        assert bool((h.grad[~valid] == 0).all()), what
