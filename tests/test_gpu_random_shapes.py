@@ -159,3 +159,58 @@ def test_lm_head_loss_over_random_shapes(pkg, dev):
         if bool(valid.any()):
             assert max_rel(h.grad, want_dh) <= 2e-2, what
         assert bool((h.grad[~valid] == 0).all()), what
+
+
+def test_expert_layer_equals_the_explicit_composition_bit_for_bit(pkg, dev):
+    # The module (token rows read in place by the gate/up launch) against routing plan -> gathered copy -> grouped pair ->
+    # SwiGLU -> grouped down -> combine, over random layer geometries: outputs and every gradient are the same bits.
+    ml, mr = pkg.fast_moe_lora, pkg.fast_moe_routing
+    G = pkg.gguf.GGUFQuantizedTensor
+    rnd = random.Random(9)
+    for case in range(30):
+        qt = rnd.choice([gb.Q8_0, gb.Q2_K, gb.Q4_K, gb.Q4_K, gb.Q4_K, gb.Q6_K, gb.IQ2_XXS])
+        qd = rnd.choice([qt, gb.Q4_K, gb.Q2_K])
+        e = rnd.choice([4, 8, 32, 64])
+        top_k = min(rnd.choice([1, 2, 6, 8]), e)
+        tokens, hidden, inter = rnd.choice([1, 5, 64, 300, 1000]), rnd.choice([256, 512, 1024]), rnd.choice([256, 512])
+        r, limit, wdt = rnd.choice([0, 4, 16]), rnd.choice([None, None, 1.5]), rnd.choice([torch.float32, torch.bfloat16])
+        what = f"case {case}: qt={qt}/{qd} e={e} top_k={top_k} tokens={tokens} hidden={hidden} inter={inter} r={r} limit={limit} {wdt}"
+        print(what, flush=True)
+        g = torch.Generator(device=dev).manual_seed(500 + case)
+        gate = G(_payload(pkg, dev, qt, e, inter, hidden, g), qt, (e, inter, hidden))
+        up = G(_payload(pkg, dev, qt, e, inter, hidden, g), qt, (e, inter, hidden))
+        down = G(_payload(pkg, dev, qd, e, hidden, inter, g), qd, (e, hidden, inter))
+        experts = ml.GGUFExperts(gate, up, down, swiglu_limit=limit)
+        layer = ml.FastGGUFMoeLora(experts, r=r, lora_alpha=2 * r) if r else None
+        params = list(layer.parameters()) if layer is not None else []
+        with torch.no_grad():
+            for name, p in (layer.named_parameters() if layer is not None else []):
+                p.copy_((torch.randn(p.shape, generator=g, device=dev) * (p.shape[-1] ** -0.5 if "lora_A" in name else 0.02)).to(torch.bfloat16))
+        x0 = torch.randn(tokens, hidden, generator=g, device=dev).to(torch.bfloat16)
+        scores = torch.randn(tokens, e, generator=g, device=dev)
+        scores[:, 0] += 1.0
+        top = torch.topk(scores, top_k, dim=-1)
+        idx, w0 = top.indices, torch.softmax(top.values, -1).to(wdt)
+        dy = torch.randn(tokens, hidden, generator=g, device=dev).to(torch.bfloat16)
+
+        def run(through_module):
+            x, w = x0.clone().requires_grad_(True), w0.clone().requires_grad_(True)
+            for p in params:
+                p.grad = None
+            if through_module:
+                out = layer(x, idx, w) if layer is not None else experts(x, idx, w)
+            else:
+                lw = layer._active_lora_weights() if layer is not None else None
+                s = lw.scaling if lw else 0.0
+                plan = mr.prepare_expert_routing(x, idx, w, e)
+                ids = torch.arange(e, dtype=torch.int64, device=dev)
+                ga, u = ml._GroupedLoraProjection.apply(plan.selected_hidden_states, gate.as_subclass(torch.Tensor), up.as_subclass(torch.Tensor), ids,
+                                                        plan.expert_end_offsets, qt, inter, lw.gate_up_a if lw else None, lw.gate_up_b if lw else None, s)
+                o = ml._GroupedLoraProjection.apply(ml.swiglu(ga, u, limit), down.as_subclass(torch.Tensor), None, ids, plan.expert_end_offsets, qd, hidden,
+                                                    lw.down_a if lw else None, lw.down_b if lw else None, s)
+                out = mr.finalize_expert_routing(o, x, plan, None).reshape(x.shape)
+            out.backward(dy)
+            return [out.detach(), x.grad, w.grad] + [p.grad.clone() for p in params]
+
+        for i, (got, want) in enumerate(zip(run(True), run(False))):
+            assert torch.equal(got, want), (what, i)
