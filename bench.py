@@ -149,9 +149,9 @@ def other_workload(name, pkg, lib, dev, args):
         labels = torch.randint(0, vocab, (rows,), device=dev, generator=g)
         labels[torch.rand(rows, device=dev, generator=g) < 0.05] = -100
         flops = 2 * 2 * rows * vocab * hidden
-        launch_flops, launches_per_step = None, None   # three kinds of launches (statistics, gradient slab, grad-input) of different sizes
+        launch_flops, launches_per_step = None, None   # launches of different sizes (statistics per chunk, one grad-input)
         workload = "configs[3]: chunked cross-entropy through a Q6_K lm_head [151936x2048], 4096 rows, chunks of 1024, loss + dHidden"
-        metric = "fwd+bwd TFLOP/s (two algorithmic GEMMs), chunked lm_head cross-entropy"
+        metric = "fwd+bwd TFLOP/s (two GEMMs), chunked lm_head cross-entropy"
 
         def step():
             hs.grad = None

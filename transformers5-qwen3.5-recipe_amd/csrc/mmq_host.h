@@ -76,6 +76,8 @@ struct MmqParams {
     const bf16_t* a[2];   // activations; [1] only for a pair in NN mode
     int64_t lda;
     RowIndex a_rows;      // NT mode only (segment 0 is the only activation matrix there)
+    int a_zero_padded;    // the rows of a hold zeros from the contraction length up to the next multiple of 64 (lda covers them):
+                          // a contraction that ends inside a 64-wide step still takes the aligned 16-byte loads
     const uint8_t* w[2];  // packed weights; [1] only for a pair
     int64_t w_row_bytes, w_expert_bytes;
     void* c[2];           // outputs; [1] only for a pair in NT mode

@@ -861,6 +861,7 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
             }
         }
     } else {  // kEpiCeStats
+        bf16_t* const logits_out = (bf16_t*)p.c[0];  // optional: the logits themselves, for a gradient pass that does not recompute them
 #pragma unroll
         for (int rb = 0; rb < LIVE; rb++) {
 #pragma unroll
@@ -874,7 +875,9 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
 #pragma unroll
                 for (int cb = 0; cb < kColBlocks; cb++) {
                     const int col = col_base + cb * 32;
-                    v[cb] = col < c.out_cols ? bf16_to_f32(to_bf16(acc[rb][cb][i])) : -INFINITY;
+                    const bf16_t logit = to_bf16(acc[rb][cb][i]);
+                    v[cb] = col < c.out_cols ? bf16_to_f32(logit) : -INFINITY;
+                    if (logits_out && row_ok && col < c.out_cols) logits_out[grow * p.ldc + col] = logit;
                     mx = fmaxf(mx, v[cb]);
                     if (row_ok && col < c.out_cols && (int64_t)(col + p.ce_col_offset) == label) p.ce_target_logit[grow] = v[cb];
                 }
@@ -963,7 +966,7 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
     c.contraction = MODE == kModeNT ? p.k : p.n;  // contraction length per segment
     c.total_steps = (MODE == kModeNN ? p.nseg : 1) * p.steps_per_seg;
     c.base = p.r_pad > 0 ? 1 : 0;
-    c.a_fast = ((p.lda & 7) == 0) && ((c.contraction & 63) == 0) &&
+    c.a_fast = ((p.lda & 7) == 0) && ((c.contraction & 63) == 0 || p.a_zero_padded) &&
                ((((uintptr_t)p.a[0]) | ((uintptr_t)p.a[MODE == kModeNN && p.nseg > 1 ? 1 : 0])) & 15) == 0;
 
     if (QT == kIQ2_XXS) {  // selector and sign tables of the decoder (6 KB)
