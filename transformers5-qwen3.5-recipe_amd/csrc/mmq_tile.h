@@ -100,7 +100,7 @@ struct TileCtx {  // wave-uniform description of the tile this workgroup compute
     uint32_t as_lds;  // LDS byte address of `as`
     bool a_fast;      // A rows can be moved with aligned 16-byte accesses and every step is whole
     const uint2* grid;
-    const float4* row_meta;  // cross-entropy epilogues: per tile row (lse, row scale, label as int bits, -), staged in LDS
+    const int* row_meta;  // cross-entropy statistics epilogue: the label of every tile row, staged in LDS
 };
 
 // (segment, first contraction index) of a step; at most two segments.
@@ -821,11 +821,10 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
     // ---- epilogue.  acc[rb][cb][i]: tile row = 32*(kWavesM*rb + wave_m) + 8*(i/4) + 4*lane_h + (i%4),
     //                                 tile col = 64*wave_n + 32*cb + lane_c
     const int col_base = c.col0 + wave_n * 64 + lane_c;
-    if (EPI == kEpiStore || EPI == kEpiAccumF32 || EPI == kEpiCeGrad) {
+    if (EPI == kEpiStore) {
         // everything that does not depend on the element is read once, up front
         const int64_t ldc = p.ldc;
-        char* const cbase = (char*)p.c[EPI == kEpiStore ? c.seg_c : 0];
-        const int64_t ce_off = p.ce_col_offset;
+        bf16_t* const cbase = (bf16_t*)p.c[c.seg_c];
         const int rows_valid = c.rows_valid;
         const bool col_ok[kColBlocks] = {col_base < c.out_cols, col_base + 32 < c.out_cols};
 #pragma unroll
@@ -837,27 +836,9 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
                 const int dr = (i >> 2) * 8 + (i & 3);  // uniform row step inside the block
                 if (r_lane + dr >= rows_valid) continue;
                 const int64_t elem = lane_elem + (int64_t)dr * ldc;
-                float lse = 0.f, rs = 0.f;
-                int64_t label = -1;
-                if (EPI == kEpiCeGrad) {
-                    const float4 meta = c.row_meta[r_lane + dr];
-                    lse = meta.x, rs = meta.y, label = (int64_t)__float_as_int(meta.z);
-                }
 #pragma unroll
-                for (int cb = 0; cb < kColBlocks; cb++) {
-                    if (!col_ok[cb]) continue;
-                    const float v = acc[rb][cb][i];
-                    if (EPI == kEpiStore) {
-                        ((bf16_t*)cbase)[elem + cb * 32] = to_bf16(v);
-                    } else if (EPI == kEpiAccumF32) {
-                        ((float*)cbase)[elem + cb * 32] += v;
-                    } else {
-                        const float logit = bf16_to_f32(to_bf16(v));  // the path's logits are bf16 values
-                        float g = __expf(logit - lse);
-                        if ((int64_t)(col_base + cb * 32) + ce_off == label) g -= 1.0f;
-                        ((bf16_t*)cbase)[elem + cb * 32] = to_bf16(g * rs);
-                    }
-                }
+                for (int cb = 0; cb < kColBlocks; cb++)
+                    if (col_ok[cb]) cbase[elem + cb * 32] = to_bf16(acc[rb][cb][i]);
             }
         }
     } else {  // kEpiCeStats
@@ -869,7 +850,7 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
                 const int r = 32 * (kWavesM * rb + wave_m) + (i >> 2) * 8 + lane_h * 4 + (i & 3);
                 const bool row_ok = r < c.rows_valid;
                 const int64_t grow = c.row_begin + (row_ok ? r : 0);
-                const int64_t label = row_ok ? (int64_t)__float_as_int(c.row_meta[r].z) : -1;
+                const int64_t label = row_ok ? (int64_t)c.row_meta[r] : -1;
                 float v[kColBlocks];
                 float mx = -INFINITY;
 #pragma unroll
@@ -940,9 +921,9 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
     c.bs = (bf16_t*)(smem_raw + kAStages * kAStageBytes);
     uint2* grid_lds = (uint2*)(smem_raw + kTileLdsBytes);  // the decoder's tables, IQ2_XXS only
     c.grid = grid_lds;
-    // what the cross-entropy epilogues need per row, read once per tile: one dependent global load per row and lane in
-    // the epilogue costs a memory round trip each
-    float4* row_meta = (float4*)(smem_raw + kTileLdsBytes + (QT == kIQ2_XXS ? Fmt<kIQ2_XXS>::kTableWords * 4 : 0));
+    // what the cross-entropy statistics epilogue needs per row, read once per tile: one dependent global load per row and
+    // lane in the epilogue costs a memory round trip each
+    int* row_meta = (int*)(smem_raw + kTileLdsBytes + (QT == kIQ2_XXS ? Fmt<kIQ2_XXS>::kTableWords * 4 : 0));
     c.row_meta = row_meta;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -1011,12 +992,8 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
                 }
             }
         }
-        if (EPI == kEpiCeStats || EPI == kEpiCeGrad) {
-            for (int r = tid; r < kTM; r += kThreadsWG) {
-                const int64_t grow = c.row_begin + min(r, c.rows_valid - 1);
-                row_meta[r] = make_float4(EPI == kEpiCeGrad ? p.lse[grow] : 0.f, EPI == kEpiCeGrad ? p.row_scale[grow] : 0.f,
-                                          __int_as_float((int)p.labels[grow]), 0.f);
-            }
+        if (EPI == kEpiCeStats) {
+            for (int r = tid; r < kTM; r += kThreadsWG) row_meta[r] = (int)p.labels[c.row_begin + min(r, c.rows_valid - 1)];
         }
         __syncthreads();  // LoRA tiles, the codebook tables and the row values are visible
     };
