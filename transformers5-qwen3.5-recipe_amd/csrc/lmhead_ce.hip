@@ -1,11 +1,10 @@
 // Chunked cross-entropy through a packed lm_head without ever holding [rows, vocab] logits.
 //
-// Per block of up to kBlockRows rows: (1) per chunk of rows, the packed-weight tile kernel runs over the whole vocabulary
-// with an epilogue that stores the bf16 logits, reduces every 128-column slab of a logits tile to (max, sum exp) per row
-// and records the target logit; a small kernel merges the slabs into log-sum-exp and the per-row loss; (2) one
-// element-wise kernel turns the block's logits into d(loss)/d(logits) in place; (3) one grad-input launch of the tile
-// kernel contracts them with the same packed rows over the whole vocabulary.  Two vocabulary-sized matmuls, as in the
-// reference, whose [chunk, vocab] logits tensor this buffer corresponds to.
+// Per block of up to kBlockRows rows: (1) the packed-weight tile kernel writes the block's bf16 logits (one launch over the
+// whole vocabulary); (2) one kernel, a workgroup per row, reads a row for its log-sum-exp, target logit and loss, then turns
+// it into d(loss)/d(logits) in place; (3) one grad-input launch of the tile kernel contracts the rows with the same packed
+// weights over the whole vocabulary.  Two vocabulary-sized matmuls, as in the reference, whose [chunk, vocab] logits tensor
+// this buffer corresponds to.
 #include <algorithm>
 
 #include "common.h"
@@ -14,10 +13,10 @@
 
 namespace ggq {
 
-// The logits of up to this many rows are kept (bf16, rows padded with zeros to a multiple of 64 columns) between the
-// statistics pass and the gradient pass: 4096 rows fill the chip with tiles of the [rows, hidden] grad-input output (a
-// 1024-row chunk makes 64 tiles for 256 compute units), at 2 bytes per row and vocabulary entry (1.2 GB for a 152k
-// vocabulary).  The caller's chunk bounds the rows of one statistics launch.
+// The logits of up to this many rows are kept (bf16, rows padded to a multiple of 64 columns): 4096 rows fill the chip with
+// tiles of the [rows, hidden] grad-input output (a 1024-row chunk makes 64 tiles for 256 compute units), at 2 bytes per row
+// and vocabulary entry (1.2 GB for a 152k vocabulary).  The caller's chunk size, which bounds the reference's [chunk, vocab]
+// logits tensor, is accepted and not needed: this block is the bound here.
 constexpr int64_t kBlockRows = 4096;
 
 // row_scale[m] = 0 for ignored rows, else 1/n_valid (mean) or 1 (sum); n_valid = 0 gives all zeros.
@@ -38,40 +37,58 @@ __global__ __launch_bounds__(1024) void ce_row_scale_kernel(const int64_t* label
     if (threadIdx.x == 0 && n_valid_out) *n_valid_out = n;
 }
 
-// One wave per row: merge the slab partials into lse, then loss = (lse - target logit) * row_scale.
-__global__ __launch_bounds__(256) void ce_finalize_kernel(const float2* partials, int ld, int nparts, const float* target_logit,
-                                                          const float* row_scale, int rows, float* lse_out, float* loss_out) {
-    const int lane = threadIdx.x & 63;
-    const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (r >= rows) return;
-    const float2* p = partials + (int64_t)r * ld;
-    float mx = -INFINITY;
-    for (int i = lane; i < nparts; i += 64) mx = fmaxf(mx, p[i].x);
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
-    float sum = 0.f;
-    for (int i = lane; i < nparts; i += 64) {
-        const float2 v = p[i];
-        if (v.y > 0.f) sum += v.y * __expf(v.x - mx);
-    }
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) sum += __shfl_xor(sum, off, 64);
-    if (lane == 0) {
-        const float lse = mx + __logf(sum);
-        lse_out[r] = lse;
-        const float rs = row_scale[r];
-        loss_out[r] = rs != 0.f ? (lse - target_logit[r]) * rs : 0.f;
-    }
+// One workgroup per row.  Pass 1: log-sum-exp of the row's logits (every lane keeps a running (max, sum) over its columns,
+// merged in lane order inside a wave and in wave order across the workgroup: deterministic), the target logit, the loss
+// (lse - target) * row_scale.  Pass 2: the row becomes (exp(logit - lse) - [column == label]) * row_scale in place, bf16;
+// the padding columns [vocab, ld) become zero.  Eight columns per lane and trip (ld is a multiple of 64).
+__device__ __forceinline__ void merge_max_sum(float& m, float& s, float m2, float s2) {
+    const float mx = fmaxf(m, m2);
+    s = (m == -INFINITY ? 0.f : s * __expf(m - mx)) + (m2 == -INFINITY ? 0.f : s2 * __expf(m2 - mx));
+    m = mx;
 }
 
-// logits -> d(loss)/d(logits) in place: (exp(logit - lse) - [column == label]) * row_scale, bf16; the padding columns
-// [vocab, ld) of every row become zero.  One workgroup per row, eight columns per lane and trip (ld is a multiple of 64).
-__global__ __launch_bounds__(256) void ce_grad_kernel(bf16_t* logits, int64_t ld, int64_t vocab, const float* lse, const float* row_scale,
-                                                      const int64_t* labels) {
+__global__ __launch_bounds__(256) void ce_loss_and_grad_kernel(bf16_t* logits, int64_t ld, int64_t vocab, const int64_t* labels, const float* row_scale,
+                                                               float* lse_out, float* loss_out) {
+    __shared__ float wave_m[4], wave_s[4];
     const int64_t row = blockIdx.x;
-    const float l = lse[row], rs = row_scale[row];
-    const int64_t label = labels[row];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint4* p = (uint4*)(logits + row * ld);
+    const int64_t label = labels[row];
+    const float rs = row_scale[row];
+    float m = -INFINITY, sum = 0.f;
+    for (int64_t c8 = threadIdx.x; c8 < ld / 8; c8 += 256) {
+        const uint4 v = p[c8];
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        float x[8];
+        float cm = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            x[e] = c8 * 8 + e < vocab ? bf16_to_f32((bf16_t)((e & 1) ? w[e >> 1] >> 16 : w[e >> 1] & 0xFFFFu)) : -INFINITY;
+            cm = fmaxf(cm, x[e]);
+        }
+        if (cm == -INFINITY) continue;  // padding only
+        float cs = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) cs += x[e] == -INFINITY ? 0.f : __expf(x[e] - cm);
+        merge_max_sum(m, sum, cm, cs);
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const float m2 = __shfl_xor(m, off, 64), s2 = __shfl_xor(sum, off, 64);
+        merge_max_sum(m, sum, m2, s2);
+    }
+    if (lane == 0) wave_m[wave] = m, wave_s[wave] = sum;
+    __syncthreads();
+    m = wave_m[0], sum = wave_s[0];
+#pragma unroll
+    for (int w = 1; w < 4; w++) merge_max_sum(m, sum, wave_m[w], wave_s[w]);
+    const float lse = m + __logf(sum);
+    if (threadIdx.x == 0) {
+        lse_out[row] = lse;
+        const float target = label >= 0 && label < vocab ? bf16_to_f32(logits[row * ld + label]) : 0.f;
+        loss_out[row] = rs != 0.f ? (lse - target) * rs : 0.f;
+    }
+    __syncthreads();  // the target logit is read before the row is overwritten
     for (int64_t c8 = threadIdx.x; c8 < ld / 8; c8 += 256) {
         const uint4 v = p[c8];
         const uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -83,7 +100,7 @@ __global__ __launch_bounds__(256) void ce_grad_kernel(bf16_t* logits, int64_t ld
             for (int h = 0; h < 2; h++) {
                 const int64_t col = c8 * 8 + 2 * e + h;
                 const float logit = bf16_to_f32((bf16_t)(h ? w[e] >> 16 : w[e] & 0xFFFFu));
-                float d = __expf(logit - l);
+                float d = __expf(logit - lse);
                 if (col == label) d -= 1.0f;
                 g[h] = col < vocab ? d * rs : 0.0f;
             }
@@ -98,11 +115,9 @@ static int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
 static int64_t padded_vocab(int64_t vocab) { return (vocab + 63) / 64 * 64; }
 
 int64_t lmhead_ce_workspace_bytes(int64_t rows, int64_t vocab, int64_t hidden, int64_t chunk) {
-    (void)hidden;
-    const int64_t rc = chunk < rows ? chunk : rows;
+    (void)hidden, (void)chunk;
     const int64_t br = std::min(rows, kBlockRows);
-    const int64_t nparts = (vocab + kBN - 1) / kBN * 2;
-    return align256(rows * 4) * 3 + align256(rc * nparts * 8) + align256(br * padded_vocab(vocab) * 2) + 1024;
+    return align256(rows * 4) * 2 + align256(br * padded_vocab(vocab) * 2) + 1024;
 }
 
 int lmhead_ce(int qt, const void* hidden, const void* packed, const int64_t* labels, int64_t rows, int64_t vocab,
@@ -114,38 +129,28 @@ int lmhead_ce(int qt, const void* hidden, const void* packed, const int64_t* lab
     if (ws_bytes < lmhead_ce_workspace_bytes(rows, vocab, hidden_dim, chunk)) return set_error(GGQ_ERR_WORKSPACE, "lmhead_ce: workspace too small");
     if (((uintptr_t)hidden | (uintptr_t)packed | (uintptr_t)grad_hidden | (uintptr_t)ws) & 15) return set_error(GGQ_ERR_ALIGN, "lmhead_ce: pointers must be 16-byte aligned");
     if (rows == 0) return GGQ_OK;
-    const int64_t rc_max = chunk < rows ? chunk : rows;
     const int64_t br_max = std::min(rows, kBlockRows);
     const int64_t ld = padded_vocab(vocab);
-    const int nparts = (int)((vocab + kBN - 1) / kBN) * 2;
     char* w = (char*)ws;
     float* row_scale = (float*)w; w += align256(rows * 4);
     float* lse = lse_out ? lse_out : (float*)w; w += align256(rows * 4);
-    float* target = (float*)w; w += align256(rows * 4);
-    float2* partials = (float2*)w; w += align256(rc_max * nparts * 8);
     bf16_t* logits = (bf16_t*)w;  // [br_max, ld]
 
     hipLaunchKernelGGL(ce_row_scale_kernel, dim3(1), dim3(1024), 0, s, labels, rows, ignore_index, reduction_mean, row_scale, n_valid_out);
     for (int64_t b0 = 0; b0 < rows; b0 += br_max) {
-        const int64_t br = std::min(rows - b0, br_max);
-        // (1) statistics and logits, chunk by chunk
-        for (int64_t r0 = b0; r0 < b0 + br; r0 += chunk) {
-            const int rc = (int)std::min(b0 + br - r0, chunk);
-            MmqParams p;
-            if (int rcode = init_params(p, qt, kModeNT, rc, (int)vocab, (int)hidden_dim, 1)) return rcode;
-            p.a[0] = (const bf16_t*)hidden + r0 * hidden_dim, p.lda = hidden_dim;
-            p.w[0] = (const uint8_t*)packed;
-            p.c[0] = logits + (r0 - b0) * ld, p.ldc = ld;
-            p.labels = labels + r0, p.ce_partials = partials, p.ce_partials_ld = nparts, p.ce_target_logit = target + r0;
-            p.ignore_index = ignore_index;
-            if (int rcode = launch_mmq(qt, kModeNT, kEpiCeStats, p, s)) return rcode;
-            hipLaunchKernelGGL(ce_finalize_kernel, dim3((rc + 3) / 4), dim3(256), 0, s, partials, nparts, nparts, target + r0, row_scale + r0, rc, lse + r0, loss_1d + r0);
-        }
-        // (2) the block's logits become the gradient with respect to them, in place
-        hipLaunchKernelGGL(ce_grad_kernel, dim3((unsigned)br), dim3(256), 0, s, logits, ld, vocab, lse + b0, row_scale + b0, labels + b0);
+        const int br = (int)std::min(rows - b0, br_max);
+        // (1) logits = hidden . W^T
+        MmqParams p;
+        if (int rcode = init_params(p, qt, kModeNT, br, (int)vocab, (int)hidden_dim, 1)) return rcode;
+        p.a[0] = (const bf16_t*)hidden + b0 * hidden_dim, p.lda = hidden_dim;
+        p.w[0] = (const uint8_t*)packed;
+        p.c[0] = logits, p.ldc = ld;
+        if (int rcode = launch_mmq(qt, kModeNT, kEpiStore, p, s)) return rcode;
+        // (2) loss per row; the logits become the gradient with respect to them
+        hipLaunchKernelGGL(ce_loss_and_grad_kernel, dim3((unsigned)br), dim3(256), 0, s, logits, ld, vocab, labels + b0, row_scale + b0, lse + b0, loss_1d + b0);
         // (3) dH = dlogits . W over the whole vocabulary
         MmqParams g;
-        if (int rcode = init_params(g, qt, kModeNN, (int)br, (int)vocab, (int)hidden_dim, 1)) return rcode;
+        if (int rcode = init_params(g, qt, kModeNN, br, (int)vocab, (int)hidden_dim, 1)) return rcode;
         g.a[0] = logits, g.lda = ld, g.a_zero_padded = 1;
         g.w[0] = (const uint8_t*)packed;
         g.c[0] = (bf16_t*)grad_hidden + b0 * hidden_dim, g.ldc = hidden_dim;

@@ -66,8 +66,7 @@ constexpr int kThreads = 1024;  // waves 0..7 run the MFMAs, waves 8..15 load an
 
 enum : int { kModeNT = 0, kModeNN = 1 };
 enum : int {
-    kEpiStore = 0,    // C (bf16) = acc
-    kEpiCeStats = 2   // per-row partial (max, sum exp) over the tile's columns + target logit; optionally C (bf16) = acc as well
+    kEpiStore = 0  // C (bf16) = acc
 };
 
 struct MmqParams {
@@ -103,12 +102,6 @@ struct MmqParams {
     int r_pad;            // multiple of 16, <= 64; 0 = no LoRA
     int lora_rank;        // NN mode: rows of the factor A that exist (the tile's rows up to r_pad are zero)
     float lora_scale;
-    // cross-entropy statistics epilogue
-    const int64_t* labels;     // [m]
-    float2* ce_partials;       // [m, ce_partials_ld] (max, sumexp)
-    float* ce_target_logit;    // [m]
-    int ce_partials_ld, ce_col_offset, ce_partial_offset;
-    int64_t ignore_index;
 };
 
 constexpr int kMaxTimedLaunches = 8192;

@@ -70,28 +70,6 @@ __device__ __forceinline__ uint4 load8_slow(const bf16_t* p, int valid) {
     return v;
 }
 
-// All-reduce over each half of a wave (lanes 0..31, 32..63): four data-parallel-primitive steps inside the rows of 16
-// lanes (neighbour, pair of a quad, mirror of 8, mirror of 16: every lane of a row ends with the row's result) and one
-// cross-lane exchange between the two rows of a half.  Five exchanges through the LDS crossbar cost several times more.
-template <int CTRL>
-static __device__ __forceinline__ float dpp_f32(float x) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
-}
-static __device__ __forceinline__ float half_wave_max(float x) {
-    x = fmaxf(x, dpp_f32<0xB1>(x));   // quad_perm [1,0,3,2]
-    x = fmaxf(x, dpp_f32<0x4E>(x));   // quad_perm [2,3,0,1]
-    x = fmaxf(x, dpp_f32<0x141>(x));  // row_half_mirror
-    x = fmaxf(x, dpp_f32<0x140>(x));  // row_mirror
-    return fmaxf(x, __shfl_xor(x, 16, 64));
-}
-static __device__ __forceinline__ float half_wave_sum(float x) {
-    x += dpp_f32<0xB1>(x);
-    x += dpp_f32<0x4E>(x);
-    x += dpp_f32<0x141>(x);
-    x += dpp_f32<0x140>(x);
-    return x + __shfl_xor(x, 16, 64);
-}
-
 struct TileCtx {  // wave-uniform description of the tile this workgroup computes
     int row_begin, rows_valid, col0, col_tile, seg_c, out_cols, contraction, total_steps, base;
     int64_t expert;
@@ -100,7 +78,6 @@ struct TileCtx {  // wave-uniform description of the tile this workgroup compute
     uint32_t as_lds;  // LDS byte address of `as`
     bool a_fast;      // A rows can be moved with aligned 16-byte accesses and every step is whole
     const uint2* grid;
-    const int* row_meta;  // cross-entropy statistics epilogue: the label of every tile row, staged in LDS
 };
 
 // (segment, first contraction index) of a step; at most two segments.
@@ -841,37 +818,6 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
                     if (col_ok[cb]) cbase[elem + cb * 32] = to_bf16(acc[rb][cb][i]);
             }
         }
-    } else {  // kEpiCeStats
-        bf16_t* const logits_out = (bf16_t*)p.c[0];  // optional: the logits themselves, for a gradient pass that does not recompute them
-#pragma unroll
-        for (int rb = 0; rb < LIVE; rb++) {
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int r = 32 * (kWavesM * rb + wave_m) + (i >> 2) * 8 + lane_h * 4 + (i & 3);
-                const bool row_ok = r < c.rows_valid;
-                const int64_t grow = c.row_begin + (row_ok ? r : 0);
-                const int64_t label = row_ok ? (int64_t)c.row_meta[r] : -1;
-                float v[kColBlocks];
-                float mx = -INFINITY;
-#pragma unroll
-                for (int cb = 0; cb < kColBlocks; cb++) {
-                    const int col = col_base + cb * 32;
-                    const bf16_t logit = to_bf16(acc[rb][cb][i]);
-                    v[cb] = col < c.out_cols ? bf16_to_f32(logit) : -INFINITY;
-                    if (logits_out && row_ok && col < c.out_cols) logits_out[grow * p.ldc + col] = logit;
-                    mx = fmaxf(mx, v[cb]);
-                    if (row_ok && col < c.out_cols && (int64_t)(col + p.ce_col_offset) == label) p.ce_target_logit[grow] = v[cb];
-                }
-                // reduce over the 32 lanes that share this row (lanes with equal lane_h)
-                mx = half_wave_max(mx);
-                float sum = 0.f;
-#pragma unroll
-                for (int cb = 0; cb < kColBlocks; cb++) sum += v[cb] == -INFINITY ? 0.f : __expf(v[cb] - mx);
-                sum = half_wave_sum(sum);
-                if (row_ok && lane_c == 0)
-                    p.ce_partials[grow * p.ce_partials_ld + p.ce_partial_offset + c.col_tile * 2 + wave_n] = make_float2(mx, sum);
-            }
-        }
     }
 }
 
@@ -921,10 +867,6 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
     c.bs = (bf16_t*)(smem_raw + kAStages * kAStageBytes);
     uint2* grid_lds = (uint2*)(smem_raw + kTileLdsBytes);  // the decoder's tables, IQ2_XXS only
     c.grid = grid_lds;
-    // what the cross-entropy statistics epilogue needs per row, read once per tile: one dependent global load per row and
-    // lane in the epilogue costs a memory round trip each
-    int* row_meta = (int*)(smem_raw + kTileLdsBytes + (QT == kIQ2_XXS ? Fmt<kIQ2_XXS>::kTableWords * 4 : 0));
-    c.row_meta = row_meta;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps control flow scalar
@@ -992,10 +934,7 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
                 }
             }
         }
-        if (EPI == kEpiCeStats) {
-            for (int r = tid; r < kTM; r += kThreadsWG) row_meta[r] = (int)p.labels[c.row_begin + min(r, c.rows_valid - 1)];
-        }
-        __syncthreads();  // LoRA tiles, the codebook tables and the row values are visible
+        __syncthreads();  // LoRA tiles and the codebook tables are visible
     };
 
     if (wave >= kCW) {
