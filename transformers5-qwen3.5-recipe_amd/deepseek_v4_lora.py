@@ -39,35 +39,35 @@ class GGUFGroupedLinear(torch.nn.Module):
 
 
 def _deepseek_v4_fixed_grouped_mmq_forward(self: GGUFGroupedLinear, input: torch.Tensor) -> torch.Tensor:
-    """The reference's replacement forward for ``GGUFGroupedLinear`` (deepseek_v4_lora.py:91-124): same guards, the grouped
-    payload viewed as ``[n_groups, out_features / n_groups, bytes]``, no logical matrix materialised."""
-    original_input_dtype = input.dtype
+    """The reference's replacement forward for ``GGUFGroupedLinear`` (deepseek_v4_lora.py:91-124), with its guards and
+    messages: the flattened payload is viewed as ``[n_groups, out_features / n_groups, bytes]`` and handed to the fixed
+    grouped operator, so the group boundary survives and no logical matrix is materialised; the result comes back in the
+    input's dtype."""
     if self.compute_dtype != torch.bfloat16:
         raise RuntimeError("DeepSeek fixed grouped MMQ requires BF16 compute_dtype.")
-    if self.input_permutation is not None or self.output_permutation is not None:
+    if not (self.input_permutation is None and self.output_permutation is None):
         raise RuntimeError("DeepSeek fixed grouped MMQ does not support layout permutations.")
-    compute_input = input.to(self.compute_dtype)
-    if not compute_input.is_contiguous() or compute_input.storage_offset() != 0:
-        compute_input = compute_input.contiguous()
-    group_out_features = self.out_features // self.n_groups
+    rows_per_group = self.out_features // self.n_groups
     payload = self.weight.as_subclass(torch.Tensor)
-    expected_payload_rows = self.n_groups * group_out_features
-    if payload.ndim != 2 or payload.shape[0] != expected_payload_rows:
-        raise RuntimeError(f"DeepSeek fixed grouped MMQ expects a flattened grouped payload with {expected_payload_rows} rows, got {tuple(payload.shape)}.")
-    packed_groups = payload.reshape(self.n_groups, group_out_features, -1)
-    output = fixed_grouped_mmq(compute_input, packed_groups, int(getattr(self.weight, "quant_type", 8)))
-    return output.to(original_input_dtype)
+    if payload.ndim != 2 or payload.shape[0] != self.n_groups * rows_per_group:
+        raise RuntimeError("DeepSeek fixed grouped MMQ expects a flattened grouped payload with "
+                           f"{self.n_groups * rows_per_group} rows, got {tuple(payload.shape)}.")
+    x = input.to(torch.bfloat16)
+    if x.storage_offset() or not x.is_contiguous():
+        x = x.contiguous()
+    block_format = int(getattr(self.weight, "quant_type", 8))
+    y = fixed_grouped_mmq(x, payload.view(self.n_groups, rows_per_group, payload.shape[1]), block_format)
+    return y if y.dtype == input.dtype else y.to(input.dtype)
 
 
 def normalize_peft_path(path: str) -> str:
-    """The pre-PEFT model path of a module or parameter (deepseek_v4_lora.py:165-175)."""
-    for prefix in ("base_model.model.", "model."):
-        if path.startswith(prefix):
-            path = path.removeprefix(prefix)
-    if path.startswith("model.layers."):
-        return path
+    """The pre-PEFT model path of a module or parameter (the mapping of deepseek_v4_lora.py:165-175): wrapper prefixes are
+    dropped one after the other, and a path that then starts at ``layers.`` gets its ``model.`` back."""
+    for wrapper_prefix in ("base_model.model.", "model."):
+        if path.startswith(wrapper_prefix):
+            path = path[len(wrapper_prefix):]
     if path.startswith("layers."):
-        return f"model.{path}"
+        path = "model." + path
     return path
 
 
