@@ -217,6 +217,34 @@ def test_routed_projection_reads_tokens_in_place(pkg, dev, top_k, rank, pair, qt
         assert_close_bf16(got[-2], o["da"], "in-place dA against the oracle")
 
 
+@pytest.mark.parametrize("shape", ["", "0", "1", "2", "3"])
+def test_q4k_grouped_identity_reproduces_decoded_rows_exactly(pkg, dev, shape, monkeypatch):
+    # One-hot rows through every Q4_K kernel shape of the grouped launches (the decoding-wave kernels by default): each
+    # output is a single product 1 * w, so the in-register decoders are compared with the oracle element by element, for
+    # arbitrary block bytes (every 6-bit scale split), in forward (pair) and in grad-input.
+    if shape:
+        monkeypatch.setenv("GGQ_GROUPED_SHAPE", shape)
+    ml = pkg.fast_moe_lora
+    e, n, k = 3, 256, 512
+    p1, p2 = _expert_payload(71, gb.Q4_K, e, n, k, "random"), _expert_payload(72, gb.Q4_K, e, n, k, "random")
+    w1 = torch.from_numpy(gb.dequantize_bf16(p1.reshape(e * n, -1), gb.Q4_K)).reshape(e, n, k)
+    w2 = torch.from_numpy(gb.dequantize_bf16(p2.reshape(e * n, -1), gb.Q4_K)).reshape(e, n, k)
+    ids = torch.arange(e, dtype=torch.int64, device=dev)
+    # forward: expert g gets the k one-hot rows; groups of 512 rows (several row tiles each)
+    x = torch.eye(k, dtype=torch.bfloat16, device=dev).repeat(e, 1)
+    ends = torch.tensor([k, 2 * k, 3 * k], dtype=torch.int32, device=dev)
+    y1, y2 = ml.grouped_mmq_pair(x, torch.from_numpy(p1).to(dev), torch.from_numpy(p2).to(dev), ids, ends, gb.Q4_K, n)
+    for g in range(e):
+        assert torch.equal(y1[g * k:(g + 1) * k].float().cpu(), w1[g].T.contiguous()), (g, "first of the pair")
+        assert torch.equal(y2[g * k:(g + 1) * k].float().cpu(), w2[g].T.contiguous()), (g, "second of the pair")
+    # grad-input: expert g gets the n one-hot cotangent rows
+    dy = torch.eye(n, dtype=torch.bfloat16, device=dev).repeat(e, 1)
+    ends_n = torch.tensor([n, 2 * n, 3 * n], dtype=torch.int32, device=dev)
+    dx = ml.grouped_mmq_grad_input(dy, torch.from_numpy(p1).to(dev), ids, ends_n, gb.Q4_K, k)
+    for g in range(e):
+        assert torch.equal(dx[g * n:(g + 1) * n].float().cpu(), w1[g]), (g, "grad-input")
+
+
 def _layer_case(seed, tokens, hidden, inter, experts, k, r, qt):
     gen = torch.Generator().manual_seed(seed)
     pg, pu = _expert_payload(seed, qt, experts, inter, hidden), _expert_payload(seed + 1000, qt, experts, inter, hidden)
