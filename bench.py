@@ -142,7 +142,7 @@ def other_workload(name, pkg, lib, dev, args):
             x.grad = a.grad = b.grad = None
             pkg.fast_lora.lora_mmq(x, payload, 12, n, a, b, 2.0).backward(dy)
     elif name == "lmhead_q6k":  # configs[3]
-        vocab, hidden, rows, chunk = 151936, 2048, 4096, 1024
+        vocab, hidden, rows, chunk = 151936, 2048, 4096, args.chunk
         payload = torch.cat([pkg.gguf.quantize_q6_k(torch.randn(min(18992, vocab - lo), hidden, generator=g, device=dev) * 0.02)
                              for lo in range(0, vocab, 18992)], dim=0)
         hs = bf(rows, hidden).requires_grad_(True)
@@ -150,8 +150,8 @@ def other_workload(name, pkg, lib, dev, args):
         labels[torch.rand(rows, device=dev, generator=g) < 0.05] = -100
         flops = 2 * 2 * rows * vocab * hidden
         launch_flops, launches_per_step = None, None   # launches of different sizes (statistics per chunk, one grad-input)
-        workload = "configs[3]: chunked cross-entropy through a Q6_K lm_head [151936x2048], 4096 rows, chunks of 1024, loss + dHidden"
-        metric = "fwd+bwd TFLOP/s (two GEMMs), chunked lm_head cross-entropy"
+        workload = f"configs[3]: chunked cross-entropy through a Q6_K lm_head [151936x2048], 4096 rows, chunks of {chunk}, loss + dHidden"
+        metric = "fwd+bwd TFLOP/s (two algorithmic GEMMs), chunked lm_head cross-entropy"
 
         def step():
             hs.grad = None
@@ -222,6 +222,7 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--chunk", type=int, default=1024, help="lmhead_q6k: rows per chunk (1024 in the BASELINE configuration; from 4096 rows on the logits of a chunk are kept)")
     ap.add_argument("--graph", type=int, default=1, help="replay the step from a captured HIP graph (1) or run it eagerly (0)")
     args = ap.parse_args()
     if args.gpus != 1:

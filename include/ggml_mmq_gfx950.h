@@ -178,10 +178,10 @@ int ggq_router_topk(const void* logits, int logits_are_bf16, int64_t tokens, int
 /* _packed_q8_linear_cross_entropy_forward (gguf_liger_loss.py:38-186): chunked mmq -> Liger
  * cross-entropy -> mmq_grad_input in one call.  labels int64 [rows];
  * loss_per_row fp32 [rows] (already divided by the number of non-ignored rows when reduction_mean);
- * grad_hidden bf16 [rows, hidden]; lse_out fp32 [rows] or NULL; n_valid_out int32[1] or NULL.  The bf16 logits of up to
- * 4096 rows at a time are kept in the workspace (the reference's [chunk, vocab] tensor), turned into their gradient in place
- * and contracted with the packed rows by one grad-input launch; `chunk` (positive) is accepted for the reference's signature
- * and does not change the result or the memory bound. */
+ * grad_hidden bf16 [rows, hidden]; lse_out fp32 [rows] or NULL; n_valid_out int32[1] or NULL.  `chunk` is the memory
+ * contract, as the reference's [chunk, vocab] logits tensor is: below 4096 rows per chunk nothing wider than 8192 vocabulary
+ * columns is ever held (the logits are recomputed for the gradient: three GEMMs); from 4096 rows per chunk on, or when one
+ * chunk covers all rows, the chunk's bf16 logits are kept in the workspace and rewritten as their gradient (two GEMMs). */
 int64_t ggq_lmhead_ce_workspace_bytes(int64_t rows, int64_t vocab, int64_t hidden_dim, int64_t chunk);
 int ggq_lmhead_cross_entropy(int qt, const void* hidden, const void* packed, const int64_t* labels, int64_t rows, int64_t vocab,
                              int64_t hidden_dim, int64_t chunk, int64_t ignore_index, int reduction_mean, float* loss_per_row,

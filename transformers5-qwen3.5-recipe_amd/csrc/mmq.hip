@@ -139,7 +139,8 @@ static int launch_one(const MmqParams& p, hipStream_t s) {
         g_timed_count++;
         (void)hipEventRecord(t->start, s);
     }
-    constexpr int kSmemBytes = Tile<SH>::kTileLdsBytes + (QT == kIQ2_XXS ? Fmt<kIQ2_XXS>::kTableWords * 4 : 0);
+    constexpr int kSmemBytes = Tile<SH>::kTileLdsBytes + (QT == kIQ2_XXS ? Fmt<kIQ2_XXS>::kTableWords * 4 : 0) +
+                               (EPI == kEpiCeStats || EPI == kEpiCeGrad ? Tile<SH>::kTM * 16 : 0);
     static bool attr_set = false;  // per instantiation; the attribute is a property of the function
     if (!attr_set) {
         hipError_t e;
@@ -229,6 +230,8 @@ static int launch_qt(int mode, int epi, const MmqParams& p, hipStream_t s) {
                 if (QT == kQ4_K && p.shape == kShapeWide) return launch_one<kQ4_K, kModeNT, kEpiStore, 1>(p, s);
                 if (QT == kQ4_K && p.shape == kShapeHalf) return launch_one<kQ4_K, kModeNT, kEpiStore, 2>(p, s);
                 return launch_one<QT, kModeNT, kEpiStore, 0>(p, s);
+            case kEpiCeStats: return launch_one<QT, kModeNT, kEpiCeStats, 0>(p, s);
+            case kEpiCeGrad: return launch_one<QT, kModeNT, kEpiCeGrad, 0>(p, s);
         }
     } else {
         switch (epi) {
@@ -237,6 +240,7 @@ static int launch_qt(int mode, int epi, const MmqParams& p, hipStream_t s) {
                 if (QT == kQ4_K && p.shape == kShapeWide) return launch_one<kQ4_K, kModeNN, kEpiStore, 1>(p, s);
                 if (QT == kQ4_K && p.shape == kShapeHalf) return launch_one<kQ4_K, kModeNN, kEpiStore, 2>(p, s);
                 return launch_one<QT, kModeNN, kEpiStore, 0>(p, s);
+            case kEpiAccumF32: return launch_one<QT, kModeNN, kEpiAccumF32, 0>(p, s);
         }
     }
     return set_error(GGQ_ERR_SHAPE, "mmq: unsupported mode/epilogue combination");

@@ -66,7 +66,10 @@ constexpr int kThreads = 1024;  // waves 0..7 run the MFMAs, waves 8..15 load an
 
 enum : int { kModeNT = 0, kModeNN = 1 };
 enum : int {
-    kEpiStore = 0  // C (bf16) = acc
+    kEpiStore = 0,     // C (bf16) = acc
+    kEpiAccumF32 = 1,  // C32 (fp32) += acc
+    kEpiCeStats = 2,   // per-row partial (max, sum exp) over the tile's columns + target logit
+    kEpiCeGrad = 3     // C (bf16) = (exp(acc - lse[m]) - [col == label[m]]) * row_scale[m]
 };
 
 struct MmqParams {
@@ -102,6 +105,14 @@ struct MmqParams {
     int r_pad;            // multiple of 16, <= 64; 0 = no LoRA
     int lora_rank;        // NN mode: rows of the factor A that exist (the tile's rows up to r_pad are zero)
     float lora_scale;
+    // cross-entropy epilogues
+    const int64_t* labels;     // [m]
+    const float* lse;          // [m]
+    const float* row_scale;    // [m]  (1/n_non_ignore or 1, 0 for ignored rows)
+    float2* ce_partials;       // [m, ce_partials_ld] (max, sumexp)
+    float* ce_target_logit;    // [m]
+    int ce_partials_ld, ce_col_offset, ce_partial_offset;
+    int64_t ignore_index;
 };
 
 constexpr int kMaxTimedLaunches = 8192;

@@ -70,6 +70,28 @@ __device__ __forceinline__ uint4 load8_slow(const bf16_t* p, int valid) {
     return v;
 }
 
+// All-reduce over each half of a wave (lanes 0..31, 32..63): four data-parallel-primitive steps inside the rows of 16
+// lanes (neighbour, pair of a quad, mirror of 8, mirror of 16: every lane of a row ends with the row's result) and one
+// cross-lane exchange between the two rows of a half.  Five exchanges through the LDS crossbar cost several times more.
+template <int CTRL>
+static __device__ __forceinline__ float dpp_f32(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
+}
+static __device__ __forceinline__ float half_wave_max(float x) {
+    x = fmaxf(x, dpp_f32<0xB1>(x));   // quad_perm [1,0,3,2]
+    x = fmaxf(x, dpp_f32<0x4E>(x));   // quad_perm [2,3,0,1]
+    x = fmaxf(x, dpp_f32<0x141>(x));  // row_half_mirror
+    x = fmaxf(x, dpp_f32<0x140>(x));  // row_mirror
+    return fmaxf(x, __shfl_xor(x, 16, 64));
+}
+static __device__ __forceinline__ float half_wave_sum(float x) {
+    x += dpp_f32<0xB1>(x);
+    x += dpp_f32<0x4E>(x);
+    x += dpp_f32<0x141>(x);
+    x += dpp_f32<0x140>(x);
+    return x + __shfl_xor(x, 16, 64);
+}
+
 struct TileCtx {  // wave-uniform description of the tile this workgroup computes
     int row_begin, rows_valid, col0, col_tile, seg_c, out_cols, contraction, total_steps, base;
     int64_t expert;
@@ -78,6 +100,7 @@ struct TileCtx {  // wave-uniform description of the tile this workgroup compute
     uint32_t as_lds;  // LDS byte address of `as`
     bool a_fast;      // A rows can be moved with aligned 16-byte accesses and every step is whole
     const uint2* grid;
+    const float4* row_meta;  // cross-entropy epilogues: per tile row (lse, row scale, label as int bits, -), staged in LDS
 };
 
 // (segment, first contraction index) of a step; at most two segments.
@@ -798,10 +821,11 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
     // ---- epilogue.  acc[rb][cb][i]: tile row = 32*(kWavesM*rb + wave_m) + 8*(i/4) + 4*lane_h + (i%4),
     //                                 tile col = 64*wave_n + 32*cb + lane_c
     const int col_base = c.col0 + wave_n * 64 + lane_c;
-    if (EPI == kEpiStore) {
+    if (EPI == kEpiStore || EPI == kEpiAccumF32 || EPI == kEpiCeGrad) {
         // everything that does not depend on the element is read once, up front
         const int64_t ldc = p.ldc;
-        bf16_t* const cbase = (bf16_t*)p.c[c.seg_c];
+        char* const cbase = (char*)p.c[EPI == kEpiStore ? c.seg_c : 0];
+        const int64_t ce_off = p.ce_col_offset;
         const int rows_valid = c.rows_valid;
         const bool col_ok[kColBlocks] = {col_base < c.out_cols, col_base + 32 < c.out_cols};
 #pragma unroll
@@ -813,9 +837,55 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
                 const int dr = (i >> 2) * 8 + (i & 3);  // uniform row step inside the block
                 if (r_lane + dr >= rows_valid) continue;
                 const int64_t elem = lane_elem + (int64_t)dr * ldc;
+                float lse = 0.f, rs = 0.f;
+                int64_t label = -1;
+                if (EPI == kEpiCeGrad) {
+                    const float4 meta = c.row_meta[r_lane + dr];
+                    lse = meta.x, rs = meta.y, label = (int64_t)__float_as_int(meta.z);
+                }
 #pragma unroll
-                for (int cb = 0; cb < kColBlocks; cb++)
-                    if (col_ok[cb]) cbase[elem + cb * 32] = to_bf16(acc[rb][cb][i]);
+                for (int cb = 0; cb < kColBlocks; cb++) {
+                    if (!col_ok[cb]) continue;
+                    const float v = acc[rb][cb][i];
+                    if (EPI == kEpiStore) {
+                        ((bf16_t*)cbase)[elem + cb * 32] = to_bf16(v);
+                    } else if (EPI == kEpiAccumF32) {
+                        ((float*)cbase)[elem + cb * 32] += v;
+                    } else {
+                        const float logit = bf16_to_f32(to_bf16(v));  // the path's logits are bf16 values
+                        float g = __expf(logit - lse);
+                        if ((int64_t)(col_base + cb * 32) + ce_off == label) g -= 1.0f;
+                        ((bf16_t*)cbase)[elem + cb * 32] = to_bf16(g * rs);
+                    }
+                }
+            }
+        }
+    } else {  // kEpiCeStats
+#pragma unroll
+        for (int rb = 0; rb < LIVE; rb++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int r = 32 * (kWavesM * rb + wave_m) + (i >> 2) * 8 + lane_h * 4 + (i & 3);
+                const bool row_ok = r < c.rows_valid;
+                const int64_t grow = c.row_begin + (row_ok ? r : 0);
+                const int64_t label = row_ok ? (int64_t)__float_as_int(c.row_meta[r].z) : -1;
+                float v[kColBlocks];
+                float mx = -INFINITY;
+#pragma unroll
+                for (int cb = 0; cb < kColBlocks; cb++) {
+                    const int col = col_base + cb * 32;
+                    v[cb] = col < c.out_cols ? bf16_to_f32(to_bf16(acc[rb][cb][i])) : -INFINITY;
+                    mx = fmaxf(mx, v[cb]);
+                    if (row_ok && col < c.out_cols && (int64_t)(col + p.ce_col_offset) == label) p.ce_target_logit[grow] = v[cb];
+                }
+                // reduce over the 32 lanes that share this row (lanes with equal lane_h)
+                mx = half_wave_max(mx);
+                float sum = 0.f;
+#pragma unroll
+                for (int cb = 0; cb < kColBlocks; cb++) sum += v[cb] == -INFINITY ? 0.f : __expf(v[cb] - mx);
+                sum = half_wave_sum(sum);
+                if (row_ok && lane_c == 0)
+                    p.ce_partials[grow * p.ce_partials_ld + p.ce_partial_offset + c.col_tile * 2 + wave_n] = make_float2(mx, sum);
             }
         }
     }
@@ -867,6 +937,10 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
     c.bs = (bf16_t*)(smem_raw + kAStages * kAStageBytes);
     uint2* grid_lds = (uint2*)(smem_raw + kTileLdsBytes);  // the decoder's tables, IQ2_XXS only
     c.grid = grid_lds;
+    // what the cross-entropy epilogues need per row, read once per tile: one dependent global load per row and lane in
+    // the epilogue costs a memory round trip each
+    float4* row_meta = (float4*)(smem_raw + kTileLdsBytes + (QT == kIQ2_XXS ? Fmt<kIQ2_XXS>::kTableWords * 4 : 0));
+    c.row_meta = row_meta;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps control flow scalar
@@ -934,7 +1008,14 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
                 }
             }
         }
-        __syncthreads();  // LoRA tiles and the codebook tables are visible
+        if (EPI == kEpiCeStats || EPI == kEpiCeGrad) {
+            for (int r = tid; r < kTM; r += kThreadsWG) {
+                const int64_t grow = c.row_begin + min(r, c.rows_valid - 1);
+                row_meta[r] = make_float4(EPI == kEpiCeGrad ? p.lse[grow] : 0.f, EPI == kEpiCeGrad ? p.row_scale[grow] : 0.f,
+                                          __int_as_float((int)p.labels[grow]), 0.f);
+            }
+        }
+        __syncthreads();  // LoRA tiles, the codebook tables and the row values are visible
     };
 
     if (wave >= kCW) {

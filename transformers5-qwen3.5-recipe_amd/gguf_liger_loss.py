@@ -4,8 +4,8 @@ Host-side mirror of the reference's ``gguf_liger_loss.py``: the same autograd ``
 (loss and d(loss)/d(hidden) are both produced in forward, backward only scales by the upstream scalar
 and rejects double backward; gguf_liger_loss.py:189-266) and the same causal-LM wrapper guards
 (:269-356).  The chunk loop itself (:103-177) runs inside one call into the kernel library, which keeps
-the bf16 logits of at most 4096 rows at a time in its workspace (the reference's [chunk, vocab] tensor), turns
-them into their gradient in place, and needs no host synchronisation for the non-ignored count.
+nothing wider than an 8192-column slab for chunks below 4096 rows and the chunk's bf16 logits (the reference's
+[chunk, vocab] tensor) from there on, and needs no host synchronisation for the non-ignored count.
 """
 
 from __future__ import annotations
