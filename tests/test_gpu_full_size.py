@@ -84,9 +84,11 @@ def test_sampled_expert_groups_at_full_size_match_an_fp32_matmul(pkg, dev):
         assert_close_bf16(xs.grad[r0:r1], want_dx.double(), f"dX of expert {e}")
 
 
-def test_lm_head_loss_at_full_size_matches_a_chunked_torch_reference(pkg, dev):
-    # Qwen's head: 151936 x 2048 in Q6_K, 4096 rows, chunks of 1024 rows
-    vocab, hidden, rows, chunk = 151936, 2048, 4096, 1024
+@pytest.mark.parametrize("chunk", [1024, 4096])
+def test_lm_head_loss_at_full_size_matches_a_chunked_torch_reference(pkg, dev, chunk):
+    # Qwen's head: 151936 x 2048 in Q6_K, 4096 rows; chunks of 1024 rows (no logits kept, the gradient recomputes them) and of
+    # 4096 rows (the chunk's logits kept and rewritten as their gradient)
+    vocab, hidden, rows = 151936, 2048, 4096
     g = torch.Generator(device=dev).manual_seed(31)
     payload = torch.cat([pkg.gguf.quantize_q6_k(torch.randn(min(18992, vocab - lo), hidden, generator=g, device=dev) * 0.02)
                          for lo in range(0, vocab, 18992)], dim=0)
