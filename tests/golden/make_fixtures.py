@@ -23,7 +23,8 @@ HERE = Path(__file__).resolve().parent
 
 def main() -> None:
     out = {}
-    for qt, name in ((gb.Q8_0, "q8_0"), (gb.Q4_K, "q4_k"), (gb.Q6_K, "q6_k"), (gb.IQ2_XXS, "iq2_xxs")):
+    for qt, name in ((gb.Q8_0, "q8_0"), (gb.Q2_K, "q2_k"), (gb.Q3_K, "q3_k"), (gb.Q4_K, "q4_k"), (gb.Q5_K, "q5_k"), (gb.Q6_K, "q6_k"),
+                     (gb.IQ2_XXS, "iq2_xxs")):
         payload = np.concatenate([make_payload(100 + qt, qt, 3, 512, "quantized"), make_payload(200 + qt, qt, 3, 512, "random")])
         out[f"{name}_payload"] = payload
         out[f"{name}_f32"] = gb.dequantize(payload, qt)

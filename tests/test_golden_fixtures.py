@@ -11,7 +11,7 @@ from oracle import gguf_blocks as gb
 from oracle import routing as rt
 
 GOLDEN = Path(__file__).resolve().parent / "golden"
-TYPES = ((gb.Q8_0, "q8_0"), (gb.Q4_K, "q4_k"), (gb.Q6_K, "q6_k"), (gb.IQ2_XXS, "iq2_xxs"))
+TYPES = ((gb.Q8_0, "q8_0"), (gb.Q2_K, "q2_k"), (gb.Q3_K, "q3_k"), (gb.Q4_K, "q4_k"), (gb.Q5_K, "q5_k"), (gb.Q6_K, "q6_k"), (gb.IQ2_XXS, "iq2_xxs"))
 
 
 @pytest.fixture(scope="module")
