@@ -180,8 +180,9 @@ int ggq_router_topk(const void* logits, int logits_are_bf16, int64_t tokens, int
  * loss_per_row fp32 [rows] (already divided by the number of non-ignored rows when reduction_mean);
  * grad_hidden bf16 [rows, hidden]; lse_out fp32 [rows] or NULL; n_valid_out int32[1] or NULL.  `chunk` is the memory
  * contract, as the reference's [chunk, vocab] logits tensor is: below 4096 rows per chunk nothing wider than 8192 vocabulary
- * columns is ever held (the logits are recomputed for the gradient: three GEMMs); from 4096 rows per chunk on, or when one
- * chunk covers all rows, the chunk's bf16 logits are kept in the workspace and rewritten as their gradient (two GEMMs). */
+ * columns is ever held (one sweep over the vocabulary with a running max and sum per row); from 4096 rows per chunk on, or
+ * when one chunk covers all rows, the chunk's bf16 logits are kept in the workspace and rewritten as their gradient.  Two
+ * vocabulary-sized GEMMs either way. */
 int64_t ggq_lmhead_ce_workspace_bytes(int64_t rows, int64_t vocab, int64_t hidden_dim, int64_t chunk);
 int ggq_lmhead_cross_entropy(int qt, const void* hidden, const void* packed, const int64_t* labels, int64_t rows, int64_t vocab,
                              int64_t hidden_dim, int64_t chunk, int64_t ignore_index, int reduction_mean, float* loss_per_row,

@@ -159,6 +159,96 @@ __global__ __launch_bounds__(256) void ce_loss_and_grad_kernel(bf16_t* logits, i
     }
 }
 
+// ---- the form that keeps no logits: one sweep over the vocabulary in blocks of kVocabBlock columns with a running
+// (max, sum exp) per row, as in a streaming softmax.  Per block and row: the block's logits (a [rows, kVocabBlock] slab
+// written by the tile kernel) become p = exp(logit - running max) in place (bf16), alpha = exp(old max - new max) rescales
+// what was accumulated so far, and the grad-input launch adds p . W_block to the fp32 accumulator it first multiplied by
+// alpha.  At the end dH = ((acc / sum) - W[label]) * row_scale.  One workgroup per row.
+__global__ __launch_bounds__(256) void ce_stream_block_kernel(bf16_t* slab, int64_t ld, int nb, int64_t v0, const int64_t* labels, float* run_max,
+                                                              float* run_sum, float* target, float* alpha) {
+    __shared__ float red[4];
+    const int64_t row = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint4* p = (uint4*)(slab + row * ld);
+    const int chunks = (nb + 63) / 64 * 8;  // the contraction of the grad-input launch runs to the next multiple of 64
+    float bm = -INFINITY;
+    for (int c8 = threadIdx.x; c8 < chunks; c8 += 256) {
+        const uint4 v = p[c8];
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+            if (c8 * 8 + e < nb) bm = fmaxf(bm, bf16_to_f32((bf16_t)((e & 1) ? w[e >> 1] >> 16 : w[e >> 1] & 0xFFFFu)));
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) bm = fmaxf(bm, __shfl_xor(bm, off, 64));
+    if (lane == 0) red[wave] = bm;
+    __syncthreads();
+    bm = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    const float m_old = run_max[row];
+    const float m_new = fmaxf(m_old, bm);
+    const int64_t label = labels[row];
+    if (threadIdx.x == 0 && label >= v0 && label < v0 + nb) target[row] = bf16_to_f32(slab[row * ld + (label - v0)]);
+    __syncthreads();  // the target logit is read before the row is overwritten
+    float sum = 0.f;
+    for (int c8 = threadIdx.x; c8 < chunks; c8 += 256) {
+        const uint4 v = p[c8];
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            float g[2];
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const float logit = bf16_to_f32((bf16_t)(h ? w[e] >> 16 : w[e] & 0xFFFFu));
+                g[h] = c8 * 8 + 2 * e + h < nb ? __expf(logit - m_new) : 0.0f;
+            }
+            o[e] = pack_bf16(g[0], g[1]);
+            // the sum runs over the rounded values the accumulator receives, so that numerator and denominator agree
+            sum += bf16_to_f32((bf16_t)(o[e] & 0xFFFFu)) + bf16_to_f32((bf16_t)(o[e] >> 16));
+        }
+        p[c8] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) sum += __shfl_xor(sum, off, 64);
+    if (lane == 0) red[wave] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const float a = m_old == -INFINITY ? 0.f : __expf(m_old - m_new);
+        alpha[row] = a;
+        run_sum[row] = run_sum[row] * a + ((red[0] + red[1]) + (red[2] + red[3]));
+        run_max[row] = m_new;
+    }
+}
+
+// Packed rows of the labels (row 0 for ignored or out-of-range labels: their gradient is zero or undefined anyway).
+__global__ __launch_bounds__(256) void gather_label_rows_kernel(const uint8_t* packed, int64_t row_bytes, const int64_t* labels, int64_t vocab, uint8_t* out) {
+    const int64_t row = blockIdx.x;
+    const int64_t label = labels[row];
+    const uint16_t* src = (const uint16_t*)(packed + (label >= 0 && label < vocab ? label : 0) * row_bytes);
+    uint16_t* dst = (uint16_t*)(out + row * row_bytes);
+    for (int64_t i = threadIdx.x; i < row_bytes / 2; i += 256) dst[i] = src[i];
+}
+
+// lse, loss and dH = ((acc / sum) - W[label]) * row_scale, rounded to bf16.  One workgroup per row.
+__global__ __launch_bounds__(256) void ce_stream_finish_kernel(const float* acc, const bf16_t* w_label, int64_t hidden, const int64_t* labels, int64_t vocab,
+                                                               const float* run_max, const float* run_sum, const float* target, const float* row_scale,
+                                                               float* lse_out, float* loss_out, bf16_t* grad_hidden) {
+    const int64_t row = blockIdx.x;
+    const float rs = row_scale[row], inv = 1.0f / run_sum[row];
+    const int64_t label = labels[row];
+    const bool has_target = label >= 0 && label < vocab;
+    if (threadIdx.x == 0) {
+        const float lse = run_max[row] + __logf(run_sum[row]);
+        lse_out[row] = lse;
+        loss_out[row] = rs != 0.f ? (lse - (has_target ? target[row] : 0.f)) * rs : 0.f;
+    }
+    for (int64_t c = threadIdx.x; c < hidden; c += 256) {
+        const float wl = has_target ? bf16_to_f32(w_label[row * hidden + c]) : 0.f;
+        grad_hidden[row * hidden + c] = to_bf16((acc[row * hidden + c] * inv - wl) * rs);
+    }
+}
+
 static int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
 
 static int64_t padded_vocab(int64_t vocab) { return (vocab + 63) / 64 * 64; }
@@ -167,10 +257,8 @@ static bool keeps_logits(int64_t rows, int64_t chunk) { return chunk >= rows || 
 
 int64_t lmhead_ce_workspace_bytes(int64_t rows, int64_t vocab, int64_t hidden, int64_t chunk) {
     if (keeps_logits(rows, chunk)) return align256(rows * 4) * 2 + align256(std::min(rows, chunk) * padded_vocab(vocab) * 2) + 1024;
-    const int64_t rc = chunk < rows ? chunk : rows;
-    const int64_t gr = std::min(rows, std::max(chunk, kGradRows));
-    const int64_t nparts = (vocab + kBN - 1) / kBN * 2;
-    return align256(rows * 4) * 3 + align256(rc * nparts * 8) + align256(gr * kVocabBlock * 2) + align256(gr * hidden * 4) + 1024;
+    const int64_t gr = std::min(rows, kGradRows);
+    return align256(rows * 4) * 6 + align256(gr * kVocabBlock * 2) + align256(gr * hidden * 4) + align256(gr * hidden * 2) * 2 + 1024;
 }
 
 // The kept-logits path: row blocks of one chunk each.
@@ -219,53 +307,55 @@ int lmhead_ce(int qt, const void* hidden, const void* packed, const int64_t* lab
     if (keeps_logits(rows, chunk))
         return lmhead_ce_kept_logits(qt, hidden, packed, labels, rows, vocab, hidden_dim, chunk, ignore_index, reduction_mean, loss_1d, grad_hidden,
                                      lse_out, n_valid_out, ws, s);
-    const int64_t rc_max = chunk < rows ? chunk : rows;
-    const int64_t gr_max = std::min(rows, std::max(chunk, kGradRows));
-    const int nparts = (int)((vocab + kBN - 1) / kBN) * 2;
+    // One sweep over the vocabulary per block of up to kGradRows rows; nothing wider than kVocabBlock columns is ever held.
+    const int64_t gr_max = std::min(rows, kGradRows);
     char* w = (char*)ws;
     float* row_scale = (float*)w; w += align256(rows * 4);
     float* lse = lse_out ? lse_out : (float*)w; w += align256(rows * 4);
     float* target = (float*)w; w += align256(rows * 4);
-    float2* partials = (float2*)w; w += align256(rc_max * nparts * 8);
-    bf16_t* dlogits = (bf16_t*)w; w += align256(gr_max * kVocabBlock * 2);
-    float* dh32 = (float*)w;
+    float* run_max = (float*)w; w += align256(rows * 4);
+    float* run_sum = (float*)w; w += align256(rows * 4);
+    float* alpha = (float*)w; w += align256(rows * 4);
+    bf16_t* slab = (bf16_t*)w; w += align256(gr_max * kVocabBlock * 2);
+    float* dh32 = (float*)w; w += align256(gr_max * hidden_dim * 4);
+    uint8_t* label_rows = (uint8_t*)w; w += align256(gr_max * hidden_dim * 2);  // packed rows are smaller than bf16 rows
+    bf16_t* w_label = (bf16_t*)w;
 
     hipLaunchKernelGGL(ce_row_scale_kernel, dim3(1), dim3(1024), 0, s, labels, rows, ignore_index, reduction_mean, row_scale, n_valid_out);
     const int64_t row_bytes = packed_row_bytes(qt, hidden_dim);
-    for (int64_t r0 = 0; r0 < rows; r0 += chunk) {
-        const int rc = (int)((rows - r0) < chunk ? (rows - r0) : chunk);
-        const bf16_t* hid = (const bf16_t*)hidden + r0 * hidden_dim;
-        MmqParams p;
-        if (int rcode = init_params(p, qt, kModeNT, rc, (int)vocab, (int)hidden_dim, 1)) return rcode;
-        p.a[0] = hid, p.lda = hidden_dim;
-        p.w[0] = (const uint8_t*)packed;
-        p.labels = labels + r0, p.ce_partials = partials, p.ce_partials_ld = nparts, p.ce_target_logit = target + r0;
-        p.ignore_index = ignore_index;
-        if (int rcode = launch_mmq(qt, kModeNT, kEpiCeStats, p, s)) return rcode;
-        hipLaunchKernelGGL(ce_finalize_kernel, dim3((rc + 3) / 4), dim3(256), 0, s, partials, nparts, nparts, target + r0, row_scale + r0, rc, lse + r0, loss_1d + r0);
-    }
-    // gradient pass: the log-sum-exp of every row is known; row blocks of up to gr_max rows
+    if (row_bytes <= 0 || row_bytes > hidden_dim * 2 || (row_bytes & 1)) return set_error(GGQ_ERR_QTYPE, "lmhead_ce: unsupported packed row size");
+    hipLaunchKernelGGL(fill_f32_kernel, dim3(grid1d(rows)), dim3(256), 0, s, run_max, rows, -INFINITY);
+    hipLaunchKernelGGL(fill_f32_kernel, dim3(grid1d(rows)), dim3(256), 0, s, run_sum, rows, 0.f);
+    hipLaunchKernelGGL(fill_f32_kernel, dim3(grid1d(rows)), dim3(256), 0, s, target, rows, 0.f);
     for (int64_t r0 = 0; r0 < rows; r0 += gr_max) {
         const int rc = (int)std::min(rows - r0, gr_max);
         const bf16_t* hid = (const bf16_t*)hidden + r0 * hidden_dim;
         hipLaunchKernelGGL(fill_f32_kernel, dim3(grid1d((int64_t)rc * hidden_dim)), dim3(256), 0, s, dh32, (int64_t)rc * hidden_dim, 0.f);
         for (int64_t v0 = 0; v0 < vocab; v0 += kVocabBlock) {
             const int nb = (int)((vocab - v0) < kVocabBlock ? (vocab - v0) : kVocabBlock);
+            // (1) the block's logits
             MmqParams g;
             if (int rcode = init_params(g, qt, kModeNT, rc, nb, (int)hidden_dim, 1)) return rcode;
             g.a[0] = hid, g.lda = hidden_dim;
             g.w[0] = (const uint8_t*)packed + v0 * row_bytes;
-            g.c[0] = dlogits, g.ldc = kVocabBlock;
-            g.labels = labels + r0, g.lse = lse + r0, g.row_scale = row_scale + r0, g.ce_col_offset = (int)v0;
-            if (int rcode = launch_mmq(qt, kModeNT, kEpiCeGrad, g, s)) return rcode;
+            g.c[0] = slab, g.ldc = kVocabBlock;
+            if (int rcode = launch_mmq(qt, kModeNT, kEpiStore, g, s)) return rcode;
+            // (2) running statistics; the slab becomes exp(logit - running max)
+            hipLaunchKernelGGL(ce_stream_block_kernel, dim3((unsigned)rc), dim3(256), 0, s, slab, kVocabBlock, nb, v0, labels + r0, run_max + r0, run_sum + r0,
+                               target + r0, alpha + r0);
+            // (3) acc = acc * alpha + p . W_block
             MmqParams b;
             if (int rcode = init_params(b, qt, kModeNN, rc, nb, (int)hidden_dim, 1)) return rcode;
-            b.a[0] = dlogits, b.lda = kVocabBlock;
+            b.a[0] = slab, b.lda = kVocabBlock, b.a_zero_padded = 1;
             b.w[0] = (const uint8_t*)packed + v0 * row_bytes;
             b.c[0] = dh32, b.ldc = hidden_dim;
+            b.row_scale = alpha + r0;
             if (int rcode = launch_mmq(qt, kModeNN, kEpiAccumF32, b, s)) return rcode;
         }
-        hipLaunchKernelGGL(f32_to_bf16_kernel, dim3(grid1d((int64_t)rc * hidden_dim)), dim3(256), 0, s, dh32, (bf16_t*)grad_hidden + r0 * hidden_dim, (int64_t)rc * hidden_dim);
+        hipLaunchKernelGGL(gather_label_rows_kernel, dim3((unsigned)rc), dim3(256), 0, s, (const uint8_t*)packed, row_bytes, labels + r0, vocab, label_rows);
+        if (int rcode = dequantize(qt, label_rows, rc, hidden_dim, w_label, 0, s)) return rcode;
+        hipLaunchKernelGGL(ce_stream_finish_kernel, dim3((unsigned)rc), dim3(256), 0, s, dh32, w_label, hidden_dim, labels + r0, vocab, run_max + r0, run_sum + r0,
+                           target + r0, row_scale + r0, lse + r0, loss_1d + r0, (bf16_t*)grad_hidden + r0 * hidden_dim);
     }
     return check_launch("lmhead_ce");
 }

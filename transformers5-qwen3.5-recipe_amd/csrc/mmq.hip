@@ -140,7 +140,7 @@ static int launch_one(const MmqParams& p, hipStream_t s) {
         (void)hipEventRecord(t->start, s);
     }
     constexpr int kSmemBytes = Tile<SH>::kTileLdsBytes + (QT == kIQ2_XXS ? Fmt<kIQ2_XXS>::kTableWords * 4 : 0) +
-                               (EPI == kEpiCeStats || EPI == kEpiCeGrad ? Tile<SH>::kTM * 16 : 0);
+                               (EPI != kEpiStore ? Tile<SH>::kTM * 16 : 0);
     static bool attr_set = false;  // per instantiation; the attribute is a property of the function
     if (!attr_set) {
         hipError_t e;

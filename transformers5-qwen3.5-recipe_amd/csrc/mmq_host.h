@@ -67,7 +67,7 @@ constexpr int kThreads = 1024;  // waves 0..7 run the MFMAs, waves 8..15 load an
 enum : int { kModeNT = 0, kModeNN = 1 };
 enum : int {
     kEpiStore = 0,     // C (bf16) = acc
-    kEpiAccumF32 = 1,  // C32 (fp32) += acc
+    kEpiAccumF32 = 1,  // C32 (fp32) = C32 * row_scale[m] + acc  (row_scale null: += acc)
     kEpiCeStats = 2,   // per-row partial (max, sum exp) over the tile's columns + target logit
     kEpiCeGrad = 3     // C (bf16) = (exp(acc - lse[m]) - [col == label[m]]) * row_scale[m]
 };

@@ -843,6 +843,7 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
                     const float4 meta = c.row_meta[r_lane + dr];
                     lse = meta.x, rs = meta.y, label = (int64_t)__float_as_int(meta.z);
                 }
+                if (EPI == kEpiAccumF32) rs = p.row_scale ? c.row_meta[r_lane + dr].y : 1.0f;
 #pragma unroll
                 for (int cb = 0; cb < kColBlocks; cb++) {
                     if (!col_ok[cb]) continue;
@@ -850,7 +851,7 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
                     if (EPI == kEpiStore) {
                         ((bf16_t*)cbase)[elem + cb * 32] = to_bf16(v);
                     } else if (EPI == kEpiAccumF32) {
-                        ((float*)cbase)[elem + cb * 32] += v;
+                        ((float*)cbase)[elem + cb * 32] = fmaf(((float*)cbase)[elem + cb * 32], rs, v);
                     } else {
                         const float logit = bf16_to_f32(to_bf16(v));  // the path's logits are bf16 values
                         float g = __expf(logit - lse);
@@ -1007,6 +1008,9 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
                     *(uint4*)&c.bs[j * kNnPitch + nn_chunk(j, ch) * 8] = v;
                 }
             }
+        }
+        if (EPI == kEpiAccumF32 && p.row_scale) {  // the factor that rescales the accumulator row before the addition
+            for (int r = tid; r < kTM; r += kThreadsWG) row_meta[r] = make_float4(0.f, p.row_scale[c.row_begin + min(r, c.rows_valid - 1)], 0.f, 0.f);
         }
         if (EPI == kEpiCeStats || EPI == kEpiCeGrad) {
             for (int r = tid; r < kTM; r += kThreadsWG) {
