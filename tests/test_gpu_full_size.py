@@ -86,7 +86,7 @@ def test_sampled_expert_groups_at_full_size_match_an_fp32_matmul(pkg, dev):
 
 @pytest.mark.parametrize("chunk", [1024, 4096])
 def test_lm_head_loss_at_full_size_matches_a_chunked_torch_reference(pkg, dev, chunk):
-    # Qwen's head: 151936 x 2048 in Q6_K, 4096 rows; chunks of 1024 rows (no logits kept, the gradient recomputes them) and of
+    # Qwen's head: 151936 x 2048 in Q6_K, 4096 rows; chunks of 1024 rows (no logits kept: one sweep over the vocabulary with a running softmax) and of
     # 4096 rows (the chunk's logits kept and rewritten as their gradient)
     vocab, hidden, rows = 151936, 2048, 4096
     g = torch.Generator(device=dev).manual_seed(31)

@@ -5,14 +5,12 @@
 //    kernel writes its bf16 logits; one kernel, a workgroup per row, reads a row for its log-sum-exp, target logit and loss
 //    and rewrites it as d(loss)/d(logits); one grad-input launch contracts the rows with the packed weights over the whole
 //    vocabulary.  Two vocabulary-sized matmuls.
-//  * smaller chunks: no logits are kept beyond a [rows, 8192] slab.  Pass 1, per chunk: the tile kernel runs over the whole
-//    vocabulary with an epilogue that reduces every 128-column slab of a logits tile to (max, sum exp) per row and records
-//    the target logit; a small kernel merges the slabs into log-sum-exp and the per-row loss.  Pass 2, per block of up to
-//    kGradRows rows, walks the vocabulary in blocks of kVocabBlock columns: the tile kernel recomputes that block's logits
-//    and its epilogue turns them into d(loss)/d(logits) (bf16, [rows of the block, kVocabBlock] only); the grad-input form
-//    of the tile kernel contracts the block with the same packed rows into an fp32 accumulator.  Three vocabulary-sized
-//    matmuls are the price of not holding the logits; a 1024-row chunk of kept logits would leave the [rows, hidden]
-//    grad-input output with 64 tiles for 256 compute units.
+//  * smaller chunks: no logits are kept beyond a [rows, 8192] slab.  Per block of up to kGradRows rows the vocabulary is
+//    swept once in blocks of kVocabBlock columns with a running (max, sum exp) per row: the tile kernel writes the block's
+//    logits into the slab; a row kernel updates the running statistics and rewrites the slab as exp(logit - running max);
+//    the grad-input form of the tile kernel adds slab . W_block to an fp32 accumulator that its epilogue first rescales
+//    by exp(old max - new max).  At the end dH = (accumulator / sum - W[label]) * row_scale.  Two vocabulary-sized
+//    matmuls here as well.
 #include <algorithm>
 
 #include "common.h"
@@ -22,9 +20,9 @@
 namespace ggq {
 
 constexpr int kVocabBlock = 8192;
-// The gradient pass takes up to this many rows at a time, whatever the caller's chunk (which bounds the statistics pass
-// and stands for the reference's [chunk, vocab] logits): 4096 rows fill the chip with tiles of the [rows, hidden]
-// grad-input output (a 1024-row chunk makes 64 tiles for 256 compute units) and cost a 64 MiB gradient slab.
+// The sweep takes up to this many rows at a time, whatever the caller's chunk (which stands for the reference's
+// [chunk, vocab] logits): 4096 rows fill the chip with tiles of the [rows, hidden] grad-input output (a 1024-row chunk
+// makes 64 tiles for 256 compute units) and cost a 64 MiB slab.
 constexpr int64_t kGradRows = 4096;
 // A chunk of at least this many rows is worth keeping the logits of: its grad-input launch fills the chip.
 constexpr int64_t kKeptLogitsRows = 4096;
