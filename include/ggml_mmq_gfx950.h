@@ -141,6 +141,18 @@ int ggq_route_plan(const void* topk_ids, int ids_are_int64, int64_t tokens, int 
                    int64_t* permutation, int64_t* inverse, int32_t* counts, int32_t* end_offsets, int64_t* active_ids,
                    int32_t* active_end_offsets, int32_t* status, void* ws, int64_t ws_bytes, void* stream);
 
+/* ggq_route_plan without a workspace and without any allocation.  No counterpart in the reference: it is for callers
+ * that cannot allocate device memory around the call (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  The sort's scratch (per-route ranks, per-chunk histograms) lives in a 2.1 MB device array
+ * inside the library, one copy per GPU, held until the process ends; its address is looked up on the first call on
+ * each device.  Limits: tokens * top_k <= 262144 routes and num_experts <= 256, otherwise the shape error (-2) is
+ * returned and nothing is launched.  All calls on one GPU share that GPU's array: calls that overlap on one GPU (two
+ * streams, two threads) race; calls on one stream are ordered and need no clearing in between.  Outputs and results
+ * are those of ggq_route_plan, bit for bit. */
+int ggq_route_plan_static(const void* topk_ids, int ids_are_int64, int64_t tokens, int top_k, int num_experts, int64_t* sorted_ids,
+                          int64_t* permutation, int64_t* inverse, int32_t* counts, int32_t* end_offsets, int64_t* active_ids,
+                          int32_t* active_end_offsets, int32_t* status, void* stream);
+
 /* _route_gather_forward_kernel (fast_moe_routing.py:101-123): selected[s] = hidden[permutation[s] / k]. */
 int ggq_route_gather_forward(const void* hidden, const int64_t* permutation, void* selected, int64_t tokens, int top_k, int hidden_dim, void* stream);
 

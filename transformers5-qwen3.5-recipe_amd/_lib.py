@@ -40,6 +40,7 @@ SIGNATURES: dict[str, tuple] = {
     "ggq_grouped_lora_mmq_backward_indexed": (_I, [_P, _P, _P, _P, _P, _P, _L, _L, _I, _L, _L, _L, _P, _L, _P, _I, _P, _P, _P, _I, _F, _P, _P, _P, _P, _L, _P]),
     "ggq_route_plan_workspace_bytes": (_L, [_L, _I, _I]),
     "ggq_route_plan": (_I, [_P, _I, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _P]),
+    "ggq_route_plan_static": (_I, [_P, _I, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
     "ggq_route_gather_forward": (_I, [_P, _P, _P, _L, _I, _I, _P]),
     "ggq_route_gather_backward": (_I, [_P, _P, _P, _L, _I, _I, _P]),
     "ggq_route_combine_forward": (_I, [_P, _P, _I, _P, _P, _L, _I, _I, _P]),

@@ -430,6 +430,15 @@ int ggq_route_plan(const void* topk_ids, int ids_are_int64, int64_t tokens, int 
                       active_ids, active_end_offsets, status, ws, ws_bytes, as_stream(stream));
 }
 
+int ggq_route_plan_static(const void* topk_ids, int ids_are_int64, int64_t tokens, int top_k, int num_experts, int64_t* sorted_ids,
+                          int64_t* permutation, int64_t* inverse, int32_t* counts, int32_t* end_offsets, int64_t* active_ids,
+                          int32_t* active_end_offsets, int32_t* status, void* stream) {
+    if (!topk_ids || !sorted_ids || !permutation || !inverse || !counts || !end_offsets || !active_ids || !active_end_offsets || !status)
+        return set_error(GGQ_ERR_NULL, "route_plan_static: null pointer");
+    return route_plan_static(topk_ids, ids_are_int64, tokens, top_k, num_experts, sorted_ids, permutation, inverse, counts, end_offsets,
+                             active_ids, active_end_offsets, status, as_stream(stream));
+}
+
 int ggq_route_gather_forward(const void* hidden, const int64_t* permutation, void* selected, int64_t tokens, int top_k, int hidden_dim, void* stream) {
     if (!hidden || !permutation || !selected) return set_error(GGQ_ERR_NULL, "route_gather_forward: null pointer");
     return route_gather_fwd(hidden, permutation, selected, tokens, top_k, hidden_dim, as_stream(stream));

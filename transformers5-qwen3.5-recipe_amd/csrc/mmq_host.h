@@ -151,6 +151,9 @@ int64_t route_plan_workspace_bytes(int64_t routes, int num_experts);
 int route_plan(const void* topk_ids, int ids_are_int64, int64_t tokens, int top_k, int num_experts,
                int64_t* sorted_ids, int64_t* permutation, int64_t* inverse, int* counts, int* end_offsets,
                int64_t* active_ids, int* active_end, int* num_active, void* ws, int64_t ws_bytes, hipStream_t s);
+int route_plan_static(const void* topk_ids, int ids_are_int64, int64_t tokens, int top_k, int num_experts,
+                      int64_t* sorted_ids, int64_t* permutation, int64_t* inverse, int* counts, int* end_offsets,
+                      int64_t* active_ids, int* active_end, int* num_active, hipStream_t s);  // no workspace: a built-in scratch array
 int route_gather_fwd(const void* hidden, const int64_t* permutation, void* selected, int64_t tokens, int top_k, int hidden_dim, hipStream_t s);
 int route_gather_bwd(const void* grad_selected, const int64_t* inverse, void* grad_hidden, int64_t tokens, int top_k, int hidden_dim, hipStream_t s);
 int route_combine_fwd(const void* expert_out, const void* weights, int w_is_bf16, const int64_t* inverse, void* out, int64_t tokens, int top_k, int hidden_dim, hipStream_t s);

@@ -3,6 +3,8 @@
 // everything is deterministic (no atomics) so a recomputed forward reproduces the same bits.
 //
 // Route r = token * k + rank.  permutation[s] = route at sorted position s; inverse[r] = s.
+#include <mutex>
+
 #include "common.h"
 #include "launch.h"
 #include "mmq_host.h"
@@ -179,6 +181,51 @@ int route_plan(const void* topk_ids, int ids_are_int64, int64_t tokens, int top_
             hipLaunchKernelGGL(route_scatter_kernel<int32_t>, dim3(chunks), dim3(kChunk), 0, s, (const int32_t*)topk_ids, routes, num_experts, local_rank, chunk_hist, expert_base, sorted_ids, permutation, inverse);
     }
     return check_launch("route_plan");
+}
+
+// ------------------------------------------------------------------------------------------------
+// The same plan without a caller workspace: the sort's scratch (per-route ranks, per-chunk histograms, expert
+// bases, per-chunk flags) lives in a file-scope device array.  Every GPU the library runs on holds its own copy
+// of the array at its own address until the process ends; the address is looked up once per device.
+constexpr int64_t kStaticPlanMaxRoutes = 1 << 18;  // 262144 routes (e.g. 32768 tokens x top-8)
+constexpr int kStaticPlanMaxExperts = 256;
+constexpr int64_t kStaticPlanInts =
+    kStaticPlanMaxRoutes + (kStaticPlanMaxRoutes / kChunk) * kStaticPlanMaxExperts + kStaticPlanMaxExperts + kStaticPlanMaxRoutes / kChunk + 4;
+static __device__ __align__(256) int scratch[kStaticPlanInts];  // 2.1 MB
+
+constexpr int kMaxDevices = 64;
+static int* scratch_ptr[kMaxDevices];  // device address of `scratch` on each device (null: not looked up yet)
+static std::mutex scratch_lock;
+
+// Device address of this device's copy of `scratch`.  The array's name is only a host-side handle: kernels and
+// copies take the address returned here.
+static int static_scratch(int** out) {
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return set_error(GGQ_ERR_RUNTIME, "route_plan_static: no current device");
+    std::lock_guard<std::mutex> guard(scratch_lock);
+    if (!scratch_ptr[device]) {
+        int* p = nullptr;
+        const hipError_t err = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || !p) return set_error(GGQ_ERR_RUNTIME, "route_plan_static: hipGetSymbolAddress failed: %s", hipGetErrorString(err));
+        scratch_ptr[device] = p;
+    }
+    *out = scratch_ptr[device];
+    return GGQ_OK;
+}
+
+int route_plan_static(const void* topk_ids, int ids_are_int64, int64_t tokens, int top_k, int num_experts,
+                      int64_t* sorted_ids, int64_t* permutation, int64_t* inverse, int* counts, int* end_offsets,
+                      int64_t* active_ids, int* active_end, int* num_active, hipStream_t s) {
+    if (tokens < 0 || top_k <= 0 || num_experts <= 0) return set_error(GGQ_ERR_SHAPE, "route_plan_static: bad shape");
+    if (tokens > kStaticPlanMaxRoutes || tokens * top_k > kStaticPlanMaxRoutes || num_experts > kStaticPlanMaxExperts)
+        return set_error(GGQ_ERR_SHAPE, "route_plan_static: at most %lld routes and %d experts fit the built-in scratch array, got %lld routes and %d experts (use route_plan with a workspace)",
+                         (long long)kStaticPlanMaxRoutes, kStaticPlanMaxExperts, (long long)(tokens * top_k), num_experts);
+    int* ws = nullptr;
+    if (int rc = static_scratch(&ws)) return rc;
+    // nothing in the scratch has to start at zero: every word the scan and scatter passes read is written by the
+    // rank pass of the same call
+    return route_plan(topk_ids, ids_are_int64, tokens, top_k, num_experts, sorted_ids, permutation, inverse, counts, end_offsets, active_ids,
+                      active_end, num_active, ws, kStaticPlanInts * (int64_t)sizeof(int), s);
 }
 
 // ------------------------------------------------------------------------------------------------
