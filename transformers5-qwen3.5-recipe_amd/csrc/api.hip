@@ -305,9 +305,8 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
     // the direct kernel moves the cotangents with aligned 16-byte accesses and takes whole groups of four 64-row steps
     // (with a LoRA term its once-per-tile operand fetch makes it no faster than the tile kernel at the shapes measured:
     // GGQ_GROUPED_SHAPE=3 still selects it)
-    const char* forced_shape = getenv("GGQ_GROUPED_SHAPE");
     const bool direct_ok = aligned16(dy1) && (!dy2 || aligned16(dy2)) && n % 64 == 0 && (nseg * (n / 64)) % 4 == 0 && n < (1 << 22) &&
-                           (!lora_a || (forced_shape && atoi(forced_shape) == kShapeDirect));
+                           (!lora_a || aligned16(lora_a)) && k % 8 == 0;
     if (int rc = init_params(p, qt, kModeNN, (int)rows, (int)n, (int)k, nseg, pick_shape(qt, rows, groups, direct_ok))) return rc;
     p.a[0] = (const bf16_t*)dy1, p.a[1] = (const bf16_t*)dy2, p.lda = n;
     p.w[0] = (const uint8_t*)packed1, p.w[1] = (const uint8_t*)packed2;

@@ -2,9 +2,12 @@
 #include "mmq_tile.h"
 #include "mmq_direct.h"
 #include "mmq_direct_nn.h"
+#include "mmq_direct8.h"
+#include "mmq_direct8_nn.h"
 #include "launch.h"
 
 #include <stdarg.h>
+#include <stdlib.h>
 #include <stdio.h>
 
 namespace ggq {
@@ -174,15 +177,20 @@ static int launch_direct(const MmqParams& p, hipStream_t s) {
         g_timed_count++;
         (void)hipEventRecord(t->start, s);
     }
-    constexpr int kSmemBytes = MODE == kModeNT ? Direct::kLdsBytes : DirectNN::kLdsBytes;
-    const void* fn = MODE == kModeNT ? (const void*)mmq_direct_q4k_kernel : (const void*)mmq_direct_nn_q4k_kernel;
+    static const bool eight = !(getenv("GGQ_DIRECT8") && atoi(getenv("GGQ_DIRECT8")) == 0);
+    const bool use8 = eight;
+    const int kSmemBytes = use8 ? (MODE == kModeNT ? Direct8::kLdsBytes : Direct8NN::kLdsBytes) : MODE == kModeNT ? Direct::kLdsBytes : DirectNN::kLdsBytes;
+    const void* fn = use8 ? (MODE == kModeNT ? (const void*)mmq_direct8_q4k_kernel : (const void*)mmq_direct8_nn_q4k_kernel)
+                          : MODE == kModeNT ? (const void*)mmq_direct_q4k_kernel : (const void*)mmq_direct_nn_q4k_kernel;
     static bool attr_set = false;  // per instantiation
     if (!attr_set) {
         if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess)
             return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", kSmemBytes);
         attr_set = true;
     }
-    if (MODE == kModeNT) hipLaunchKernelGGL(mmq_direct_q4k_kernel, dim3((unsigned)grid), dim3(Direct::kThreadsWG), kSmemBytes, s, p);
+    if (use8 && MODE == kModeNN) hipLaunchKernelGGL(mmq_direct8_nn_q4k_kernel, dim3((unsigned)grid), dim3(Direct8NN::kThreadsWG), kSmemBytes, s, p);
+    else if (use8) hipLaunchKernelGGL(mmq_direct8_q4k_kernel, dim3((unsigned)grid), dim3(Direct8::kThreadsWG), kSmemBytes, s, p);
+    else if (MODE == kModeNT) hipLaunchKernelGGL(mmq_direct_q4k_kernel, dim3((unsigned)grid), dim3(Direct::kThreadsWG), kSmemBytes, s, p);
     else hipLaunchKernelGGL(mmq_direct_nn_q4k_kernel, dim3((unsigned)grid), dim3(DirectNN::kThreadsWG), kSmemBytes, s, p);
     if (t) (void)hipEventRecord(t->stop, s);
     return check_launch(MODE == kModeNT ? "mmq_direct_q4k_kernel" : "mmq_direct_nn_q4k_kernel");
