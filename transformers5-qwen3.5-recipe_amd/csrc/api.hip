@@ -88,14 +88,15 @@ static int pick_shape(int qt, int64_t rows, int64_t groups, bool direct_ok) {
     return forced == kShapeHalf ? kShapeHalf : kShapeWide;
 }
 
-// Direct shape: a workgroup walks up to four column tiles of its row tile, fewer while that leaves compute units
-// without work.  GGQ_DIRECT_TILES_PER_WG is a tuning aid, read per call.
-static int direct_tiles_per_wg(int64_t rows, int64_t groups, int col_tiles) {
+// Direct shape: a workgroup walks a run of column tiles of its row tile as one stream of steps.  Short tiles (few
+// contraction steps) gain from runs of four (the next tile's first loads are in flight while a tile finishes); with
+// long tiles one tile per workgroup balances the compute units better (the tiles with the most rows are dispatched
+// first).  Fewer per run while that leaves compute units without work.
+static int direct_tiles_per_wg(int64_t rows, int64_t groups, int col_tiles, int steps_per_tile) {
     const int64_t row_tiles = groups > 0 ? std::max<int64_t>(groups, rows / kDirectBM) : (rows + kDirectBM - 1) / kDirectBM;
-    int per_wg = 4;
+    int per_wg = steps_per_tile >= 32 ? 1 : 4;
     while (per_wg > 1 && row_tiles * ((col_tiles + per_wg - 1) / per_wg) < 256) per_wg >>= 1;
-    const char* e = getenv("GGQ_DIRECT_TILES_PER_WG");
-    return e && atoi(e) > 0 ? atoi(e) : per_wg;
+    return per_wg;
 }
 
 // A dense layer's factor gradients deal their rows to at most this many workgroups per column block (fp32 partial sums
@@ -208,7 +209,7 @@ static int grouped_forward(const char* what, const void* x, RowIndex x_index, co
     p.a[0] = (const bf16_t*)x, p.lda = k, p.a_rows = x_index;
     p.w[0] = (const uint8_t*)packed1, p.w[1] = (const uint8_t*)packed2;
     p.c[0] = y1, p.c[1] = y2, p.ldc = n;
-    if (p.shape == kShapeDirect) p.col_tiles_per_wg = direct_tiles_per_wg(rows, groups, nseg * p.col_tiles_per_seg);
+    if (p.shape == kShapeDirect) p.col_tiles_per_wg = direct_tiles_per_wg(rows, groups, nseg * p.col_tiles_per_seg, p.steps_per_seg);
 
     const TileDesc* tiles64 = nullptr;
     const int* num_tiles64 = nullptr;
@@ -224,13 +225,16 @@ static int grouped_forward(const char* what, const void* x, RowIndex x_index, co
         const int max128 = wide ? (int)groups : (int)(rows / bm_main + groups);
         max_tall = wide ? (int)std::min<int64_t>(rows / kBM + groups, rows / (kWideBM + 1) + rows / kBM + 1) : 0;
         max_tiles64 = (int)(rows / 64 + groups);
+        const bool direct = p.shape == kShapeDirect;  // its workgroups take the tiles with the most rows first
         TileDesc* t128 = (TileDesc*)bump.take((int64_t)max128 * sizeof(TileDesc));
+        TileDesc* t_sorted = direct ? (TileDesc*)bump.take((int64_t)max128 * sizeof(TileDesc)) : nullptr;
         t_tall = wide ? (TileDesc*)bump.take((int64_t)max_tall * sizeof(TileDesc)) : nullptr;
         TileDesc* t64 = lora_a ? (TileDesc*)bump.take((int64_t)max_tiles64 * sizeof(TileDesc)) : nullptr;
         int* counts = (int*)bump.take(16);
-        if (!t128 || !counts || (lora_a && !t64) || (wide && !t_tall)) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
+        if (!t128 || !counts || (lora_a && !t64) || (wide && !t_tall) || (direct && !t_sorted)) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
         RowTileTables tb{};
-        tb.add(bm_main, 0, wide ? kWideBM : 0x7FFFFFFF, t128, counts);
+        tb.add(bm_main, 0, wide ? kWideBM : 0x7FFFFFFF, t128, counts, t_sorted);
+        if (direct) t128 = t_sorted;
         if (wide) tb.add(kBM, kWideBM, 0x7FFFFFFF, t_tall, counts + 2), n_tall = counts + 2;
         if (lora_a) tb.add(64, 0, 0x7FFFFFFF, t64, counts + 1);
         if (int rc = build_row_tile_tables(expert_ids, end_offsets, (int)groups, tb, nullptr, 0, s)) return rc;
@@ -311,7 +315,7 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
     p.a[0] = (const bf16_t*)dy1, p.a[1] = (const bf16_t*)dy2, p.lda = n;
     p.w[0] = (const uint8_t*)packed1, p.w[1] = (const uint8_t*)packed2;
     p.c[0] = dx, p.ldc = k;
-    if (p.shape == kShapeDirect) p.col_tiles_per_wg = direct_tiles_per_wg(rows, groups, p.col_tiles_per_seg);
+    if (p.shape == kShapeDirect) p.col_tiles_per_wg = direct_tiles_per_wg(rows, groups, p.col_tiles_per_seg, nseg * p.steps_per_seg);
 
     const TileDesc* tiles64 = nullptr;
     const int* num_tiles64 = nullptr;
@@ -326,14 +330,17 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
         const int max128 = wide ? (int)groups : (int)(rows / bm_main + groups);
         max_tall = wide ? (int)std::min<int64_t>(rows / kBM + groups, rows / (kWideBM + 1) + rows / kBM + 1) : 0;
         max_tiles64 = (int)(rows / 64 + groups);
+        const bool direct = p.shape == kShapeDirect;  // its workgroups take the tiles with the most rows first
         TileDesc* t128 = (TileDesc*)bump.take((int64_t)max128 * sizeof(TileDesc));
+        TileDesc* t_sorted = direct ? (TileDesc*)bump.take((int64_t)max128 * sizeof(TileDesc)) : nullptr;
         t_tall = wide ? (TileDesc*)bump.take((int64_t)max_tall * sizeof(TileDesc)) : nullptr;
         TileDesc* t64 = lora_a ? (TileDesc*)bump.take((int64_t)max_tiles64 * sizeof(TileDesc)) : nullptr;
         int* counts = (int*)bump.take(16);
         int* rg = lora_a ? (int*)bump.take(experts * 2 * 4) : nullptr;
-        if (!t128 || !counts || (lora_a && (!t64 || !rg)) || (wide && !t_tall)) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
+        if (!t128 || !counts || (lora_a && (!t64 || !rg)) || (wide && !t_tall) || (direct && !t_sorted)) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
         RowTileTables tb{};
-        tb.add(bm_main, 0, wide ? kWideBM : 0x7FFFFFFF, t128, counts);
+        tb.add(bm_main, 0, wide ? kWideBM : 0x7FFFFFFF, t128, counts, t_sorted);
+        if (direct) t128 = t_sorted;
         if (wide) tb.add(kBM, kWideBM, 0x7FFFFFFF, t_tall, counts + 2), n_tall = counts + 2;
         if (lora_a) tb.add(64, 0, 0x7FFFFFFF, t64, counts + 1);
         if (int rc = build_row_tile_tables(expert_ids, end_offsets, (int)groups, tb, rg, (int)experts, s)) return rc;

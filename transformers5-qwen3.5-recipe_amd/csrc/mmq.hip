@@ -79,6 +79,60 @@ __global__ __launch_bounds__(256) void build_row_tiles_kernel(const int64_t* exp
         __syncthreads();
     }
     if (tid == 0) *tb.num_tiles[t] = base;
+    TileDesc* by_size = tb.by_size[t];
+    if (!by_size) return;
+    // Stable bucket sort by the number of 32-row blocks, largest first: thread i takes the i-th contiguous share of the
+    // table; per-thread bucket counts are scanned over the threads, bucket after bucket.
+    __syncthreads();  // the table written above is visible to the whole workgroup
+    constexpr int kBuckets = 8;  // tiles of up to 256 rows
+    __shared__ int bucket_count[kBuckets][256];
+    __shared__ int bucket_base[kBuckets];
+    const int total = base;
+    const int share = (total + 255) / 256, i0 = min(total, tid * share), i1 = min(total, i0 + share);
+    int mine[kBuckets];
+#pragma unroll
+    for (int b = 0; b < kBuckets; b++) mine[b] = 0;
+    for (int i = i0; i < i1; i++) {
+        const int bucket = kBuckets - min(kBuckets, max(1, (tiles[i].row_end - tiles[i].row_begin + 31) >> 5));
+#pragma unroll
+        for (int b = 0; b < kBuckets; b++) mine[b] += bucket == b;
+    }
+#pragma unroll
+    for (int b = 0; b < kBuckets; b++) bucket_count[b][tid] = mine[b];
+    __syncthreads();
+    if (tid < kBuckets) {  // exclusive scan over the threads of one bucket (256 entries: serial is a few microseconds at most)
+        int run = 0;
+        for (int j = 0; j < 256; j++) {
+            const int v = bucket_count[tid][j];
+            bucket_count[tid][j] = run;
+            run += v;
+        }
+        bucket_base[tid] = run;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int run = 0;
+        for (int b = 0; b < kBuckets; b++) {
+            const int v = bucket_base[b];
+            bucket_base[b] = run;
+            run += v;
+        }
+    }
+    __syncthreads();
+    int at[kBuckets];
+#pragma unroll
+    for (int b = 0; b < kBuckets; b++) at[b] = bucket_base[b] + bucket_count[b][tid];
+    for (int i = i0; i < i1; i++) {
+        const TileDesc d = tiles[i];
+        const int bucket = kBuckets - min(kBuckets, max(1, (d.row_end - d.row_begin + 31) >> 5));
+        int pos = 0;
+#pragma unroll
+        for (int b = 0; b < kBuckets; b++) {
+            if (bucket == b) pos = at[b];
+            at[b] += bucket == b;
+        }
+        by_size[pos] = d;
+    }
 }
 
 int build_row_tile_tables(const int64_t* expert_ids, const int32_t* end_offsets, int groups, const RowTileTables& tb,
@@ -163,9 +217,10 @@ template <int MODE>
 static int launch_direct(const MmqParams& p, hipStream_t s) {
     const int col_tiles = (MODE == kModeNT ? p.nseg : 1) * p.col_tiles_per_seg;
     if (p.col_tiles_per_wg < 1) return set_error(GGQ_ERR_SHAPE, "mmq: column tiles per workgroup must be at least 1");
-    const int64_t total = (int64_t)p.max_row_tiles * ((col_tiles + p.col_tiles_per_wg - 1) / p.col_tiles_per_wg);
+    // row tiles are dealt round-robin over the eight XCDs; each XCD walks its row tiles' column-tile runs
+    const int64_t total = (int64_t)((p.max_row_tiles + 7) / 8) * ((col_tiles + p.col_tiles_per_wg - 1) / p.col_tiles_per_wg);
     if (total <= 0) return GGQ_OK;
-    const int64_t grid = (total + 7) / 8 * 8;
+    const int64_t grid = total * 8;
     if (grid > 0x7FFFFFF0) return set_error(GGQ_ERR_SHAPE, "mmq: too many tiles for one launch");
     if (MODE == kModeNN && ((p.n & 63) || ((p.nseg * p.steps_per_seg) & 3)))
         return set_error(GGQ_ERR_SHAPE, "mmq: the direct grad-input kernel needs whole groups of four 64-row steps");

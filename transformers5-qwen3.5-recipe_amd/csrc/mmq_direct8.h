@@ -332,12 +332,11 @@ struct Direct8 {
         const int col_tiles = p.nseg * p.col_tiles_per_seg;
         const int chunks = (col_tiles + p.col_tiles_per_wg - 1) / p.col_tiles_per_wg;
         const int row_tiles = p.tiles ? min(*p.num_tiles, p.max_row_tiles) : p.max_row_tiles;
-        const int units = row_tiles * chunks;
-        const int per_xcd = (units + 7) >> 3;
+        // Row tile rt runs on XCD rt % 8 (the table lists the tiles with the most rows first: every XCD gets its
+        // share of them, and takes its own in that order); the column-tile runs of a row tile follow one another there.
         const int slot = (int)(blockIdx.x >> 3);
-        const int unit = (int)(blockIdx.x & 7) * per_xcd + slot;
-        if (slot >= per_xcd || unit >= units) return;
-        const int row_tile = unit / chunks, chunk = unit - row_tile * chunks;
+        const int row_tile = (slot / chunks) * 8 + (int)(blockIdx.x & 7), chunk = slot % chunks;
+        if (row_tile >= row_tiles) return;
         RowCtx c;
         int row_end;
         if (p.tiles) {

@@ -211,17 +211,21 @@ struct Direct8NN {
         open_a();
         request_a(std::integral_constant<int, 0>{});
 
-        auto sub_step = [&](const bf16x8_t& b0, int next_stage_off, int next_i, auto&& piece, auto&& request) __attribute__((always_inline)) {
+        // One sub-step: the row blocks' MFMAs one by one, each followed by the read of its operand of the following
+        // sub-step (into the registers it has just released) and by whatever `slot` puts behind that MFMA.
+        auto sub_step = [&](const bf16x8_t& b0, int next_stage_off, int next_i, auto&& slot) __attribute__((always_inline)) {
             const uint8_t* src = a_row + next_stage_off + a_koff[next_i];
-#pragma unroll
-            for (int rb = 0; rb < LIVE; rb++) {
-                acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b0, ao[rb], acc[rb], 0, 0, 0);
-                if (rb == 0) request();
-                ao[rb] = *(const bf16x8_t*)(src + rb * 32 * kARowBytes);
-                if (0 * LIVE / 2 == rb) piece(std::integral_constant<int, 0>{});
-                if (1 * LIVE / 2 == rb) piece(std::integral_constant<int, 1>{});
-                __builtin_amdgcn_sched_barrier(0);
-            }
+            auto one = [&](auto rb_c) __attribute__((always_inline)) {
+                constexpr int RB = decltype(rb_c)::value;
+                if constexpr (RB < LIVE) {
+                    acc[RB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b0, ao[RB], acc[RB], 0, 0, 0);
+                    ao[RB] = *(const bf16x8_t*)(src + RB * 32 * kARowBytes);
+                    slot(rb_c);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            };
+            one(std::integral_constant<int, 0>{}), one(std::integral_constant<int, 1>{}), one(std::integral_constant<int, 2>{});
+            one(std::integral_constant<int, 3>{}), one(std::integral_constant<int, 4>{}), one(std::integral_constant<int, 5>{});
         };
         bool stores_behind = false;  // the tile before this one went out through the staged store path
         int relax = 0;               // steps of this tile whose wait still allows for the stores of the tile before
@@ -244,19 +248,33 @@ struct Direct8NN {
                     raw_fetch(w_rd);
                     const int a_rd_next = a_rd == (kStages - 1) * kStageBytes ? 0 : a_rd + kStageBytes;
                     __builtin_amdgcn_sched_barrier(0);
+                    // The next step's weight row of this lane is decoded in eight pieces (one quant word = four columns
+                    // each) spread evenly over the 3 LIVE MFMA slots of the first three sub-steps, so that the block is
+                    // complete before the phase ends; its transposing reads are spread over the last sub-step's slots and
+                    // have landed when the next step starts.
                     uint32_t o[4];
-                    auto piece_of = [&](auto q_c) __attribute__((always_inline)) {
-                        return [&, q_c](auto k_c) __attribute__((always_inline)) {
-                            constexpr int Q = decltype(q_c)::value, K = decltype(k_c)::value;
-                            const u32x4_t& src = Q < 2 ? rq0 : rq1;
-                            if (Q == 0 && K == 0) sub_block_scale(rh, wave, dl, nm);
-                            decode_word(src[2 * (Q & 1) + K], nib_mask, dl, nm, o + 2 * K);
-                            if (K == 1) *(uint4*)(d_my_row + Q * 16) = make_uint4(o[0], o[1], o[2], o[3]);
+                    auto decode_piece = [&](auto hp_c) __attribute__((always_inline)) {
+                        constexpr int HP = decltype(hp_c)::value, Q = HP >> 1, K = HP & 1;
+                        const u32x4_t& src = Q < 2 ? rq0 : rq1;
+                        if (HP == 0) sub_block_scale(rh, wave, dl, nm);
+                        decode_word(src[2 * (Q & 1) + K], nib_mask, dl, nm, o + 2 * K);
+                        if (K == 1) *(uint4*)(d_my_row + Q * 16) = make_uint4(o[0], o[1], o[2], o[3]);
+                    };
+                    auto decode_slots = [&](auto i_c) __attribute__((always_inline)) {  // sub-step I's share
+                        return [&, i_c](auto rb_c) __attribute__((always_inline)) {
+                            constexpr int T = decltype(i_c)::value * LIVE + decltype(rb_c)::value;
+                            auto maybe = [&](auto hp_c) __attribute__((always_inline)) {
+                                if constexpr (decltype(hp_c)::value * 3 * LIVE / 8 == T) decode_piece(hp_c);
+                            };
+                            maybe(std::integral_constant<int, 0>{}), maybe(std::integral_constant<int, 1>{}), maybe(std::integral_constant<int, 2>{}), maybe(std::integral_constant<int, 3>{});
+                            maybe(std::integral_constant<int, 4>{}), maybe(std::integral_constant<int, 5>{}), maybe(std::integral_constant<int, 6>{}), maybe(std::integral_constant<int, 7>{});
+                            if constexpr (decltype(rb_c)::value == 0 && decltype(i_c)::value == 0) request_a(std::integral_constant<int, 1>{});
+                            if constexpr (decltype(rb_c)::value == 0 && decltype(i_c)::value == 1) request_a(std::integral_constant<int, 2>{});
                         };
                     };
-                    sub_step(b[0], a_rd, 1, piece_of(std::integral_constant<int, 0>{}), [&]() __attribute__((always_inline)) { request_a(std::integral_constant<int, 1>{}); });
-                    sub_step(b[1], a_rd, 2, piece_of(std::integral_constant<int, 1>{}), [&]() __attribute__((always_inline)) { request_a(std::integral_constant<int, 2>{}); });
-                    sub_step(b[2], a_rd, 3, piece_of(std::integral_constant<int, 2>{}), [&]() __attribute__((always_inline)) {});
+                    sub_step(b[0], a_rd, 1, decode_slots(std::integral_constant<int, 0>{}));
+                    sub_step(b[1], a_rd, 2, decode_slots(std::integral_constant<int, 1>{}));
+                    sub_step(b[2], a_rd, 3, decode_slots(std::integral_constant<int, 2>{}));
                     // End of the phase: all but the requests of this phase (and, with four stages, the one before it)
                     // have landed - this wave's parts of the next step's A stage and of the packed bytes of the step
                     // after it.  Behind the barrier every wave's parts have, and every wave is done with the stages the
@@ -267,13 +285,19 @@ struct Direct8NN {
                     else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBehind) : "memory");
                     lds_barrier();
                     open_a();
-                    sub_step(b[3], a_rd_next, 0, piece_of(std::integral_constant<int, 3>{}), [&]() __attribute__((always_inline)) {
-                        request_w();
-                        request_a(std::integral_constant<int, 0>{});
+                    bf16x8_t* bn = bops[P ^ 1];
+                    sub_step(b[3], a_rd_next, 0, [&](auto rb_c) __attribute__((always_inline)) {
+                        constexpr int RB = decltype(rb_c)::value;
+                        if constexpr (RB == 0) {
+                            request_w();
+                            request_a(std::integral_constant<int, 0>{});
+                        }
+                        // the next step's operands: its rows are in the block (LDS accesses of a wave execute in order), and
+                        // the writes of the step after it come behind these reads
+#pragma unroll
+                        for (int ks = 0; ks < 4; ks++)
+                            if (ks * LIVE / 4 == RB) bn[ks] = read_tr(tr_src + ks * 16 * kDecPitch, kDecPitch);
                     });
-                    // the next step's operands: its rows are in the block now (LDS accesses of a wave execute in order),
-                    // and the writes of the step after it come behind these reads
-                    read_b(bops[P ^ 1]);
                     a_rd = a_rd_next;
                     w_rd = w_rd == (kStages - 1) * kRawStageBytes ? 0 : w_rd + kRawStageBytes;
                     relax--;
@@ -364,12 +388,11 @@ struct Direct8NN {
         const int col_tiles = p.col_tiles_per_seg;
         const int chunks = (col_tiles + p.col_tiles_per_wg - 1) / p.col_tiles_per_wg;
         const int row_tiles = p.tiles ? min(*p.num_tiles, p.max_row_tiles) : p.max_row_tiles;
-        const int units = row_tiles * chunks;
-        const int per_xcd = (units + 7) >> 3;
+        // Row tile rt runs on XCD rt % 8 (the table lists the tiles with the most rows first: every XCD gets its
+        // share of them, and takes its own in that order); the column-tile runs of a row tile follow one another there.
         const int slot = (int)(blockIdx.x >> 3);
-        const int unit = (int)(blockIdx.x & 7) * per_xcd + slot;
-        if (slot >= per_xcd || unit >= units) return;
-        const int row_tile = unit / chunks, chunk = unit - row_tile * chunks;
+        const int row_tile = (slot / chunks) * 8 + (int)(blockIdx.x & 7), chunk = slot % chunks;
+        if (row_tile >= row_tiles) return;
         RowCtx c;
         int row_end;
         if (p.tiles) {

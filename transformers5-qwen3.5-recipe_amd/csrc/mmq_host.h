@@ -137,8 +137,12 @@ struct RowTileTables {
     int bm[3], min_rows[3], max_rows[3];
     TileDesc* tiles[3];
     int* num_tiles[3];
-    void add(int bm_, int min_rows_, int max_rows_, TileDesc* tiles_, int* num_tiles_) {
+    // not null: the table also goes here ordered by descending number of 32-row blocks (ties in group order), so that
+    // workgroups dispatched in table order take the most expensive tiles first
+    TileDesc* by_size[3];
+    void add(int bm_, int min_rows_, int max_rows_, TileDesc* tiles_, int* num_tiles_, TileDesc* by_size_ = nullptr) {
         bm[count] = bm_, min_rows[count] = min_rows_, max_rows[count] = max_rows_, tiles[count] = tiles_, num_tiles[count] = num_tiles_;
+        by_size[count] = by_size_;
         count++;
     }
 };
