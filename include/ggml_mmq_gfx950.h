@@ -190,15 +190,23 @@ int ggq_router_topk(const void* logits, int logits_are_bf16, int64_t tokens, int
 /* _packed_q8_linear_cross_entropy_forward (gguf_liger_loss.py:38-186): chunked mmq -> Liger
  * cross-entropy -> mmq_grad_input in one call.  labels int64 [rows];
  * loss_per_row fp32 [rows] (already divided by the number of non-ignored rows when reduction_mean);
- * grad_hidden bf16 [rows, hidden]; lse_out fp32 [rows] or NULL; n_valid_out int32[1] or NULL.  `chunk` is the memory
- * contract, as the reference's [chunk, vocab] logits tensor is: below 4096 rows per chunk nothing wider than 8192 vocabulary
- * columns is ever held (one sweep over the vocabulary with a running max and sum per row); from 4096 rows per chunk on, or
- * when one chunk covers all rows, the chunk's bf16 logits are kept in the workspace and rewritten as their gradient.  Two
- * vocabulary-sized GEMMs either way. */
+ * grad_hidden bf16 [rows, hidden]; lse_out fp32 [rows] or NULL;
+ * status_out int32[2] or NULL: {number of rows that count, number of labels outside [0, vocab) other than ignore_index}.
+ *   Such labels are treated as ignored (no loss, no gradient) and only reported here: nothing on the host waits for them.
+ * predicted_tokens int64 [rows] or NULL: the row's argmax over the bf16 logits (the first maximum), -1 for rows that do not
+ *   count; token_correct fp32 [rows] or NULL: 1 where the argmax is the label, else 0 (Liger's RETURN_PREDICTED_TOKENS /
+ *   RETURN_TOKEN_ACCURACY outputs, gguf_liger_loss.py:92-100, 117-185; the accuracy is sum(token_correct) / status_out[0]).
+ * Memory: `chunk` stands for the reference's [chunk, vocab] logits tensor.  From 4096 rows per chunk on, or when one chunk
+ * covers all rows, the chunk's bf16 logits are kept in the workspace and rewritten as their gradient.  Below that nothing wider
+ * than 8192 vocabulary columns is held (one sweep over the vocabulary with a running max, sum and argmax per row), but the
+ * sweep takes min(rows, 4096) rows at a time whatever the chunk: the workspace then holds a [min(rows, 4096), 8192] bf16 slab,
+ * an fp32 [min(rows, 4096), hidden] accumulator and two bf16-sized [.., hidden] label-row buffers (about 128 MiB at hidden 2048),
+ * for chunk 64 as for chunk 1024.  Two vocabulary-sized GEMMs either way. */
 int64_t ggq_lmhead_ce_workspace_bytes(int64_t rows, int64_t vocab, int64_t hidden_dim, int64_t chunk);
 int ggq_lmhead_cross_entropy(int qt, const void* hidden, const void* packed, const int64_t* labels, int64_t rows, int64_t vocab,
                              int64_t hidden_dim, int64_t chunk, int64_t ignore_index, int reduction_mean, float* loss_per_row,
-                             void* grad_hidden, float* lse_out, int32_t* n_valid_out, void* ws, int64_t ws_bytes, void* stream);
+                             void* grad_hidden, float* lse_out, int32_t* status_out, int64_t* predicted_tokens, float* token_correct, void* ws,
+                             int64_t ws_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -46,3 +46,23 @@ def linear_cross_entropy(hidden, w, labels, ignore_index=-100, reduction="mean",
         loss_1d[r0:r1] = (lse - xy) * scale * v.to(torch.float64)
         dh[r0:r1] = p @ w
     return loss_1d.sum(), dh, loss_1d, lse_all
+
+
+def predicted_tokens(hidden, w, labels, ignore_index=-100, chunk=1024):
+    """Liger's RETURN_PREDICTED_TOKENS / RETURN_TOKEN_ACCURACY outputs as the reference's loop collects them
+    (gguf_liger_loss.py:92-101, 117-185): per row the argmax of the bf16 logits, the FIRST maximum (the kernel scans the
+    vocabulary in ascending blocks and takes a later block only for a strictly larger maximum), -1 on ignored rows;
+    accuracy = rows whose argmax is the label / rows that count (0 when none does, where the reference divides by zero).
+    Returns (predicted int64 [rows], accuracy float)."""
+    rows = hidden.shape[0]
+    valid = labels != ignore_index
+    pred = torch.full((rows,), -1, dtype=torch.int64)
+    for r0 in range(0, rows, chunk):
+        r1 = min(r0 + chunk, rows)
+        logits = bf16_round64(hidden[r0:r1].to(torch.float64) @ w.T)
+        best = logits.max(dim=1, keepdim=True).values
+        first = torch.where(logits == best, torch.arange(logits.shape[1])[None, :], logits.shape[1]).min(dim=1).values
+        pred[r0:r1] = torch.where(valid[r0:r1], first, torch.full_like(first, -1))
+    n = int(valid.sum())
+    acc = float(((pred == labels) & valid).sum()) / n if n else 0.0
+    return pred, acc

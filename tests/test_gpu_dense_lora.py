@@ -108,7 +108,9 @@ def test_dense_guards(pkg, dev):
     with pytest.raises(TypeError):
         fl.mmq(x.float(), p, gb.Q4_K, 8)
     with pytest.raises(ValueError):
-        fl.mmq(x, p, 10, 8)  # Q2_K: not implemented, must not be routed anywhere else
+        fl.mmq(x, torch.zeros(8, 82, dtype=torch.uint8, device=dev), 22, 8)  # IQ2_S: no kernel here, must not be routed anywhere else
+    with pytest.raises(ValueError):
+        fl.mmq(x, torch.zeros(8, 8 * 18, dtype=torch.uint8, device=dev), 2, 8)  # Q4_0 with a byte count that would fit: no kernel
     with pytest.raises(ValueError):
         fl.mmq(x, p, gb.Q4_K, 9)  # payload rows do not match out_features
     with pytest.raises(ValueError):

@@ -42,7 +42,9 @@ def test_dequantize_expert_stack_and_constant_payload(pkg, dev):
 def test_dequantize_rejects_bad_operands(pkg, dev):
     p = torch.zeros(4, 144, dtype=torch.uint8, device=dev)
     with pytest.raises(ValueError):
-        pkg.gguf.dequantize_gguf_tensor(p, 11, torch.bfloat16)  # Q3_K: no native decoder
+        pkg.gguf.dequantize_gguf_tensor(torch.zeros(4, 82, dtype=torch.uint8, device=dev), 22, torch.bfloat16)  # IQ2_S (82-byte blocks): no decoder here
+    with pytest.raises(ValueError):
+        pkg.gguf.dequantize_gguf_tensor(p, 2, torch.bfloat16)  # Q4_0: no decoder here
     with pytest.raises(TypeError):
         pkg.gguf.dequantize_gguf_tensor(p, gb.Q4_K, torch.float16)
     with pytest.raises(ValueError):

@@ -68,3 +68,26 @@ def test_uniform_logits_closed_form():
     assert torch.allclose(loss_1d, lse)
     # sum over vocab of (1/V - onehot) is 0, and every weight row is the same: dh = 0
     assert float(dh.abs().max()) < 1e-6
+
+
+def test_predicted_tokens_first_maximum_and_accuracy():
+    # distinct logits: torch.argmax; tied logits: a brute-force scan that keeps the first maximum
+    g = torch.Generator().manual_seed(11)
+    hid = torch.randn(9, 16, generator=g).to(torch.bfloat16)
+    w = torch.randn(40, 16, generator=g).to(torch.bfloat16).double()
+    labels = torch.randint(0, 40, (9,), generator=g)
+    labels[2] = -100
+    logits = ce.bf16_round64(hid.double() @ w.T)
+    pred, acc = ce.predicted_tokens(hid, w, labels, -100, chunk=4)
+    for r in range(9):
+        best, arg = None, -1
+        for c in range(40):
+            if best is None or float(logits[r, c]) > best:
+                best, arg = float(logits[r, c]), c
+        assert int(pred[r]) == (-1 if r == 2 else arg)
+    counted = [r for r in range(9) if r != 2]
+    assert abs(acc - sum(int(pred[r]) == int(labels[r]) for r in counted) / len(counted)) < 1e-12
+    hid[:] = 0  # every logit equal: the first column
+    pred, acc = ce.predicted_tokens(hid, w, labels, -100)
+    assert pred.tolist() == [0, 0, -1, 0, 0, 0, 0, 0, 0]
+    assert ce.predicted_tokens(hid, w, torch.full((9,), -100), -100)[1] == 0.0

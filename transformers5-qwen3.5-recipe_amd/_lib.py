@@ -51,7 +51,7 @@ SIGNATURES: dict[str, tuple] = {
     "ggq_swiglu_clamped_forward": (_I, [_P, _P, _P, _L, _F, _P]),
     "ggq_swiglu_clamped_backward": (_I, [_P, _P, _P, _P, _P, _L, _F, _P]),
     "ggq_lmhead_ce_workspace_bytes": (_L, [_L, _L, _L, _L]),
-    "ggq_lmhead_cross_entropy": (_I, [_I, _P, _P, _P, _L, _L, _L, _L, _L, _I, _P, _P, _P, _P, _P, _L, _P]),
+    "ggq_lmhead_cross_entropy": (_I, [_I, _P, _P, _P, _L, _L, _L, _L, _L, _I, _P, _P, _P, _P, _P, _P, _P, _L, _P]),
 }
 
 

@@ -30,7 +30,7 @@ bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 int check_weights(const char* what, int qt, const void* w, int64_t k) {
     if (!w) return set_error(GGQ_ERR_NULL, "%s: packed weight pointer is null", what);
-    if (packed_row_bytes(qt, k) < 0) return set_error(GGQ_ERR_QTYPE, "%s: unsupported GGML type id %d (supported: 8, 12, 14, 16)", what, qt);
+    if (packed_row_bytes(qt, k) < 0) return set_error(GGQ_ERR_QTYPE, "%s: unsupported GGML type id %d (supported: 8, 10, 11, 12, 13, 14, 16)", what, qt);
     if (!aligned16(w)) return set_error(GGQ_ERR_ALIGN, "%s: packed weights must be 16-byte aligned", what);
     return GGQ_OK;
 }
@@ -500,10 +500,11 @@ int64_t ggq_lmhead_ce_workspace_bytes(int64_t rows, int64_t vocab, int64_t hidde
 
 int ggq_lmhead_cross_entropy(int qt, const void* hidden, const void* packed, const int64_t* labels, int64_t rows, int64_t vocab,
                              int64_t hidden_dim, int64_t chunk, int64_t ignore_index, int reduction_mean, float* loss_per_row,
-                             void* grad_hidden, float* lse_out, int32_t* n_valid_out, void* ws, int64_t ws_bytes, void* stream) {
+                             void* grad_hidden, float* lse_out, int32_t* status_out, int64_t* predicted_tokens, float* token_correct, void* ws,
+                             int64_t ws_bytes, void* stream) {
     if (int rc = check_weights("lmhead_cross_entropy", qt, packed, hidden_dim)) return rc;
     return lmhead_ce(qt, hidden, packed, labels, rows, vocab, hidden_dim, chunk, ignore_index, reduction_mean, loss_per_row,
-                     grad_hidden, lse_out, n_valid_out, ws, ws_bytes, as_stream(stream));
+                     grad_hidden, lse_out, status_out, predicted_tokens, token_correct, ws, ws_bytes, as_stream(stream));
 }
 
 }  // extern "C"

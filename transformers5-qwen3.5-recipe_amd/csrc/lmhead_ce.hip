@@ -27,56 +27,34 @@ constexpr int64_t kGradRows = 4096;
 // A chunk of at least this many rows is worth keeping the logits of: its grad-input launch fills the chip.
 constexpr int64_t kKeptLogitsRows = 4096;
 
-// row_scale[m] = 0 for ignored rows, else 1/n_valid (mean) or 1 (sum); n_valid = 0 gives all zeros.
-__global__ __launch_bounds__(1024) void ce_row_scale_kernel(const int64_t* labels, int64_t rows, int64_t ignore_index,
-                                                             int mean, float* row_scale, int* n_valid_out) {
-    __shared__ int partial[1024];
-    int c = 0;
-    for (int64_t i = threadIdx.x; i < rows; i += 1024) c += labels[i] != ignore_index;
-    partial[threadIdx.x] = c;
+// row_scale[m] = 0 for ignored rows, else 1/n_valid (mean) or 1 (sum); n_valid = 0 gives all zeros.  A label outside
+// [0, vocab) that is not ignore_index is treated as ignored (no loss, no gradient) and counted in status[1].
+__device__ __forceinline__ bool label_counts(int64_t label, int64_t vocab, int64_t ignore_index) {
+    return label != ignore_index && label >= 0 && label < vocab;
+}
+__global__ __launch_bounds__(1024) void ce_row_scale_kernel(const int64_t* labels, int64_t rows, int64_t vocab, int64_t ignore_index,
+                                                             int mean, float* row_scale, int* status) {
+    __shared__ int partial[1024], partial_bad[1024];
+    int c = 0, bad = 0;
+    for (int64_t i = threadIdx.x; i < rows; i += 1024) {
+        const int64_t l = labels[i];
+        c += label_counts(l, vocab, ignore_index);
+        bad += l != ignore_index && (l < 0 || l >= vocab);
+    }
+    partial[threadIdx.x] = c, partial_bad[threadIdx.x] = bad;
     __syncthreads();
     for (int off = 512; off >= 1; off >>= 1) {
-        if ((int)threadIdx.x < off) partial[threadIdx.x] += partial[threadIdx.x + off];
+        if ((int)threadIdx.x < off) partial[threadIdx.x] += partial[threadIdx.x + off], partial_bad[threadIdx.x] += partial_bad[threadIdx.x + off];
         __syncthreads();
     }
     const int n = partial[0];
     const float scale = n == 0 ? 0.f : (mean ? 1.0f / (float)n : 1.0f);
-    for (int64_t i = threadIdx.x; i < rows; i += 1024) row_scale[i] = labels[i] != ignore_index ? scale : 0.f;
-    if (threadIdx.x == 0 && n_valid_out) *n_valid_out = n;
-}
-
-// One wave per row: merge the slab partials into lse, then loss = (lse - target logit) * row_scale.
-__global__ __launch_bounds__(256) void ce_finalize_kernel(const float2* partials, int ld, int nparts, const float* target_logit,
-                                                          const float* row_scale, int rows, float* lse_out, float* loss_out) {
-    const int lane = threadIdx.x & 63;
-    const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (r >= rows) return;
-    const float2* p = partials + (int64_t)r * ld;
-    float mx = -INFINITY;
-    for (int i = lane; i < nparts; i += 64) mx = fmaxf(mx, p[i].x);
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
-    float sum = 0.f;
-    for (int i = lane; i < nparts; i += 64) {
-        const float2 v = p[i];
-        if (v.y > 0.f) sum += v.y * __expf(v.x - mx);
-    }
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) sum += __shfl_xor(sum, off, 64);
-    if (lane == 0) {
-        const float lse = mx + __logf(sum);
-        lse_out[r] = lse;
-        const float rs = row_scale[r];
-        loss_out[r] = rs != 0.f ? (lse - target_logit[r]) * rs : 0.f;
-    }
+    for (int64_t i = threadIdx.x; i < rows; i += 1024) row_scale[i] = label_counts(labels[i], vocab, ignore_index) ? scale : 0.f;
+    if (threadIdx.x == 0 && status) status[0] = n, status[1] = partial_bad[0];
 }
 
 __global__ void fill_f32_kernel(float* p, int64_t n, float v) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = v;
-}
-
-__global__ void f32_to_bf16_kernel(const float* src, bf16_t* dst, int64_t n) {
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) dst[i] = to_bf16(src[i]);
 }
 
 static unsigned grid1d(int64_t n) {
@@ -94,15 +72,24 @@ __device__ __forceinline__ void merge_max_sum(float& m, float& s, float m2, floa
     m = mx;
 }
 
+// (value, column) of the better of two candidates: the larger value, and among equal values the smaller column (the first
+// maximum of the row, the choice of an argmax that scans the columns in order)
+__device__ __forceinline__ void merge_arg(float& v, int& i, float v2, int i2) {
+    if (v2 > v || (v2 == v && i2 < i)) v = v2, i = i2;
+}
+
 __global__ __launch_bounds__(256) void ce_loss_and_grad_kernel(bf16_t* logits, int64_t ld, int64_t vocab, const int64_t* labels, const float* row_scale,
-                                                               float* lse_out, float* loss_out) {
-    __shared__ float wave_m[4], wave_s[4];
+                                                               float* lse_out, float* loss_out, int64_t ignore_index, int64_t* predicted, float* correct) {
+    __shared__ float wave_m[4], wave_s[4], wave_bv[4];
+    __shared__ int wave_bi[4];
     const int64_t row = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint4* p = (uint4*)(logits + row * ld);
     const int64_t label = labels[row];
     const float rs = row_scale[row];
     float m = -INFINITY, sum = 0.f;
+    float bv = -INFINITY;  // this lane's best logit and its column (its columns come in ascending order: strict > keeps the first)
+    int bi = 0x7FFFFFFF;
     for (int64_t c8 = threadIdx.x; c8 < ld / 8; c8 += 256) {
         const uint4 v = p[c8];
         const uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -114,6 +101,12 @@ __global__ __launch_bounds__(256) void ce_loss_and_grad_kernel(bf16_t* logits, i
             cm = fmaxf(cm, x[e]);
         }
         if (cm == -INFINITY) continue;  // padding only
+        if (cm > bv) {
+            bv = cm;
+#pragma unroll
+            for (int e = 7; e >= 0; e--)
+                if (x[e] == cm) bi = (int)(c8 * 8 + e);
+        }
         float cs = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; e++) cs += x[e] == -INFINITY ? 0.f : __expf(x[e] - cm);
@@ -124,7 +117,13 @@ __global__ __launch_bounds__(256) void ce_loss_and_grad_kernel(bf16_t* logits, i
         const float m2 = __shfl_xor(m, off, 64), s2 = __shfl_xor(sum, off, 64);
         merge_max_sum(m, sum, m2, s2);
     }
-    if (lane == 0) wave_m[wave] = m, wave_s[wave] = sum;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const float v2 = __shfl_xor(bv, off, 64);
+        const int i2 = __shfl_xor(bi, off, 64);
+        merge_arg(bv, bi, v2, i2);
+    }
+    if (lane == 0) wave_m[wave] = m, wave_s[wave] = sum, wave_bv[wave] = bv, wave_bi[wave] = bi;
     __syncthreads();
     m = wave_m[0], sum = wave_s[0];
 #pragma unroll
@@ -132,8 +131,14 @@ __global__ __launch_bounds__(256) void ce_loss_and_grad_kernel(bf16_t* logits, i
     const float lse = m + __logf(sum);
     if (threadIdx.x == 0) {
         lse_out[row] = lse;
-        const float target = label >= 0 && label < vocab ? bf16_to_f32(logits[row * ld + label]) : 0.f;
+        const bool counts = label_counts(label, vocab, ignore_index);
+        const float target = counts ? bf16_to_f32(logits[row * ld + label]) : 0.f;
         loss_out[row] = rs != 0.f ? (lse - target) * rs : 0.f;
+        bv = wave_bv[0], bi = wave_bi[0];
+#pragma unroll
+        for (int w = 1; w < 4; w++) merge_arg(bv, bi, wave_bv[w], wave_bi[w]);
+        if (predicted) predicted[row] = counts ? (int64_t)bi : -1;
+        if (correct) correct[row] = counts && (int64_t)bi == label ? 1.0f : 0.0f;
     }
     __syncthreads();  // the target logit is read before the row is overwritten
     for (int64_t c8 = threadIdx.x; c8 < ld / 8; c8 += 256) {
@@ -148,7 +153,7 @@ __global__ __launch_bounds__(256) void ce_loss_and_grad_kernel(bf16_t* logits, i
                 const int64_t col = c8 * 8 + 2 * e + h;
                 const float logit = bf16_to_f32((bf16_t)(h ? w[e] >> 16 : w[e] & 0xFFFFu));
                 float d = __expf(logit - lse);
-                if (col == label) d -= 1.0f;
+                if (col == label && rs != 0.f) d -= 1.0f;
                 g[h] = col < vocab ? d * rs : 0.0f;
             }
             o[e] = pack_bf16(g[0], g[1]);
@@ -163,8 +168,9 @@ __global__ __launch_bounds__(256) void ce_loss_and_grad_kernel(bf16_t* logits, i
 // what was accumulated so far, and the grad-input launch adds p . W_block to the fp32 accumulator it first multiplied by
 // alpha.  At the end dH = ((acc / sum) - W[label]) * row_scale.  One workgroup per row.
 __global__ __launch_bounds__(256) void ce_stream_block_kernel(bf16_t* slab, int64_t ld, int nb, int64_t v0, const int64_t* labels, float* run_max,
-                                                              float* run_sum, float* target, float* alpha) {
+                                                              float* run_sum, float* target, float* alpha, int64_t* run_arg) {
     __shared__ float red[4];
+    __shared__ int red_i[4];
     const int64_t row = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint4* p = (uint4*)(slab + row * ld);
@@ -186,9 +192,10 @@ __global__ __launch_bounds__(256) void ce_stream_block_kernel(bf16_t* slab, int6
     const float m_old = run_max[row];
     const float m_new = fmaxf(m_old, bm);
     const int64_t label = labels[row];
-    if (threadIdx.x == 0 && label >= v0 && label < v0 + nb) target[row] = bf16_to_f32(slab[row * ld + (label - v0)]);
+    if (threadIdx.x == 0 && label >= v0 && label < v0 + nb) target[row] = bf16_to_f32(slab[row * ld + (label - v0)]);  // (an ignore_index inside the range is masked by its zero row scale)
     __syncthreads();  // the target logit is read before the row is overwritten
     float sum = 0.f;
+    int first = 0x7FFFFFFF;  // first column of the block that holds the block's maximum
     for (int c8 = threadIdx.x; c8 < chunks; c8 += 256) {
         const uint4 v = p[c8];
         const uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -199,7 +206,9 @@ __global__ __launch_bounds__(256) void ce_stream_block_kernel(bf16_t* slab, int6
 #pragma unroll
             for (int h = 0; h < 2; h++) {
                 const float logit = bf16_to_f32((bf16_t)(h ? w[e] >> 16 : w[e] & 0xFFFFu));
-                g[h] = c8 * 8 + 2 * e + h < nb ? __expf(logit - m_new) : 0.0f;
+                const int col = c8 * 8 + 2 * e + h;
+                if (col < nb && logit == bm) first = min(first, col);
+                g[h] = col < nb ? __expf(logit - m_new) : 0.0f;
             }
             o[e] = pack_bf16(g[0], g[1]);
             // the sum runs over the rounded values the accumulator receives, so that numerator and denominator agree
@@ -209,9 +218,13 @@ __global__ __launch_bounds__(256) void ce_stream_block_kernel(bf16_t* slab, int6
     }
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) sum += __shfl_xor(sum, off, 64);
-    if (lane == 0) red[wave] = sum;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) first = min(first, __shfl_xor(first, off, 64));
+    if (lane == 0) red[wave] = sum, red_i[wave] = first;
     __syncthreads();
     if (threadIdx.x == 0) {
+        // a later block takes the argmax over only with a strictly larger maximum: equal maxima keep the first column
+        if (run_arg && bm > m_old) run_arg[row] = v0 + min(min(red_i[0], red_i[1]), min(red_i[2], red_i[3]));
         const float a = m_old == -INFINITY ? 0.f : __expf(m_old - m_new);
         alpha[row] = a;
         run_sum[row] = run_sum[row] * a + ((red[0] + red[1]) + (red[2] + red[3]));
@@ -231,15 +244,21 @@ __global__ __launch_bounds__(256) void gather_label_rows_kernel(const uint8_t* p
 // lse, loss and dH = ((acc / sum) - W[label]) * row_scale, rounded to bf16.  One workgroup per row.
 __global__ __launch_bounds__(256) void ce_stream_finish_kernel(const float* acc, const bf16_t* w_label, int64_t hidden, const int64_t* labels, int64_t vocab,
                                                                const float* run_max, const float* run_sum, const float* target, const float* row_scale,
-                                                               float* lse_out, float* loss_out, bf16_t* grad_hidden) {
+                                                               float* lse_out, float* loss_out, bf16_t* grad_hidden, int64_t ignore_index,
+                                                               const int64_t* run_arg, int64_t* predicted, float* correct) {
     const int64_t row = blockIdx.x;
     const float rs = row_scale[row], inv = 1.0f / run_sum[row];
     const int64_t label = labels[row];
-    const bool has_target = label >= 0 && label < vocab;
+    const bool has_target = label_counts(label, vocab, ignore_index);
     if (threadIdx.x == 0) {
         const float lse = run_max[row] + __logf(run_sum[row]);
         lse_out[row] = lse;
         loss_out[row] = rs != 0.f ? (lse - (has_target ? target[row] : 0.f)) * rs : 0.f;
+        if (run_arg) {
+            const int64_t arg = run_arg[row];
+            if (correct) correct[row] = has_target && arg == label ? 1.0f : 0.0f;
+            if (predicted) predicted[row] = has_target ? arg : -1;  // (may be the running storage itself: read first)
+        }
     }
     for (int64_t c = threadIdx.x; c < hidden; c += 256) {
         const float wl = has_target ? bf16_to_f32(w_label[row * hidden + c]) : 0.f;
@@ -256,13 +275,13 @@ static bool keeps_logits(int64_t rows, int64_t chunk) { return chunk >= rows || 
 int64_t lmhead_ce_workspace_bytes(int64_t rows, int64_t vocab, int64_t hidden, int64_t chunk) {
     if (keeps_logits(rows, chunk)) return align256(rows * 4) * 2 + align256(std::min(rows, chunk) * padded_vocab(vocab) * 2) + 1024;
     const int64_t gr = std::min(rows, kGradRows);
-    return align256(rows * 4) * 6 + align256(gr * kVocabBlock * 2) + align256(gr * hidden * 4) + align256(gr * hidden * 2) * 2 + 1024;
+    return align256(rows * 4) * 6 + align256(rows * 8) + align256(gr * kVocabBlock * 2) + align256(gr * hidden * 4) + align256(gr * hidden * 2) * 2 + 1024;
 }
 
 // The kept-logits path: row blocks of one chunk each.
 static int lmhead_ce_kept_logits(int qt, const void* hidden, const void* packed, const int64_t* labels, int64_t rows, int64_t vocab,
                                  int64_t hidden_dim, int64_t chunk, int64_t ignore_index, int reduction_mean, float* loss_1d,
-                                 void* grad_hidden, float* lse_out, int* n_valid_out, void* ws, hipStream_t s) {
+                                 void* grad_hidden, float* lse_out, int* n_valid_out, int64_t* predicted, float* correct, void* ws, hipStream_t s) {
     const int64_t br_max = std::min(rows, chunk);
     const int64_t ld = padded_vocab(vocab);
     char* w = (char*)ws;
@@ -270,7 +289,7 @@ static int lmhead_ce_kept_logits(int qt, const void* hidden, const void* packed,
     float* lse = lse_out ? lse_out : (float*)w; w += align256(rows * 4);
     bf16_t* logits = (bf16_t*)w;  // [br_max, ld]
 
-    hipLaunchKernelGGL(ce_row_scale_kernel, dim3(1), dim3(1024), 0, s, labels, rows, ignore_index, reduction_mean, row_scale, n_valid_out);
+    hipLaunchKernelGGL(ce_row_scale_kernel, dim3(1), dim3(1024), 0, s, labels, rows, vocab, ignore_index, reduction_mean, row_scale, n_valid_out);
     for (int64_t b0 = 0; b0 < rows; b0 += br_max) {
         const int br = (int)std::min(rows - b0, br_max);
         // (1) logits = hidden . W^T
@@ -281,7 +300,8 @@ static int lmhead_ce_kept_logits(int qt, const void* hidden, const void* packed,
         p.c[0] = logits, p.ldc = ld;
         if (int rcode = launch_mmq(qt, kModeNT, kEpiStore, p, s)) return rcode;
         // (2) loss per row; the logits become the gradient with respect to them
-        hipLaunchKernelGGL(ce_loss_and_grad_kernel, dim3((unsigned)br), dim3(256), 0, s, logits, ld, vocab, labels + b0, row_scale + b0, lse + b0, loss_1d + b0);
+        hipLaunchKernelGGL(ce_loss_and_grad_kernel, dim3((unsigned)br), dim3(256), 0, s, logits, ld, vocab, labels + b0, row_scale + b0, lse + b0, loss_1d + b0,
+                           ignore_index, predicted ? predicted + b0 : nullptr, correct ? correct + b0 : nullptr);
         // (3) dH = dlogits . W over the whole vocabulary
         MmqParams g;
         if (int rcode = init_params(g, qt, kModeNN, br, (int)vocab, (int)hidden_dim, 1)) return rcode;
@@ -295,7 +315,7 @@ static int lmhead_ce_kept_logits(int qt, const void* hidden, const void* packed,
 
 int lmhead_ce(int qt, const void* hidden, const void* packed, const int64_t* labels, int64_t rows, int64_t vocab,
               int64_t hidden_dim, int64_t chunk, int64_t ignore_index, int reduction_mean, float* loss_1d,
-              void* grad_hidden, float* lse_out, int* n_valid_out, void* ws, int64_t ws_bytes, hipStream_t s) {
+              void* grad_hidden, float* lse_out, int* n_valid_out, int64_t* predicted, float* correct, void* ws, int64_t ws_bytes, hipStream_t s) {
     if (rows < 0 || vocab <= 0 || hidden_dim <= 0 || chunk <= 0) return set_error(GGQ_ERR_SHAPE, "lmhead_ce: bad shape");
     if (rows >= (1 << 30) || vocab >= (1 << 30)) return set_error(GGQ_ERR_SHAPE, "lmhead_ce: shape too large");
     if (!hidden || !packed || !labels || !loss_1d || !grad_hidden || !ws) return set_error(GGQ_ERR_NULL, "lmhead_ce: null pointer");
@@ -304,7 +324,7 @@ int lmhead_ce(int qt, const void* hidden, const void* packed, const int64_t* lab
     if (rows == 0) return GGQ_OK;
     if (keeps_logits(rows, chunk))
         return lmhead_ce_kept_logits(qt, hidden, packed, labels, rows, vocab, hidden_dim, chunk, ignore_index, reduction_mean, loss_1d, grad_hidden,
-                                     lse_out, n_valid_out, ws, s);
+                                     lse_out, n_valid_out, predicted, correct, ws, s);
     // One sweep over the vocabulary per block of up to kGradRows rows; nothing wider than kVocabBlock columns is ever held.
     const int64_t gr_max = std::min(rows, kGradRows);
     char* w = (char*)ws;
@@ -314,12 +334,13 @@ int lmhead_ce(int qt, const void* hidden, const void* packed, const int64_t* lab
     float* run_max = (float*)w; w += align256(rows * 4);
     float* run_sum = (float*)w; w += align256(rows * 4);
     float* alpha = (float*)w; w += align256(rows * 4);
+    int64_t* run_arg = (predicted || correct) ? (int64_t*)w : nullptr; w += align256(rows * 8);  // running argmax column per row
     bf16_t* slab = (bf16_t*)w; w += align256(gr_max * kVocabBlock * 2);
     float* dh32 = (float*)w; w += align256(gr_max * hidden_dim * 4);
     uint8_t* label_rows = (uint8_t*)w; w += align256(gr_max * hidden_dim * 2);  // packed rows are smaller than bf16 rows
     bf16_t* w_label = (bf16_t*)w;
 
-    hipLaunchKernelGGL(ce_row_scale_kernel, dim3(1), dim3(1024), 0, s, labels, rows, ignore_index, reduction_mean, row_scale, n_valid_out);
+    hipLaunchKernelGGL(ce_row_scale_kernel, dim3(1), dim3(1024), 0, s, labels, rows, vocab, ignore_index, reduction_mean, row_scale, n_valid_out);
     const int64_t row_bytes = packed_row_bytes(qt, hidden_dim);
     if (row_bytes <= 0 || row_bytes > hidden_dim * 2 || (row_bytes & 1)) return set_error(GGQ_ERR_QTYPE, "lmhead_ce: unsupported packed row size");
     hipLaunchKernelGGL(fill_f32_kernel, dim3(grid1d(rows)), dim3(256), 0, s, run_max, rows, -INFINITY);
@@ -340,7 +361,7 @@ int lmhead_ce(int qt, const void* hidden, const void* packed, const int64_t* lab
             if (int rcode = launch_mmq(qt, kModeNT, kEpiStore, g, s)) return rcode;
             // (2) running statistics; the slab becomes exp(logit - running max)
             hipLaunchKernelGGL(ce_stream_block_kernel, dim3((unsigned)rc), dim3(256), 0, s, slab, kVocabBlock, nb, v0, labels + r0, run_max + r0, run_sum + r0,
-                               target + r0, alpha + r0);
+                               target + r0, alpha + r0, run_arg ? run_arg + r0 : nullptr);
             // (3) acc = acc * alpha + p . W_block
             MmqParams b;
             if (int rcode = init_params(b, qt, kModeNN, rc, nb, (int)hidden_dim, 1)) return rcode;
@@ -353,7 +374,8 @@ int lmhead_ce(int qt, const void* hidden, const void* packed, const int64_t* lab
         hipLaunchKernelGGL(gather_label_rows_kernel, dim3((unsigned)rc), dim3(256), 0, s, (const uint8_t*)packed, row_bytes, labels + r0, vocab, label_rows);
         if (int rcode = dequantize(qt, label_rows, rc, hidden_dim, w_label, 0, s)) return rcode;
         hipLaunchKernelGGL(ce_stream_finish_kernel, dim3((unsigned)rc), dim3(256), 0, s, dh32, w_label, hidden_dim, labels + r0, vocab, run_max + r0, run_sum + r0,
-                           target + r0, row_scale + r0, lse + r0, loss_1d + r0, (bf16_t*)grad_hidden + r0 * hidden_dim);
+                           target + r0, row_scale + r0, lse + r0, loss_1d + r0, (bf16_t*)grad_hidden + r0 * hidden_dim, ignore_index,
+                           run_arg ? run_arg + r0 : nullptr, predicted ? predicted + r0 : nullptr, correct ? correct + r0 : nullptr);
     }
     return check_launch("lmhead_ce");
 }

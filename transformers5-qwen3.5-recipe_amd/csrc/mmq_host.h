@@ -170,7 +170,7 @@ int swiglu_bwd(const void* gate, const void* up, const void* dh, void* dgate, vo
 int64_t lmhead_ce_workspace_bytes(int64_t rows, int64_t vocab, int64_t hidden, int64_t chunk);
 int lmhead_ce(int qt, const void* hidden, const void* packed, const int64_t* labels, int64_t rows, int64_t vocab,
               int64_t hidden_dim, int64_t chunk, int64_t ignore_index, int reduction_mean, float* loss_1d,
-              void* grad_hidden, float* lse_out, int* n_valid_out, void* ws, int64_t ws_bytes, hipStream_t s);
+              void* grad_hidden, float* lse_out, int* n_valid_out, int64_t* predicted, float* correct, void* ws, int64_t ws_bytes, hipStream_t s);
 
 int dequantize(int qt, const void* payload, int64_t rows, int64_t k, void* out, int out_f32, hipStream_t stream);
 

@@ -18,8 +18,8 @@ import torch
 from . import _lib
 from .gguf import GGML_QUANT_SIZES, GGUFQuantizedTensor, row_bytes
 
-# GGML type ids with native kernels here (the reference's wheel also lists 10, 11, 13, 22:
-# fast_lora.py:24-27; those are not implemented and are rejected, never routed elsewhere).
+# GGML type ids with native kernels here: 8, 10, 11, 12, 13, 14, 16.  The reference's wheel also lists 22 (IQ2_S,
+# fast_lora.py:24-27), which is not implemented and is rejected, never routed elsewhere.
 _NATIVE_MMQ_QUANT_TYPES = frozenset(GGML_QUANT_SIZES)
 
 

@@ -21,9 +21,17 @@ from .gguf import GGUFQuantizedTensor, row_bytes
 _PACKED_LM_HEAD_CHUNK_SIZE = 256
 
 
+# set to True to wait for the device after every loss call and raise on labels outside [0, vocab) that are not
+# ignore_index (the kernels treat such labels as ignored and only count them, so that no call has to synchronise)
+VALIDATE_LABELS = False
+
+
 def _packed_linear_cross_entropy_forward(input: torch.Tensor, packed_weight: torch.Tensor, target: torch.Tensor, quant_type: int,
-                                         out_features: int, chunk_size: int, ignore_index: int, reduction: str):
-    """Returns (loss, grad_input, loss_1d, lse, n_non_ignore tensor)."""
+                                         out_features: int, chunk_size: int, ignore_index: int, reduction: str,
+                                         return_token_accuracy: bool = False, return_predicted_tokens: bool = False):
+    """Returns (loss, grad_input, loss_1d, lse, status, token_accuracy, predicted_tokens); status is an int32[2] device tensor
+    {rows that count, labels out of range}.  token_accuracy = correct argmax rows / rows that count (gguf_liger_loss.py:180-185),
+    predicted_tokens int64 [rows] with -1 on ignored rows (:97-101); both None unless asked for."""
     if input.ndim != 2:
         raise ValueError(f"Packed LM-head loss expects two-dimensional hidden states, got {input.shape}.")
     if input.dtype != torch.bfloat16:
@@ -48,50 +56,68 @@ def _packed_linear_cross_entropy_forward(input: torch.Tensor, packed_weight: tor
     grad_input = torch.zeros_like(input)
     loss_1d = torch.zeros(rows, dtype=torch.float32, device=dev)
     lse = torch.zeros(rows, dtype=torch.float32, device=dev)
-    n_valid = torch.zeros(1, dtype=torch.int32, device=dev)
+    status = torch.zeros(2, dtype=torch.int32, device=dev)
+    correct = torch.zeros(rows, dtype=torch.float32, device=dev) if return_token_accuracy else None
+    predicted = torch.full((rows,), -1, dtype=torch.int64, device=dev) if return_predicted_tokens else None
     if rows:
         lib = _lib.load()
         ws = torch.empty(lib.ggq_lmhead_ce_workspace_bytes(rows, out_features, hidden, chunk_size), dtype=torch.uint8, device=dev)
         _lib.check(lib.ggq_lmhead_cross_entropy(quant_type, input.data_ptr(), packed_weight.data_ptr(), target.data_ptr(), rows, out_features,
                                                hidden, chunk_size, ignore_index, int(reduction == "mean"), loss_1d.data_ptr(),
-                                               grad_input.data_ptr(), lse.data_ptr(), n_valid.data_ptr(), ws.data_ptr(), ws.numel(),
-                                               _lib.stream_handle(dev)))
-    return torch.sum(loss_1d), grad_input, loss_1d, lse, n_valid
+                                               grad_input.data_ptr(), lse.data_ptr(), status.data_ptr(), _lib.ptr(predicted), _lib.ptr(correct),
+                                               ws.data_ptr(), ws.numel(), _lib.stream_handle(dev)))
+        if VALIDATE_LABELS and int(status[1]):
+            raise ValueError(f"{int(status[1])} labels lie outside [0, {out_features}) and are not ignore_index={ignore_index}")
+    token_accuracy = None
+    if return_token_accuracy:
+        # (no rows that count: 0 / 0 in the reference, gguf_liger_loss.py:183; defined as 0 here, like the loss)
+        token_accuracy = torch.sum(correct) / torch.clamp(status[0], min=1).to(torch.float32)
+    return torch.sum(loss_1d), grad_input, loss_1d, lse, status, token_accuracy, predicted
 
 
 class _PackedLinearCrossEntropyFunction(torch.autograd.Function):
     """Fused loss over a frozen packed lm_head (counterpart of
-    ``_PackedQ8LigerLinearCrossEntropyFunction``, gguf_liger_loss.py:189-266)."""
+    ``_PackedQ8LigerLinearCrossEntropyFunction``, gguf_liger_loss.py:189-266): returns (loss, token_accuracy,
+    predicted_tokens), the last two None unless asked for and never differentiable."""
 
     @staticmethod
-    def forward(ctx, input, packed_weight, target, quant_type, out_features, chunk_size, ignore_index, reduction):
-        loss, grad_input, _, _, _ = _packed_linear_cross_entropy_forward(
-            input, packed_weight, target, quant_type, out_features, chunk_size, ignore_index, reduction)
+    def forward(ctx, input, packed_weight, target, quant_type, out_features, chunk_size, ignore_index, reduction,
+                return_token_accuracy=False, return_predicted_tokens=False):
+        loss, grad_input, _, _, _, token_accuracy, predicted = _packed_linear_cross_entropy_forward(
+            input, packed_weight, target, quant_type, out_features, chunk_size, ignore_index, reduction,
+            return_token_accuracy, return_predicted_tokens)
         ctx.save_for_backward(grad_input.detach())
-        return loss
+        ctx.mark_non_differentiable(*[t for t in (token_accuracy, predicted) if t is not None])
+        return loss, token_accuracy, predicted
 
     @staticmethod
-    def backward(ctx, grad_output):
+    def backward(ctx, grad_output, grad_accuracy=None, grad_predicted=None):
         if torch.is_grad_enabled():
             raise RuntimeError("Packed GGUF LM-head loss does not support higher-order gradients")
         (grad_input,) = ctx.saved_tensors
         # the saved gradient assumes an upstream gradient of one; rescale only when it is not
         grad_input = grad_input * grad_output.to(grad_input.dtype)
-        return grad_input, None, None, None, None, None, None, None
+        return grad_input, None, None, None, None, None, None, None, None, None
 
 
 def packed_linear_cross_entropy(hidden_states, packed_weight, target, quant_type, out_features, chunk_size=_PACKED_LM_HEAD_CHUNK_SIZE,
-                                ignore_index=-100, reduction="mean") -> torch.Tensor:
-    return _PackedLinearCrossEntropyFunction.apply(hidden_states, packed_weight.as_subclass(torch.Tensor), target, int(quant_type),
-                                                   int(out_features), int(chunk_size), int(ignore_index), reduction)
+                                ignore_index=-100, reduction="mean", return_token_accuracy=False, return_predicted_tokens=False):
+    """The loss; with either flag set, the triple (loss, token_accuracy, predicted_tokens)."""
+    loss, token_accuracy, predicted = _PackedLinearCrossEntropyFunction.apply(
+        hidden_states, packed_weight.as_subclass(torch.Tensor), target, int(quant_type), int(out_features), int(chunk_size),
+        int(ignore_index), reduction, bool(return_token_accuracy), bool(return_predicted_tokens))
+    if return_token_accuracy or return_predicted_tokens:
+        return loss, token_accuracy, predicted
+    return loss
 
 
 def _packed_for_causal_lm_loss(hidden_states: torch.Tensor, lm_head: GGUFLinear, labels: torch.Tensor, hidden_size: int,
                                num_items_in_batch: int | torch.Tensor | None = None, ignore_index: int = -100,
                                shift_labels: torch.Tensor | None = None, final_logit_softcapping: float | None = None,
-                               chunk_size: int = _PACKED_LM_HEAD_CHUNK_SIZE, **kwargs: Any) -> torch.Tensor:
-    """Causal-LM loss entry: option guards, label shift, mean vs sum/num_items
-    (gguf_liger_loss.py:269-356).  Unlike the reference, any hidden size that is a multiple of 64 and
+                               return_token_accuracy: bool = False, return_predicted_tokens: bool = False,
+                               chunk_size: int = _PACKED_LM_HEAD_CHUNK_SIZE, **kwargs: Any):
+    """Causal-LM loss entry: option guards, label shift, mean vs sum/num_items, optional token accuracy and predicted
+    tokens (gguf_liger_loss.py:269-356).  Unlike the reference, any hidden size that is a multiple of 64 and
     any natively supported GGML type is accepted (the reference validates 2048 / Q6_K only, :315-323)."""
     if kwargs.get("return_z_loss", False):
         raise RuntimeError("Packed GGUF LM-head loss does not support z-loss output.")
@@ -107,8 +133,6 @@ def _packed_for_causal_lm_loss(hidden_states: torch.Tensor, lm_head: GGUFLinear,
         raise RuntimeError("Packed GGUF LM-head loss does not support LSE square scaling.")
     if final_logit_softcapping is not None:
         raise RuntimeError("Packed GGUF LM-head loss does not support logit softcapping.")
-    if kwargs.get("return_token_accuracy", False) or kwargs.get("return_predicted_tokens", False):
-        raise RuntimeError("Packed GGUF LM-head loss does not produce token accuracy or predicted tokens.")
     if kwargs.get("accum_dtype") not in {None, torch.float32}:
         raise RuntimeError("Packed GGUF LM-head loss supports only FP32 internal accumulation.")
     if not isinstance(lm_head.weight, GGUFQuantizedTensor):
@@ -127,8 +151,11 @@ def _packed_for_causal_lm_loss(hidden_states: torch.Tensor, lm_head: GGUFLinear,
     hidden_states = hidden_states.reshape(-1, hidden_size)
     shift_labels = shift_labels.reshape(-1).to(hidden_states.device)
     reduction = "sum" if num_items_in_batch is not None else "mean"
-    loss = packed_linear_cross_entropy(hidden_states, lm_head.weight, shift_labels, lm_head.weight.quant_type, lm_head.out_features,
-                                       chunk_size, ignore_index, reduction)
+    loss, token_accuracy, predicted_tokens = _PackedLinearCrossEntropyFunction.apply(
+        hidden_states, lm_head.weight.as_subclass(torch.Tensor), shift_labels, int(lm_head.weight.quant_type), int(lm_head.out_features),
+        int(chunk_size), int(ignore_index), reduction, bool(return_token_accuracy), bool(return_predicted_tokens))
     if num_items_in_batch is not None:
         loss = loss / num_items_in_batch
+    if return_token_accuracy or return_predicted_tokens:
+        return loss, None, token_accuracy, predicted_tokens  # (loss, z_loss, accuracy, tokens), gguf_liger_loss.py:352-353
     return loss
