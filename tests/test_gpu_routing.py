@@ -44,6 +44,12 @@ def test_route_plan_all_routes_to_one_expert_and_bad_ids(pkg, dev):
     idx[7, 3] = 99  # outside [0, 16): clamped for memory safety and reported
     *_, status = pkg.fast_moe_routing.build_route_plan(idx.to(dev), 16)
     assert int(status[1]) == 1
+    pkg.fast_moe_routing.VALIDATE_EXPERT_IDS = True  # the debugging switch turns the flag into an error (and a synchronisation)
+    try:
+        with pytest.raises(ValueError):
+            pkg.fast_moe_routing.build_route_plan(idx.to(dev), 16)
+    finally:
+        pkg.fast_moe_routing.VALIDATE_EXPERT_IDS = False
 
 
 @pytest.mark.parametrize("tokens,k,hidden", [(2048, 8, 2048), (257, 6, 4096), (8, 4, 2048), (64, 8, 4096), (5, 1, 256)])

@@ -126,6 +126,21 @@ def fixed_grouped_mmq(x: torch.Tensor, packed_groups: torch.Tensor, quant_type: 
     return _FixedGroupedMmq.apply(x, packed_groups.as_subclass(torch.Tensor), int(quant_type))
 
 
+def fixed_grouped_mmq_grad_input(grad_output: torch.Tensor, packed_groups: torch.Tensor, quant_type: int, in_features: int) -> torch.Tensor:
+    """Input gradient of ``fixed_grouped_mmq``: [..., groups, n] x packed [groups, n, bytes] -> [..., groups, in_features]."""
+    packed_groups = packed_groups.as_subclass(torch.Tensor)
+    _lib.require_device_tensor(grad_output, "fixed grouped cotangent", torch.bfloat16)
+    _lib.require_device_tensor(packed_groups, "fixed grouped payload", torch.uint8)
+    groups, n_group = packed_groups.shape[0], packed_groups.shape[1]
+    if grad_output.ndim < 2 or tuple(grad_output.shape[-2:]) != (groups, n_group) or packed_groups.shape[2] != row_bytes(quant_type, in_features):
+        raise ValueError(f"fixed grouped cotangent {tuple(grad_output.shape)} does not fit packed groups {tuple(packed_groups.shape)} of type {quant_type}")
+    rows = grad_output.numel() // (groups * n_group)
+    dx = torch.empty(*grad_output.shape[:-1], in_features, dtype=torch.bfloat16, device=grad_output.device)
+    _lib.check(_lib.load().ggq_fixed_grouped_mmq_grad_input(grad_output.data_ptr(), packed_groups.data_ptr(), quant_type, rows, groups, n_group, in_features,
+                                                            dx.data_ptr(), _lib.stream_handle(grad_output.device)))
+    return dx
+
+
 def _workspace(device, rows: int, groups: int, experts: int, n_total: int, k: int, r: int) -> torch.Tensor:
     nbytes = _lib.load().ggq_lora_workspace_bytes(rows, groups, experts, n_total, k, r)
     return torch.empty(nbytes, dtype=torch.uint8, device=device)

@@ -18,6 +18,11 @@ import torch
 from . import _lib
 
 
+# set to True to wait for the device after every plan and raise on expert ids outside [0, num_experts) (the sort clamps such
+# ids so that no access leaves its buffers and only flags them in ``status[1]``, so that no call has to synchronise)
+VALIDATE_EXPERT_IDS = False
+
+
 @dataclass(frozen=True)
 class ExpertRoutingPlan:
     selected_hidden_states: torch.Tensor | None  # [routes, hidden] bf16, expert-sorted (None: prepared with gather=False)
@@ -61,6 +66,8 @@ def build_route_plan(top_k_index: torch.Tensor, num_experts: int):
                                   sorted_ids.data_ptr(), perm.data_ptr(), inv.data_ptr(), counts.data_ptr(), ends.data_ptr(),
                                   active_ids.data_ptr(), active_ends.data_ptr(), status.data_ptr(), ws.data_ptr(), ws.numel(),
                                   _lib.stream_handle(dev)))
+    if VALIDATE_EXPERT_IDS and int(status[1]):
+        raise ValueError(f"expert ids outside [0, {num_experts}) in the top-k index matrix")
     return sorted_ids, perm, inv, counts, ends, active_ids, active_ends, status
 
 
