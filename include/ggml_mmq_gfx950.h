@@ -41,6 +41,12 @@ const char* ggq_last_error(void);
 int ggq_profile_begin(void);
 int ggq_profile_end(float* ms, int* qt, int* mode, int* epilogue, int capacity);
 
+/* Test aid with no counterpart in the reference: force the kernel family of the grouped Q4_K launches that follow (0 = tall
+ * tiles, 1 = the wide / tall tile mix, 3 = the kernels whose MFMA waves decode the weights themselves, wherever their operand
+ * conditions hold; -1 = the library's own choice, the default).  A process-wide setting, not thread safe; results are the
+ * same to the stated tolerances whatever is chosen. */
+int ggq_debug_force_grouped_shape(int shape);
+
 /* fast_lora.py:24-31 (_NATIVE_MMQ_QUANT_TYPES / supports_native_mmq): 1 if this library has kernels
  * for the GGML type id. */
 int ggq_supports_quant_type(int qt);

@@ -26,3 +26,15 @@ def dev():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     return torch.device("cuda:0")
+
+
+@pytest.fixture
+def force_grouped_shape(pkg):
+    """Forces the kernel family of the grouped Q4_K launches for one test ("" / None = the library's own choice)."""
+    lib = pkg._lib.load()
+
+    def force(shape):
+        pkg._lib.check(lib.ggq_debug_force_grouped_shape(-1 if shape in ("", None) else int(shape)))
+
+    yield force
+    lib.ggq_debug_force_grouped_shape(-1)

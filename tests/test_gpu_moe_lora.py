@@ -107,16 +107,13 @@ def test_constant_byte_iq2_xxs_experts(pkg, dev):
     torch.testing.assert_close(h.grad.double().cpu(), want["dx"], rtol=1e-2, atol=1e-2)
 
 
-@pytest.mark.parametrize("qt,r,shape,n", [(gb.Q4_K, 16, "", 192), (gb.Q4_K, 16, "", 256), (gb.Q4_K, 16, "3", 256), (gb.Q4_K, 16, "1", 256), (gb.Q4_K, 16, "2", 192),
+@pytest.mark.parametrize("qt,r,shape,n", [(gb.Q4_K, 16, "", 192), (gb.Q4_K, 16, "", 256), (gb.Q4_K, 16, "3", 256), (gb.Q4_K, 16, "1", 256), (gb.Q4_K, 16, "0", 192),
                                           (gb.Q8_0, 4, "", 192), (gb.Q6_K, 8, "", 192), (gb.IQ2_XXS, 16, "", 192)])
-def test_grouped_lora_projection_all_gradients(pkg, dev, qt, r, shape, n, monkeypatch):
+def test_grouped_lora_projection_all_gradients(pkg, dev, qt, r, shape, n, force_grouped_shape):
     # ragged groups including empty experts, a group larger than one 128-row tile, and inactive planes.
-    # Q4_K runs forward in the kernel whose MFMA waves decode the weights themselves; shape "3" with n = 256 also the
-    # grad-input (that kernel takes contraction lengths in whole groups of four 64-row steps, and is the default only
-    # without a LoRA term); shape "1": the wide / tall tile mix, "2": the 128 x 128 tiles (two workgroups per
-    # compute unit)
-    if shape:
-        monkeypatch.setenv("GGQ_GROUPED_SHAPE", shape)
+    # Q4_K runs in the kernels whose MFMA waves decode the weights themselves (the grad-input one takes an even number of
+    # whole 64-row contraction steps: n = 192 as a pair, n = 256); shape "1": the wide / tall tile mix, "0": tall tiles
+    force_grouped_shape(shape)
     ml = pkg.fast_moe_lora
     e_total, k = 8, 512
     sizes = [0, 150, 3, 0, 129, 1, 64, 0]
@@ -159,14 +156,13 @@ def test_grouped_lora_projection_all_gradients(pkg, dev, qt, r, shape, n, monkey
 
 @pytest.mark.parametrize("top_k,rank,pair,qt,shape", [(8, 16, True, gb.Q4_K, ""), (3, 4, True, gb.Q4_K, ""), (1, 16, False, gb.Q4_K, ""),
                                                       (8, 0, True, gb.Q4_K, ""), (8, 16, True, gb.Q4_K, "1"), (3, 16, True, gb.Q4_K, "0"),
-                                                      (2, 8, True, gb.Q4_K, "2"), (8, 16, True, gb.Q6_K, ""), (3, 4, False, gb.IQ2_XXS, "")])
-def test_routed_projection_reads_tokens_in_place(pkg, dev, top_k, rank, pair, qt, shape, monkeypatch):
+                                                      (2, 8, True, gb.Q4_K, "0"), (8, 16, True, gb.Q6_K, ""), (3, 4, False, gb.IQ2_XXS, "")])
+def test_routed_projection_reads_tokens_in_place(pkg, dev, top_k, rank, pair, qt, shape, force_grouped_shape):
     # The gate/up launch that reads the token matrix through the routing permutation against the same launch on the
     # gathered copy: outputs, token gradients (summed over each token's routes) and factor gradients are the same bits.
     # Skewed routing: some experts receive no route, one receives more than a 192-row tile.  Every kernel shape of the
     # forward launch takes the index (the decoding-wave kernel by default for Q4_K, the tile kernels otherwise).
-    if shape:
-        monkeypatch.setenv("GGQ_GROUPED_SHAPE", shape)
+    force_grouped_shape(shape)
     ml, mr = pkg.fast_moe_lora, pkg.fast_moe_routing
     tokens, k, n, experts = 211, 512, 256, 12
     gen = torch.Generator().manual_seed(977 + top_k)
@@ -217,13 +213,12 @@ def test_routed_projection_reads_tokens_in_place(pkg, dev, top_k, rank, pair, qt
         assert_close_bf16(got[-2], o["da"], "in-place dA against the oracle")
 
 
-@pytest.mark.parametrize("shape", ["", "0", "1", "2", "3"])
-def test_q4k_grouped_identity_reproduces_decoded_rows_exactly(pkg, dev, shape, monkeypatch):
+@pytest.mark.parametrize("shape", ["", "0", "1", "3"])
+def test_q4k_grouped_identity_reproduces_decoded_rows_exactly(pkg, dev, shape, force_grouped_shape):
     # One-hot rows through every Q4_K kernel shape of the grouped launches (the decoding-wave kernels by default): each
     # output is a single product 1 * w, so the in-register decoders are compared with the oracle element by element, for
     # arbitrary block bytes (every 6-bit scale split), in forward (pair) and in grad-input.
-    if shape:
-        monkeypatch.setenv("GGQ_GROUPED_SHAPE", shape)
+    force_grouped_shape(shape)
     ml = pkg.fast_moe_lora
     e, n, k = 3, 256, 512
     p1, p2 = _expert_payload(71, gb.Q4_K, e, n, k, "random"), _expert_payload(72, gb.Q4_K, e, n, k, "random")

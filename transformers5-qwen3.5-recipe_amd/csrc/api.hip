@@ -3,7 +3,6 @@
 #include "../../include/ggml_mmq_gfx950.h"
 
 #include <algorithm>
-#include <stdlib.h>
 
 #include "launch.h"
 #include "mmq_host.h"
@@ -27,6 +26,8 @@ struct Bump {  // carve 256-byte aligned pieces out of the caller's workspace
 };
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+int g_shape_override = -1;  // ggq_debug_force_grouped_shape: -1 = the automatic choice
 
 int check_weights(const char* what, int qt, const void* w, int64_t k) {
     if (!w) return set_error(GGQ_ERR_NULL, "%s: packed weight pointer is null", what);
@@ -55,6 +56,12 @@ int ggq_profile_end(float* ms, int* qt, int* mode, int* epilogue, int capacity) 
     return profile_end(ms, qt, mode, epilogue, capacity);
 }
 
+int ggq_debug_force_grouped_shape(int shape) {
+    if (shape != -1 && shape != kShapeTall && shape != kShapeWide && shape != kShapeDirect) return set_error(GGQ_ERR_SHAPE, "debug_force_grouped_shape: unknown shape %d", shape);
+    g_shape_override = shape;
+    return GGQ_OK;
+}
+
 int ggq_supports_quant_type(int qt) { return packed_row_bytes(qt, 256) > 0 ? 1 : 0; }
 
 int64_t ggq_row_bytes(int qt, int64_t k) { return block_multiple(qt, k) ? packed_row_bytes(qt, k) : -1; }
@@ -75,17 +82,15 @@ static int launch_wide_and_tall(int qt, int mode, MmqParams& p, int rows, int n,
     return launch_mmq_mixed(mode, p, s);
 }
 
-// Q4_K forward over expert groups that average at most 256 rows runs the direct kernel when `direct_ok`;
-// otherwise groups that average at most 192 rows run the Q4_K tile kernel in its wide shape, mixed with tall
-// tiles for their larger groups.  GGQ_GROUPED_SHAPE is a tuning aid, read per call: 0 = tall tiles, 1 = the
-// wide / tall mix, 2 = half tiles, 3 = the direct kernel (forward) whatever the group sizes.
+// Q4_K over expert groups that average at most 256 rows runs the direct kernels (the MFMA waves decode the weights
+// themselves) when the operands allow (`direct_ok`); otherwise groups that average at most 192 rows run the Q4_K tile kernel
+// in its wide shape, mixed with tall tiles for their larger groups; everything else runs tall tiles.
 static int pick_shape(int qt, int64_t rows, int64_t groups, bool direct_ok) {
     if (qt != 12 /* GGML Q4_K */) return kShapeTall;
-    const char* e = getenv("GGQ_GROUPED_SHAPE");
-    const int forced = e && *e ? atoi(e) : -1;
+    const int forced = g_shape_override;  // a test aid
     if (direct_ok && (forced == kShapeDirect || (forced < 0 && groups > 0 && rows <= 256 * groups))) return kShapeDirect;
     if (forced == kShapeTall || !(groups > 0 && rows <= 192 * groups)) return kShapeTall;
-    return forced == kShapeHalf ? kShapeHalf : kShapeWide;
+    return kShapeWide;
 }
 
 // Direct shape: a workgroup walks a run of column tiles of its row tile as one stream of steps.  Short tiles (few
@@ -306,10 +311,8 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
     Bump bump{(char*)ws, ws_bytes, 0};
 
     MmqParams p;
-    // the direct kernel moves the cotangents with aligned 16-byte accesses and takes whole groups of four 64-row steps
-    // (with a LoRA term its once-per-tile operand fetch makes it no faster than the tile kernel at the shapes measured:
-    // GGQ_GROUPED_SHAPE=3 still selects it)
-    const bool direct_ok = aligned16(dy1) && (!dy2 || aligned16(dy2)) && n % 64 == 0 && (nseg * (n / 64)) % 4 == 0 && n < (1 << 22) &&
+    // the direct kernel moves the cotangents with aligned 16-byte accesses and takes an even number of whole 64-row steps
+    const bool direct_ok = aligned16(dy1) && (!dy2 || aligned16(dy2)) && n % 64 == 0 && (nseg * (n / 64)) % 2 == 0 && n < (1 << 22) &&
                            (!lora_a || aligned16(lora_a)) && k % 8 == 0;
     if (int rc = init_params(p, qt, kModeNN, (int)rows, (int)n, (int)k, nseg, pick_shape(qt, rows, groups, direct_ok))) return rc;
     p.a[0] = (const bf16_t*)dy1, p.a[1] = (const bf16_t*)dy2, p.lda = n;

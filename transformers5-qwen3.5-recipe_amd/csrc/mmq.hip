@@ -1,13 +1,10 @@
 // Host launchers for the packed-weight tile kernel, the expert row-tile table and the error state.
 #include "mmq_tile.h"
-#include "mmq_direct.h"
-#include "mmq_direct_nn.h"
 #include "mmq_direct8.h"
 #include "mmq_direct8_nn.h"
 #include "launch.h"
 
 #include <stdarg.h>
-#include <stdlib.h>
 #include <stdio.h>
 
 namespace ggq {
@@ -200,14 +197,10 @@ static int launch_one(const MmqParams& p, hipStream_t s) {
                                (EPI != kEpiStore ? Tile<SH>::kTM * 16 : 0);
     static bool attr_set = false;  // per instantiation; the attribute is a property of the function
     if (!attr_set) {
-        hipError_t e;
-        if constexpr (SH == kShapeHalf) e = hipFuncSetAttribute((const void*)mmq_half_kernel<QT, MODE, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
-        else e = hipFuncSetAttribute((const void*)mmq_tile_kernel<QT, MODE, EPI, SH>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
-        if (e != hipSuccess) return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", kSmemBytes);
+        if (hipFuncSetAttribute((const void*)mmq_tile_kernel<QT, MODE, EPI, SH>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess) return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", kSmemBytes);
         attr_set = true;
     }
-    if constexpr (SH == kShapeHalf) hipLaunchKernelGGL((mmq_half_kernel<QT, MODE, EPI>), dim3((unsigned)grid), dim3(Tile<kShapeHalf>::kThreadsWG), kSmemBytes, s, p);
-    else hipLaunchKernelGGL((mmq_tile_kernel<QT, MODE, EPI, SH>), dim3((unsigned)grid), dim3(kThreads), kSmemBytes, s, p);
+    hipLaunchKernelGGL((mmq_tile_kernel<QT, MODE, EPI, SH>), dim3((unsigned)grid), dim3(kThreads), kSmemBytes, s, p);
     if (t) (void)hipEventRecord(t->stop, s);
     return check_launch("mmq_tile_kernel");
 }
@@ -222,8 +215,8 @@ static int launch_direct(const MmqParams& p, hipStream_t s) {
     if (total <= 0) return GGQ_OK;
     const int64_t grid = total * 8;
     if (grid > 0x7FFFFFF0) return set_error(GGQ_ERR_SHAPE, "mmq: too many tiles for one launch");
-    if (MODE == kModeNN && ((p.n & 63) || ((p.nseg * p.steps_per_seg) & 3)))
-        return set_error(GGQ_ERR_SHAPE, "mmq: the direct grad-input kernel needs whole groups of four 64-row steps");
+    if (MODE == kModeNN && ((p.n & 63) || ((p.nseg * p.steps_per_seg) & 1)))
+        return set_error(GGQ_ERR_SHAPE, "mmq: the direct grad-input kernel needs an even number of whole 64-row steps");
     TimedLaunch* t = nullptr;
     if (g_timing && g_timed_count < kMaxTimedLaunches) {
         t = &g_timed[g_timed_count];
@@ -232,23 +225,18 @@ static int launch_direct(const MmqParams& p, hipStream_t s) {
         g_timed_count++;
         (void)hipEventRecord(t->start, s);
     }
-    static const bool eight = !(getenv("GGQ_DIRECT8") && atoi(getenv("GGQ_DIRECT8")) == 0);
-    const bool use8 = eight;
-    const int kSmemBytes = use8 ? (MODE == kModeNT ? Direct8::kLdsBytes : Direct8NN::kLdsBytes) : MODE == kModeNT ? Direct::kLdsBytes : DirectNN::kLdsBytes;
-    const void* fn = use8 ? (MODE == kModeNT ? (const void*)mmq_direct8_q4k_kernel : (const void*)mmq_direct8_nn_q4k_kernel)
-                          : MODE == kModeNT ? (const void*)mmq_direct_q4k_kernel : (const void*)mmq_direct_nn_q4k_kernel;
+    constexpr int kSmemBytes = MODE == kModeNT ? Direct8::kLdsBytes : Direct8NN::kLdsBytes;
+    const void* fn = MODE == kModeNT ? (const void*)mmq_direct8_q4k_kernel : (const void*)mmq_direct8_nn_q4k_kernel;
     static bool attr_set = false;  // per instantiation
     if (!attr_set) {
         if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess)
             return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", kSmemBytes);
         attr_set = true;
     }
-    if (use8 && MODE == kModeNN) hipLaunchKernelGGL(mmq_direct8_nn_q4k_kernel, dim3((unsigned)grid), dim3(Direct8NN::kThreadsWG), kSmemBytes, s, p);
-    else if (use8) hipLaunchKernelGGL(mmq_direct8_q4k_kernel, dim3((unsigned)grid), dim3(Direct8::kThreadsWG), kSmemBytes, s, p);
-    else if (MODE == kModeNT) hipLaunchKernelGGL(mmq_direct_q4k_kernel, dim3((unsigned)grid), dim3(Direct::kThreadsWG), kSmemBytes, s, p);
-    else hipLaunchKernelGGL(mmq_direct_nn_q4k_kernel, dim3((unsigned)grid), dim3(DirectNN::kThreadsWG), kSmemBytes, s, p);
+    if (MODE == kModeNT) hipLaunchKernelGGL(mmq_direct8_q4k_kernel, dim3((unsigned)grid), dim3(Direct8::kThreadsWG), kSmemBytes, s, p);
+    else hipLaunchKernelGGL(mmq_direct8_nn_q4k_kernel, dim3((unsigned)grid), dim3(Direct8NN::kThreadsWG), kSmemBytes, s, p);
     if (t) (void)hipEventRecord(t->stop, s);
-    return check_launch(MODE == kModeNT ? "mmq_direct_q4k_kernel" : "mmq_direct_nn_q4k_kernel");
+    return check_launch(MODE == kModeNT ? "mmq_direct8_q4k_kernel" : "mmq_direct8_nn_q4k_kernel");
 }
 
 template <int MODE>
@@ -291,17 +279,13 @@ static int launch_qt(int mode, int epi, const MmqParams& p, hipStream_t s) {
             case kEpiStore:
                 if (QT == kQ4_K && p.shape == kShapeDirect) return launch_direct<kModeNT>(p, s);
                 if (QT == kQ4_K && p.shape == kShapeWide) return launch_one<kQ4_K, kModeNT, kEpiStore, 1>(p, s);
-                if (QT == kQ4_K && p.shape == kShapeHalf) return launch_one<kQ4_K, kModeNT, kEpiStore, 2>(p, s);
                 return launch_one<QT, kModeNT, kEpiStore, 0>(p, s);
-            case kEpiCeStats: return launch_one<QT, kModeNT, kEpiCeStats, 0>(p, s);
-            case kEpiCeGrad: return launch_one<QT, kModeNT, kEpiCeGrad, 0>(p, s);
         }
     } else {
         switch (epi) {
             case kEpiStore:
                 if (QT == kQ4_K && p.shape == kShapeDirect) return launch_direct<kModeNN>(p, s);
                 if (QT == kQ4_K && p.shape == kShapeWide) return launch_one<kQ4_K, kModeNN, kEpiStore, 1>(p, s);
-                if (QT == kQ4_K && p.shape == kShapeHalf) return launch_one<kQ4_K, kModeNN, kEpiStore, 2>(p, s);
                 return launch_one<QT, kModeNN, kEpiStore, 0>(p, s);
             case kEpiAccumF32: return launch_one<QT, kModeNN, kEpiAccumF32, 0>(p, s);
         }

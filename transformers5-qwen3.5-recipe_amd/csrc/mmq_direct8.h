@@ -1,17 +1,26 @@
-// Q4_K forward ("NT") tile kernel with register decoding and TWO waves per SIMD.
+// Q4_K forward ("NT") tile kernel in which the waves that issue the MFMAs decode the packed weights themselves.
 //
 //   C[m, n] = sum_k A[m, k] * W[n, k]  (+ s * LA[m, :] . LB[n, :])
 //
-// Same data flow as the four-wave direct kernel (mmq_direct.h): the waves that issue the MFMAs decode the packed
-// weights themselves, in registers, straight into MFMA operands; the A tile goes global -> LDS directly through a
-// ring of four stages; a workgroup walks a run of column tiles of its row tile as one stream of steps.  The
-// difference is the split of the 192 x 256 tile: a workgroup is 512 lanes = eight waves, two per SIMD with 256
-// registers each, and wave w owns the 32 columns at 32 w of every row (up to six 32-row blocks of 32x32x16
-// accumulators).  A single wave issues at most one instruction per four to five cycles, whatever its kind, so a
-// step's decode arithmetic, LDS reads, loads and waits (about eight instructions per MFMA) cannot hide behind
-// that wave's own MFMAs; with two waves per SIMD one wave's MFMAs run while the other decodes, reads and waits.
-// Every weight is still decoded exactly once per row tile; the price is that all eight waves read the whole A
-// tile from LDS (twice the operand traffic of the four-wave split, well inside the LDS bandwidth).
+// A workgroup is 512 lanes = eight waves, two per SIMD with 256 registers each, and computes tiles of up to 192 rows x
+// 256 columns; wave w owns the 32 columns at 32 w of every row: up to six 32-row blocks of MFMA 32x32x16 accumulators.
+// The kernel is instantiated per number of live 32-row blocks, so an expert group of any size up to 192 rows is one row
+// tile and issues no MFMA on empty blocks.  Per contraction step of 64
+//   * the A tile goes global -> LDS directly (no registers), three steps ahead, through a ring of four stages; rows are
+//     unpadded with XOR-swizzled 16-byte slots (a_slot), every wave reads all of them;
+//   * the packed quant bytes go global -> LDS directly as well, half a 256-wide block (two steps) of the wave's 32
+//     columns at a time, four lanes per row so that a row's bytes are requested by adjacent lanes, into a ring of three
+//     wave-private buffers; block headers are loaded into registers;
+//   * a lane reads its 16 quant bytes of the step from its wave's buffer and decodes them in registers into the operands
+//     of the step's four MFMA sub-steps (mmq_direct.h).  No decoded weight ever touches LDS.
+// A single wave issues at most one instruction per four to five cycles, whatever its kind, so a step's decode
+// arithmetic, LDS reads, requests and waits (about eight instructions per MFMA) cannot hide behind that wave's own
+// MFMAs; with two waves per SIMD one wave's MFMAs run while the other decodes, reads and waits.
+// The weights are the MFMA's first operand, so a lane's accumulator registers hold four consecutive columns of one row;
+// a finished row block goes through a wave-private LDS block and leaves as 64-byte row pieces.  The LoRA term is added
+// there.  A workgroup takes a run of column tiles of its row tile and treats their steps as one stream, so the requests
+// of a tile's first steps are in flight while the tile before it finishes.  The requests are inline-asm loads the
+// compiler does not track; the step waits for them with exact counts (vector memory operations complete in issue order).
 #pragma once
 #include "mmq_direct.h"
 

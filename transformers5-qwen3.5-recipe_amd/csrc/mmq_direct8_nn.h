@@ -261,7 +261,7 @@ struct Direct8NN {
                         if (K == 1) *(uint4*)(d_my_row + Q * 16) = make_uint4(o[0], o[1], o[2], o[3]);
                     };
                     auto decode_slots = [&](auto i_c) __attribute__((always_inline)) {  // sub-step I's share
-                        return [&, i_c](auto rb_c) __attribute__((always_inline)) {
+                        return [&](auto rb_c) __attribute__((always_inline)) {
                             constexpr int T = decltype(i_c)::value * LIVE + decltype(rb_c)::value;
                             auto maybe = [&](auto hp_c) __attribute__((always_inline)) {
                                 if constexpr (decltype(hp_c)::value * 3 * LIVE / 8 == T) decode_piece(hp_c);

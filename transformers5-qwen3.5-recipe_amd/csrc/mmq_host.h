@@ -59,17 +59,15 @@ struct FactorGradParams {
 
 constexpr int kBM = 256, kBN = 128, kBK = 64;  // the tall tile shape (dense launches, large expert groups)
 constexpr int kWideBM = 128, kWideBN = 256;    // the wide tile shape (Q4_K expert groups of about a hundred rows)
-constexpr int kDirectBM = 192, kDirectBN = 256;  // the direct shape (Q4_K forward: the MFMA waves decode the weights themselves)
-constexpr int kShapeTall = 0, kShapeWide = 1, kShapeHalf = 2, kShapeDirect = 3;
+constexpr int kDirectBM = 192, kDirectBN = 256;  // the direct shape (Q4_K expert groups: the MFMA waves decode the weights themselves)
+constexpr int kShapeTall = 0, kShapeWide = 1, kShapeDirect = 3;
 constexpr int kLdsStride = kBK + 8;  // bf16 elements per LDS row: 144 bytes keeps 128-bit reads conflict-free
 constexpr int kThreads = 1024;  // waves 0..7 run the MFMAs, waves 8..15 load and decode
 
 enum : int { kModeNT = 0, kModeNN = 1 };
 enum : int {
     kEpiStore = 0,     // C (bf16) = acc
-    kEpiAccumF32 = 1,  // C32 (fp32) = C32 * row_scale[m] + acc  (row_scale null: += acc)
-    kEpiCeStats = 2,   // per-row partial (max, sum exp) over the tile's columns + target logit
-    kEpiCeGrad = 3     // C (bf16) = (exp(acc - lse[m]) - [col == label[m]]) * row_scale[m]
+    kEpiAccumF32 = 1   // C32 (fp32) = C32 * row_scale[m] + acc  (row_scale null: += acc)
 };
 
 struct MmqParams {
@@ -97,7 +95,7 @@ struct MmqParams {
     int max_row_tiles2;
     int col_tiles_per_seg2;
     int col_tiles_per_wg;   // direct shape: column tiles one workgroup walks through (>= 1)
-    int shape;  // kShapeTall / kShapeWide / kShapeHalf / kShapeDirect: which kernel the sizes above are for
+    int shape;  // kShapeTall / kShapeWide / kShapeDirect: which kernel the sizes above are for
     // LoRA
     const bf16_t* la;     // [rows, r_pad]  (x A^T in NT, dY B in NN)
     const bf16_t* lb;     // per expert: NT [cols_total, r_pad] (rows of B); NN [lora_rank, k] (the factor A as it is)
@@ -105,14 +103,7 @@ struct MmqParams {
     int r_pad;            // multiple of 16, <= 64; 0 = no LoRA
     int lora_rank;        // NN mode: rows of the factor A that exist (the tile's rows up to r_pad are zero)
     float lora_scale;
-    // cross-entropy epilogues
-    const int64_t* labels;     // [m]
-    const float* lse;          // [m]
-    const float* row_scale;    // [m]  (1/n_non_ignore or 1, 0 for ignored rows)
-    float2* ce_partials;       // [m, ce_partials_ld] (max, sumexp)
-    float* ce_target_logit;    // [m]
-    int ce_partials_ld, ce_col_offset, ce_partial_offset;
-    int64_t ignore_index;
+    const float* row_scale;    // accumulate epilogue: [m] factors of the old accumulator rows (null: 1)
 };
 
 constexpr int kMaxTimedLaunches = 8192;

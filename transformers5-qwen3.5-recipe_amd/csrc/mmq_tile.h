@@ -100,7 +100,7 @@ struct TileCtx {  // wave-uniform description of the tile this workgroup compute
     uint32_t as_lds;  // LDS byte address of `as`
     bool a_fast;      // A rows can be moved with aligned 16-byte accesses and every step is whole
     const uint2* grid;
-    const float4* row_meta;  // cross-entropy epilogues: per tile row (lse, row scale, label as int bits, -), staged in LDS
+    const float* row_scale;  // accumulate epilogue: the tile rows' factors, staged in LDS
 };
 
 // (segment, first contraction index) of a step; at most two segments.
@@ -117,21 +117,18 @@ __device__ __forceinline__ void step_origin(const MmqParams& p, int step, int& s
 // row blocks wave_m and wave_m + kWavesM and the 64 columns at 64 * wave_n.
 template <int SH>
 struct Tile {
-static constexpr int kTM = SH == 0 ? 256 : 128, kTN = SH == 1 ? 256 : 128;
+static constexpr int kTM = SH == 0 ? 256 : 128, kTN = SH == 0 ? 128 : 256;
 static constexpr int kWavesM = kTM / 64, kWavesN = kTN / 64;
-// SH = 2: 128 x 128 ("half"): four consumer and four producer waves, half the registers and less than half
-// the LDS of a compute unit, so two workgroups share one: each has its own barrier, and one's waits, set-up
-// and stores run under the other's steps.
-static constexpr int kCW = kWavesM * kWavesN;       // consumer waves (8, 8, 4), as many producer waves
+static constexpr int kCW = kWavesM * kWavesN;       // consumer waves (8), as many producer waves
 static constexpr int kProducerLanes = 64 * kCW;
 static constexpr int kThreadsWG = 128 * kCW;
 static constexpr int kAStageBytes = kTM * kARowBytes;   // 32 KB / 16 KB
 // LDS ring of A tiles: the loads of a step are issued kAStages - 1 steps ahead of its MFMAs.  Memory latency
 // under load is about two thousand cycles; the wide shape's short steps need the longer ring.
-static constexpr int kAStages = SH == 0 ? 3 : SH == 1 ? 5 : 2;
+static constexpr int kAStages = SH == 0 ? 3 : 5;
 static constexpr int kAhead = kAStages - 1;
 static constexpr int kAGroups = kTM / 8;                // 8-row groups (one direct-to-LDS instruction each)
-static constexpr int kGroupsPerWave = kAGroups / kCW;   // groups one consumer wave moves per step (4 / 2 / 4)
+static constexpr int kGroupsPerWave = kAGroups / kCW;   // groups one consumer wave moves per step (4 / 2)
 // W buffer: forward [output column][64 + 8]; grad-input [contraction row][columns + 32], as the rows are
 // decoded (the consumers transpose on the way out of LDS).  Sized for the larger of the two.
 static constexpr int kNnPitch = kTN + 32;
@@ -140,7 +137,7 @@ static constexpr int kNnPitch = kTN + 32;
 // row and run, and would otherwise meet four deep on the same banks) hit distinct banks, while the four
 // rows of a transposing read keep their 32-byte pieces on distinct banks.
 static __device__ __forceinline__ int nn_chunk(int row, int q) {
-    const int sw = SH == 0 ? (((row >> 2) & 3) ^ (row & 1)) : SH == 1 ? ((row & 1) ^ (((q >> 4) & 1) << 1)) : (row & 3);
+    const int sw = SH == 0 ? (((row >> 2) & 3) ^ (row & 1)) : ((row & 1) ^ (((q >> 4) & 1) << 1));
     return q ^ sw;
 }
 static constexpr int kBTile = kTN * kLdsStride > kBK * kNnPitch ? kTN * kLdsStride : kBK * kNnPitch;  // bf16 elements
@@ -821,11 +818,10 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
     // ---- epilogue.  acc[rb][cb][i]: tile row = 32*(kWavesM*rb + wave_m) + 8*(i/4) + 4*lane_h + (i%4),
     //                                 tile col = 64*wave_n + 32*cb + lane_c
     const int col_base = c.col0 + wave_n * 64 + lane_c;
-    if (EPI == kEpiStore || EPI == kEpiAccumF32 || EPI == kEpiCeGrad) {
+    {
         // everything that does not depend on the element is read once, up front
         const int64_t ldc = p.ldc;
         char* const cbase = (char*)p.c[EPI == kEpiStore ? c.seg_c : 0];
-        const int64_t ce_off = p.ce_col_offset;
         const int rows_valid = c.rows_valid;
         const bool col_ok[kColBlocks] = {col_base < c.out_cols, col_base + 32 < c.out_cols};
 #pragma unroll
@@ -837,56 +833,15 @@ static __device__ __forceinline__ void consume(const MmqParams& p, const TileCtx
                 const int dr = (i >> 2) * 8 + (i & 3);  // uniform row step inside the block
                 if (r_lane + dr >= rows_valid) continue;
                 const int64_t elem = lane_elem + (int64_t)dr * ldc;
-                float lse = 0.f, rs = 0.f;
-                int64_t label = -1;
-                if (EPI == kEpiCeGrad) {
-                    const float4 meta = c.row_meta[r_lane + dr];
-                    lse = meta.x, rs = meta.y, label = (int64_t)__float_as_int(meta.z);
-                }
-                if (EPI == kEpiAccumF32) rs = p.row_scale ? c.row_meta[r_lane + dr].y : 1.0f;
+                float rs = 1.0f;
+                if (EPI == kEpiAccumF32 && p.row_scale) rs = c.row_scale[r_lane + dr];
 #pragma unroll
                 for (int cb = 0; cb < kColBlocks; cb++) {
                     if (!col_ok[cb]) continue;
                     const float v = acc[rb][cb][i];
-                    if (EPI == kEpiStore) {
-                        ((bf16_t*)cbase)[elem + cb * 32] = to_bf16(v);
-                    } else if (EPI == kEpiAccumF32) {
-                        ((float*)cbase)[elem + cb * 32] = fmaf(((float*)cbase)[elem + cb * 32], rs, v);
-                    } else {
-                        const float logit = bf16_to_f32(to_bf16(v));  // the path's logits are bf16 values
-                        float g = __expf(logit - lse);
-                        if ((int64_t)(col_base + cb * 32) + ce_off == label) g -= 1.0f;
-                        ((bf16_t*)cbase)[elem + cb * 32] = to_bf16(g * rs);
-                    }
+                    if (EPI == kEpiStore) ((bf16_t*)cbase)[elem + cb * 32] = to_bf16(v);
+                    else ((float*)cbase)[elem + cb * 32] = fmaf(((float*)cbase)[elem + cb * 32], rs, v);
                 }
-            }
-        }
-    } else {  // kEpiCeStats
-#pragma unroll
-        for (int rb = 0; rb < LIVE; rb++) {
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int r = 32 * (kWavesM * rb + wave_m) + (i >> 2) * 8 + lane_h * 4 + (i & 3);
-                const bool row_ok = r < c.rows_valid;
-                const int64_t grow = c.row_begin + (row_ok ? r : 0);
-                const int64_t label = row_ok ? (int64_t)__float_as_int(c.row_meta[r].z) : -1;
-                float v[kColBlocks];
-                float mx = -INFINITY;
-#pragma unroll
-                for (int cb = 0; cb < kColBlocks; cb++) {
-                    const int col = col_base + cb * 32;
-                    v[cb] = col < c.out_cols ? bf16_to_f32(to_bf16(acc[rb][cb][i])) : -INFINITY;
-                    mx = fmaxf(mx, v[cb]);
-                    if (row_ok && col < c.out_cols && (int64_t)(col + p.ce_col_offset) == label) p.ce_target_logit[grow] = v[cb];
-                }
-                // reduce over the 32 lanes that share this row (lanes with equal lane_h)
-                mx = half_wave_max(mx);
-                float sum = 0.f;
-#pragma unroll
-                for (int cb = 0; cb < kColBlocks; cb++) sum += v[cb] == -INFINITY ? 0.f : __expf(v[cb] - mx);
-                sum = half_wave_sum(sum);
-                if (row_ok && lane_c == 0)
-                    p.ce_partials[grow * p.ce_partials_ld + p.ce_partial_offset + c.col_tile * 2 + wave_n] = make_float2(mx, sum);
             }
         }
     }
@@ -938,10 +893,10 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
     c.bs = (bf16_t*)(smem_raw + kAStages * kAStageBytes);
     uint2* grid_lds = (uint2*)(smem_raw + kTileLdsBytes);  // the decoder's tables, IQ2_XXS only
     c.grid = grid_lds;
-    // what the cross-entropy epilogues need per row, read once per tile: one dependent global load per row and lane in
-    // the epilogue costs a memory round trip each
-    float4* row_meta = (float4*)(smem_raw + kTileLdsBytes + (QT == kIQ2_XXS ? Fmt<kIQ2_XXS>::kTableWords * 4 : 0));
-    c.row_meta = row_meta;
+    // the accumulate epilogue's factor per tile row, read once per tile: one dependent global load per row and lane in the
+    // epilogue costs a memory round trip each
+    float* row_scale = (float*)(smem_raw + kTileLdsBytes + (QT == kIQ2_XXS ? Fmt<kIQ2_XXS>::kTableWords * 4 : 0));
+    c.row_scale = row_scale;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps control flow scalar
@@ -1010,14 +965,7 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
             }
         }
         if (EPI == kEpiAccumF32 && p.row_scale) {  // the factor that rescales the accumulator row before the addition
-            for (int r = tid; r < kTM; r += kThreadsWG) row_meta[r] = make_float4(0.f, p.row_scale[c.row_begin + min(r, c.rows_valid - 1)], 0.f, 0.f);
-        }
-        if (EPI == kEpiCeStats || EPI == kEpiCeGrad) {
-            for (int r = tid; r < kTM; r += kThreadsWG) {
-                const int64_t grow = c.row_begin + min(r, c.rows_valid - 1);
-                row_meta[r] = make_float4(EPI == kEpiCeGrad ? p.lse[grow] : 0.f, EPI == kEpiCeGrad ? p.row_scale[grow] : 0.f,
-                                          __int_as_float((int)p.labels[grow]), 0.f);
-            }
+            for (int r = tid; r < kTM; r += kThreadsWG) row_scale[r] = p.row_scale[c.row_begin + min(r, c.rows_valid - 1)];
         }
         __syncthreads();  // LoRA tiles, the codebook tables and the row values are visible
     };
@@ -1043,12 +991,6 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
 template <int QT, int MODE, int EPI, int SH>
 __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_waves_per_eu(4, 4))) void mmq_tile_kernel(const MmqParams p) {
     Tile<SH>::template run<QT, MODE, EPI>(p);
-}
-
-// The half shape: eight waves, two workgroups to a compute unit.
-template <int QT, int MODE, int EPI>
-__global__ __launch_bounds__(512, 2) __attribute__((amdgpu_waves_per_eu(4, 4))) void mmq_half_kernel(const MmqParams p) {
-    Tile<kShapeHalf>::template run<QT, MODE, EPI>(p);
 }
 
 // Grouped launch with both shapes in one grid: wide tiles for the row tiles of table `tiles`, tall tiles
