@@ -27,6 +27,75 @@ import __graft_entry__
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
+SEED = 19260817  # + the index of the BASELINE configuration; every input is drawn on the host from this seed
+
+_TYPE_NAMES = {8: "Q8_0", 10: "Q2_K", 11: "Q3_K", 12: "Q4_K", 13: "Q5_K", 14: "Q6_K", 16: "IQ2_XXS"}
+
+
+def kernel_name(qt: int, mode: int, epi: int, shape: int) -> str:
+    """Name of the kernel a profiled launch ran, from the record ggq_profile_end returns for it."""
+    direction = "forward" if mode == 0 else "grad_input"
+    if shape == 3:
+        return "mmq_direct8_q4k_kernel (Q4_K, forward)" if mode == 0 else "mmq_direct8_nn_q4k_kernel (Q4_K, grad_input)"
+    if shape == 4:
+        return f"mmq_mixed_kernel<Q4_K, {direction}, store>"
+    return f"mmq_tile_kernel<{_TYPE_NAMES.get(qt, qt)}, {direction}, {'store' if epi == 0 else 'accumulate_f32'}, {'tall' if shape == 0 else 'wide'}>"
+
+
+def profiled_launches(lib, cap=8192):
+    """[(kernel name, ms)] of the launches recorded since ggq_profile_begin."""
+    ms, qt, mode, epi, shape = (ctypes.c_float * cap)(), (ctypes.c_int * cap)(), (ctypes.c_int * cap)(), (ctypes.c_int * cap)(), (ctypes.c_int * cap)()
+    n = max(lib.ggq_profile_end(ms, qt, mode, epi, shape, cap), 0)
+    return [(kernel_name(qt[j], mode[j], epi[j], shape[j]), ms[j]) for j in range(n)]
+
+
+def measured_traffic(kernel: str):
+    """(bytes per launch, source file) of a kernel's HBM traffic from the committed counter summaries: lines
+    'bench.traffic_bytes <kernel name, spaces as written> = <bytes>' in profiles/*pmc_traffic.txt; (None, None) when the
+    kernel that ran has no such line (the counters are collected offline, in runs of their own)."""
+    import glob
+
+    root = os.path.dirname(os.path.abspath(__file__))
+    for path in sorted(glob.glob(os.path.join(root, "profiles", "*pmc_traffic.txt"))):
+        with open(path) as f:
+            for line in f:
+                if line.startswith("bench.traffic_bytes ") and "=" in line:
+                    name, value = line[len("bench.traffic_bytes "):].rsplit("=", 1)
+                    if name.strip() == kernel:
+                        return float(value), os.path.relpath(path, root)
+    return None, None
+
+
+def host_randn(gen, *shape, std=1.0, dtype=torch.float32, device=None):
+    t = torch.randn(*shape, generator=gen) * std
+    return t.to(dtype).to(device) if device is not None else t.to(dtype)
+
+
+def device_ceilings(pkg, lib, dev, x_samples, w_samples):
+    """What this box sustains, next to the nominal peaks: the bf16 MFMA rate of a register-only loop with operands drawn
+    from the workload's activations and decoded weights (and with all-zero operands: the device is power limited and its
+    clock depends on the data), and the rate of a device-to-device copy."""
+    out = {}
+    tf = ctypes.c_float()
+    n = min(x_samples.numel(), w_samples.numel()) // 8 * 8
+    a, b = x_samples.reshape(-1)[:n].contiguous(), w_samples.reshape(-1)[:n].contiguous()
+    st = pkg._lib.stream_handle(dev)
+    if lib.ggq_measure_mfma_ceiling(a.data_ptr(), b.data_ptr(), n, 20000, ctypes.byref(tf), st) == 0:
+        out["mfma_bf16_tflops_workload_values"] = tf.value
+    z = torch.zeros(n, dtype=torch.bfloat16, device=dev)
+    if lib.ggq_measure_mfma_ceiling(z.data_ptr(), z.data_ptr(), n, 20000, ctypes.byref(tf), st) == 0:
+        out["mfma_bf16_tflops_zero_values"] = tf.value
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(5):
+        dst.copy_(src)
+    e1.record()
+    torch.cuda.synchronize()
+    out["device_copy_gb_per_s"] = 5 * 2 * src.numel() / (e0.elapsed_time(e1) * 1e-3) / 1e9  # bytes read + bytes written
+    return out
 
 CFG = dict(tokens=4096, hidden=2048, inter=512, experts=256, top_k=8, rank=16, alpha=32.0)
 
@@ -44,16 +113,17 @@ def packed_weight_bytes(cfg) -> int:
     return cfg["experts"] * (2 * cfg["inter"] * cfg["hidden"] + cfg["hidden"] * cfg["inter"]) * 144 // 256
 
 
-def build_workload(pkg, dev, cfg, seed=19260817 + 2):
-    g = torch.Generator(device=dev).manual_seed(seed)
+def build_workload(pkg, dev, cfg, seed=SEED + 2):
+    """Every value is drawn on the host from one CPU generator (the bytes are the same on every box) and copied over; the
+    fp32 expert weights are quantized to Q4_K on the device in slices of 32 experts."""
+    g = torch.Generator().manual_seed(seed)
     e, h, i, r = cfg["experts"], cfg["hidden"], cfg["inter"], cfg["rank"]
     G = pkg.gguf.GGUFQuantizedTensor
 
     def packed(shape):
         out = []
-        for lo in range(0, e, 32):  # quantize in slices to bound the fp32 staging memory
-            w = torch.randn((min(32, e - lo),) + shape, generator=g, device=dev) * 0.02
-            out.append(pkg.gguf.quantize_q4_k(w))
+        for lo in range(0, e, 32):  # in slices, to bound the fp32 staging memory
+            out.append(pkg.gguf.quantize_q4_k(host_randn(g, min(32, e - lo), *shape, std=0.02, device=dev)))
         return torch.cat(out, dim=0)
 
     gate = G(packed((i, h)), 12, (e, i, h))
@@ -62,16 +132,16 @@ def build_workload(pkg, dev, cfg, seed=19260817 + 2):
     experts = pkg.fast_moe_lora.GGUFExperts(gate, up, down)
     layer = pkg.fast_moe_lora.FastGGUFMoeLora(experts, r=r, lora_alpha=cfg["alpha"])
     with torch.no_grad():
-        layer.lora_A["default"].weight.copy_((torch.randn(e, r, h, generator=g, device=dev) * h ** -0.5).to(torch.bfloat16))
-        layer.lora_B["default"].weight.copy_((torch.randn(e, 2 * i, r, generator=g, device=dev) * 0.01).to(torch.bfloat16))
-        layer.lora_A_down["default"].weight.copy_((torch.randn(e, r, i, generator=g, device=dev) * i ** -0.5).to(torch.bfloat16))
-        layer.lora_B_down["default"].weight.copy_((torch.randn(e, h, r, generator=g, device=dev) * 0.01).to(torch.bfloat16))
-    x = torch.randn(cfg["tokens"], h, generator=g, device=dev).to(torch.bfloat16).requires_grad_(True)
-    logits = torch.randn(cfg["tokens"], e, generator=g, device=dev)
-    top = torch.topk(logits, cfg["top_k"], dim=-1)
-    idx = top.indices
-    weights = torch.softmax(top.values, dim=-1).requires_grad_(True)
-    dy = torch.randn(cfg["tokens"], h, generator=g, device=dev).to(torch.bfloat16)
+        layer.lora_A["default"].weight.copy_(host_randn(g, e, r, h, std=h ** -0.5, dtype=torch.bfloat16))
+        layer.lora_B["default"].weight.copy_(host_randn(g, e, 2 * i, r, std=0.01, dtype=torch.bfloat16))
+        layer.lora_A_down["default"].weight.copy_(host_randn(g, e, r, i, std=i ** -0.5, dtype=torch.bfloat16))
+        layer.lora_B_down["default"].weight.copy_(host_randn(g, e, h, r, std=0.01, dtype=torch.bfloat16))
+    x = host_randn(g, cfg["tokens"], h, dtype=torch.bfloat16, device=dev).requires_grad_(True)
+    logits = host_randn(g, cfg["tokens"], e)
+    top = torch.topk(logits, cfg["top_k"], dim=-1)  # on the host: ties (none in practice) resolve the same way everywhere
+    idx = top.indices.to(dev)
+    weights = torch.softmax(top.values, dim=-1).to(dev).requires_grad_(True)
+    dy = host_randn(g, cfg["tokens"], h, dtype=torch.bfloat16, device=dev)
     return layer, x, idx, weights, dy
 
 
@@ -123,14 +193,15 @@ def cpu_baseline(cfg, sample_experts=64, repeats=21):
 def other_workload(name, pkg, lib, dev, args):
     """The other BASELINE configurations, timed the same way (eager launches): not the headline line, but the same JSON
     shape, so that their kernels can be traced with the same command."""
-    g = torch.Generator(device=dev).manual_seed(3)
+    g = torch.Generator().manual_seed(SEED + {"dense_q4k": 1, "lmhead_q6k": 3, "moe_iq2xxs": 4}.get(name, 0))  # host generator: same bytes on every box
+    gd = torch.Generator(device=dev).manual_seed(SEED)  # only for the arbitrary-byte IQ2_XXS payloads (1.7 GB of them)
 
     def bf(*shape, std=1.0):
-        return (torch.randn(*shape, generator=g, device=dev) * std).to(torch.bfloat16)
+        return host_randn(g, *shape, std=std, dtype=torch.bfloat16, device=dev)
 
     if name == "dense_q4k":  # configs[1]
         n, k, rows = 4096, 2048, 4096
-        payload = pkg.gguf.quantize_q4_k(torch.randn(n, k, generator=g, device=dev) * 0.02)
+        payload = pkg.gguf.quantize_q4_k(host_randn(g, n, k, std=0.02, device=dev))
         x, a, b = bf(rows, k).requires_grad_(True), bf(16, k, std=k ** -0.5).requires_grad_(True), bf(n, 16, std=0.01).requires_grad_(True)
         dy = bf(rows, n)
         flops = 2 * 2 * rows * n * k + 3 * 2 * rows * 16 * (n + k)
@@ -143,11 +214,12 @@ def other_workload(name, pkg, lib, dev, args):
             pkg.fast_lora.lora_mmq(x, payload, 12, n, a, b, 2.0).backward(dy)
     elif name == "lmhead_q6k":  # configs[3]
         vocab, hidden, rows, chunk = 151936, 2048, 4096, args.chunk
-        payload = torch.cat([pkg.gguf.quantize_q6_k(torch.randn(min(18992, vocab - lo), hidden, generator=g, device=dev) * 0.02)
+        payload = torch.cat([pkg.gguf.quantize_q6_k(host_randn(g, min(18992, vocab - lo), hidden, std=0.02, device=dev))
                              for lo in range(0, vocab, 18992)], dim=0)
         hs = bf(rows, hidden).requires_grad_(True)
-        labels = torch.randint(0, vocab, (rows,), device=dev, generator=g)
-        labels[torch.rand(rows, device=dev, generator=g) < 0.05] = -100
+        labels = torch.randint(0, vocab, (rows,), generator=g)
+        labels[torch.rand(rows, generator=g) < 0.05] = -100
+        labels = labels.to(dev)
         flops = 2 * 2 * rows * vocab * hidden
         launch_flops, launches_per_step = None, None   # launches of different sizes (statistics per chunk, one grad-input)
         workload = f"configs[3]: chunked cross-entropy through a Q6_K lm_head [151936x2048], 4096 rows, chunks of {chunk}, loss + dHidden"
@@ -159,16 +231,16 @@ def other_workload(name, pkg, lib, dev, args):
     elif name == "moe_iq2xxs":  # configs[4], routed experts
         tokens, hidden, inter, e, top_k, r = 2048, 4096, 2048, 256, 8, 16
         G = pkg.gguf.GGUFQuantizedTensor
-        gate = G(pkg.gguf.random_iq2_xxs((e, inter, hidden), g, dev), 16, (e, inter, hidden))
-        up = G(pkg.gguf.random_iq2_xxs((e, inter, hidden), g, dev), 16, (e, inter, hidden))
-        down = G(pkg.gguf.random_iq2_xxs((e, hidden, inter), g, dev), 16, (e, hidden, inter))
+        gate = G(pkg.gguf.random_iq2_xxs((e, inter, hidden), gd, dev), 16, (e, inter, hidden))
+        up = G(pkg.gguf.random_iq2_xxs((e, inter, hidden), gd, dev), 16, (e, inter, hidden))
+        down = G(pkg.gguf.random_iq2_xxs((e, hidden, inter), gd, dev), 16, (e, hidden, inter))
         layer = pkg.fast_moe_lora.FastGGUFMoeLora(pkg.fast_moe_lora.GGUFExperts(gate, up, down), r=r, lora_alpha=32)
         with torch.no_grad():
             for pname, p in layer.named_parameters():
                 p.copy_(bf(*p.shape, std=p.shape[-1] ** -0.5 if "lora_A" in pname else 0.01))
         x = bf(tokens, hidden).requires_grad_(True)
-        top = torch.topk(torch.randn(tokens, e, generator=g, device=dev), top_k, dim=-1)
-        idx, weights = top.indices, torch.softmax(top.values, dim=-1).requires_grad_(True)
+        top = torch.topk(host_randn(g, tokens, e), top_k, dim=-1)
+        idx, weights = top.indices.to(dev), torch.softmax(top.values, dim=-1).to(dev).requires_grad_(True)
         dy = bf(tokens, hidden)
         routes = tokens * top_k
         flops = 2 * 2 * routes * (2 * inter * hidden + hidden * inter) + 3 * 2 * routes * r * ((hidden + 2 * inter) + (inter + hidden))
@@ -198,15 +270,17 @@ def other_workload(name, pkg, lib, dev, args):
     for _ in range(prof_steps):
         step()
     torch.cuda.synchronize()
-    cap = 8192
-    ms, qt, mode, epi = (ctypes.c_float * cap)(), (ctypes.c_int * cap)(), (ctypes.c_int * cap)(), (ctypes.c_int * cap)()
-    n_l = max(lib.ggq_profile_end(ms, qt, mode, epi, cap), 0)
-    tile_ms = sum(ms[j] for j in range(n_l)) / prof_steps
+    launches = profiled_launches(lib)
+    n_l = len(launches)
+    tile_ms = sum(t for _, t in launches) / prof_steps
+    by_kernel = {}
+    for nm, t in launches:
+        by_kernel.setdefault(nm, []).append(t)
     roofline = None
     if launch_flops is not None and n_l:
         avg_ms = tile_ms / launches_per_step
         achieved = launch_flops / (avg_ms * 1e-3) / 1e12
-        roofline = {"bound": "mfma", "kernel": "packed-weight tile kernels (all launches of the step)", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
+        roofline = {"bound": "mfma", "kernel": " + ".join(sorted(by_kernel)), "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
                     "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "avg_launch_ms": avg_ms, "launches_timed": n_l}
     print(json.dumps({
         "metric": metric, "value": flops / (ms_per_step * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -285,28 +359,23 @@ def main() -> None:
     for _ in range(prof_steps):
         step()
     torch.cuda.synchronize()
-    cap = 8192
-    ms = (ctypes.c_float * cap)()
-    qt = (ctypes.c_int * cap)()
-    mode = (ctypes.c_int * cap)()
-    epi = (ctypes.c_int * cap)()
-    n = lib.ggq_profile_end(ms, qt, mode, epi, cap)
+    launches = profiled_launches(lib)
     fl = algorithmic_flops(cfg)
-    per_mode = {0: [], 1: []}
-    for j in range(max(n, 0)):
-        per_mode[mode[j]].append(ms[j])
-    names = {0: "mmq_direct_q4k_kernel (Q4_K, forward, store)", 1: "mmq_mixed_kernel<Q4_K, grad_input, store>"}
-    dominant = max(per_mode, key=lambda m: sum(per_mode[m]))
-    launches = len(per_mode[dominant])
-    avg_ms = sum(per_mode[dominant]) / max(launches, 1)
-    # each step launches the kernel twice per direction: gate/up (pair) and down
+    by_kernel = {}
+    for nm, t in launches:
+        by_kernel.setdefault(nm, []).append(t)
+    dominant = max(by_kernel, key=lambda k: sum(by_kernel[k])) if by_kernel else "none"
+    n_launches = len(by_kernel.get(dominant, []))
+    avg_ms = sum(by_kernel.get(dominant, [])) / max(n_launches, 1)
+    # each step launches a direction's kernel twice: gate/up (pair) and down; the figure is their average
     flops_per_launch = (fl["gate_up"] + fl["down"]) / 2
-    achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12 if launches else 0.0
-    kernel_ms_per_step = {names[m]: sum(v) / prof_steps for m, v in per_mode.items()}
-    # HBM bytes per launch (fetched + written, average of the gate/up and down launches) from the FETCH_SIZE /
-    # WRITE_SIZE counter runs summarised in profiles/mmq_direct_and_mixed_q4k_grouped_moe_lora_step.pmc_traffic.txt;
-    # the counters are collected offline, so this figure only changes when that profile is redone.
-    traffic_bytes = {0: 572.1e6 + 100.7e6, 1: 343.6e6 + 83.9e6}[dominant]
+    achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12 if n_launches else 0.0
+    kernel_ms_per_step = {k: sum(v) / prof_steps for k, v in by_kernel.items()}
+    traffic_bytes, traffic_source = measured_traffic(dominant)
+    # operands with the workload's statistics for the on-box MFMA ceiling: token activations and decoded expert weights
+    with torch.no_grad():
+        w_samples = pkg.gguf.dequantize_gguf_tensor(layer.base_layer.gate_proj.as_subclass(torch.Tensor)[0].contiguous(), 12, torch.bfloat16)
+    ceilings = device_ceilings(pkg, lib, dev, x.detach(), w_samples)
 
     result = {
         "metric": "fwd+bwd TFLOP/s and weight GB/s, Q4_K grouped-MoE LoRA; % of MI355X roofline",
@@ -326,10 +395,12 @@ def main() -> None:
         "weight_gb_per_s": 2 * packed_weight_bytes(cfg) / (ms_per_step * 1e-3) / 1e9,
         "pct_of_mfma_peak": 100.0 * fl["total"] / (ms_per_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
         "pct_of_hbm_peak_weights": 100.0 * 2 * packed_weight_bytes(cfg) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
-        "roofline": {"bound": "mfma", "kernel": names[dominant], "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic_bytes, "avg_launch_ms": avg_ms, "launches_timed": launches,
-                     "flops_per_launch": flops_per_launch},
+        "roofline": {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic_bytes, "traffic_source": traffic_source, "avg_launch_ms": avg_ms,
+                     "launches_timed": n_launches, "flops_per_launch": flops_per_launch},
         "tile_kernel_ms_per_step": kernel_ms_per_step,
+        "ceilings_on_this_box": ceilings,
+        "frac_of_measured_mfma_ceiling": achieved / ceilings["mfma_bf16_tflops_workload_values"] if ceilings.get("mfma_bf16_tflops_workload_values") else None,
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg)

@@ -34,12 +34,21 @@ extern "C" {
 const char* ggq_last_error(void);
 
 /* Kernel timing aid (the reference profiles with Kineto module ranges, deepseek_v4_profiler.py:39-74):
- * between begin and end every launch of the packed-weight tile kernel is bracketed by HIP events on
+ * between begin and end every launch of a packed-weight matmul kernel is bracketed by HIP events on
  * its stream.  ggq_profile_end synchronises on them and fills host arrays (milliseconds, GGML type id,
- * mode 0 = forward / 1 = grad-input, epilogue id) for up to `capacity` launches; returns the number
- * written or a negative error.  Not thread safe; at most 8192 launches are recorded. */
+ * mode 0 = forward / 1 = grad-input, epilogue id 0 = store / 1 = fp32 accumulate, and - unless `shape` is NULL - the kernel
+ * family: 0 = tall tiles, 1 = wide tiles, 3 = the kernels whose MFMA waves decode the weights, 4 = one launch of wide and
+ * tall tiles) for up to `capacity` launches; returns the number written or a negative error.  Not thread safe; at most
+ * 8192 launches are recorded. */
 int ggq_profile_begin(void);
-int ggq_profile_end(float* ms, int* qt, int* mode, int* epilogue, int capacity);
+int ggq_profile_end(float* ms, int* qt, int* mode, int* epilogue, int* shape, int capacity);
+
+/* Measurement aid with no counterpart in the reference: the bf16 MFMA rate (TFLOP/s, into the HOST float tflops_out) a
+ * register-only loop of 32x32x16 MFMAs sustains on this device when its operands are drawn from the two device sample
+ * buffers (`elems` bf16 values each, at least 4096, 16-byte aligned).  The device is power limited and its clock depends on
+ * the operand values, so this - measured with a workload's own activations and decoded weights - is that workload's
+ * MFMA-bound ceiling.  Synchronous: allocates 256 bytes, times `iters` loop trips with HIP events on `stream` and waits. */
+int ggq_measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64_t elems, int iters, float* tflops_out, void* stream);
 
 /* Test aid with no counterpart in the reference: force the kernel family of the grouped Q4_K launches that follow (0 = tall
  * tiles, 1 = the wide / tall tile mix, 3 = the kernels whose MFMA waves decode the weights themselves, wherever their operand

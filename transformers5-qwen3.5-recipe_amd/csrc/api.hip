@@ -51,9 +51,13 @@ const char* ggq_last_error(void) { return last_error(); }
 
 int ggq_profile_begin(void) { return profile_begin(); }
 
-int ggq_profile_end(float* ms, int* qt, int* mode, int* epilogue, int capacity) {
+int ggq_profile_end(float* ms, int* qt, int* mode, int* epilogue, int* shape, int capacity) {
     if (!ms || !qt || !mode || !epilogue) return set_error(GGQ_ERR_NULL, "profile_end: null pointer");
-    return profile_end(ms, qt, mode, epilogue, capacity);
+    return profile_end(ms, qt, mode, epilogue, shape, capacity);
+}
+
+int ggq_measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64_t elems, int iters, float* tflops_out, void* stream) {
+    return measure_mfma_ceiling(a_samples, b_samples, elems, iters, tflops_out, as_stream(stream));
 }
 
 int ggq_debug_force_grouped_shape(int shape) {

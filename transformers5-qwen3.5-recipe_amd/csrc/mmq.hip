@@ -151,7 +151,7 @@ int build_row_tiles(const int64_t* expert_ids, const int32_t* end_offsets, int g
 // Optional per-launch timing of the tile kernel with HIP events on the launch stream (off by default).
 struct TimedLaunch {
     hipEvent_t start, stop;
-    int qt, mode, epi;
+    int qt, mode, epi, shape;
 };
 static TimedLaunch g_timed[kMaxTimedLaunches];
 static int g_timed_count = 0;
@@ -163,14 +163,18 @@ int profile_begin() {
     return GGQ_OK;
 }
 
-int profile_end(float* ms, int* qt, int* mode, int* epi, int capacity) {
+int profile_end(float* ms, int* qt, int* mode, int* epi, int* shape, int capacity) {
     g_timing = false;
     int n = 0;
     for (int i = 0; i < g_timed_count; i++) {
         float t = 0.f;
         if (hipEventSynchronize(g_timed[i].stop) != hipSuccess || hipEventElapsedTime(&t, g_timed[i].start, g_timed[i].stop) != hipSuccess)
             return set_error(GGQ_ERR_RUNTIME, "profile_end: event query failed");
-        if (n < capacity) ms[n] = t, qt[n] = g_timed[i].qt, mode[n] = g_timed[i].mode, epi[n] = g_timed[i].epi, n++;
+        if (n < capacity) {
+            ms[n] = t, qt[n] = g_timed[i].qt, mode[n] = g_timed[i].mode, epi[n] = g_timed[i].epi;
+            if (shape) shape[n] = g_timed[i].shape;
+            n++;
+        }
         (void)hipEventDestroy(g_timed[i].start);
         (void)hipEventDestroy(g_timed[i].stop);
     }
@@ -189,7 +193,7 @@ static int launch_one(const MmqParams& p, hipStream_t s) {
     if (g_timing && g_timed_count < kMaxTimedLaunches) {
         t = &g_timed[g_timed_count];
         if (hipEventCreate(&t->start) != hipSuccess || hipEventCreate(&t->stop) != hipSuccess) return set_error(GGQ_ERR_RUNTIME, "mmq: event creation failed");
-        t->qt = QT, t->mode = MODE, t->epi = EPI;
+        t->qt = QT, t->mode = MODE, t->epi = EPI, t->shape = SH;
         g_timed_count++;
         (void)hipEventRecord(t->start, s);
     }
@@ -221,7 +225,7 @@ static int launch_direct(const MmqParams& p, hipStream_t s) {
     if (g_timing && g_timed_count < kMaxTimedLaunches) {
         t = &g_timed[g_timed_count];
         if (hipEventCreate(&t->start) != hipSuccess || hipEventCreate(&t->stop) != hipSuccess) return set_error(GGQ_ERR_RUNTIME, "mmq: event creation failed");
-        t->qt = kQ4_K, t->mode = MODE, t->epi = kEpiStore;
+        t->qt = kQ4_K, t->mode = MODE, t->epi = kEpiStore, t->shape = kShapeDirect;
         g_timed_count++;
         (void)hipEventRecord(t->start, s);
     }
@@ -252,7 +256,7 @@ static int launch_mixed_mode(const MmqParams& p, hipStream_t s) {
     if (g_timing && g_timed_count < kMaxTimedLaunches) {
         t = &g_timed[g_timed_count];
         if (hipEventCreate(&t->start) != hipSuccess || hipEventCreate(&t->stop) != hipSuccess) return set_error(GGQ_ERR_RUNTIME, "mmq: event creation failed");
-        t->qt = kQ4_K, t->mode = MODE, t->epi = kEpiStore;
+        t->qt = kQ4_K, t->mode = MODE, t->epi = kEpiStore, t->shape = kShapeMixed;
         g_timed_count++;
         (void)hipEventRecord(t->start, s);
     }

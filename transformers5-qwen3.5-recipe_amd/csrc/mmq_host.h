@@ -61,6 +61,7 @@ constexpr int kBM = 256, kBN = 128, kBK = 64;  // the tall tile shape (dense lau
 constexpr int kWideBM = 128, kWideBN = 256;    // the wide tile shape (Q4_K expert groups of about a hundred rows)
 constexpr int kDirectBM = 192, kDirectBN = 256;  // the direct shape (Q4_K expert groups: the MFMA waves decode the weights themselves)
 constexpr int kShapeTall = 0, kShapeWide = 1, kShapeDirect = 3;
+constexpr int kShapeMixed = 4;  // (profile records only: one launch of wide and tall tiles)
 constexpr int kLdsStride = kBK + 8;  // bf16 elements per LDS row: 144 bytes keeps 128-bit reads conflict-free
 constexpr int kThreads = 1024;  // waves 0..7 run the MFMAs, waves 8..15 load and decode
 
@@ -108,7 +109,8 @@ struct MmqParams {
 
 constexpr int kMaxTimedLaunches = 8192;
 int profile_begin();
-int profile_end(float* ms, int* qt, int* mode, int* epi, int capacity);
+int profile_end(float* ms, int* qt, int* mode, int* epi, int* shape, int capacity);
+int measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64_t elems, int iters, float* tflops_out, hipStream_t s);
 const char* last_error();
 int launch_mmq(int qt, int mode, int epi, const MmqParams& p, hipStream_t s);
 int launch_mmq_mixed(int mode, const MmqParams& p, hipStream_t s);  // Q4_K, store epilogue, tiles + tiles2
