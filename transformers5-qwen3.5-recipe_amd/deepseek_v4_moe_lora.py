@@ -7,7 +7,9 @@ from typing import Any
 
 import torch
 
-from .fast_moe_lora import FastGGUFMoeLora, GGUFExperts, _ExpertLoraWeights, qwen3_5_moe_gguf_mmq_lora_forward
+from .deepseek_v4_lora import DEEPSEEK_V4_TARGET_MODULES_PATTERN
+from .fast_moe_lora import (ALL_GGUF_EXPERTS_FUNCTIONS, FastGGUFMoeLora, GGUFExperts, _ExpertLoraWeights, _register_expert_wrapper,
+                            qwen3_5_moe_gguf_mmq_lora_forward)
 
 EXPERTS_IMPLEMENTATION = "deepseek_v4_gguf_dequant_aiter_lora"
 
@@ -15,6 +17,8 @@ EXPERTS_IMPLEMENTATION = "deepseek_v4_gguf_dequant_aiter_lora"
 class DeepseekV4GGUFExperts(GGUFExperts):
     """Packed DeepSeek-V4 experts (stand-in for the fork's class of that name): split gate / up / down payloads and the
     model's ``swiglu_limit`` (the activation clamps gate to at most the limit and up to [-limit, limit])."""
+
+    experts_implementation = EXPERTS_IMPLEMENTATION
 
     def __init__(self, gate_proj, up_proj, down_proj, swiglu_limit: float, compute_dtype: torch.dtype = torch.bfloat16):
         if not swiglu_limit or swiglu_limit <= 0:
@@ -29,6 +33,16 @@ def deepseek_v4_gguf_dequant_aiter_lora_forward(self: Any, hidden_states: torch.
     if not isinstance(self, DeepseekV4GGUFExperts):
         raise TypeError(f"{EXPERTS_IMPLEMENTATION} requires DeepseekV4GGUFExperts, got {type(self).__name__}.")
     return qwen3_5_moe_gguf_mmq_lora_forward(self, hidden_states, top_k_index, top_k_weights, _deepseek_v4_gguf_lora_weights)
+
+
+ALL_GGUF_EXPERTS_FUNCTIONS[EXPERTS_IMPLEMENTATION] = deepseek_v4_gguf_dequant_aiter_lora_forward
+
+
+def register_deepseek_v4_moe_lora(lora_config, model: torch.nn.Module):
+    """Registers DeepSeek's expert forward and its config-local wrapper (deepseek_v4_moe_lora.py:66-95): a string
+    ``target_modules`` must be the exact DeepSeek pattern (which already names "experts"), a collection gets "experts" added."""
+    return _register_expert_wrapper(lora_config, model, EXPERTS_IMPLEMENTATION, deepseek_v4_gguf_dequant_aiter_lora_forward, DeepseekV4GGUFExperts,
+                                    DeepseekV4GGUFMoeLora, "DeepSeek V4 GGUF MoE LoRA", exact_pattern=DEEPSEEK_V4_TARGET_MODULES_PATTERN)
 
 
 class DeepseekV4GGUFMoeLora(FastGGUFMoeLora):

@@ -207,6 +207,14 @@ def _fused_lora_add(result, x, lora_A: torch.nn.Linear, lora_B: torch.nn.Linear,
     return out
 
 
+def _layer_input(x: torch.Tensor) -> torch.Tensor:
+    """What a layer hands to the operators, which take only contiguous 16-byte aligned operands and copy nothing themselves:
+    callers of a layer (a model's forward) may pass views, so the layer makes the bounded copy."""
+    if not x.is_contiguous():
+        return x.contiguous()
+    return x.clone() if x.data_ptr() % 16 else x
+
+
 class GGUFLinear(torch.nn.Module):
     """Frozen linear layer whose weight stays packed (stand-in for the fork's ``GGUFLinear``; exposes
     the attributes fast_lora.py:137-162 and gguf_liger_loss.py:305-324 read)."""
@@ -226,38 +234,106 @@ class GGUFLinear(torch.nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self.compute_dtype != torch.bfloat16:
             raise RuntimeError("The packed GGUF MMQ linear path requires BF16 compute_dtype.")
-        y = mmq(x, self.weight, self.weight.quant_type, self.out_features)
+        y = mmq(_layer_input(x), self.weight, self.weight.quant_type, self.out_features)
         if self.bias is not None:
             y = y + self.bias.to(device=y.device, dtype=y.dtype)
         return y
 
 
+_WRAPPER_OPTIONS = ("lora_dropout", "use_rslora", "use_dora", "lora_bias", "init_lora_weights", "alora_invocation_tokens")
+
+
+def _new_factors(wrapper: torch.nn.Module, adapter_name: str, in_features: int, out_features: int, r: int, lora_alpha: float, opts: dict,
+                 device, dtype) -> None:
+    """lora_A / lora_B / scaling of one adapter under PEFT's names and shapes.  ``init_lora_weights``: True gives A
+    Kaiming-uniform (a = sqrt 5) and B zero, "gaussian" A ~ N(0, 1/r) and B zero, False a non-zero delta for tests
+    (A Kaiming-uniform, B ~ N(0, 0.02))."""
+    if r <= 0:
+        raise ValueError(f"LoRA rank must be positive, got {r}")
+    if opts["use_dora"] or opts["alora_invocation_tokens"] is not None:
+        raise ValueError("the fast LoRA wrappers do not support DoRA or aLoRA variants")
+    if opts["lora_bias"]:
+        raise ValueError("the fast LoRA wrappers do not support LoRA bias")
+    wrapper.lora_A = torch.nn.ModuleDict({adapter_name: torch.nn.Linear(in_features, r, bias=False, device=device, dtype=dtype)})
+    wrapper.lora_B = torch.nn.ModuleDict({adapter_name: torch.nn.Linear(r, out_features, bias=False, device=device, dtype=dtype)})
+    init = opts["init_lora_weights"]
+    if init is True or init is False:
+        torch.nn.init.kaiming_uniform_(wrapper.lora_A[adapter_name].weight, a=math.sqrt(5))
+    elif init == "gaussian":
+        torch.nn.init.normal_(wrapper.lora_A[adapter_name].weight, std=1 / r)
+    else:
+        raise ValueError(f"the fast LoRA wrappers do not support init_lora_weights={init!r}")
+    if init is False:
+        torch.nn.init.normal_(wrapper.lora_B[adapter_name].weight, std=0.02)
+    else:
+        torch.nn.init.zeros_(wrapper.lora_B[adapter_name].weight)
+    wrapper.r = {adapter_name: r}
+    wrapper.lora_alpha = {adapter_name: lora_alpha}
+    wrapper.scaling = {adapter_name: lora_alpha / (math.sqrt(r) if opts["use_rslora"] else r)}
+    wrapper.active_adapter = adapter_name
+    wrapper.disable_adapters = False
+    wrapper.merged = False
+
+
+class FastLoraLinear(torch.nn.Module):
+    """LoRA wrapper for an ordinary floating ``torch.nn.Linear`` (counterpart of fast_lora.py:68-124): the base layer's own
+    forward, then the fused residual ``_fused_lora_add``.  Framework operators only: nothing here is packed.  Constructed the
+    way PEFT constructs a registered wrapper: ``(base_layer, adapter_name, config=..., r=..., lora_alpha=..., **kwargs)``."""
+
+    def __init__(self, base_layer: torch.nn.Module, adapter_name: str = "default", *, r: int, lora_alpha: float, config: Any = None,
+                 **kwargs: Any):
+        super().__init__()
+        if not isinstance(adapter_name, str):
+            raise TypeError("the second argument is the adapter's name; pass r= and lora_alpha= by keyword")
+        from .peft_compat import adapter_options
+
+        opts = adapter_options(config, kwargs, _WRAPPER_OPTIONS)
+        self.base_layer = base_layer
+        w = base_layer.weight
+        _new_factors(self, adapter_name, base_layer.in_features, base_layer.out_features, r, lora_alpha, opts, w.device, w.dtype)
+        p = float(opts["lora_dropout"])
+        self.lora_dropout = torch.nn.ModuleDict({adapter_name: torch.nn.Dropout(p) if p > 0.0 else torch.nn.Identity()})
+
+    def get_base_layer(self) -> torch.nn.Module:
+        return self.base_layer
+
+    def forward(self, x: torch.Tensor, *args: Any, **kwargs: Any) -> torch.Tensor:
+        result = self.base_layer(x, *args, **kwargs)
+        if self.disable_adapters:
+            return result
+        name = self.active_adapter
+        return _fused_lora_add(result, x, self.lora_A[name], self.lora_B[name], self.lora_dropout[name], self.scaling[name])
+
+
 class FastGGUFLoraLinear(torch.nn.Module):
-    """LoRA wrapper for a frozen packed ``GGUFLinear`` (counterpart of fast_lora.py:127-175).
+    """LoRA wrapper for a frozen packed ``GGUFLinear`` (counterpart of fast_lora.py:127-175), constructed like
+    ``FastLoraLinear``.
 
     One adapter, no dropout, no DoRA: the configurations the reference's fast path accepts
     (fast_lora.py:82-94); anything else is rejected rather than served by a slower route."""
 
-    def __init__(self, base_layer: GGUFLinear, r: int, lora_alpha: float, adapter_name: str = "default",
-                 use_rslora: bool = False, lora_dropout: float = 0.0):
+    def __init__(self, base_layer: GGUFLinear, adapter_name: str = "default", *, r: int, lora_alpha: float, config: Any = None,
+                 **kwargs: Any):
         super().__init__()
-        if r <= 0 or r > 64:
+        if not isinstance(adapter_name, str):
+            raise TypeError("the second argument is the adapter's name; pass r= and lora_alpha= by keyword")
+        from .peft_compat import adapter_options
+
+        opts = adapter_options(config, kwargs, _WRAPPER_OPTIONS)
+        if r > 64:
             raise ValueError(f"LoRA rank must be in 1..64, got {r}")
-        if lora_dropout != 0.0:
+        if float(opts["lora_dropout"]) != 0.0:
             raise ValueError("the packed LoRA linear requires lora_dropout=0")
         if not isinstance(base_layer.weight, GGUFQuantizedTensor) or not supports_native_mmq(base_layer.weight):
             raise TypeError("FastGGUFLoraLinear requires a packed weight of a natively supported GGML type")
         if base_layer.input_permutation is not None or base_layer.output_permutation is not None:
             raise RuntimeError("the packed GGUF MMQ linear path does not support layout permutations")
         self.base_layer = base_layer
-        dev, dt = base_layer.weight.device, base_layer.compute_dtype
-        self.lora_A = torch.nn.ModuleDict({adapter_name: torch.nn.Linear(base_layer.in_features, r, bias=False, device=dev, dtype=dt)})
-        self.lora_B = torch.nn.ModuleDict({adapter_name: torch.nn.Linear(r, base_layer.out_features, bias=False, device=dev, dtype=dt)})
-        torch.nn.init.kaiming_uniform_(self.lora_A[adapter_name].weight, a=math.sqrt(5))
-        torch.nn.init.zeros_(self.lora_B[adapter_name].weight)
-        self.scaling = {adapter_name: lora_alpha / (math.sqrt(r) if use_rslora else r)}
-        self.active_adapter = adapter_name
-        self.disable_adapters = False
+        _new_factors(self, adapter_name, base_layer.in_features, base_layer.out_features, r, lora_alpha, opts, base_layer.weight.device,
+                     base_layer.compute_dtype)
+
+    def get_base_layer(self) -> torch.nn.Module:
+        return self.base_layer
 
     def forward(self, x: torch.Tensor, *args: Any, **kwargs: Any) -> torch.Tensor:
         if args or kwargs:
@@ -268,7 +344,7 @@ class FastGGUFLoraLinear(torch.nn.Module):
         if self.disable_adapters:
             return base(x)
         name = self.active_adapter
-        y = lora_mmq(x, base.weight, base.weight.quant_type, base.out_features, self.lora_A[name].weight, self.lora_B[name].weight, self.scaling[name])
+        y = lora_mmq(_layer_input(x), base.weight, base.weight.quant_type, base.out_features, self.lora_A[name].weight, self.lora_B[name].weight, self.scaling[name])
         if base.bias is not None:
             y = y + base.bias.to(device=y.device, dtype=y.dtype)
         return y
@@ -278,6 +354,18 @@ class FastGGUFLoraLinear(torch.nn.Module):
 
     def unmerge(self) -> None:
         raise RuntimeError("GGUF LoRA adapters cannot be unmerged because merging is unsupported.")
+
+
+def register_fast_lora(lora_config):
+    """Registers the linear wrappers on one LoRA config (fast_lora.py:178-200): config-local, through the config's
+    ``_register_custom_module``; nothing is patched process-wide.  ``GGUFLinear`` comes first so that a packed layer never
+    falls to the float wrapper."""
+    register = getattr(lora_config, "_register_custom_module", None)
+    if register is None:
+        raise RuntimeError("This PEFT version has no LoraConfig._register_custom_module API. "
+                           "Cannot install fast LoRA without a global monkey patch.")
+    register({GGUFLinear: FastGGUFLoraLinear, torch.nn.Linear: FastLoraLinear})
+    return lora_config
 
 
 # ------------------------------------------------------------------------------------------------

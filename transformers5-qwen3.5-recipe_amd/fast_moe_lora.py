@@ -28,6 +28,10 @@ from .gguf import GGUFQuantizedTensor, row_bytes
 
 EXPERTS_IMPLEMENTATION = "qwen3_5_moe_gguf_mmq_lora"
 
+# name -> forward(experts, hidden_states, top_k_index, top_k_weights, lora_weights): the registry packed expert modules look
+# their forward up in (stand-in for the fork's ``ALL_GGUF_EXPERTS_FUNCTIONS``, which fast_moe_lora.py:797-799 fills)
+ALL_GGUF_EXPERTS_FUNCTIONS: dict[str, Any] = {}
+
 
 # ------------------------------------------------------------------------------------------------
 def _check_grouped(x, payload, expert_indices, expert_offsets, quant_type, n, k, what):
@@ -354,8 +358,13 @@ class GGUFExperts(torch.nn.Module):
     def _apply_split_gate(self, gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
         return swiglu(gate, up, self.swiglu_limit)
 
+    experts_implementation = EXPERTS_IMPLEMENTATION
+
     def forward(self, hidden_states, top_k_index, top_k_weights, lora_weights: _ExpertLoraWeights | None = None):
-        return qwen3_5_moe_gguf_mmq_lora_forward(self, hidden_states, top_k_index, top_k_weights, lora_weights)
+        fn = ALL_GGUF_EXPERTS_FUNCTIONS.get(self.experts_implementation)
+        if fn is None:
+            raise RuntimeError(f"experts implementation {self.experts_implementation!r} is not registered")
+        return fn(self, hidden_states, top_k_index, top_k_weights, lora_weights)
 
 
 def qwen3_5_moe_gguf_mmq_lora_forward(self: GGUFExperts, hidden_states: torch.Tensor, top_k_index: torch.Tensor,
@@ -405,6 +414,61 @@ def qwen3_5_moe_gguf_mmq_lora_forward(self: GGUFExperts, hidden_states: torch.Te
     return finalize_expert_routing(output, hidden_states, routing_plan, execution_plan.output_mask).reshape(hidden_states.shape)
 
 
+ALL_GGUF_EXPERTS_FUNCTIONS[EXPERTS_IMPLEMENTATION] = qwen3_5_moe_gguf_mmq_lora_forward
+
+
+def set_gguf_experts_implementation(model: torch.nn.Module, name: str, experts_type: type = GGUFExperts) -> list[str]:
+    """Points every packed expert module of ``model`` at a registered forward (what the fork's
+    ``model.set_experts_implementation`` does for its GGUF expert modules, fast_moe_lora.py:800).  The model's own method is
+    called too when it has one and knows the name; stock transformers knows only its own registry and refuses others, which
+    is not an error here.  Returns the module paths."""
+    if name not in ALL_GGUF_EXPERTS_FUNCTIONS:
+        raise ValueError(f"experts implementation {name!r} is not registered")
+    setter = getattr(model, "set_experts_implementation", None)
+    if callable(setter):
+        try:
+            setter(name)
+        except ValueError:
+            pass
+    paths = []
+    for path, module in model.named_modules():
+        if isinstance(module, experts_type):
+            module.experts_implementation = name
+            paths.append(path)
+    return paths
+
+
+def _register_expert_wrapper(lora_config, model: torch.nn.Module, name: str, forward, experts_type: type, wrapper: type, what: str,
+                             exact_pattern: str | None = None):
+    register = getattr(lora_config, "_register_custom_module", None)
+    if register is None:
+        raise RuntimeError("This PEFT version has no LoraConfig._register_custom_module API. "
+                           f"Cannot install {what} without a global PEFT monkey patch.")
+    if getattr(lora_config, "target_parameters", None):
+        raise ValueError("Persistent GGUF expert LoRA targets the complete 'experts' module, not target_parameters.")
+    if isinstance(lora_config.target_modules, str):
+        if exact_pattern is None:
+            raise TypeError(f"{what} requires an explicit target_modules collection, not a regex string.")
+        if lora_config.target_modules != exact_pattern:
+            raise ValueError("DeepSeek V4 LoRA uses one exact indexer-excluding target pattern.")
+    else:
+        target_modules = set(lora_config.target_modules or ())
+        target_modules.add("experts")
+        lora_config.__dict__["target_modules"] = target_modules
+    ALL_GGUF_EXPERTS_FUNCTIONS[name] = forward
+    set_gguf_experts_implementation(model, name, experts_type)
+    register({experts_type: wrapper})
+    return lora_config
+
+
+def register_fast_moe_lora(lora_config, model: torch.nn.Module):
+    """Registers the packed expert forward process-wide and the expert LoRA wrapper on one config
+    (fast_moe_lora.py:773-802): "experts" joins ``target_modules``, every ``GGUFExperts`` of ``model`` is pointed at
+    ``EXPERTS_IMPLEMENTATION``, and the config maps ``GGUFExperts`` to ``FastGGUFMoeLora``."""
+    return _register_expert_wrapper(lora_config, model, EXPERTS_IMPLEMENTATION, qwen3_5_moe_gguf_mmq_lora_forward, GGUFExperts,
+                                    FastGGUFMoeLora, "fast GGUF MoE LoRA")
+
+
 class _ExpertFactor(torch.nn.Module):
     """One expert factor family as a module with a ``weight`` (fast_moe_lora.py:463-470), so adapter checkpoints carry the
     reference's key names (``...lora_A_down.<adapter>.weight``)."""
@@ -420,15 +484,24 @@ class FastGGUFMoeLora(torch.nn.Module):
 
     adapter_layer_names = ("lora_A", "lora_B", "lora_A_down", "lora_B_down")
 
-    def __init__(self, base_layer: GGUFExperts, adapter_name: str = "default", *, r: int, lora_alpha: float,
-                 use_rslora: bool = False, lora_dropout: float = 0.0, init_lora_weights: bool | str = True):
+    def __init__(self, base_layer: GGUFExperts, adapter_name: str = "default", *, r: int, lora_alpha: float, config: Any = None,
+                 **kwargs: Any):
         super().__init__()
+        from .peft_compat import adapter_options
+
+        opts = adapter_options(config, kwargs, ("lora_dropout", "use_rslora", "use_dora", "lora_bias", "init_lora_weights",
+                                                "alora_invocation_tokens"))
+        use_rslora, init_lora_weights = opts["use_rslora"], opts["init_lora_weights"]
         if not isinstance(base_layer, GGUFExperts):
             raise TypeError(f"Fast GGUF MoE LoRA requires GGUFExperts, got {type(base_layer).__name__}.")
         if r <= 0 or r > 64:
             raise ValueError(f"LoRA rank must be in 1..64, got {r}.")
-        if lora_dropout != 0.0:
+        if float(opts["lora_dropout"]) != 0.0:
             raise ValueError("Fast GGUF MoE LoRA currently requires lora_dropout=0.")
+        if opts["lora_bias"]:
+            raise ValueError("Fast GGUF MoE LoRA does not support LoRA bias.")
+        if opts["use_dora"] or opts["alora_invocation_tokens"] is not None:
+            raise ValueError("Fast GGUF MoE LoRA does not support DoRA or aLoRA variants.")
         self.base_layer = base_layer
         e, h, i = base_layer.num_experts, base_layer.hidden_dim, base_layer.intermediate_dim
         dev, dt = base_layer.gate_proj.device, base_layer.compute_dtype
@@ -454,6 +527,9 @@ class FastGGUFMoeLora(torch.nn.Module):
         if init_lora_weights is not False:
             torch.nn.init.zeros_(self.lora_B[adapter_name].weight)
             torch.nn.init.zeros_(self.lora_B_down[adapter_name].weight)
+
+    def get_base_layer(self) -> torch.nn.Module:
+        return self.base_layer
 
     def _active_lora_weights(self) -> _ExpertLoraWeights | None:
         if self.disable_adapters:

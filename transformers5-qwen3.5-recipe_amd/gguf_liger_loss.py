@@ -159,3 +159,148 @@ def _packed_for_causal_lm_loss(hidden_states: torch.Tensor, lm_head: GGUFLinear,
     if return_token_accuracy or return_predicted_tokens:
         return loss, None, token_accuracy, predicted_tokens  # (loss, z_loss, accuracy, tokens), gguf_liger_loss.py:352-353
     return loss
+
+
+# ------------------------------------------------------------------------------------------------
+# Model-level installation (gguf_liger_loss.py:359-532 of the reference): a replacement forward for the causal-LM class
+# that never builds the [tokens, vocab] logits while training, and the function that binds it to one loaded model.
+def _causal_lm_output_class():
+    """``MoeCausalLMOutputWithPast`` with the two extra fields of Liger's output class (gguf_liger_loss.py:502-512); a plain
+    attribute/dict container with the same field names when transformers is not importable."""
+    from dataclasses import dataclass, fields
+
+    try:
+        from transformers.modeling_outputs import MoeCausalLMOutputWithPast
+    except ImportError:
+        @dataclass
+        class PackedMoeCausalLMOutputWithPast:
+            loss: Any = None
+            aux_loss: Any = None
+            logits: Any = None
+            past_key_values: Any = None
+            hidden_states: Any = None
+            attentions: Any = None
+            router_logits: Any = None
+            token_accuracy: Any = None
+            predicted_tokens: Any = None
+
+            def __getitem__(self, key):
+                if isinstance(key, str):
+                    return getattr(self, key)
+                return tuple(getattr(self, f.name) for f in fields(self) if getattr(self, f.name) is not None)[key]
+
+        return PackedMoeCausalLMOutputWithPast
+
+    @dataclass
+    class PackedMoeCausalLMOutputWithPast(MoeCausalLMOutputWithPast):
+        token_accuracy: torch.Tensor | None = None
+        predicted_tokens: torch.Tensor | None = None
+
+    return PackedMoeCausalLMOutputWithPast
+
+
+_OUTPUT_CLASS = None
+
+
+def _output_class():
+    global _OUTPUT_CLASS
+    if _OUTPUT_CLASS is None:
+        _OUTPUT_CLASS = _causal_lm_output_class()
+    return _OUTPUT_CLASS
+
+
+def _router_aux_loss(self, outputs, attention_mask):
+    """The load-balancing term of the model family (gguf_liger_loss.py:472-481): transformers' own function, which the
+    stock forward of the same class calls."""
+    from transformers.models.qwen3_5_moe.modeling_qwen3_5_moe import load_balancing_loss_func
+
+    return load_balancing_loss_func(outputs.router_logits, self.num_experts, self.num_experts_per_tok, attention_mask)
+
+
+def gguf_liger_lce_forward(self, input_ids=None, attention_mask=None, position_ids=None, past_key_values=None, inputs_embeds=None,
+                           labels=None, use_cache=None, output_attentions=None, output_hidden_states=None, output_router_logits=None,
+                           mm_token_type_ids=None, cache_position=None, logits_to_keep: int | torch.Tensor = 0, skip_logits: bool | None = None,
+                           return_dict: bool | None = None, **kwargs: Any):
+    """Causal-LM forward over a packed lm_head (the flow and guards of gguf_liger_loss.py:359-512).  While training with labels
+    the loss comes from the chunked packed cross-entropy and ``logits`` stays None; otherwise the head runs as a layer and
+    the model's own ``loss_function`` is used.  ``self`` needs ``model``, ``lm_head``, ``config``, ``loss_function``,
+    ``vocab_size`` and, for the router term, ``num_experts``, ``num_experts_per_tok`` and ``router_aux_loss_coef``.
+    Arguments that are None are not forwarded to ``self.model``, so that model classes without them keep working."""
+    config = self.config
+    output_router_logits = output_router_logits if output_router_logits is not None else getattr(config, "output_router_logits", False)
+    return_dict = return_dict if return_dict is not None else getattr(config, "use_return_dict", True)
+    optional = dict(attention_mask=attention_mask, position_ids=position_ids, past_key_values=past_key_values, inputs_embeds=inputs_embeds,
+                    use_cache=use_cache, output_attentions=output_attentions, output_hidden_states=output_hidden_states,
+                    mm_token_type_ids=mm_token_type_ids, cache_position=cache_position)
+    shift_labels = kwargs.pop("shift_labels", None)
+    loss_kwargs = dict(kwargs)
+    outputs = self.model(input_ids=input_ids, output_router_logits=output_router_logits,
+                         **{k: v for k, v in optional.items() if v is not None}, **kwargs)
+    hidden_states = outputs.last_hidden_state
+    if hidden_states is None:
+        raise RuntimeError("Qwen model did not return hidden states")
+    slice_indices = slice(-logits_to_keep, None) if isinstance(logits_to_keep, int) else logits_to_keep
+    kept_hidden_states = hidden_states[:, slice_indices, :]
+    logits = loss = token_accuracy = predicted_tokens = None
+    have_labels = labels is not None or shift_labels is not None
+    if skip_logits is None:
+        skip_logits = self.training and have_labels
+    if skip_logits and not (isinstance(logits_to_keep, int) and logits_to_keep == 0):
+        raise RuntimeError("Packed GGUF LM-head loss requires logits_to_keep=0 during training.")
+    if skip_logits and not have_labels:
+        raise RuntimeError("Packed GGUF LM-head loss requires labels or shift_labels.")
+    if self.training and not skip_logits and have_labels:
+        raise RuntimeError("Packed GGUF training with labels requires the no-full-logits fused loss.")
+    if skip_logits:
+        if not isinstance(self.lm_head, GGUFLinear):
+            raise TypeError(f"GGUF-aware Liger loss requires a GGUFLinear LM head, got {type(self.lm_head).__name__}.")
+        if self.lm_head.bias is not None:
+            raise RuntimeError("GGUF-aware Liger loss currently requires a bias-free LM head.")
+        result = _packed_for_causal_lm_loss(hidden_states=kept_hidden_states, lm_head=self.lm_head, labels=labels, shift_labels=shift_labels,
+                                            hidden_size=config.hidden_size, **loss_kwargs)
+        if isinstance(result, tuple):
+            loss, _, token_accuracy, predicted_tokens = result
+        else:
+            loss = result
+    else:
+        logits = self.lm_head(kept_hidden_states)
+        if have_labels:
+            loss = self.loss_function(logits=logits, labels=labels, shift_labels=shift_labels, vocab_size=self.vocab_size, **loss_kwargs)
+    aux_loss = None
+    if output_router_logits:
+        aux_loss = _router_aux_loss(self, outputs, attention_mask)
+        if labels is not None:
+            if loss is None:
+                raise RuntimeError("router auxiliary loss requires a primary loss")
+            loss = loss + self.router_aux_loss_coef * aux_loss.to(loss.device)
+    if not return_dict:
+        output = (logits,) + tuple(outputs[1:])
+        output = ((aux_loss,) + output) if aux_loss is not None else output
+        output = ((loss,) + output) if loss is not None else output
+        output = output + (token_accuracy,) if token_accuracy is not None else output
+        return output + (predicted_tokens,) if predicted_tokens is not None else output
+    return _output_class()(loss=loss, aux_loss=aux_loss, logits=logits, past_key_values=getattr(outputs, "past_key_values", None),
+                           hidden_states=getattr(outputs, "hidden_states", None), attentions=getattr(outputs, "attentions", None),
+                           router_logits=getattr(outputs, "router_logits", None), token_accuracy=token_accuracy,
+                           predicted_tokens=predicted_tokens)
+
+
+def _unwrapped_causal_lm(model: torch.nn.Module, class_name: str, what: str) -> torch.nn.Module:
+    get_base_model = getattr(model, "get_base_model", None)
+    target = get_base_model() if callable(get_base_model) else model
+    if not any(c.__name__ == class_name for c in type(target).__mro__):
+        raise TypeError(f"{what} requires {class_name} after unwrapping PEFT, got {type(target).__name__}.")
+    if not isinstance(target.lm_head, GGUFLinear):
+        raise TypeError(f"{what} requires GGUFLinear, got {type(target.lm_head).__name__}.")
+    return target
+
+
+def apply_gguf_liger_fused_linear_cross_entropy(model: torch.nn.Module) -> torch.nn.Module:
+    """Binds ``gguf_liger_lce_forward`` to one loaded text model (gguf_liger_loss.py:515-532): a PEFT wrapper is unwrapped
+    through ``get_base_model``, the model must be a ``Qwen3_5MoeForCausalLM`` (by class name anywhere in its MRO, so that
+    the fork's and upstream's classes both qualify) whose ``lm_head`` is a packed ``GGUFLinear``.  Returns the patched model."""
+    from types import MethodType
+
+    target = _unwrapped_causal_lm(model, "Qwen3_5MoeForCausalLM", "GGUF-aware Liger loss")
+    target.forward = MethodType(gguf_liger_lce_forward, target)
+    return target
