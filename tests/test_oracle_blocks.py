@@ -143,6 +143,37 @@ def test_iq2xxs_grid_structure():
     assert int(((n19 == 2) & (n2b == 0)).sum()) == 28 and int(((n19 == 0) & (n2b == 1)).sum()) == 8
 
 
+# The same 256 points in a second encoding, typed separately from the byte table: eight 2-bit digits per point, least
+# significant first, digit 0 / 1 / 2 = magnitude 0x08 / 0x19 / 0x2b (the form in which the public ggml quantizer source lists
+# its IQ2_XXS lattice points).  It pins nothing against upstream, but a typing slip in one entry of either table fails here.
+_IQ2XXS_GRID_DIGITS = (
+    0, 2, 5, 8, 10, 17, 20, 32, 34, 40, 42, 65, 68, 80, 88, 97,
+    100, 128, 130, 138, 162, 257, 260, 272, 277, 320, 388, 408, 512, 514, 546, 642,
+    1025, 1028, 1040, 1057, 1060, 1088, 1090, 1096, 1120, 1153, 1156, 1168, 1188, 1280, 1282, 1288,
+    1312, 1350, 1385, 1408, 1425, 1545, 1552, 1600, 1668, 1700, 2048, 2053, 2056, 2068, 2088, 2113,
+    2116, 2128, 2130, 2184, 2308, 2368, 2562, 2580, 4097, 4100, 4112, 4129, 4160, 4192, 4228, 4240,
+    4245, 4352, 4360, 4384, 4432, 4442, 4480, 4644, 4677, 5120, 5128, 5152, 5157, 5193, 5248, 5400,
+    5474, 5632, 5654, 6145, 6148, 6160, 6208, 6273, 6400, 6405, 6560, 6737, 8192, 8194, 8202, 8260,
+    8289, 8320, 8322, 8489, 8520, 8704, 8706, 9217, 9220, 9232, 9280, 9302, 9472, 9537, 9572, 9872,
+    10248, 10272, 10388, 10820, 16385, 16388, 16400, 16408, 16417, 16420, 16448, 16456, 16470, 16480, 16513, 16516,
+    16528, 16640, 16672, 16737, 16768, 16773, 16897, 16912, 16968, 16982, 17000, 17408, 17416, 17440, 17536, 17561,
+    17682, 17700, 17920, 18433, 18436, 18448, 18496, 18501, 18688, 18776, 18785, 18818, 19013, 19088, 20480, 20488,
+    20497, 20505, 20512, 20608, 20616, 20740, 20802, 20900, 21137, 21648, 21650, 21770, 22017, 22100, 22528, 22545,
+    22553, 22628, 22848, 23048, 24580, 24592, 24640, 24680, 24832, 24917, 25112, 25184, 25600, 25605, 25872, 25874,
+    25988, 26690, 32768, 32770, 32778, 32833, 32898, 33028, 33048, 33088, 33297, 33793, 33796, 33808, 33813, 33856,
+    33888, 34048, 34118, 34196, 34313, 34368, 34400, 34818, 35076, 35345, 36868, 36880, 36900, 36928, 37025, 37142,
+    37248, 37445, 37888, 37922, 37956, 38225, 39041, 39200, 40962, 41040, 41093, 41225, 41472, 42008, 43088, 43268,
+)
+
+
+def test_iq2xxs_grid_agrees_with_its_digit_encoding():
+    assert len(_IQ2XXS_GRID_DIGITS) == 256
+    magnitude = {0: 0x08, 1: 0x19, 2: 0x2B}
+    for i, (digits, point) in enumerate(zip(_IQ2XXS_GRID_DIGITS, IQ2XXS_GRID)):
+        expanded = sum(magnitude[(digits >> (2 * j)) & 3] << (8 * j) for j in range(8))  # digit 3 does not occur: KeyError
+        assert expanded == point, (i, digits, hex(point))
+
+
 @pytest.mark.parametrize("qt", [gb.Q8_0, gb.Q2_K, gb.Q3_K, gb.Q4_K, gb.Q5_K, gb.Q6_K, gb.IQ2_XXS])
 def test_numpy_and_c_agree_on_arbitrary_bytes(qt):
     payload = gb.random_payload(np.random.default_rng(qt), qt, 23, 1024)
