@@ -181,6 +181,29 @@ int ggq_route_combine_forward(const void* expert_out, const void* weights, int w
 /* _route_combine_backward_kernel (fast_moe_routing.py:197-226); either gradient may be NULL. */
 int ggq_route_combine_backward(const void* expert_out, const void* weights, int weights_are_bf16, const int64_t* permutation, const void* grad_out, void* grad_expert_out, void* grad_weights, int64_t tokens, int top_k, int hidden_dim, void* stream);
 
+/* The combine's backward folded into the down projection's (what _RouteCombine.backward, fast_moe_routing.py:197-226 /
+ * :276-300, followed by grouped_mmq_grad_input and the grouped LoRA GEMMs, fast_moe_lora.py:255-262 and :42-151, compute in
+ * several passes): grad_out is the [tokens, n] cotangent of the COMBINED output, and expert-sorted row i stands for
+ * weights[permutation[i]] * grad_out[permutation[i] / top_k] without that [rows, n] matrix ever being written.
+ * dx_unscaled [rows, k] = grad_out[token] . W[expert] + LoRA term, WITHOUT the routing weight (ggq_swiglu_backward_routed
+ * applies it); d_lora_a / d_lora_b (may be NULL) include it.  x [rows, k] and xa are the projection's forward input and its
+ * x . A^T.  Workspace as for ggq_grouped_lora_mmq_backward. */
+int ggq_grouped_lora_mmq_backward_routed_output(const void* grad_out, int64_t tokens, const int64_t* permutation, int top_k,
+                                                const void* weights, int weights_are_bf16, const void* packed,
+                                                const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts,
+                                                int qt, int64_t rows, int64_t n, int64_t k, const void* x, const void* xa,
+                                                const void* lora_a, const void* lora_b, int r, float scale, void* dx_unscaled,
+                                                void* d_lora_a, void* d_lora_b, void* ws, int64_t ws_bytes, void* stream);
+
+/* The second half of that backward: dh_unweighted [rows, inter] is dx_unscaled above, the cotangent of
+ * h = silu(gate) * up (limit > 0: the clamped form) before the routing weight.  Writes dgate, dup for the cotangent
+ * weights[permutation[i]] * dh_unweighted[i], and grad_weights[permutation[i]] = <dh_unweighted[i], h[i]> (fp32 sum; equal
+ * to the <grad_out[token], expert_out[i]> of fast_moe_routing.py:217-224 up to rounding; NULL: not wanted), in the
+ * weights' type. */
+int ggq_swiglu_backward_routed(const void* gate, const void* up, const void* dh_unweighted, const void* weights, int weights_are_bf16,
+                               const int64_t* permutation, void* dgate, void* dup, void* grad_weights, int64_t rows, int inter, float limit,
+                               void* stream);
+
 /* GGUFExperts._apply_split_gate (fork; called at fast_moe_lora.py:747): h = silu(gate) * up, and its
  * autograd.  elems = rows * intermediate. */
 int ggq_swiglu_forward(const void* gate, const void* up, void* h, int64_t elems, void* stream);

@@ -35,9 +35,12 @@ def weights_bf16(payload: np.ndarray, qt: int) -> torch.Tensor:
     return torch.from_numpy(gb.dequantize_bf16(payload, qt)).to(torch.float64)
 
 
-def lora_linear(x, w, a=None, b=None, s=1.0, dy=None):
+def lora_linear(x, w, a=None, b=None, s=1.0, dy=None, row_weight=None):
     """x [M,K] bf16, w [N,K] float64 (bf16 values), a [r,K], b [N,r] bf16, dy [M,N] bf16.
-    Returns dict(y, xa, dx, da, db) in float64 (xa holds bf16 values)."""
+    Returns dict(y, xa, dx, da, db) in float64 (xa holds bf16 values).
+    ``row_weight`` [M] float64: row i's cotangent is row_weight[i] * dy[i] without that product being stored (the order of
+    the backward that folds the expert combine into the down projection): dx stays UNWEIGHTED, the factor gradients carry the
+    weight on their rank-r operand, which is rounded to bf16 again."""
     x64 = x.to(torch.float64)
     out = {"y": x64 @ w.T}
     if a is not None:
@@ -51,8 +54,11 @@ def lora_linear(x, w, a=None, b=None, s=1.0, dy=None):
         if a is not None:
             t = bf16_round(dy64 @ b64)
             out["dx"] = out["dx"] + s * (t @ a64)
+            xa_b = out["xa"]
+            if row_weight is not None:
+                t, xa_b = bf16_round(t * row_weight[:, None]), bf16_round(xa_b * row_weight[:, None])
             out["da"] = s * (t.T @ x64)
-            out["db"] = s * (dy64.T @ out["xa"])
+            out["db"] = s * (dy64.T @ xa_b)
     return out
 
 
@@ -62,7 +68,7 @@ def group_bounds(offsets) -> list[tuple[int, int]]:
     return list(zip([0] + ends[:-1], ends))
 
 
-def grouped_lora_linear(x, w_all, experts, offsets, a_all=None, b_all=None, s=1.0, dy=None):
+def grouped_lora_linear(x, w_all, experts, offsets, a_all=None, b_all=None, s=1.0, dy=None, row_weight=None):
     """Per-group loop of :func:`lora_linear`.  w_all [E,N,K] float64, a_all [E,r,K], b_all [E,N,r].
     experts: active expert ids; offsets: cumulative ends.  Factor gradients cover all E planes and are
     zero for inactive experts (test_fast_moe_lora.py:331-333)."""
@@ -83,6 +89,7 @@ def grouped_lora_linear(x, w_all, experts, offsets, a_all=None, b_all=None, s=1.
             x[r0:r1], w_all[e],
             None if a_all is None else a_all[e], None if b_all is None else b_all[e], s,
             None if dy is None else dy[r0:r1],
+            None if row_weight is None else row_weight[r0:r1],
         )
         res["y"][r0:r1] = part["y"]
         if "xa" in part:
@@ -103,26 +110,37 @@ def silu_mul(gate: torch.Tensor, up: torch.Tensor, limit: float | None = None) -
     return gate * torch.sigmoid(gate) * up
 
 
-def expert_layer(x_sorted, experts, offsets, wg, wu, wd, a_gu, b_gu, a_d, b_d, s, dy=None):
+def expert_layer(x_sorted, experts, offsets, wg, wu, wd, a_gu, b_gu, a_d, b_d, s, dy=None, row_weight=None, limit=None):
     """Expert-sorted rows through gate/up -> SiLU*up -> down with LoRA on both projections
     (fast_moe_lora.py:722-763).  wg, wu [E,I,H]; wd [E,H,I]; a_gu [E,r,H]; b_gu [E,2I,r];
     a_d [E,r,I]; b_d [E,H,r].  Intermediates are rounded to bf16 where the path stores them
-    (gate, up, h).  Returns float64 tensors."""
+    (gate, up, h).  Returns float64 tensors.
+    With ``row_weight`` [rows] (the routing weight of each sorted row) ``dy`` is the UNWEIGHTED cotangent of the down
+    projection's rows: its grad-input is rounded to bf16 unweighted ("dh_unweighted"), the activation's backward runs on
+    row_weight * that, and "dw" = <dh_unweighted, h> per row is the routing weight's gradient (the same number as
+    <dy, out> of the row, by associativity).  ``limit``: the clamped activation (no gradient into a clamped input)."""
     inter = wg.shape[1]
     w_gu = torch.cat([wg, wu], dim=1)
     gu = grouped_lora_linear(x_sorted, w_gu, experts, offsets, a_gu, b_gu, s)
     gate = bf16_round(gu["y"][:, :inter])
     up = bf16_round(gu["y"][:, inter:])
-    h = bf16_round(silu_mul(gate, up))
+    h = bf16_round(silu_mul(gate, up, limit))
     h_bf = h.to(torch.bfloat16)
-    dn = grouped_lora_linear(h_bf, wd, experts, offsets, a_d, b_d, s, dy)
+    dn = grouped_lora_linear(h_bf, wd, experts, offsets, a_d, b_d, s, dy, row_weight)
     res = {"gate": gate, "up": up, "h": h, "out": dn["y"]}
     if dy is None:
         return res
     dh = bf16_round(dn["dx"])
-    sig = torch.sigmoid(gate)
-    dgate = bf16_round(dh * up * (sig * (1 + gate * (1 - sig))))
-    dup = bf16_round(dh * gate * sig)
+    if row_weight is not None:
+        res["dh_unweighted"], res["dw"] = dh, (dh * h).sum(dim=1)
+        dh = dh * row_weight[:, None]
+    gc, uc = (gate, up) if limit is None else (gate.clamp(max=limit), up.clamp(min=-limit, max=limit))
+    sig = torch.sigmoid(gc)
+    dgate = bf16_round(dh * uc * (sig * (1 + gc * (1 - sig))))
+    dup = bf16_round(dh * gc * sig)
+    if limit is not None:
+        dgate = torch.where(gate <= limit, dgate, torch.zeros_like(dgate))
+        dup = torch.where((up >= -limit) & (up <= limit), dup, torch.zeros_like(dup))
     dgu = torch.cat([dgate, dup], dim=1).to(torch.bfloat16)
     back = grouped_lora_linear(x_sorted, w_gu, experts, offsets, a_gu, b_gu, s, dgu)
     res.update(dh=dh, dgate=dgate, dup=dup, dx=back["dx"], da_gu=back["da"], db_gu=back["db"],

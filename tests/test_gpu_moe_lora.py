@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import ALL_TYPES, TYPE_NAMES, assert_close_bf16, bf16_randn, make_payload
+from helpers import max_rel, ALL_TYPES, TYPE_NAMES, assert_close_bf16, bf16_randn, make_payload
 from oracle import gguf_blocks as gb
 from oracle import lora_matmul as ref
 from oracle import routing as rref
@@ -255,19 +255,27 @@ def _layer_case(seed, tokens, hidden, inter, experts, k, r, qt):
     return pg, pu, pd, x, idx, w, a_gu, b_gu, a_d, b_d, dy
 
 
-def _oracle_layer(pg, pu, pd, x, idx, w, a_gu, b_gu, a_d, b_d, dy, qt, s, experts):
+def _oracle_layer(pg, pu, pd, x, idx, w, a_gu, b_gu, a_d, b_d, dy, qt, s, experts, fused=False):
     tokens, k = idx.shape
     sorted_ids, perm, inv = rref.plan(idx)
     counts = rref.expert_counts(idx, experts)
     ends = torch.cumsum(counts.long(), 0).int()
     sel = rref.gather_forward(x, perm, k)
-    # backward through combine first: dO rows for the sorted layout
-    d_o = (dy.float()[perm // k] * rref.bf16(w).reshape(-1)[perm][:, None]).to(torch.bfloat16)
-    res = ref.expert_layer(sel, torch.arange(experts), ends, ref.weights_bf16(pg, qt), ref.weights_bf16(pu, qt),
-                           ref.weights_bf16(pd, qt), a_gu, b_gu, a_d, b_d, s, d_o)
+    weights = (ref.weights_bf16(pg, qt), ref.weights_bf16(pu, qt), ref.weights_bf16(pd, qt))
+    if fused:
+        # the order of the fused backward: the tokens' cotangent rows unweighted, the routing weight after the grad-input
+        row_weight = rref.bf16(w).reshape(-1)[perm].double()  # the path applies routing weights at bf16 precision
+        res = ref.expert_layer(sel, torch.arange(experts), ends, *weights, a_gu, b_gu, a_d, b_d, s, dy[perm // k], row_weight=row_weight)
+        dw = torch.zeros(tokens * k, dtype=torch.float64)
+        dw[perm] = res["dw"]
+        dw = dw.reshape(tokens, k)
+    else:
+        # backward through combine first: dO rows for the sorted layout
+        d_o = (dy.float()[perm // k] * rref.bf16(w).reshape(-1)[perm][:, None]).to(torch.bfloat16)
+        res = ref.expert_layer(sel, torch.arange(experts), ends, *weights, a_gu, b_gu, a_d, b_d, s, d_o)
+        _, dw = rref.combine_backward(dy, ref.bf16_round(res["out"]).to(torch.bfloat16), w, perm)
     out = rref.combine_forward(ref.bf16_round(res["out"]).to(torch.bfloat16), w, inv)
     dx_tok = rref.gather_backward(ref.bf16_round(res["dx"]).to(torch.bfloat16), inv, tokens, k)
-    _, dw = rref.combine_backward(dy, ref.bf16_round(res["out"]).to(torch.bfloat16), w, perm)
     return out, dx_tok, dw, res
 
 
@@ -277,11 +285,15 @@ def _oracle_layer(pg, pu, pd, x, idx, w, a_gu, b_gu, a_d, b_d, dy, qt, s, expert
     (gb.IQ2_XXS, 64, 512, 512, 8, 2, 16),
     (gb.Q8_0, 40, 256, 128, 4, 2, 8),
 ])
-def test_expert_layer_forward_backward(pkg, dev, qt, tokens, hidden, inter, experts, k, r):
+@pytest.mark.parametrize("fused", [True, False])
+def test_expert_layer_forward_backward(pkg, dev, qt, tokens, hidden, inter, experts, k, r, fused, monkeypatch):
+    # fused: activation + down projection + combine as one autograd node whose backward never forms the [routes, hidden]
+    # cotangent; otherwise the three nodes of the reference's structure.  Both against the same oracle layer.
     ml, G = pkg.fast_moe_lora, pkg.gguf.GGUFQuantizedTensor
+    monkeypatch.setattr(ml, "FUSE_GATED_DOWN_COMBINE", fused)
     s = 32.0 / r
     pg, pu, pd, x, idx, w, a_gu, b_gu, a_d, b_d, dy = _layer_case(97531, tokens, hidden, inter, experts, k, r, qt)
-    want_out, want_dx, want_dw, res = _oracle_layer(pg, pu, pd, x, idx, w, a_gu, b_gu, a_d, b_d, dy, qt, s, experts)
+    want_out, want_dx, want_dw, res = _oracle_layer(pg, pu, pd, x, idx, w, a_gu, b_gu, a_d, b_d, dy, qt, s, experts, fused)
     mod = ml.GGUFExperts(G(torch.from_numpy(pg).to(dev), qt, (experts, inter, hidden)), G(torch.from_numpy(pu).to(dev), qt, (experts, inter, hidden)),
                          G(torch.from_numpy(pd).to(dev), qt, (experts, hidden, inter)))
     layer = ml.FastGGUFMoeLora(mod, r=r, lora_alpha=32)
@@ -364,3 +376,43 @@ def test_clamped_swiglu_forward_and_gradients(pkg, dev, limit):
     assert float(gd.grad[0, 0]) == 0.0 and float(ud.grad[0, 0]) == 0.0 and float(ud.grad[0, 1]) == 0.0
     with pytest.raises(ValueError):
         ml.swiglu(gd, ud, 0.0)
+
+
+@pytest.mark.parametrize("limit", [None, 1.5])
+@pytest.mark.parametrize("weights_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("qt,with_lora", [(gb.Q4_K, True), (gb.Q6_K, True), (gb.Q4_K, False)])
+def test_fused_gated_down_combine_against_the_separate_nodes(pkg, dev, monkeypatch, limit, weights_dtype, qt, with_lora):
+    # one autograd node for activation + down projection + combine against the three separate ones: the forward gives the
+    # same bits, the gradients agree to rounding (the fused backward applies the routing weight after the grad-input matmul
+    # instead of before it, and takes the weights' gradient from the 512-wide side of the projection)
+    ml, G = pkg.fast_moe_lora, pkg.gguf.GGUFQuantizedTensor
+    tokens, hidden, inter, experts, k, r = 200, 512, 256, 12, 4, 16
+    pg, pu, pd, x, idx, w, a_gu, b_gu, a_d, b_d, dy = _layer_case(4242, tokens, hidden, inter, experts, k, r, qt)
+    mod = ml.GGUFExperts(G(torch.from_numpy(pg).to(dev), qt, (experts, inter, hidden)), G(torch.from_numpy(pu).to(dev), qt, (experts, inter, hidden)),
+                         G(torch.from_numpy(pd).to(dev), qt, (experts, hidden, inter)), swiglu_limit=limit)
+    layer = ml.FastGGUFMoeLora(mod, r=r, lora_alpha=32)
+    with torch.no_grad():
+        layer.lora_A["default"].weight.copy_(a_gu.to(dev)); layer.lora_B["default"].weight.copy_(b_gu.to(dev))
+        layer.lora_A_down["default"].weight.copy_(a_d.to(dev)); layer.lora_B_down["default"].weight.copy_(b_d.to(dev))
+    layer.disable_adapters = not with_lora
+    results = {}
+    for fused in (True, False):
+        monkeypatch.setattr(ml, "FUSE_GATED_DOWN_COMBINE", fused)
+        for p in layer.parameters():
+            p.grad = None
+        xd = (3.0 * x).to(dev).requires_grad_(True)  # wide enough activations for the clamp to bite
+        wd = w.to(weights_dtype).to(dev).requires_grad_(True)
+        out = layer(xd, idx.to(dev), wd)
+        out.backward(dy.to(dev))
+        results[fused] = (out, xd.grad, wd.grad, [None if p.grad is None else p.grad.clone() for p in layer.parameters()])
+    (out1, dx1, dw1, g1), (out0, dx0, dw0, g0) = results[True], results[False]
+    assert torch.equal(out1, out0)
+    assert dw1.dtype == weights_dtype
+    # (each order is held to a few bf16 steps of its own oracle in test_expert_layer_forward_backward; the two orders round
+    # at different places, so against each other only the path's tolerance holds)
+    assert max_rel(dx1, dx0) <= 2e-2 and max_rel(dw1, dw0) <= 2e-2
+    for a, b, (name, _) in zip(g1, g0, layer.named_parameters()):
+        if with_lora:
+            assert max_rel(a, b) <= 2e-2, name
+        else:
+            assert a is None and b is None

@@ -110,3 +110,52 @@ def test_expert_layer_matches_unrounded_autograd_within_bf16_tolerance():
     torch.nn.functional.silu(g).sum().backward()
     sig = torch.sigmoid(g.detach())
     assert torch.allclose(g.grad, sig * (1 + g.detach() * (1 - sig)), atol=1e-12)
+
+
+def test_expert_layer_with_row_weights_matches_autograd_of_the_weighted_sum():
+    # the order of the backward that folds the combine into the down projection: the cotangent arrives unweighted, the
+    # weight is applied after the grad-input.  Pinned by autograd of sum_r w_r <dy_r, out_r> in float64 without roundings:
+    # input and factor gradients within the bf16 tolerance, and the weight gradient <dh_unweighted, h> against d/dw_r.
+    gen = torch.Generator().manual_seed(8)
+    e, h, i, r, s = 3, 64, 32, 4, 2.0
+    experts, offsets = [0, 2], [5, 9]
+    rows = offsets[-1]
+    rng = np.random.default_rng(8)
+    wg, wu = (lm.weights_bf16(gb.quantize((rng.standard_normal((e * i, h)) * 0.1).astype(np.float32), gb.Q8_0), gb.Q8_0).reshape(e, i, h) for _ in range(2))
+    wd = lm.weights_bf16(gb.quantize((rng.standard_normal((e * h, i)) * 0.1).astype(np.float32), gb.Q8_0), gb.Q8_0).reshape(e, h, i)
+    x = torch.randn(rows, h, generator=gen).to(torch.bfloat16)
+    dy = torch.randn(rows, h, generator=gen).to(torch.bfloat16)
+    w = torch.rand(rows, generator=gen).double() + 0.1
+    a_gu = (torch.randn(e, r, h, generator=gen) * h ** -0.5).to(torch.bfloat16)
+    b_gu = (torch.randn(e, 2 * i, r, generator=gen) * 0.1).to(torch.bfloat16)
+    a_d = (torch.randn(e, r, i, generator=gen) * i ** -0.5).to(torch.bfloat16)
+    b_d = (torch.randn(e, h, r, generator=gen) * 0.1).to(torch.bfloat16)
+    # the clamp is a discontinuity of the gradient: put the limit in the middle of the widest gap between the gate / up
+    # magnitudes, so that the bf16 rounding of gate and up moves no value across it
+    plain = lm.expert_layer(x, experts, offsets, wg, wu, wd, a_gu, b_gu, a_d, b_d, s)
+    mags = torch.cat([plain["gate"].reshape(-1), plain["up"].reshape(-1)]).abs().sort().values
+    mags = mags[(mags > 0.3) & (mags < 1.0)]
+    gap = int((mags[1:] - mags[:-1]).argmax())
+    limit = float((mags[gap] + mags[gap + 1]) / 2)
+    assert float(mags[gap + 1] - mags[gap]) > 0.01  # bf16 rounding moves a value of this size by at most 0.002
+    for lim in (None, limit):
+        got = lm.expert_layer(x, experts, offsets, wg, wu, wd, a_gu, b_gu, a_d, b_d, s, dy, row_weight=w, limit=lim)
+        leaves = [t.double().clone().requires_grad_(True) for t in (x, a_gu, b_gu, a_d, b_d, w)]
+        xr, agr, bgr, adr, bdr, wr = leaves
+        row_expert = [0] * 5 + [2] * 4
+        total = 0.0
+        for row, ex in enumerate(row_expert):
+            gu = xr[row] @ torch.cat([wg[ex], wu[ex]]).T + s * ((xr[row] @ agr[ex].T) @ bgr[ex].T)
+            hid = lm.silu_mul(gu[:i], gu[i:], lim)
+            out = hid @ wd[ex].T + s * ((hid @ adr[ex].T) @ bdr[ex].T)
+            total = total + wr[row] * (out * dy[row].double()).sum()
+        total.backward()
+        assert max_rel(got["dx"], xr.grad) < 2e-2
+        assert max_rel(got["dw"], wr.grad) < 2e-2
+        for name, leaf in (("da_gu", agr), ("db_gu", bgr), ("da_d", adr), ("db_d", bdr)):
+            assert max_rel(got[name], leaf.grad) < 2e-2, (name, lim)
+        # the same layer with the weight folded into the cotangent beforehand (the reference's order) agrees to rounding
+        pre = lm.expert_layer(x, experts, offsets, wg, wu, wd, a_gu, b_gu, a_d, b_d, s, (dy.double() * w[:, None]).to(torch.bfloat16), limit=lim)
+        for name in ("dx", "da_gu", "db_gu", "da_d", "db_d"):
+            assert max_rel(got[name], pre[name]) < 2e-2, (name, lim)
+    assert (got["gate"] > limit).any() or (got["up"].abs() > limit).any()  # the clamp was exercised

@@ -298,8 +298,14 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
                             const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts, int qt,
                             int64_t rows, int64_t n, int64_t k, const void* x, RowIndex x_index, const void* xa, const void* lora_a,
                             const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b, void* ws,
-                            int64_t ws_bytes, void* stream) {
+                            int64_t ws_bytes, void* stream, RowIndex dy_index = RowIndex{}, const void* row_weights = nullptr,
+                            int row_weights_are_bf16 = 0) {
+    // dy_index: row i of the launch is row dy_index.source(i) of dy1 (one cotangent matrix), and, with row_weights, stands
+    // for weights[dy_index.row_index[i]] times that row: dx comes out WITHOUT that factor (the caller applies it), the
+    // factor gradients with it (it is put on their small operand, dy.B or xa)
     hipStream_t s = as_stream(stream);
+    if (dy_index.on() && (dy2 || (uint64_t)dy_index.index_rows * (uint64_t)n * 2 >= (1ull << 32)))
+        return set_error(GGQ_ERR_SHAPE, "%s: an indexed cotangent is one matrix under 4 GiB", what);
     if (rows < 0 || n <= 0 || k <= 0 || rows >= (1ll << 31) || n >= (1ll << 30) || k >= (1ll << 30)) return set_error(GGQ_ERR_SHAPE, "%s: bad shape rows=%lld n=%lld k=%lld", what, (long long)rows, (long long)n, (long long)k);
     if (int rc = check_weights(what, qt, packed1, k)) return rc;
     if (packed2 && !aligned16(packed2)) return set_error(GGQ_ERR_ALIGN, "%s: packed weights must be 16-byte aligned", what);
@@ -319,7 +325,7 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
     const bool direct_ok = aligned16(dy1) && (!dy2 || aligned16(dy2)) && n % 64 == 0 && (nseg * (n / 64)) % 2 == 0 && n < (1 << 22) &&
                            (!lora_a || aligned16(lora_a)) && k % 8 == 0;
     if (int rc = init_params(p, qt, kModeNN, (int)rows, (int)n, (int)k, nseg, pick_shape(qt, rows, groups, direct_ok))) return rc;
-    p.a[0] = (const bf16_t*)dy1, p.a[1] = (const bf16_t*)dy2, p.lda = n;
+    p.a[0] = (const bf16_t*)dy1, p.a[1] = (const bf16_t*)dy2, p.lda = n, p.a_rows = dy_index;
     p.w[0] = (const uint8_t*)packed1, p.w[1] = (const uint8_t*)packed2;
     p.c[0] = dx, p.ldc = k;
     if (p.shape == kShapeDirect) p.col_tiles_per_wg = direct_tiles_per_wg(rows, groups, p.col_tiles_per_seg, nseg * p.steps_per_seg);
@@ -360,7 +366,7 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
         if (!dyb) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
         if (rows > 0) {
             SkinnyNtParams sp{};
-            sp.in[0] = (const bf16_t*)dy1, sp.in[1] = (const bf16_t*)dy2, sp.ld_in = n;
+            sp.in[0] = (const bf16_t*)dy1, sp.in[1] = (const bf16_t*)dy2, sp.ld_in = n, sp.in_rows = dy_index;
             sp.f = (const bf16_t*)lora_b, sp.ldf = r, sp.f_expert_elems = (int64_t)r * ntot, sp.f_natural = 1;
             sp.out = dyb;
             sp.m = (int)rows, sp.c = (int)n, sp.r = r, sp.nseg = nseg;
@@ -385,8 +391,9 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
         if (d_lora_b) {
             FactorGradParams fp{};
             fp.partials = partials, fp.partials_bytes = partials_bytes;
-            fp.in[0] = (const bf16_t*)dy1, fp.in[1] = (const bf16_t*)dy2, fp.ld_in = n;
+            fp.in[0] = (const bf16_t*)dy1, fp.in[1] = (const bf16_t*)dy2, fp.ld_in = n, fp.in_rows = dy_index;
             fp.s = (const bf16_t*)xa, fp.out = (bf16_t*)d_lora_b, fp.out_expert_elems = ntot * r;
+            fp.s_weights = row_weights, fp.s_weight_index = dy_index.row_index, fp.s_weights_are_bf16 = row_weights_are_bf16;
             fp.ranges = ranges, fp.m = (int)rows, fp.c = (int)n, fp.r = r, fp.nseg = nseg, fp.out_j_major = 0, fp.scale = scale;
             if (int rc = factor_grad(fp, rp, experts, s)) return rc;
         }
@@ -395,6 +402,7 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
             fp.partials = partials, fp.partials_bytes = partials_bytes;
             fp.in[0] = (const bf16_t*)x, fp.ld_in = k, fp.in_rows = x_index;
             fp.s = dyb, fp.out = (bf16_t*)d_lora_a, fp.out_expert_elems = (int64_t)r * k;
+            fp.s_weights = row_weights, fp.s_weight_index = dy_index.row_index, fp.s_weights_are_bf16 = row_weights_are_bf16;
             fp.ranges = ranges, fp.m = (int)rows, fp.c = (int)k, fp.r = r, fp.nseg = 1, fp.out_j_major = 1, fp.scale = scale;
             if (int rc = factor_grad(fp, rp, experts, s)) return rc;
         }
@@ -427,6 +435,24 @@ int ggq_grouped_lora_mmq_backward_indexed(const void* dy1, const void* dy2, cons
     return grouped_backward(what, dy1, dy2, packed1, packed2, expert_ids, end_offsets, groups, experts, qt, rows, n, k, x,
                             RowIndex{row_index, index_div, (int)x_rows}, xa, lora_a, lora_b, r, scale, dx, d_lora_a, d_lora_b, ws, ws_bytes,
                             stream);
+}
+
+// The backward of a projection whose output rows were scaled by routing weights and summed per token (the expert FFN's
+// down projection followed by the combine): grad_out is the [tokens, n] cotangent of the COMBINED output; expert-sorted
+// row i stands for weights[permutation[i]] * grad_out[permutation[i] / top_k].  dx_unscaled is dy . W (+ LoRA term) of
+// the unweighted token rows; d_lora_a / d_lora_b carry the weights.
+int ggq_grouped_lora_mmq_backward_routed_output(const void* grad_out, int64_t tokens, const int64_t* permutation, int top_k,
+                                                const void* weights, int weights_are_bf16, const void* packed,
+                                                const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts,
+                                                int qt, int64_t rows, int64_t n, int64_t k, const void* x, const void* xa,
+                                                const void* lora_a, const void* lora_b, int r, float scale, void* dx_unscaled,
+                                                void* d_lora_a, void* d_lora_b, void* ws, int64_t ws_bytes, void* stream) {
+    const char* what = "grouped_lora_mmq_backward_routed_output";
+    if (!permutation || !weights) return set_error(GGQ_ERR_NULL, "%s: null permutation or weights", what);
+    if (tokens <= 0 || tokens >= (1ll << 31) || top_k <= 0 || rows != tokens * top_k) return set_error(GGQ_ERR_SHAPE, "%s: rows must be tokens * top_k", what);
+    return grouped_backward(what, grad_out, nullptr, packed, nullptr, expert_ids, end_offsets, groups, experts, qt, rows, n, k, x, RowIndex{}, xa,
+                            lora_a, lora_b, r, scale, dx_unscaled, d_lora_a, d_lora_b, ws, ws_bytes, stream,
+                            RowIndex{permutation, top_k, (int)tokens}, weights, weights_are_bf16);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -486,6 +512,13 @@ int ggq_swiglu_clamped_forward(const void* gate, const void* up, void* h, int64_
 int ggq_swiglu_backward(const void* gate, const void* up, const void* dh, void* dgate, void* dup, int64_t elems, void* stream) {
     if (!gate || !up || !dh || !dgate || !dup) return set_error(GGQ_ERR_NULL, "swiglu_backward: null pointer");
     return swiglu_bwd(gate, up, dh, dgate, dup, elems, 0.0f, as_stream(stream));
+}
+
+int ggq_swiglu_backward_routed(const void* gate, const void* up, const void* dh_unweighted, const void* weights, int weights_are_bf16,
+                               const int64_t* permutation, void* dgate, void* dup, void* grad_weights, int64_t rows, int inter, float limit,
+                               void* stream) {
+    if (!gate || !up || !dh_unweighted || !weights || !permutation || !dgate || !dup) return set_error(GGQ_ERR_NULL, "swiglu_backward_routed: null pointer");
+    return swiglu_bwd_routed(gate, up, dh_unweighted, weights, weights_are_bf16, permutation, dgate, dup, grad_weights, rows, inter, limit, as_stream(stream));
 }
 
 int ggq_swiglu_clamped_backward(const void* gate, const void* up, const void* dh, void* dgate, void* dup, int64_t elems, float limit, void* stream) {

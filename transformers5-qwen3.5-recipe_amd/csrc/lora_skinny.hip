@@ -325,7 +325,17 @@ __global__ __launch_bounds__(256) void factor_grad_kernel(FactorGradParams p) {
                 vin[u][cb] = load8g(in + (int64_t)src * p.ld_in + tcc, r < row_end ? p.c - tcc : 0, vec);
             }
             vs[u] = make_uint4(0, 0, 0, 0);
-            if (sr < 32 && m0 + 32 * u + sr < row_end) vs[u] = *(const uint4*)(p.s + (int64_t)(m0 + 32 * u + sr) * rp + sch * 8);
+            if (sr < 32 && m0 + 32 * u + sr < row_end) {
+                const int64_t row = m0 + 32 * u + sr;
+                vs[u] = *(const uint4*)(p.s + row * rp + sch * 8);
+                if (p.s_weights) {
+                    const int64_t wi = p.s_weight_index[row];
+                    // (routing weights act at bf16 precision everywhere on the path)
+                    const float w = p.s_weights_are_bf16 ? bf16_to_f32(((const bf16_t*)p.s_weights)[wi]) : bf16_to_f32(to_bf16(((const float*)p.s_weights)[wi]));
+                    vs[u] = make_uint4(pack_bf16(bf16_lo(vs[u].x) * w, bf16_hi(vs[u].x) * w), pack_bf16(bf16_lo(vs[u].y) * w, bf16_hi(vs[u].y) * w),
+                                       pack_bf16(bf16_lo(vs[u].z) * w, bf16_hi(vs[u].z) * w), pack_bf16(bf16_lo(vs[u].w) * w, bf16_hi(vs[u].w) * w));
+                }
+            }
         }
 #pragma unroll
         for (int u = 0; u < 4; u++) {

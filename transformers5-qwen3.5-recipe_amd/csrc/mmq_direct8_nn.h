@@ -86,7 +86,10 @@ struct Direct8NN {
         for (int i = 0; i < NI; i++) {
             const int r = 64 * i + (tid >> 3), s = tid & 7;
             const int kc = s ^ ((r >> 1) & 7);
-            a_voff[i] = (uint32_t)(((int64_t)min(r, c.rows_valid - 1) * p.lda + kc * 8) * 2);
+            const int rr = min(r, c.rows_valid - 1);
+            // with a row index (one cotangent matrix read through it) the lane offsets carry the whole stored row
+            const int src = p.a_rows.on() ? p.a_rows.source(c.row_begin + rr) : rr;
+            a_voff[i] = (uint32_t)(((int64_t)src * p.lda + kc * 8) * 2);
         }
         // packed bytes of a step: lane t of the workgroup moves quant chunk (t % 8) ^ swizzle of weight row t / 8
         // (the 16-byte chunks of a row are XOR-swizzled like an A row's: the per-row reads below meet no bank conflict);
@@ -99,7 +102,7 @@ struct Direct8NN {
         int w_tile_i = ct0, w_step_i = 0, w_wr = 0;
         auto step_src_a = [&](int st) __attribute__((always_inline)) {
             const int seg = st >= sps ? 1 : 0, local = st - seg * sps;
-            return (seg ? p.a[1] : p.a[0]) + (int64_t)c.row_begin * p.lda + local * 64;
+            return (seg ? p.a[1] : p.a[0]) + (p.a_rows.on() ? 0 : (int64_t)c.row_begin * p.lda) + local * 64;
         };
         auto step_src_w = [&](int ct, int st) __attribute__((always_inline)) {
             const int seg = st >= sps ? 1 : 0, local = st - seg * sps;

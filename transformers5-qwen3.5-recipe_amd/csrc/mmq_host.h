@@ -44,6 +44,10 @@ struct FactorGradParams {
     int64_t ld_in;
     RowIndex in_rows;     // segment 0 only (nseg == 1 when set)
     const bf16_t* s;      // [m, r_pad]
+    // optional factor per row of s: row i is scaled by weights[index[i]] (fp32 or bf16 weights) and rounded to bf16 again
+    const void* s_weights;
+    const int64_t* s_weight_index;
+    int s_weights_are_bf16;
     bf16_t* out;          // per expert: [nseg*c][r] (out_j_major = 0) or [r][nseg*c] (= 1)
     int64_t out_expert_elems;
     const int* ranges;    // per expert (row_begin, row_end); null: all m rows, one expert
@@ -74,7 +78,7 @@ enum : int {
 struct MmqParams {
     const bf16_t* a[2];   // activations; [1] only for a pair in NN mode
     int64_t lda;
-    RowIndex a_rows;      // NT mode only (segment 0 is the only activation matrix there)
+    RowIndex a_rows;      // rows of a[0] read through an index (one segment only; the matrix stays under 4 GiB)
     int a_zero_padded;    // the rows of a hold zeros from the contraction length up to the next multiple of 64 (lda covers them):
                           // a contraction that ends inside a 64-wide step still takes the aligned 16-byte loads
     const uint8_t* w[2];  // packed weights; [1] only for a pair
@@ -159,6 +163,8 @@ int router_topk(const void* logits, int logits_are_bf16, int64_t tokens, int num
                 int64_t* indices, void* weights, int weights_mode, float scale, hipStream_t s);
 int swiglu_fwd(const void* gate, const void* up, void* h, int64_t elems, float limit, hipStream_t s);
 int swiglu_bwd(const void* gate, const void* up, const void* dh, void* dgate, void* dup, int64_t elems, float limit, hipStream_t s);
+int swiglu_bwd_routed(const void* gate, const void* up, const void* dh, const void* weights, int w_is_bf16, const int64_t* permutation,
+                      void* dgate, void* dup, void* grad_weights, int64_t routes, int inter, float limit, hipStream_t s);
 
 int64_t lmhead_ce_workspace_bytes(int64_t rows, int64_t vocab, int64_t hidden, int64_t chunk);
 int lmhead_ce(int qt, const void* hidden, const void* packed, const int64_t* labels, int64_t rows, int64_t vocab,

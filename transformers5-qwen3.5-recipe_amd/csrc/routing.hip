@@ -453,6 +453,72 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const uint4* gate, cons
     }
 }
 
+// Backward of h = silu(gate) * up for rows whose cotangent arrives without its routing weight: one wave per expert-sorted
+// row s, route = permutation[s], w = weights[route].  With d = the unweighted cotangent row, the gradient of the weight is
+// sum_j d[j] * h[j] (h recomputed exactly as the forward rounds it), accumulated in fp32 in a fixed lane-strided order and
+// reduced by a butterfly, and dgate / dup are those of the cotangent w * d (the product is not rounded in between).
+__global__ __launch_bounds__(256) void swiglu_bwd_routed_kernel(const uint4* gate, const uint4* up, const uint4* dh, const void* weights,
+                                                                int w_is_bf16, const int64_t* permutation, uint4* dgate, uint4* dup,
+                                                                void* grad_weights, int64_t routes, int chunks_per_row, float limit) {
+    const float hi = limit > 0.0f ? limit : INFINITY;
+    const int lane = threadIdx.x & 63;
+    const int64_t s = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (s >= routes) return;
+    const int64_t route = permutation[s];
+    const float w = load_weight(weights, w_is_bf16, route);
+    float dot = 0.f;
+    for (int ch = lane; ch < chunks_per_row; ch += 64) {
+        const int64_t i = s * chunks_per_row + ch;
+        const uint4 g = gate[i], u = up[i], d = dh[i];
+        const uint32_t gv[4] = {g.x, g.y, g.z, g.w}, uv[4] = {u.x, u.y, u.z, u.w}, dv[4] = {d.x, d.y, d.z, d.w};
+        uint32_t rg[4], ru[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            float og[2], ou[2], hh[2], dd[2];
+#pragma unroll
+            for (int hlf = 0; hlf < 2; hlf++) {
+                const float xr = hlf ? bf16_hi(gv[e]) : bf16_lo(gv[e]);
+                const float ur = hlf ? bf16_hi(uv[e]) : bf16_lo(uv[e]);
+                dd[hlf] = hlf ? bf16_hi(dv[e]) : bf16_lo(dv[e]);
+                const float x = fminf(xr, hi), uu = fminf(fmaxf(ur, -hi), hi);
+                const float den = 1.0f + __expf(-x);
+                hh[hlf] = (x / den) * uu;  // the forward's expression, rounded below as the forward stores it
+                const float sig = 1.0f / den;
+                const float dw = dd[hlf] * w;
+                og[hlf] = xr <= hi ? dw * uu * (sig * (1.0f + x * (1.0f - sig))) : 0.0f;
+                ou[hlf] = (ur >= -hi && ur <= hi) ? dw * x * sig : 0.0f;
+            }
+            const uint32_t hb = pack_bf16(hh[0], hh[1]);
+            dot = fmaf(dd[0], bf16_lo(hb), dot);
+            dot = fmaf(dd[1], bf16_hi(hb), dot);
+            rg[e] = pack_bf16(og[0], og[1]);
+            ru[e] = pack_bf16(ou[0], ou[1]);
+        }
+        dgate[i] = make_uint4(rg[0], rg[1], rg[2], rg[3]);
+        dup[i] = make_uint4(ru[0], ru[1], ru[2], ru[3]);
+    }
+    if (grad_weights) {
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) dot += __shfl_xor(dot, off, 64);
+        if (lane == 0) {
+            if (w_is_bf16) ((bf16_t*)grad_weights)[route] = to_bf16(dot);
+            else ((float*)grad_weights)[route] = dot;
+        }
+    }
+}
+
+int swiglu_bwd_routed(const void* gate, const void* up, const void* dh, const void* weights, int w_is_bf16, const int64_t* permutation,
+                      void* dgate, void* dup, void* grad_weights, int64_t routes, int inter, float limit, hipStream_t s) {
+    if (inter <= 0 || inter % 8) return set_error(GGQ_ERR_SHAPE, "swiglu_backward_routed: row width must be a positive multiple of 8");
+    if (((uintptr_t)gate | (uintptr_t)up | (uintptr_t)dh | (uintptr_t)dgate | (uintptr_t)dup) & 15) return set_error(GGQ_ERR_ALIGN, "swiglu_backward_routed: buffers must be 16-byte aligned");
+    if (routes == 0) return GGQ_OK;
+    const int64_t grid = (routes + 3) / 4;
+    if (grid > 0x7FFFFFFF) return set_error(GGQ_ERR_SHAPE, "swiglu_backward_routed: too many routes");
+    hipLaunchKernelGGL(swiglu_bwd_routed_kernel, dim3((unsigned)grid), dim3(256), 0, s, (const uint4*)gate, (const uint4*)up, (const uint4*)dh, weights,
+                       w_is_bf16, permutation, (uint4*)dgate, (uint4*)dup, grad_weights, routes, inter / 8, limit);
+    return check_launch("swiglu_backward_routed");
+}
+
 int swiglu_fwd(const void* gate, const void* up, void* h, int64_t elems, float limit, hipStream_t s) {
     if (elems % 8) return set_error(GGQ_ERR_SHAPE, "swiglu: element count must be a multiple of 8");
     if (((uintptr_t)gate | (uintptr_t)up | (uintptr_t)h) & 15) return set_error(GGQ_ERR_ALIGN, "swiglu: buffers must be 16-byte aligned");

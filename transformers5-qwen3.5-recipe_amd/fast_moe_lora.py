@@ -296,6 +296,73 @@ def swiglu(gate: torch.Tensor, up: torch.Tensor, limit: float | None = None) -> 
     return _SwiGLU.apply(gate, up, limit)
 
 
+# set to False to run the activation, the down projection and the combine as three autograd nodes (the reference's structure)
+FUSE_GATED_DOWN_COMBINE = True
+
+
+class _RoutedGatedDownProjection(torch.autograd.Function):
+    """silu(gate) * up, the down projection with its LoRA delta, and the weighted sum of every token's routes
+    (fast_moe_lora.py:747-770 with fast_moe_routing.py:431-459) as ONE autograd node.  The forward runs the same three
+    launches as the separate nodes and gives the same bits.  The backward never forms the [routes, hidden] cotangent of the
+    expert output: the grad-input launch reads the tokens' cotangent rows through the permutation and leaves the routing
+    weight out, the activation's backward applies it and computes the routing weights' gradient as
+    <unweighted dH[route], h[route]>, which equals the reference's <dOut[token], expert_out[route]>
+    (fast_moe_routing.py:217-224) up to rounding; the factor gradients carry the weight on their rank-r operand."""
+
+    @staticmethod
+    def forward(ctx, gate, up, limit, payload, expert_indices, expert_offsets, quant_type, out_features, lora_a, lora_b, scaling,
+                routing_weights, permutation, inverse_permutation):
+        _lib.require_device_tensor(gate, "gate", torch.bfloat16)
+        _lib.require_device_tensor(up, "up", torch.bfloat16)
+        lib, stream = _lib.load(), _lib.stream_handle(gate.device)
+        act = torch.empty_like(gate)
+        if limit is None:
+            _lib.check(lib.ggq_swiglu_forward(gate.data_ptr(), up.data_ptr(), act.data_ptr(), gate.numel(), stream))
+        else:
+            _lib.check(lib.ggq_swiglu_clamped_forward(gate.data_ptr(), up.data_ptr(), act.data_ptr(), gate.numel(), float(limit), stream))
+        y, _, xa = _grouped_forward(act, payload, None, expert_indices, expert_offsets, quant_type, out_features, lora_a, lora_b, scaling)
+        tokens, top_k = routing_weights.shape
+        out = torch.empty(tokens, out_features, dtype=y.dtype, device=y.device)
+        _lib.check(lib.ggq_route_combine_forward(y.data_ptr(), routing_weights.data_ptr(), int(routing_weights.dtype == torch.bfloat16),
+                                                 inverse_permutation.data_ptr(), out.data_ptr(), tokens, top_k, out_features, stream))
+        ctx.has_lora = lora_a is not None
+        ctx.save_for_backward(gate, up, act, payload, expert_indices, expert_offsets, routing_weights, permutation,
+                              *((xa, lora_a, lora_b) if ctx.has_lora else ()))
+        ctx.meta = (float(limit or 0.0), int(quant_type), int(out_features), float(scaling))
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        if torch.is_grad_enabled():
+            raise RuntimeError("packed grouped MMQ does not support higher-order gradients")
+        gate, up, act, payload, expert_indices, expert_offsets, routing_weights, permutation, *rest = ctx.saved_tensors
+        xa, lora_a, lora_b = rest if ctx.has_lora else (None, None, None)
+        limit, quant_type, n, scaling = ctx.meta
+        grad_out = grad_out.contiguous()
+        _lib.require_device_tensor(grad_out, "combined output cotangent", torch.bfloat16)
+        rows, k = act.shape
+        tokens, top_k = routing_weights.shape
+        experts = payload.shape[0]
+        r = 0 if lora_a is None else lora_a.shape[1]
+        dev = act.device
+        lib, stream = _lib.load(), _lib.stream_handle(dev)
+        d_act = torch.empty(rows, k, dtype=torch.bfloat16, device=dev)
+        da = torch.empty_like(lora_a) if (ctx.has_lora and ctx.needs_input_grad[8]) else None
+        db = torch.empty_like(lora_b) if (ctx.has_lora and ctx.needs_input_grad[9]) else None
+        w_bf16 = int(routing_weights.dtype == torch.bfloat16)
+        ws = _lora_ws(dev, rows, expert_indices.numel(), experts, n, k, r)
+        _lib.check(lib.ggq_grouped_lora_mmq_backward_routed_output(
+            grad_out.data_ptr(), tokens, permutation.data_ptr(), top_k, routing_weights.data_ptr(), w_bf16, payload.data_ptr(),
+            expert_indices.data_ptr(), expert_offsets.data_ptr(), expert_indices.numel(), experts, quant_type, rows, n, k, act.data_ptr(),
+            _lib.ptr(xa), _lib.ptr(lora_a), _lib.ptr(lora_b), r, scaling, d_act.data_ptr(), _lib.ptr(da), _lib.ptr(db), ws.data_ptr(),
+            ws.numel(), stream))
+        dgate, dup = torch.empty_like(gate), torch.empty_like(up)
+        dw = torch.empty_like(routing_weights) if ctx.needs_input_grad[11] else None
+        _lib.check(lib.ggq_swiglu_backward_routed(gate.data_ptr(), up.data_ptr(), d_act.data_ptr(), routing_weights.data_ptr(), w_bf16,
+                                                  permutation.data_ptr(), dgate.data_ptr(), dup.data_ptr(), _lib.ptr(dw), rows, k, limit, stream))
+        return dgate, dup, None, None, None, None, None, None, da, db, None, dw, None, None
+
+
 # ------------------------------------------------------------------------------------------------
 def _group_sizes_from_offsets(offsets: torch.Tensor) -> torch.Tensor:
     if offsets.ndim != 1:
@@ -407,6 +474,13 @@ def qwen3_5_moe_gguf_mmq_lora_forward(self: GGUFExperts, hidden_states: torch.Te
         gate, up = _GroupedLoraProjection.apply(
             selected, _as_payload(self.gate_proj), _as_payload(self.up_proj), expert_indices, expert_offsets,
             int(self.gate_proj.quant_type), self.intermediate_dim, lw.gate_up_a if lw else None, lw.gate_up_b if lw else None, s)
+    if (FUSE_GATED_DOWN_COMBINE and execution_plan.output_mask is None and type(self)._apply_split_gate is GGUFExperts._apply_split_gate
+            and routing_plan.routing_weights.is_contiguous()):
+        combined = _RoutedGatedDownProjection.apply(
+            gate, up, self.swiglu_limit, _as_payload(self.down_proj), expert_indices, expert_offsets, int(self.down_proj.quant_type),
+            self.hidden_dim, lw.down_a if lw else None, lw.down_b if lw else None, s, routing_plan.routing_weights, routing_plan.permutation,
+            routing_plan.inverse_permutation)
+        return combined.to(hidden_states.dtype).reshape(hidden_states.shape)
     intermediate = self._apply_split_gate(gate, up)
     output = _GroupedLoraProjection.apply(
         intermediate, _as_payload(self.down_proj), None, expert_indices, expert_offsets, int(self.down_proj.quant_type),
