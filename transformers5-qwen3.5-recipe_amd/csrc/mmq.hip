@@ -28,22 +28,39 @@ int check_launch(const char* what) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// Row-tile tables.  One workgroup per table; groups are walked 256 at a time with an LDS prefix sum, so
+// Inclusive prefix sum over the 256 threads of the workgroup: a shuffle scan inside each wave, then the wave totals
+// through LDS (one barrier; `totals` must not be reused before the next barrier of the caller).
+__device__ __forceinline__ int block_scan_inclusive(int v, int tid, int* totals) {
+    const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int u = __shfl_up(v, off, 64);
+        if (lane >= off) v += u;
+    }
+    if (lane == 63) totals[wave] = v;
+    __syncthreads();
+    int before = 0;
+#pragma unroll
+    for (int w = 0; w < 3; w++) before += w < wave ? totals[w] : 0;
+    return v + before;
+}
+
+// Row-tile tables.  One workgroup per table; groups are walked 256 at a time with a prefix sum, so
 // a table is in group order and identical from run to run.  Table t keeps the groups with
 // min_rows[t] < rows <= max_rows[t] and cuts them into tiles of bm[t] rows.
 __global__ __launch_bounds__(256) void build_row_tiles_kernel(const int64_t* expert_ids, const int32_t* end_offsets,
                                                               int groups, RowTileTables tb, int* expert_ranges,
                                                               int num_experts) {
-    __shared__ int scan[256];
-    __shared__ int base;
+    __shared__ int totals[2][4];
     const int tid = threadIdx.x, t = blockIdx.x;
     const int bm = tb.bm[t], min_rows = tb.min_rows[t], max_rows = tb.max_rows[t];
     TileDesc* tiles = tb.tiles[t];
     if (expert_ranges && t == 0) {
         for (int e = tid; e < num_experts; e += 256) expert_ranges[2 * e] = expert_ranges[2 * e + 1] = 0;
+        __syncthreads();  // (the ranges of the listed groups are written below, by other threads)
     }
-    if (tid == 0) base = 0;
-    __syncthreads();
+    int base = 0;  // tiles of the groups walked so far (the same value in every thread)
+    int flip = 0;
     for (int g0 = 0; g0 < groups; g0 += 256) {
         const int g = g0 + tid;
         int r0 = 0, r1 = 0, count = 0, expert = 0;
@@ -57,33 +74,24 @@ __global__ __launch_bounds__(256) void build_row_tiles_kernel(const int64_t* exp
                 if (e >= 0 && e < num_experts) expert_ranges[2 * e] = r0, expert_ranges[2 * e + 1] = r1;
             }
         }
-        scan[tid] = count;
-        __syncthreads();
-        for (int off = 1; off < 256; off <<= 1) {  // inclusive Hillis-Steele scan
-            int v = tid >= off ? scan[tid - off] : 0;
-            __syncthreads();
-            scan[tid] += v;
-            __syncthreads();
-        }
-        const int first = base + scan[tid] - count;
+        const int incl = block_scan_inclusive(count, tid, totals[flip]);
+        const int first = base + incl - count;
         for (int i = 0; i < count; i++) {
             TileDesc d;
             d.group = g, d.row_begin = r0 + i * bm, d.row_end = min(r1, r0 + (i + 1) * bm), d.expert = expert;
             tiles[first + i] = d;
         }
-        __syncthreads();
-        if (tid == 255) base += scan[255];
-        __syncthreads();
+        base += totals[flip][0] + totals[flip][1] + totals[flip][2] + totals[flip][3];
+        flip ^= 1;  // the next round's totals go to the other row: no barrier needed between the rounds
     }
     if (tid == 0) *tb.num_tiles[t] = base;
     TileDesc* by_size = tb.by_size[t];
     if (!by_size) return;
     // Stable bucket sort by the number of 32-row blocks, largest first: thread i takes the i-th contiguous share of the
-    // table; per-thread bucket counts are scanned over the threads, bucket after bucket.
+    // table; the per-thread bucket counts are scanned over the threads, bucket after bucket.
     __syncthreads();  // the table written above is visible to the whole workgroup
     constexpr int kBuckets = 8;  // tiles of up to 256 rows
-    __shared__ int bucket_count[kBuckets][256];
-    __shared__ int bucket_base[kBuckets];
+    __shared__ int bucket_totals[kBuckets][4];
     const int total = base;
     const int share = (total + 255) / 256, i0 = min(total, tid * share), i1 = min(total, i0 + share);
     int mine[kBuckets];
@@ -94,31 +102,14 @@ __global__ __launch_bounds__(256) void build_row_tiles_kernel(const int64_t* exp
 #pragma unroll
         for (int b = 0; b < kBuckets; b++) mine[b] += bucket == b;
     }
+    int at[kBuckets];  // position of this thread's first tile of bucket b
+    int run = 0;
 #pragma unroll
-    for (int b = 0; b < kBuckets; b++) bucket_count[b][tid] = mine[b];
-    __syncthreads();
-    if (tid < kBuckets) {  // exclusive scan over the threads of one bucket (256 entries: serial is a few microseconds at most)
-        int run = 0;
-        for (int j = 0; j < 256; j++) {
-            const int v = bucket_count[tid][j];
-            bucket_count[tid][j] = run;
-            run += v;
-        }
-        bucket_base[tid] = run;
+    for (int b = 0; b < kBuckets; b++) {
+        const int incl = block_scan_inclusive(mine[b], tid, bucket_totals[b]);
+        at[b] = run + incl - mine[b];
+        run += bucket_totals[b][0] + bucket_totals[b][1] + bucket_totals[b][2] + bucket_totals[b][3];
     }
-    __syncthreads();
-    if (tid == 0) {
-        int run = 0;
-        for (int b = 0; b < kBuckets; b++) {
-            const int v = bucket_base[b];
-            bucket_base[b] = run;
-            run += v;
-        }
-    }
-    __syncthreads();
-    int at[kBuckets];
-#pragma unroll
-    for (int b = 0; b < kBuckets; b++) at[b] = bucket_base[b] + bucket_count[b][tid];
     for (int i = i0; i < i1; i++) {
         const TileDesc d = tiles[i];
         const int bucket = kBuckets - min(kBuckets, max(1, (d.row_end - d.row_begin + 31) >> 5));
