@@ -83,16 +83,17 @@ static int launch_wide_and_tall(int qt, int mode, MmqParams& p, int rows, int n,
     MmqParams sizes;
     if (int rc = init_params(sizes, qt, mode, rows, n, k, nseg, kShapeTall)) return rc;
     p.tiles2 = tall, p.num_tiles2 = num_tall, p.max_row_tiles2 = max_tall, p.col_tiles_per_seg2 = sizes.col_tiles_per_seg;
-    return launch_mmq_mixed(mode, p, s);
+    return launch_mmq_mixed(qt, mode, p, s);
 }
 
 // Q4_K over expert groups that average at most 256 rows runs the direct kernels (the MFMA waves decode the weights
-// themselves) when the operands allow (`direct_ok`); otherwise groups that average at most 192 rows run the Q4_K tile kernel
-// in its wide shape, mixed with tall tiles for their larger groups; everything else runs tall tiles.
+// themselves) when the operands allow (`direct_ok`); otherwise, and for every other block format, groups that average at
+// most 192 rows run the tile kernel in its wide shape, mixed with tall tiles for their larger groups; everything else runs
+// tall tiles.
 static int pick_shape(int qt, int64_t rows, int64_t groups, bool direct_ok) {
-    if (qt != 12 /* GGML Q4_K */) return kShapeTall;
     const int forced = g_shape_override;  // a test aid
-    if (direct_ok && (forced == kShapeDirect || (forced < 0 && groups > 0 && rows <= 256 * groups))) return kShapeDirect;
+    const bool q4k = qt == 12;            // GGML Q4_K: the only block format with decoding-wave kernels
+    if (q4k && direct_ok && (forced == kShapeDirect || (forced < 0 && groups > 0 && rows <= 256 * groups))) return kShapeDirect;
     if (forced == kShapeTall || !(groups > 0 && rows <= 192 * groups)) return kShapeTall;
     return kShapeWide;
 }

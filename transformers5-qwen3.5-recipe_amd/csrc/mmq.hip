@@ -234,7 +234,7 @@ static int launch_direct(const MmqParams& p, hipStream_t s) {
     return check_launch(MODE == kModeNT ? "mmq_direct8_q4k_kernel" : "mmq_direct8_nn_q4k_kernel");
 }
 
-template <int MODE>
+template <int QT, int MODE>
 static int launch_mixed_mode(const MmqParams& p, hipStream_t s) {
     const int segs = MODE == kModeNT ? p.nseg : 1;
     // per XCD: ceil(wide units / 8) * wide column tiles + ceil(tall units / 8) * tall column tiles slots
@@ -247,24 +247,36 @@ static int launch_mixed_mode(const MmqParams& p, hipStream_t s) {
     if (g_timing && g_timed_count < kMaxTimedLaunches) {
         t = &g_timed[g_timed_count];
         if (hipEventCreate(&t->start) != hipSuccess || hipEventCreate(&t->stop) != hipSuccess) return set_error(GGQ_ERR_RUNTIME, "mmq: event creation failed");
-        t->qt = kQ4_K, t->mode = MODE, t->epi = kEpiStore, t->shape = kShapeMixed;
+        t->qt = QT, t->mode = MODE, t->epi = kEpiStore, t->shape = kShapeMixed;
         g_timed_count++;
         (void)hipEventRecord(t->start, s);
     }
-    constexpr int kSmemBytes = Tile<kShapeWide>::kTileLdsBytes > Tile<kShapeTall>::kTileLdsBytes ? Tile<kShapeWide>::kTileLdsBytes : Tile<kShapeTall>::kTileLdsBytes;
-    static bool attr_set = false;
+    constexpr int kSmemBytes = (Tile<kShapeWide>::kTileLdsBytes > Tile<kShapeTall>::kTileLdsBytes ? Tile<kShapeWide>::kTileLdsBytes : Tile<kShapeTall>::kTileLdsBytes) +
+                               (QT == kIQ2_XXS ? Fmt<kIQ2_XXS>::kTableWords * 4 : 0);
+    static bool attr_set = false;  // per instantiation
     if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)mmq_mixed_kernel<kQ4_K, MODE, kEpiStore>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess)
+        if (hipFuncSetAttribute((const void*)mmq_mixed_kernel<QT, MODE, kEpiStore>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess)
             return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", kSmemBytes);
         attr_set = true;
     }
-    hipLaunchKernelGGL((mmq_mixed_kernel<kQ4_K, MODE, kEpiStore>), dim3((unsigned)grid), dim3(kThreads), kSmemBytes, s, p);
+    hipLaunchKernelGGL((mmq_mixed_kernel<QT, MODE, kEpiStore>), dim3((unsigned)grid), dim3(kThreads), kSmemBytes, s, p);
     if (t) (void)hipEventRecord(t->stop, s);
     return check_launch("mmq_mixed_kernel");
 }
 
-int launch_mmq_mixed(int mode, const MmqParams& p, hipStream_t s) {
-    return mode == kModeNT ? launch_mixed_mode<kModeNT>(p, s) : launch_mixed_mode<kModeNN>(p, s);
+int launch_mmq_mixed(int qt, int mode, const MmqParams& p, hipStream_t s) {
+#define GGQ_MIXED(QT) return mode == kModeNT ? launch_mixed_mode<QT, kModeNT>(p, s) : launch_mixed_mode<QT, kModeNN>(p, s)
+    switch (qt) {
+        case kQ8_0: GGQ_MIXED(kQ8_0);
+        case kQ2_K: GGQ_MIXED(kQ2_K);
+        case kQ3_K: GGQ_MIXED(kQ3_K);
+        case kQ4_K: GGQ_MIXED(kQ4_K);
+        case kQ5_K: GGQ_MIXED(kQ5_K);
+        case kQ6_K: GGQ_MIXED(kQ6_K);
+        case kIQ2_XXS: GGQ_MIXED(kIQ2_XXS);
+    }
+#undef GGQ_MIXED
+    return set_error(GGQ_ERR_QTYPE, "unsupported GGML type id %d", qt);
 }
 
 template <int QT>
@@ -273,14 +285,14 @@ static int launch_qt(int mode, int epi, const MmqParams& p, hipStream_t s) {
         switch (epi) {
             case kEpiStore:
                 if (QT == kQ4_K && p.shape == kShapeDirect) return launch_direct<kModeNT>(p, s);
-                if (QT == kQ4_K && p.shape == kShapeWide) return launch_one<kQ4_K, kModeNT, kEpiStore, 1>(p, s);
+                if (p.shape == kShapeWide) return launch_one<QT, kModeNT, kEpiStore, 1>(p, s);
                 return launch_one<QT, kModeNT, kEpiStore, 0>(p, s);
         }
     } else {
         switch (epi) {
             case kEpiStore:
                 if (QT == kQ4_K && p.shape == kShapeDirect) return launch_direct<kModeNN>(p, s);
-                if (QT == kQ4_K && p.shape == kShapeWide) return launch_one<kQ4_K, kModeNN, kEpiStore, 1>(p, s);
+                if (p.shape == kShapeWide) return launch_one<QT, kModeNN, kEpiStore, 1>(p, s);
                 return launch_one<QT, kModeNN, kEpiStore, 0>(p, s);
             case kEpiAccumF32: return launch_one<QT, kModeNN, kEpiAccumF32, 0>(p, s);
         }
@@ -311,7 +323,7 @@ int init_params(MmqParams& p, int qt, int mode, int m, int n, int k, int nseg, i
     p.m = m, p.n = n, p.k = k, p.nseg = nseg;
     p.w_row_bytes = packed_row_bytes(qt, k);
     p.w_expert_bytes = p.w_row_bytes * n;
-    if (shape != kShapeTall && qt != kQ4_K) shape = kShapeTall;  // the other shapes exist for Q4_K only
+    if (shape == kShapeDirect && qt != kQ4_K) shape = kShapeTall;  // the decoding-wave kernels exist for Q4_K only
     const int bm = shape == kShapeDirect ? kDirectBM : shape == kShapeTall ? kBM : kWideBM;
     const int bn = shape == kShapeDirect ? kDirectBN : shape == kShapeWide ? kWideBN : kBN;
     p.shape = shape;

@@ -117,7 +117,7 @@ int profile_end(float* ms, int* qt, int* mode, int* epi, int* shape, int capacit
 int measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64_t elems, int iters, float* tflops_out, hipStream_t s);
 const char* last_error();
 int launch_mmq(int qt, int mode, int epi, const MmqParams& p, hipStream_t s);
-int launch_mmq_mixed(int mode, const MmqParams& p, hipStream_t s);  // Q4_K, store epilogue, tiles + tiles2
+int launch_mmq_mixed(int qt, int mode, const MmqParams& p, hipStream_t s);  // Q4_K, store epilogue, tiles + tiles2
 int init_params(MmqParams& p, int qt, int mode, int m, int n, int k, int nseg, int shape = kShapeTall);
 
 int pad_factor(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int r, int r_pad, bool transpose, hipStream_t s);

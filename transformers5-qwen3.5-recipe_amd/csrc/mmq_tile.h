@@ -412,6 +412,53 @@ static __device__ __forceinline__ void produce(const MmqParams& p, const TileCtx
     lds_barrier();
 }
 
+// ---- Wide shape, every block format but Q4_K: all 512 producer lanes work on every step, one 32-wide run each
+// (forward: lane = (output column ptid / 2, run 2 * step + ptid % 2); grad-input: lane = (contraction row ptid / 8, run
+// ptid % 8 of the tile's 256 columns, so that the eight lanes of a row read adjacent bytes)).  A step is decoded and
+// stored in its own phase; its register set is reloaded for a later step as soon as it is decoded.
+// Expert groups of a few dozen rows give the consumers little to do per step, so the tile's time is the producers' chain
+// of load, decode, store and barrier: the wide tile runs that chain once per 256 output columns instead of once per 128.
+template <int QT, int MODE, class AfterIssue>
+static __device__ __forceinline__ void produce_all(const MmqParams& p, const TileCtx& c, int ptid, AfterIssue&& after_issue) {
+    static_assert(SH == 1, "the wide shape's producer");
+    ProducerLane l;
+    l.ptid = ptid;
+    l.lane = MODE == kModeNN ? (ptid >> 3) : (ptid & 63);
+    l.pw = MODE == kModeNN ? (ptid & 7) : (ptid >> 6);
+    l.w_ksub_nn = min((c.col0 >> 5) + l.pw, (p.k >> 5) - 1);
+    l.w_row_nt = min(c.col0 + (ptid >> 1), p.n - 1);
+    const int steps = c.total_steps;
+    uint32_t wv[16];
+    int stage = c.base, buf = c.base;
+    // The packed bytes of a step are requested kDepth steps ahead, in as many register sets as the block format's packed run
+    // allows (a step cannot take less than the memory latency / kDepth; measured, two sets and eight differ by 2 % at 64
+    // rows per group, so the latency is not what paces these tiles).
+    constexpr int kRawRegs = (int)(sizeof(typename Fmt<QT>::Raw) / 4);
+    constexpr int kDepth = kRawRegs <= 4 ? 8 : kRawRegs <= 12 ? 4 : 2;
+    typename Fmt<QT>::Raw raw[kDepth];
+#pragma unroll
+    for (int i = 0; i < kDepth; i++) w_issue_run<QT, MODE>(p, c, l, min(i, steps - 1), raw[i]);  // unconditional: a load under a branch is drained at the join
+    after_issue();
+    auto phase = [&](typename Fmt<QT>::Raw& r, int u) __attribute__((always_inline)) {
+        if (!c.a_fast && ptid < 256) fill_a_slow<MODE>(p, c, l, u, stage);
+        Fmt<QT>::pin(r);
+        Fmt<QT>::decode(r, MODE == kModeNT ? 2 * u + (ptid & 1) : l.w_ksub_nn, wv, c.grid);
+#pragma unroll
+        for (int i = 0; i < 16; i++) asm volatile("" : "+v"(wv[i]));  // the decode stays in front of the reload and the barrier
+        w_issue_run<QT, MODE>(p, c, l, min(u + kDepth, steps - 1), r);
+        w_store_run<MODE>(c, l, buf, wv);
+        lds_barrier();
+        stage = stage == kAStages - 1 ? 0 : stage + 1;
+        buf ^= 1;
+    };
+    for (int u = 0; u < steps; u += kDepth) {
+#pragma unroll
+        for (int i = 0; i < kDepth; i++)
+            if (u + i < steps) phase(raw[i], u + i);
+    }
+    lds_barrier();
+}
+
 // ---- Q4_K: both producer quartets (512 lanes) work on every step, half a run each.  The decode of a
 // step is the longest thing between two barriers when an expert group has few rows; splitting it over
 // all eight producer waves halves it.
@@ -972,6 +1019,7 @@ static __device__ __forceinline__ void run_tile(const MmqParams& p, const TileDe
 
     if (wave >= kCW) {
         if (QT == kQ4_K) produce_q4k<MODE>(p, c, tid - kProducerLanes, wave - kCW, lora_tiles);
+        else if constexpr (SH == 1) produce_all<QT, MODE>(p, c, tid - kProducerLanes, lora_tiles);
         else if (wave < 12) produce<QT, MODE, 0>(p, c, tid & 255, wave & 3, lora_tiles);
         else produce<QT, MODE, 1>(p, c, tid & 255, wave & 3, lora_tiles);
     } else {
