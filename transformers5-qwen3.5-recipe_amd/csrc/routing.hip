@@ -464,12 +464,16 @@ __global__ __launch_bounds__(256) void swiglu_bwd_routed_kernel(const uint4* gat
     const int lane = threadIdx.x & 63;
     const int64_t s = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (s >= routes) return;
+    // the row's first chunks are requested before the route's weight, which hangs on two dependent loads
+    const bool first = lane < chunks_per_row;
+    const int64_t i0 = s * chunks_per_row + (first ? lane : 0);
+    uint4 g = gate[i0], u = up[i0], d = dh[i0];
     const int64_t route = permutation[s];
     const float w = load_weight(weights, w_is_bf16, route);
     float dot = 0.f;
     for (int ch = lane; ch < chunks_per_row; ch += 64) {
         const int64_t i = s * chunks_per_row + ch;
-        const uint4 g = gate[i], u = up[i], d = dh[i];
+        if (ch != lane) g = gate[i], u = up[i], d = dh[i];
         const uint32_t gv[4] = {g.x, g.y, g.z, g.w}, uv[4] = {u.x, u.y, u.z, u.w}, dv[4] = {d.x, d.y, d.z, d.w};
         uint32_t rg[4], ru[4];
 #pragma unroll
