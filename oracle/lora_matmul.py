@@ -146,3 +146,26 @@ def expert_layer(x_sorted, experts, offsets, wg, wu, wd, a_gu, b_gu, a_d, b_d, s
     res.update(dh=dh, dgate=dgate, dup=dup, dx=back["dx"], da_gu=back["da"], db_gu=back["db"],
                da_d=dn["da"], db_d=dn["db"])
     return res
+
+
+def grouped_mm(lhs, rhs, group_sizes, dy=None):
+    """The grouped product the reference takes from AITER (``gmm``, fast_moe_lora.py:42-52) and its two gradients (``gmm``
+    against the transposed planes, :55-68; ``ptgmm``, :71-87), as the per-group loop the reference's tests use
+    (test_fast_moe_lora.py:106-130).  lhs [M,K], rhs [E,K,N], group_sizes [E] (consecutive row groups; rows no group covers
+    give zero rows and take no part in any gradient), dy [M,N].  float64; returns dict(out, dlhs, drhs)."""
+    lhs64, rhs64 = lhs.to(torch.float64), rhs.to(torch.float64)
+    m, n = lhs64.shape[0], rhs64.shape[2]
+    out = {"out": torch.zeros((m, n), dtype=torch.float64)}
+    if dy is not None:
+        dy64 = dy.to(torch.float64)
+        out["dlhs"] = torch.zeros_like(lhs64)
+        out["drhs"] = torch.zeros_like(rhs64)
+    r0 = 0
+    for e, size in enumerate(int(v) for v in group_sizes):
+        r1 = min(m, r0 + max(size, 0))
+        out["out"][r0:r1] = lhs64[r0:r1] @ rhs64[e]
+        if dy is not None:
+            out["dlhs"][r0:r1] = dy64[r0:r1] @ rhs64[e].T
+            out["drhs"][e] = lhs64[r0:r1].T @ dy64[r0:r1]
+        r0 = r1
+    return out

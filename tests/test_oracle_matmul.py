@@ -159,3 +159,28 @@ def test_expert_layer_with_row_weights_matches_autograd_of_the_weighted_sum():
         for name in ("dx", "da_gu", "db_gu", "da_d", "db_d"):
             assert max_rel(got[name], pre[name]) < 2e-2, (name, lim)
     assert (got["gate"] > limit).any() or (got["up"].abs() > limit).any()  # the clamp was exercised
+
+
+def test_grouped_mm_matches_autograd_of_the_group_loop():
+    """The closed-form gradients of the grouped product (a transposed operand or a group boundary off by one fails here),
+    rows no group covers included."""
+    gen = torch.Generator().manual_seed(31)
+    m, k, n, sizes = 11, 5, 4, [3, 0, 4, 2]  # two rows left over
+    lhs = torch.randint(-4, 5, (m, k), generator=gen).double().requires_grad_(True)
+    rhs = torch.randint(-4, 5, (len(sizes), k, n), generator=gen).double().requires_grad_(True)
+    dy = torch.randint(-4, 5, (m, n), generator=gen).double()
+    pieces, r0 = [], 0
+    for e, size in enumerate(sizes):
+        pieces.append(lhs[r0:r0 + size] @ rhs[e])
+        r0 += size
+    pieces.append(torch.zeros(m - r0, n, dtype=torch.float64))
+    out = torch.cat(pieces)
+    dlhs, drhs = torch.autograd.grad(out, (lhs, rhs), dy)
+    got = lm.grouped_mm(lhs.detach(), rhs.detach(), sizes, dy)
+    assert torch.equal(got["out"], out.detach())
+    assert torch.equal(got["dlhs"], dlhs)
+    assert torch.equal(got["drhs"], drhs)
+    assert torch.count_nonzero(got["drhs"][1]) == 0 and torch.count_nonzero(got["dlhs"][r0:]) == 0
+    # sizes running past the last row are clipped
+    clipped = lm.grouped_mm(lhs.detach(), rhs.detach(), [3, 0, 4, 100], dy)
+    assert torch.equal(clipped["out"][:7], out.detach()[:7]) and torch.equal(clipped["out"][7:], lhs.detach()[7:] @ rhs.detach()[3])

@@ -151,3 +151,24 @@ def test_operator_entries_give_the_package_results(pkg, dev):
     xg = bf16_randn(gen, 11, 8, 256).to(dev)
     assert torch.equal(fixed_grouped_mmq(xg, pg), pkg.fast_lora.fixed_grouped_mmq(xg, pg, gb.Q8_0))
     assert torch.equal(ops.fixed_grouped_mmq.default(xg, pg.as_subclass(torch.Tensor), gb.Q8_0), pkg.fast_lora.fixed_grouped_mmq(xg, pg, gb.Q8_0))
+
+
+def test_grouped_mm_stands_in_for_the_aiter_import_and_checks_its_operands(pkg):
+    """``from aiter.ops.triton.gmm import gmm, ptgmm`` (fast_moe_lora.py:22) resolves to the package's functions once
+    installed; their operand checks run without a device."""
+    import importlib
+    import sys
+
+    gm = pkg.grouped_mm
+    gm.install_as_aiter_gmm()
+    gm.install_as_aiter_gmm()  # idempotent
+    mod = importlib.import_module("aiter.ops.triton.gmm")
+    assert mod.gmm is gm.gmm and mod.ptgmm is gm.ptgmm
+    assert sys.modules["aiter"].ops.triton.gmm is mod
+    sizes = torch.tensor([2, 2, 2], dtype=torch.int32)
+    with pytest.raises(ValueError, match="expects lhs"):
+        gm.aiter_grouped_mm(torch.zeros(6, 4, 1, dtype=torch.bfloat16), torch.zeros(3, 4, 5, dtype=torch.bfloat16), sizes)
+    with pytest.raises(ValueError, match="expert mismatch"):
+        gm.aiter_grouped_mm(torch.zeros(6, 4, dtype=torch.bfloat16), torch.zeros(2, 4, 5, dtype=torch.bfloat16), sizes)
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        gm.aiter_grouped_mm(torch.zeros(6, 4, dtype=torch.bfloat16), torch.zeros(3, 4, 5, dtype=torch.bfloat16), sizes)

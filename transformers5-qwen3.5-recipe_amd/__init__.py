@@ -8,6 +8,6 @@ tensors; ``torch_ggml_ops`` registers the reference's operator names on these ke
 twins of the dense, expert and loss surfaces; ``_lib`` binds the shared library.
 """
 
-from . import _lib, deepseek_v4_liger_loss, deepseek_v4_lora, deepseek_v4_moe_lora, fast_lora, fast_moe_lora, fast_moe_ranking, fast_moe_routing, gguf, gguf_file, gguf_liger_loss, peft_compat, torch_ggml_ops  # noqa: F401
+from . import _lib, deepseek_v4_liger_loss, deepseek_v4_lora, deepseek_v4_moe_lora, fast_lora, fast_moe_lora, fast_moe_ranking, fast_moe_routing, gguf, gguf_file, gguf_liger_loss, grouped_mm, peft_compat, torch_ggml_ops  # noqa: F401
 
 __all__ = ["_lib", "deepseek_v4_liger_loss", "deepseek_v4_lora", "deepseek_v4_moe_lora", "fast_lora", "fast_moe_lora", "fast_moe_ranking", "fast_moe_routing", "gguf", "gguf_file", "gguf_liger_loss", "torch_ggml_ops"]

@@ -24,9 +24,13 @@ import torch
 from . import _lib
 from .fast_lora import _NATIVE_MMQ_QUANT_TYPES, supports_native_mmq
 from .fast_moe_routing import ExpertRoutingPlan, finalize_expert_routing, prepare_expert_routing
-from .gguf import GGUFQuantizedTensor, row_bytes
+from .gguf import GGUFQuantizedTensor, dequantize_gguf_tensor, row_bytes
+from .grouped_mm import aiter_grouped_mm, gmm, lora_grouped_linear
 
 EXPERTS_IMPLEMENTATION = "qwen3_5_moe_gguf_mmq_lora"
+# the reference's own structure under the reference's own name (fast_moe_lora.py:38): base projections and LoRA deltas as
+# separate grouped products, and expert weights that have no packed kernel served by decode + gmm
+SEPARATED_EXPERTS_IMPLEMENTATION = "qwen3_5_moe_gguf_mmq_aiter_lora"
 
 # name -> forward(experts, hidden_states, top_k_index, top_k_weights, lora_weights): the registry packed expert modules look
 # their forward up in (stand-in for the fork's ``ALL_GGUF_EXPERTS_FUNCTIONS``, which fast_moe_lora.py:797-799 fills)
@@ -402,12 +406,16 @@ class GGUFExperts(torch.nn.Module):
     has_bias = False
     has_gate = True
 
-    def __init__(self, gate_proj: GGUFQuantizedTensor, up_proj: GGUFQuantizedTensor, down_proj: GGUFQuantizedTensor,
-                 compute_dtype: torch.dtype = torch.bfloat16, swiglu_limit: float | None = None):
+    def __init__(self, gate_proj: GGUFQuantizedTensor | torch.Tensor, up_proj: GGUFQuantizedTensor | torch.Tensor,
+                 down_proj: GGUFQuantizedTensor | torch.Tensor, compute_dtype: torch.dtype = torch.bfloat16, swiglu_limit: float | None = None):
         super().__init__()
         self.swiglu_limit = swiglu_limit  # DeepSeek's config.swiglu_limit; None: plain silu(gate) * up
-        e, i, h = gate_proj.logical_shape
-        if tuple(up_proj.logical_shape) != (e, i, h) or tuple(down_proj.logical_shape) != (e, h, i):
+
+        def logical(w):  # plain floating-point planes are taken by the separated implementation only
+            return tuple(w.logical_shape) if isinstance(w, GGUFQuantizedTensor) else tuple(w.shape)
+
+        e, i, h = logical(gate_proj)
+        if logical(up_proj) != (e, i, h) or logical(down_proj) != (e, h, i):
             raise ValueError("expert projections must be gate/up [E,I,H] and down [E,H,I]")
         self.gate_proj, self.up_proj, self.down_proj = gate_proj, up_proj, down_proj
         self.num_experts, self.hidden_dim, self.intermediate_dim = e, h, i
@@ -444,6 +452,8 @@ def qwen3_5_moe_gguf_mmq_lora_forward(self: GGUFExperts, hidden_states: torch.Te
     for w in (self.gate_proj, self.up_proj, self.down_proj):
         if w.requires_grad:
             raise RuntimeError("Fast GGUF expert execution requires frozen packed base weights.")
+        if not isinstance(w, GGUFQuantizedTensor):
+            raise RuntimeError(f"{EXPERTS_IMPLEMENTATION} takes packed expert weights; {SEPARATED_EXPERTS_IMPLEMENTATION} also takes floating-point ones.")
         if not supports_native_mmq(w):
             raise RuntimeError(f"GGML type id {w.quant_type} has no native grouped MMQ kernel.")
     if self.compute_dtype != torch.bfloat16:
@@ -489,6 +499,109 @@ def qwen3_5_moe_gguf_mmq_lora_forward(self: GGUFExperts, hidden_states: torch.Te
 
 
 ALL_GGUF_EXPERTS_FUNCTIONS[EXPERTS_IMPLEMENTATION] = qwen3_5_moe_gguf_mmq_lora_forward
+
+
+# ------------------------------------------------------------------------------------------------
+def _dequantize_selected_experts(weight: Any, expert_indices: torch.Tensor, dtype: torch.dtype, device: torch.device) -> torch.Tensor:
+    """Dense [G, N, K] planes of the selected experts (fast_moe_lora.py:154-172): packed planes are decoded, floating-point
+    ones copied; anything else is an error."""
+    if isinstance(weight, GGUFQuantizedTensor):
+        payload = weight.as_subclass(torch.Tensor)
+        selected = payload.index_select(0, expert_indices.to(payload.device))
+        return dequantize_gguf_tensor(selected, weight.quant_type, dtype=dtype, device=device)
+    if not weight.is_floating_point():
+        raise RuntimeError("GGUF expert weights must be packed or floating point before grouped execution.")
+    return weight.index_select(0, expert_indices.to(weight.device)).to(device=device, dtype=dtype)
+
+
+class _UnpackedExpertProjection(torch.autograd.Function):
+    """The branch of the reference's ``_AiterGGUFExpertProjection`` for weights without a packed kernel
+    (fast_moe_lora.py:230-247, 264-287): decode or copy the selected experts' planes, then ``gmm``; the input's gradient is a
+    ``gmm`` against the same planes, which are decoded again instead of being kept.  The weights get no gradient."""
+
+    @staticmethod
+    def forward(ctx, hidden_states, weight, expert_indices, group_sizes, compute_dtype):
+        if weight.requires_grad:
+            raise RuntimeError("Fast GGUF expert execution requires frozen packed base weights.")
+        if compute_dtype != torch.bfloat16:
+            raise RuntimeError("Grouped expert execution requires BF16 compute dtype.")
+        ctx.input_dtype = hidden_states.dtype
+        ctx.compute_dtype = compute_dtype
+        hidden_states = hidden_states.to(compute_dtype).contiguous()
+        dense = _dequantize_selected_experts(weight, expert_indices, compute_dtype, hidden_states.device)
+        ctx.weight = weight
+        ctx.save_for_backward(expert_indices, group_sizes)
+        return gmm(hidden_states, dense.transpose(1, 2), group_sizes, preferred_element_type=compute_dtype)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        grad_hidden = None
+        if ctx.needs_input_grad[0]:
+            expert_indices, group_sizes = ctx.saved_tensors
+            dense = _dequantize_selected_experts(ctx.weight, expert_indices, ctx.compute_dtype, grad_output.device)
+            grad_hidden = gmm(grad_output.contiguous(), dense, group_sizes, preferred_element_type=ctx.compute_dtype).to(ctx.input_dtype)
+        return grad_hidden, None, None, None, None
+
+
+def _base_grouped_linear(hidden_states, weight, expert_indices, expert_offsets, group_sizes, compute_dtype):
+    """One frozen expert projection (fast_moe_lora.py:175-288): the packed kernel where the block format has one."""
+    if isinstance(weight, GGUFQuantizedTensor) and supports_native_mmq(weight):
+        if compute_dtype != torch.bfloat16:
+            raise RuntimeError("Grouped GGUF MMQ requires BF16 compute dtype.")
+        return grouped_mmq(hidden_states, weight, expert_indices, expert_offsets, int(weight.quant_type), int(weight.logical_shape[-2]))
+    return _UnpackedExpertProjection.apply(hidden_states, weight, expert_indices, group_sizes, compute_dtype)
+
+
+def _base_grouped_pair(hidden_states, first_weight, second_weight, expert_indices, expert_offsets, group_sizes, compute_dtype):
+    """The gate/up pair (fast_moe_lora.py:291-395): one paired packed launch where both halves share a native block format,
+    two single projections otherwise."""
+    packed = [isinstance(w, GGUFQuantizedTensor) and supports_native_mmq(w) for w in (first_weight, second_weight)]
+    if all(packed) and first_weight.quant_type == second_weight.quant_type:
+        if tuple(first_weight.logical_shape) != tuple(second_weight.logical_shape):
+            raise RuntimeError("Paired grouped GGUF MMQ requires matching logical shapes.")
+        if compute_dtype != torch.bfloat16:
+            raise RuntimeError("Grouped GGUF MMQ requires BF16 compute dtype.")
+        return grouped_mmq_pair(hidden_states, first_weight, second_weight, expert_indices, expert_offsets, int(first_weight.quant_type),
+                                int(first_weight.logical_shape[-2]))
+    return (_base_grouped_linear(hidden_states, first_weight, expert_indices, expert_offsets, group_sizes, compute_dtype),
+            _base_grouped_linear(hidden_states, second_weight, expert_indices, expert_offsets, group_sizes, compute_dtype))
+
+
+def qwen3_5_moe_gguf_mmq_aiter_lora_forward(self: GGUFExperts, hidden_states: torch.Tensor, top_k_index: torch.Tensor,
+                                            top_k_weights: torch.Tensor, lora_weights: _ExpertLoraWeights | None = None) -> torch.Tensor:
+    """The expert FFN in the reference's own order (fast_moe_lora.py:685-770): base projections, then each LoRA delta as two
+    grouped products (``lora_grouped_linear``) added with ``alpha=scaling``; every intermediate is a bf16 tensor of its own.
+    Slower than ``qwen3_5_moe_gguf_mmq_lora_forward`` (which folds the deltas into the packed-weight launches), but it also
+    takes expert weights that are plain floating-point tensors."""
+    if not isinstance(self, GGUFExperts):
+        raise TypeError(f"{SEPARATED_EXPERTS_IMPLEMENTATION} requires GGUFExperts, got {type(self).__name__}.")
+    if self.projection_layout != "split_gate_up" or self.has_bias or not self.has_gate:
+        raise RuntimeError("The GGUF LoRA path requires split, bias-free gate/up expert projections.")
+    compute_hidden_states = self._prepare_expert_hidden_states(hidden_states)
+    routing_plan = prepare_expert_routing(compute_hidden_states, top_k_index, top_k_weights, self.num_experts)
+    execution_plan = self._prepare_expert_execution(routing_plan, "grouped_mm")
+    if execution_plan.offsets is None:
+        raise RuntimeError("GGUF LoRA requires grouped expert offsets.")
+    selected = routing_plan.selected_hidden_states
+    expert_indices = execution_plan.expert_indices.to(device=selected.device, dtype=torch.long).contiguous()
+    expert_offsets = execution_plan.offsets.to(device=selected.device, dtype=torch.int32).contiguous()
+    group_sizes = _group_sizes_from_offsets(expert_offsets)
+
+    gate, up = _base_grouped_pair(selected, self.gate_proj, self.up_proj, expert_indices, expert_offsets, group_sizes, self.compute_dtype)
+    lw = lora_weights
+    if lw is not None:
+        lora_group_sizes = _complete_group_sizes(group_sizes, expert_indices, self.num_experts)
+        gate_delta, up_delta = lora_grouped_linear(selected, lw.gate_up_a, lw.gate_up_b, lora_group_sizes).chunk(2, dim=-1)
+        gate = torch.add(gate, gate_delta, alpha=lw.scaling)
+        up = torch.add(up, up_delta, alpha=lw.scaling)
+    intermediate = self._apply_split_gate(gate.contiguous(), up.contiguous())
+    output = _base_grouped_linear(intermediate, self.down_proj, expert_indices, expert_offsets, group_sizes, self.compute_dtype)
+    if lw is not None:
+        output = torch.add(output, lora_grouped_linear(intermediate, lw.down_a, lw.down_b, lora_group_sizes), alpha=lw.scaling)
+    return finalize_expert_routing(output, hidden_states, routing_plan, execution_plan.output_mask).reshape(hidden_states.shape)
+
+
+ALL_GGUF_EXPERTS_FUNCTIONS[SEPARATED_EXPERTS_IMPLEMENTATION] = qwen3_5_moe_gguf_mmq_aiter_lora_forward
 
 
 def set_gguf_experts_implementation(model: torch.nn.Module, name: str, experts_type: type = GGUFExperts) -> list[str]:
