@@ -33,6 +33,7 @@ CASES = [  # m, k, n, group sizes
     (100, 128, 128, [30, 20]),                       # 50 rows no group covers: zero rows
     (64, 96, 80, [50, 50]),                          # sizes past the last row are clipped
     (1, 8, 8, [1]),
+    (1500, 24, 40, [3, 0] * 500),                    # a thousand groups: the plan's threads walk several groups each
 ]
 
 
