@@ -172,3 +172,36 @@ def test_grouped_mm_stands_in_for_the_aiter_import_and_checks_its_operands(pkg):
         gm.aiter_grouped_mm(torch.zeros(6, 4, dtype=torch.bfloat16), torch.zeros(2, 4, 5, dtype=torch.bfloat16), sizes)
     with pytest.raises(RuntimeError, match="ROCm device"):
         gm.aiter_grouped_mm(torch.zeros(6, 4, dtype=torch.bfloat16), torch.zeros(3, 4, 5, dtype=torch.bfloat16), sizes)
+
+
+@pytest.mark.gpu
+def test_operator_entries_compose_with_torch_compile(pkg, dev):
+    """``torch.compile`` composition (docs/plan_qwen3.5.md:125-150): a function over the dispatcher entries is traced through
+    their FakeTensor kernels and registered autograd (the ``aot_eager`` backend: no code generation involved) and gives the
+    eager bits, forward and backward."""
+    pkg.torch_ggml_ops.install()
+    ops = torch.ops.torch_ggml_ops
+    gen = torch.Generator().manual_seed(9)
+    n, k, e = 128, 256, 3
+    p = torch.from_numpy(make_payload(21, gb.Q4_K, n, k)).to(dev)
+    sizes = [20, 0, 45]
+    ids = torch.arange(e, dtype=torch.int64, device=dev)
+    ends = torch.tensor(np.cumsum(sizes), dtype=torch.int32, device=dev)
+    p1 = torch.from_numpy(make_payload(22, gb.Q4_K, e * n, k)).reshape(e, n, -1).to(dev)
+    p2 = torch.from_numpy(make_payload(23, gb.Q4_K, e * n, k)).reshape(e, n, -1).to(dev)
+
+    def fn(x, xs):
+        y = ops.mmq(x, p, gb.Q4_K, n)
+        a, b = ops.grouped_mmq_pair(xs, p1, p2, ids, ends, gb.Q4_K, n)
+        return y.float().square().mean() + (a.float() * torch.sigmoid(b.float())).mean()
+
+    compiled = torch.compile(fn, backend="aot_eager", fullgraph=True)
+    x0, xs0 = bf16_randn(gen, 2, 9, k).to(dev), bf16_randn(gen, sum(sizes), k).to(dev)
+    results = []
+    for f in (fn, compiled):
+        x, xs = x0.clone().requires_grad_(True), xs0.clone().requires_grad_(True)
+        out = f(x, xs)
+        out.backward()
+        results.append((out.detach(), x.grad, xs.grad))
+    for got, want in zip(results[1], results[0]):
+        assert torch.equal(got, want)
