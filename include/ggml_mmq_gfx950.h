@@ -205,20 +205,20 @@ int ggq_swiglu_backward_routed(const void* gate, const void* up, const void* dh_
                                void* stream);
 
 /* AITER's grouped products as the reference calls them (gmm / ptgmm, fast_moe_lora.py:22, 42-87; _AiterGroupedMM :90-151),
- * for bf16 matrices with no packed weight: the LoRA factors of an expert layer (:674-682) and expert weights without a
+ * for bf16 or fp16 matrices (is_f16; both operands and the output share the type) with no packed weight: the LoRA factors of an expert layer (:674-682) and expert weights without a
  * packed kernel (:230-247).  group_sizes [experts] int32 on the device: consecutive row groups of lhs, group e owning
  * rhs[e].  Sizes are clipped to m, negative ones count as zero; rows no group covers give zero output rows.
- *   ggq_gmm:   out [m, n] bf16: out[i] = lhs[i] . rhs[e], lhs [m, k] row-major, rhs[e] stored [n][k] (rhs_k_contiguous = 1:
+ *   ggq_gmm:   out [m, n]: out[i] = lhs[i] . rhs[e], lhs [m, k] row-major, rhs[e] stored [n][k] (rhs_k_contiguous = 1:
  *              the reference's `factor.transpose(1, 2)` of an [E, n, k] factor) or [k][n] (0: its grad-input call, :53-68).
- *   ggq_ptgmm: out [experts, k, n] bf16: out[e] = lhs[rows of e]^T . grad_out[rows of e] (:71-87); experts without rows
+ *   ggq_ptgmm: out [experts, k, n]: out[e] = lhs[rows of e]^T . grad_out[rows of e] (:71-87); experts without rows
  *              get zeros, every plane is written.
- * fp32 accumulation, one rounding to bf16.  Any k and n (16-byte loads when k resp. n is a multiple of 8 and the base
+ * fp32 accumulation, one rounding to the 16-bit type.  Any k and n (16-byte loads when k resp. n is a multiple of 8 and the base
  * addresses are 16-byte aligned).  ws: ggq_gmm_workspace_bytes(experts) bytes of device memory, 4-byte aligned. */
 int64_t ggq_gmm_workspace_bytes(int64_t experts);
 int ggq_gmm(const void* lhs, const void* rhs, const int32_t* group_sizes, void* out, int64_t m, int64_t k, int64_t n, int64_t experts,
-            int rhs_k_contiguous, void* ws, int64_t ws_bytes, void* stream);
+            int rhs_k_contiguous, int is_f16, void* ws, int64_t ws_bytes, void* stream);
 int ggq_ptgmm(const void* lhs, const void* grad_out, const int32_t* group_sizes, void* out, int64_t m, int64_t k, int64_t n, int64_t experts,
-              void* ws, int64_t ws_bytes, void* stream);
+              int is_f16, void* ws, int64_t ws_bytes, void* stream);
 
 /* GGUFExperts._apply_split_gate (fork; called at fast_moe_lora.py:747): h = silu(gate) * up, and its
  * autograd.  elems = rows * intermediate. */

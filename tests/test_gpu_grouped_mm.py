@@ -70,6 +70,35 @@ def test_gmm_and_ptgmm_against_the_group_loop(pkg, dev, m, k, n, sizes, k_contig
         r0 = min(m, r0 + size)
 
 
+def test_half_precision_operands(pkg, dev):
+    """The reference's wrapper admits fp16 as well (fast_moe_lora.py:116-119): same relations, fp16 roundings."""
+    gm = pkg.grouped_mm
+    gen = torch.Generator().manual_seed(17)
+    m, k, n, sizes = 300, 72, 40, [130, 0, 1, 169]
+    lhs = torch.randn(m, k, generator=gen).half()
+    planes = (0.5 * torch.randn(len(sizes), k, n, generator=gen)).half()
+    dy = torch.randn(m, n, generator=gen).half()
+    want = ref.grouped_mm(lhs, planes, sizes, dy)
+    gs = torch.tensor(sizes, dtype=torch.int32, device=dev)
+    tol = lambda w, mag: 2.0 ** -11 * w.abs() + 2.0 ** -18 * mag + 1e-30  # half an fp16 ulp + the fp32 sum's noise
+
+    def close(got, w, mag, what):
+        assert got.dtype == torch.float16
+        bad = (got.double().cpu() - w).abs() > tol(w, mag)
+        assert not bad.any(), f"{what}: {int(bad.sum())} of {bad.numel()} off"
+
+    mag = ref.grouped_mm(lhs.abs(), planes.abs(), sizes, dy.abs())
+    for rhs_d in (planes.to(dev), planes.transpose(1, 2).contiguous().to(dev).transpose(1, 2)):
+        close(gm.gmm(lhs.to(dev), rhs_d, gs), want["out"], mag["out"], "gmm fp16")
+    close(gm.gmm(dy.to(dev), planes.to(dev).transpose(1, 2), gs), want["dlhs"], ref.grouped_mm(dy.abs(), planes.abs().transpose(1, 2), sizes)["out"], "gmm fp16 transposed planes")
+    close(gm.ptgmm(lhs.to(dev).T, dy.to(dev), gs), want["drhs"], mag["drhs"], "ptgmm fp16")
+    lhs_d, planes_d = lhs.to(dev).requires_grad_(True), planes.to(dev).requires_grad_(True)
+    out = gm.aiter_grouped_mm(lhs_d, planes_d, gs)
+    out.backward(dy.to(dev))
+    close(lhs_d.grad, want["dlhs"], ref.grouped_mm(dy.abs(), planes.abs().transpose(1, 2), sizes)["out"], "autograd d lhs fp16")
+    close(planes_d.grad, want["drhs"], mag["drhs"], "autograd d planes fp16")
+
+
 def test_unaligned_bases_take_the_element_path(pkg, dev):
     gm = pkg.grouped_mm
     gen = torch.Generator().manual_seed(5)
@@ -137,14 +166,16 @@ def test_grouped_mm_rejects_layout_repairs(pkg, dev):
         torch.autograd.grad(output, (valid_lhs, valid_factor), strided)
     with pytest.raises(ValueError, match="contiguous int32"):
         gm.aiter_grouped_mm(valid_lhs, valid_factor.transpose(1, 2), sizes.long())
-    with pytest.raises(TypeError, match="BF16"):
+    with pytest.raises(TypeError, match="FP16/BF16"):
         gm.aiter_grouped_mm(valid_lhs.float(), valid_factor.float().transpose(1, 2), sizes)
+    with pytest.raises(TypeError, match="FP16/BF16"):
+        gm.aiter_grouped_mm(valid_lhs, valid_factor.half().transpose(1, 2), sizes)
     with pytest.raises(ValueError, match="K mismatch"):
         gm.aiter_grouped_mm(valid_lhs[:, :8].contiguous(), valid_factor.transpose(1, 2), sizes)
     with pytest.raises(ValueError, match="dense"):
         gm.gmm(valid_lhs, torch.randn(3, 16, 8, device=dev, dtype=torch.bfloat16)[:, :, ::2], sizes)
     lib = pkg._lib.load()
-    assert lib.ggq_gmm(valid_lhs.data_ptr(), factor.data_ptr(), sizes.data_ptr(), output.data_ptr(), 6, 16, 4, 3, 1, sizes.data_ptr(), 4, None) == -6
+    assert lib.ggq_gmm(valid_lhs.data_ptr(), factor.data_ptr(), sizes.data_ptr(), output.data_ptr(), 6, 16, 4, 3, 1, 0, sizes.data_ptr(), 4, None) == -6
     assert b"workspace" in lib.ggq_last_error()
 
 

@@ -56,8 +56,8 @@ SIGNATURES: dict[str, tuple] = {
     "ggq_grouped_lora_mmq_backward_routed_output": (_I, [_P, _L, _P, _I, _P, _I, _P, _P, _P, _L, _L, _I, _L, _L, _L, _P, _P, _P, _P, _I, _F, _P, _P, _P,
                                                          _P, _L, _P]),
     "ggq_gmm_workspace_bytes": (_L, [_L]),
-    "ggq_gmm": (_I, [_P, _P, _P, _P, _L, _L, _L, _L, _I, _P, _L, _P]),
-    "ggq_ptgmm": (_I, [_P, _P, _P, _P, _L, _L, _L, _L, _P, _L, _P]),
+    "ggq_gmm": (_I, [_P, _P, _P, _P, _L, _L, _L, _L, _I, _I, _P, _L, _P]),
+    "ggq_ptgmm": (_I, [_P, _P, _P, _P, _L, _L, _L, _L, _I, _P, _L, _P]),
     "ggq_lmhead_ce_workspace_bytes": (_L, [_L, _L, _L, _L]),
     "ggq_lmhead_cross_entropy": (_I, [_I, _P, _P, _P, _L, _L, _L, _L, _L, _I, _P, _P, _P, _P, _P, _P, _P, _L, _P]),
 }

@@ -531,13 +531,13 @@ int ggq_swiglu_clamped_backward(const void* gate, const void* up, const void* dh
 int64_t ggq_gmm_workspace_bytes(int64_t experts) { return grouped_gemm_workspace_bytes(experts); }
 
 int ggq_gmm(const void* lhs, const void* rhs, const int32_t* group_sizes, void* out, int64_t m, int64_t k, int64_t n, int64_t experts, int rhs_k_contiguous,
-            void* ws, int64_t ws_bytes, void* stream) {
-    return grouped_gemm(lhs, rhs, group_sizes, out, m, k, n, experts, rhs_k_contiguous, ws, ws_bytes, as_stream(stream));
+            int is_f16, void* ws, int64_t ws_bytes, void* stream) {
+    return grouped_gemm(lhs, rhs, group_sizes, out, m, k, n, experts, rhs_k_contiguous, is_f16, ws, ws_bytes, as_stream(stream));
 }
 
-int ggq_ptgmm(const void* lhs, const void* grad_out, const int32_t* group_sizes, void* out, int64_t m, int64_t k, int64_t n, int64_t experts, void* ws,
-              int64_t ws_bytes, void* stream) {
-    return grouped_gemm_transposed(lhs, grad_out, group_sizes, out, m, k, n, experts, ws, ws_bytes, as_stream(stream));
+int ggq_ptgmm(const void* lhs, const void* grad_out, const int32_t* group_sizes, void* out, int64_t m, int64_t k, int64_t n, int64_t experts, int is_f16,
+              void* ws, int64_t ws_bytes, void* stream) {
+    return grouped_gemm_transposed(lhs, grad_out, group_sizes, out, m, k, n, experts, is_f16, ws, ws_bytes, as_stream(stream));
 }
 
 int ggq_router_topk(const void* logits, int logits_are_bf16, int64_t tokens, int num_experts, int top_k, const float* correction_bias,

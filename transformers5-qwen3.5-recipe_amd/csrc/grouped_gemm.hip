@@ -1,4 +1,4 @@
-// Grouped bf16 matrix products over row groups, with no packed weight involved: what the reference takes from AITER's
+// Grouped bf16 (or fp16) matrix products over row groups, with no packed weight involved: what the reference takes from AITER's
 // gmm / ptgmm (fast_moe_lora.py:22, 42-87) for its LoRA factors and for expert weights that have no packed kernel.
 //
 //   gmm:    out[i, :]  = lhs[i, :] . rhs[e]            for the rows i of group e   (rhs[e] is [k, n], either index contiguous)
@@ -21,6 +21,18 @@ namespace ggq {
 namespace {
 
 typedef short v4i16_t __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+
+// the two 16-bit element types of the entry points (the reference's wrapper admits both, fast_moe_lora.py:116-119)
+template <bool F16>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    if (F16) {
+        const f16x2_t v = {(_Float16)lo, (_Float16)hi};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    return pack_bf16(lo, hi);
+}
 typedef __attribute__((address_space(3))) v4i16_t* lds_v4i16_ptr;
 
 constexpr int kT = 128;          // output tile edge
@@ -88,7 +100,7 @@ __device__ __forceinline__ bf16x8_t operand(const bf16_t* tile, int first, int l
 }
 
 // out[i, j] = sum over t in [0, t_len) of R(i, t) * C(j, t) for the tile's rows i < rows.outer_valid and columns j < cols.outer_valid.
-template <bool ROWS_TR, bool COLS_TR>
+template <bool ROWS_TR, bool COLS_TR, bool F16>
 __device__ __forceinline__ void tile_product(const Operand& rows, const Operand& cols, int t_len, bf16_t* out, int64_t ld_out) {
     __shared__ __attribute__((aligned(16))) bf16_t r_t[2][kTileElems];
     __shared__ __attribute__((aligned(16))) bf16_t c_t[2][kTileElems];
@@ -123,7 +135,10 @@ __device__ __forceinline__ void tile_product(const Operand& rows, const Operand&
         for (int ib = 0; ib < 4; ib++) {
             const bf16x8_t r_op = operand<ROWS_TR>(r_t[buf], wi * 64 + ib * 16, li, lq);
 #pragma unroll
-            for (int jb = 0; jb < 4; jb++) acc[ib][jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(c_op[jb], r_op, acc[ib][jb], 0, 0, 0);
+            for (int jb = 0; jb < 4; jb++) {
+                if (F16) acc[ib][jb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, c_op[jb]), __builtin_bit_cast(f16x8_t, r_op), acc[ib][jb], 0, 0, 0);
+                else acc[ib][jb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(c_op[jb], r_op, acc[ib][jb], 0, 0, 0);
+            }
         }
         buf ^= 1;
     }
@@ -138,11 +153,11 @@ __device__ __forceinline__ void tile_product(const Operand& rows, const Operand&
             const int j = wj * 64 + jb * 16 + 4 * lq;
             bf16_t* dst = out + (int64_t)i * ld_out + j;
             if (vec4 && j + 3 < cols.outer_valid) {
-                *(uint2*)dst = make_uint2(pack_bf16(acc[ib][jb][0], acc[ib][jb][1]), pack_bf16(acc[ib][jb][2], acc[ib][jb][3]));
+                *(uint2*)dst = make_uint2(pack2<F16>(acc[ib][jb][0], acc[ib][jb][1]), pack2<F16>(acc[ib][jb][2], acc[ib][jb][3]));
             } else {
 #pragma unroll
                 for (int v = 0; v < 4; v++)
-                    if (j + v < cols.outer_valid) dst[v] = to_bf16(acc[ib][jb][v]);
+                    if (j + v < cols.outer_valid) dst[v] = (bf16_t)(pack2<F16>(acc[ib][jb][v], 0.0f) & 0xFFFFu);
             }
         }
     }
@@ -215,7 +230,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_plan_kernel(const int32_t* g
     }
 }
 
-template <bool RHS_TR>
+template <bool RHS_TR, bool F16>
 __global__ __launch_bounds__(256) void gmm_kernel(GroupedGemmParams p) {
     const int col_tiles = (p.n + kT - 1) / kT;
     const int rt = (int)(blockIdx.x / col_tiles), ct = (int)(blockIdx.x % col_tiles);
@@ -249,9 +264,10 @@ __global__ __launch_bounds__(256) void gmm_kernel(GroupedGemmParams p) {
         cols.ld = p.k;
         cols.vec = (p.k & 7) == 0 && (((uintptr_t)p.rhs & 15) == 0);
     }
-    tile_product<false, RHS_TR>(rows, cols, no_expert ? 0 : p.k, p.out + (int64_t)r0 * p.n + c0, p.n);
+    tile_product<false, RHS_TR, F16>(rows, cols, no_expert ? 0 : p.k, p.out + (int64_t)r0 * p.n + c0, p.n);
 }
 
+template <bool F16>
 __global__ __launch_bounds__(256) void ptgmm_kernel(GroupedGemmParams p) {
     const int col_tiles = (p.n + kT - 1) / kT, row_tiles = (p.k + kT - 1) / kT;
     const int per_expert = col_tiles * row_tiles;
@@ -267,7 +283,7 @@ __global__ __launch_bounds__(256) void ptgmm_kernel(GroupedGemmParams p) {
     cols.ld = p.n;
     cols.outer_valid = min(kT, p.n - ct * kT);
     cols.vec = (p.n & 7) == 0 && (((uintptr_t)p.rhs & 15) == 0);
-    tile_product<true, true>(rows, cols, row_end - row_begin, p.out + ((int64_t)e * p.k + kt * kT) * p.n + ct * kT, p.n);
+    tile_product<true, true, F16>(rows, cols, row_end - row_begin, p.out + ((int64_t)e * p.k + kt * kT) * p.n + ct * kT, p.n);
 }
 
 int check_common(const char* what, const void* lhs, const void* rhs, const int32_t* group_sizes, const void* out, int64_t m, int64_t k, int64_t n,
@@ -277,7 +293,7 @@ int check_common(const char* what, const void* lhs, const void* rhs, const int32
     if (m > INT32_MAX - 2 * kT || k > INT32_MAX - 2 * kT || n > INT32_MAX - 2 * kT || experts > (1 << 24))
         return set_error(GGQ_ERR_SHAPE, "%s: a size exceeds the 32-bit index range of the kernels", what);
     if (!group_sizes || !ws || (!lhs && m * k > 0) || (!rhs && rhs_elems > 0) || (!out && out_elems > 0)) return set_error(GGQ_ERR_NULL, "%s: null pointer", what);
-    if (((uintptr_t)lhs | (uintptr_t)rhs | (uintptr_t)out) & 1) return set_error(GGQ_ERR_ALIGN, "%s: bf16 matrices must be 2-byte aligned", what);
+    if (((uintptr_t)lhs | (uintptr_t)rhs | (uintptr_t)out) & 1) return set_error(GGQ_ERR_ALIGN, "%s: matrices must be 2-byte aligned", what);
     if (ws_bytes < grouped_gemm_workspace_bytes(experts))
         return set_error(GGQ_ERR_WORKSPACE, "%s: workspace of %lld bytes, %lld needed", what, (long long)ws_bytes, (long long)grouped_gemm_workspace_bytes(experts));
     if (((uintptr_t)ws | (uintptr_t)group_sizes) & 3) return set_error(GGQ_ERR_ALIGN, "%s: group sizes and workspace must be 4-byte aligned", what);
@@ -289,7 +305,7 @@ int check_common(const char* what, const void* lhs, const void* rhs, const int32
 int64_t grouped_gemm_workspace_bytes(int64_t experts) { return experts < 1 ? -1 : (2 * experts + 4) * (int64_t)sizeof(int32_t); }
 
 int grouped_gemm(const void* lhs, const void* rhs, const int32_t* group_sizes, void* out, int64_t m, int64_t k, int64_t n, int64_t experts, int rhs_k_contiguous,
-                 void* ws, int64_t ws_bytes, hipStream_t stream) {
+                 int is_f16, void* ws, int64_t ws_bytes, hipStream_t stream) {
     if (int rc = check_common("gmm", lhs, rhs, group_sizes, out, m, k, n, experts, experts * k * n, m * n, ws, ws_bytes)) return rc;
     if (m == 0 || n == 0) return GGQ_OK;
     GroupedGemmParams p;
@@ -300,13 +316,15 @@ int grouped_gemm(const void* lhs, const void* rhs, const int32_t* group_sizes, v
     const int64_t row_tiles = (m + kT - 1) / kT + experts + 1, col_tiles = (n + kT - 1) / kT;
     if (row_tiles * col_tiles > INT32_MAX) return set_error(GGQ_ERR_SHAPE, "gmm: %lld tiles exceed the grid limit", (long long)(row_tiles * col_tiles));
     const dim3 grid((unsigned)(row_tiles * col_tiles));
-    if (rhs_k_contiguous) hipLaunchKernelGGL(gmm_kernel<false>, grid, dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL(gmm_kernel<true>, grid, dim3(256), 0, stream, p);
+    if (rhs_k_contiguous && is_f16) hipLaunchKernelGGL((gmm_kernel<false, true>), grid, dim3(256), 0, stream, p);
+    else if (rhs_k_contiguous) hipLaunchKernelGGL((gmm_kernel<false, false>), grid, dim3(256), 0, stream, p);
+    else if (is_f16) hipLaunchKernelGGL((gmm_kernel<true, true>), grid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((gmm_kernel<true, false>), grid, dim3(256), 0, stream, p);
     return check_launch("gmm");
 }
 
 int grouped_gemm_transposed(const void* lhs, const void* grad_out, const int32_t* group_sizes, void* out, int64_t m, int64_t k, int64_t n, int64_t experts,
-                            void* ws, int64_t ws_bytes, hipStream_t stream) {
+                            int is_f16, void* ws, int64_t ws_bytes, hipStream_t stream) {
     if (int rc = check_common("ptgmm", lhs, grad_out, group_sizes, out, m, k, n, experts, m * n, experts * k * n, ws, ws_bytes)) return rc;
     if (k == 0 || n == 0) return GGQ_OK;
     GroupedGemmParams p;
@@ -316,7 +334,8 @@ int grouped_gemm_transposed(const void* lhs, const void* grad_out, const int32_t
     if (int rc = check_launch("grouped_gemm_plan")) return rc;
     const int64_t tiles = experts * ((k + kT - 1) / kT) * ((n + kT - 1) / kT);
     if (tiles > INT32_MAX) return set_error(GGQ_ERR_SHAPE, "ptgmm: %lld tiles exceed the grid limit", (long long)tiles);
-    hipLaunchKernelGGL(ptgmm_kernel, dim3((unsigned)tiles), dim3(256), 0, stream, p);
+    if (is_f16) hipLaunchKernelGGL(ptgmm_kernel<true>, dim3((unsigned)tiles), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(ptgmm_kernel<false>, dim3((unsigned)tiles), dim3(256), 0, stream, p);
     return check_launch("ptgmm");
 }
 

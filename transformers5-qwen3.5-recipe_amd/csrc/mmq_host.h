@@ -173,12 +173,12 @@ int lmhead_ce(int qt, const void* hidden, const void* packed, const int64_t* lab
 
 int dequantize(int qt, const void* payload, int64_t rows, int64_t k, void* out, int out_f32, hipStream_t stream);
 
-// Grouped bf16 products without packed weights (grouped_gemm.hip): out[rows of e] = lhs[rows of e] . rhs[e] with rhs[e] stored
+// Grouped bf16 / fp16 products without packed weights (grouped_gemm.hip): out[rows of e] = lhs[rows of e] . rhs[e] with rhs[e] stored
 // [n][k] (rhs_k_contiguous) or [k][n]; and out[e] = lhs[rows of e]^T . grad_out[rows of e].
 int64_t grouped_gemm_workspace_bytes(int64_t experts);
 int grouped_gemm(const void* lhs, const void* rhs, const int32_t* group_sizes, void* out, int64_t m, int64_t k, int64_t n, int64_t experts, int rhs_k_contiguous,
-                 void* ws, int64_t ws_bytes, hipStream_t stream);
+                 int is_f16, void* ws, int64_t ws_bytes, hipStream_t stream);
 int grouped_gemm_transposed(const void* lhs, const void* grad_out, const int32_t* group_sizes, void* out, int64_t m, int64_t k, int64_t n, int64_t experts,
-                            void* ws, int64_t ws_bytes, hipStream_t stream);
+                            int is_f16, void* ws, int64_t ws_bytes, hipStream_t stream);
 
 }  // namespace ggq

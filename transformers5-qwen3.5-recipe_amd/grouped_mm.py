@@ -7,7 +7,8 @@ They exist for code written against the reference's surface (its ``_lora_grouped
 projection of expert weights that have no packed kernel, :230-247, which ``expert_projection_without_packed_kernel`` in
 ``fast_moe_lora`` restates).  AITER itself is not importable where this package is tested, so ``gmm`` / ``ptgmm`` follow the
 reference's call sites (argument order, the ``lhs.T`` convention of ``ptgmm``, ``preferred_element_type`` / ``config``
-keywords) and its tests (test_fast_moe_lora.py:280-360), not AITER's source.  bf16 only: the reference also admits fp16.
+keywords) and its tests (test_fast_moe_lora.py:280-360), not AITER's source.  bf16 or fp16 (both operands alike), as the
+reference's wrapper admits (fast_moe_lora.py:116-119).
 """
 
 from __future__ import annotations
@@ -19,6 +20,9 @@ import types
 import torch
 
 from . import _lib
+
+
+_DTYPES = (torch.float16, torch.bfloat16)
 
 
 def _require_device(t: torch.Tensor, name: str) -> None:
@@ -45,10 +49,10 @@ def gmm(lhs: torch.Tensor, rhs: torch.Tensor, group_sizes: torch.Tensor, preferr
     strides equal to 1 (a contiguous [E, K, N] tensor or the ``.transpose(1, 2)`` of a contiguous [E, N, K] one), group_sizes
     [E] int32 on the device.  ``config`` (AITER's tile choice, moe_gmm_configs.py) is accepted and ignored."""
     _require_device(lhs, "gmm lhs")
-    if lhs.dtype != torch.bfloat16 or rhs.dtype != torch.bfloat16 or rhs.device != lhs.device:
-        raise TypeError(f"gmm requires matching BF16 inputs on one device, got {lhs.dtype} and {rhs.dtype}.")
-    if preferred_element_type not in (None, torch.bfloat16):
-        raise TypeError(f"gmm writes BF16, got preferred_element_type={preferred_element_type}.")
+    if lhs.dtype not in _DTYPES or rhs.dtype != lhs.dtype or rhs.device != lhs.device:
+        raise TypeError(f"gmm requires matching FP16/BF16 inputs on one device, got {lhs.dtype} and {rhs.dtype}.")
+    if preferred_element_type not in (None, lhs.dtype):
+        raise TypeError(f"gmm writes its inputs' type {lhs.dtype}, got preferred_element_type={preferred_element_type}.")
     if lhs.ndim != 2 or rhs.ndim != 3 or lhs.shape[1] != rhs.shape[1]:
         raise ValueError(f"gmm expects lhs [M,K] and rhs [E,K,N], got {tuple(lhs.shape)} and {tuple(rhs.shape)}.")
     if lhs.stride() != (lhs.shape[1], 1) and lhs.numel() > 0:
@@ -64,11 +68,11 @@ def gmm(lhs: torch.Tensor, rhs: torch.Tensor, group_sizes: torch.Tensor, preferr
         k_contiguous = 1  # [E, N, K] seen through transpose(1, 2)
     else:
         raise ValueError(f"gmm rhs must be a dense [E,K,N] tensor or the transpose(1, 2) of a dense [E,N,K] one, got strides {rhs.stride()}.")
-    out = torch.empty((m, n), dtype=torch.bfloat16, device=lhs.device)
+    out = torch.empty((m, n), dtype=lhs.dtype, device=lhs.device)
     ws = _workspace(lhs.device, experts)
     lib, stream = _lib.load(), _lib.stream_handle(lhs.device)
     _lib.check(lib.ggq_gmm(lhs.data_ptr(), rhs.data_ptr(), group_sizes.data_ptr(), out.data_ptr(), m, k, n, experts, k_contiguous,
-                           ws.data_ptr(), ws.numel(), stream))
+                           int(lhs.dtype == torch.float16), ws.data_ptr(), ws.numel(), stream))
     return out
 
 
@@ -78,10 +82,10 @@ def ptgmm(lhs: torch.Tensor, rhs: torch.Tensor, group_sizes: torch.Tensor, prefe
     reference passes ``lhs.T``, fast_moe_lora.py:76-87), rhs [M, N] row-major.  Returns [E, K, N]; groups without rows get
     zeros."""
     _require_device(rhs, "ptgmm rhs")
-    if lhs.dtype != torch.bfloat16 or rhs.dtype != torch.bfloat16 or lhs.device != rhs.device:
-        raise TypeError(f"ptgmm requires matching BF16 inputs on one device, got {lhs.dtype} and {rhs.dtype}.")
-    if preferred_element_type not in (None, torch.bfloat16):
-        raise TypeError(f"ptgmm writes BF16, got preferred_element_type={preferred_element_type}.")
+    if lhs.dtype not in _DTYPES or rhs.dtype != lhs.dtype or lhs.device != rhs.device:
+        raise TypeError(f"ptgmm requires matching FP16/BF16 inputs on one device, got {lhs.dtype} and {rhs.dtype}.")
+    if preferred_element_type not in (None, lhs.dtype):
+        raise TypeError(f"ptgmm writes its inputs' type {lhs.dtype}, got preferred_element_type={preferred_element_type}.")
     if lhs.ndim != 2 or rhs.ndim != 2 or lhs.shape[1] != rhs.shape[0]:
         raise ValueError(f"ptgmm expects lhs [K,M] and rhs [M,N], got {tuple(lhs.shape)} and {tuple(rhs.shape)}.")
     k, m = lhs.shape
@@ -92,11 +96,11 @@ def ptgmm(lhs: torch.Tensor, rhs: torch.Tensor, group_sizes: torch.Tensor, prefe
         raise ValueError("ptgmm rhs must be row-major.")
     experts = group_sizes.numel()
     _check_group_sizes(group_sizes, experts, rhs.device)
-    out = torch.empty((experts, k, n), dtype=torch.bfloat16, device=rhs.device)
+    out = torch.empty((experts, k, n), dtype=rhs.dtype, device=rhs.device)
     ws = _workspace(rhs.device, experts)
     lib, stream = _lib.load(), _lib.stream_handle(rhs.device)
-    _lib.check(lib.ggq_ptgmm(lhs.data_ptr(), rhs.data_ptr(), group_sizes.data_ptr(), out.data_ptr(), m, k, n, experts, ws.data_ptr(),
-                             ws.numel(), stream))
+    _lib.check(lib.ggq_ptgmm(lhs.data_ptr(), rhs.data_ptr(), group_sizes.data_ptr(), out.data_ptr(), m, k, n, experts,
+                             int(rhs.dtype == torch.float16), ws.data_ptr(), ws.numel(), stream))
     return out
 
 
@@ -112,8 +116,8 @@ class _AiterGroupedMM(torch.autograd.Function):
             raise ValueError(f"Grouped-MM K mismatch: lhs has {lhs.shape[1]}, rhs has {rhs.shape[1]}.")
         if rhs.shape[0] != group_sizes.numel():
             raise ValueError(f"Grouped-MM expert mismatch: rhs has {rhs.shape[0]}, group_sizes has {group_sizes.numel()}.")
-        if lhs.dtype != torch.bfloat16 or rhs.dtype != lhs.dtype:
-            raise TypeError(f"AITER grouped MM requires matching BF16 inputs, got {lhs.dtype} and {rhs.dtype}.")
+        if lhs.dtype not in _DTYPES or rhs.dtype != lhs.dtype:
+            raise TypeError(f"AITER grouped MM requires matching FP16/BF16 inputs, got {lhs.dtype} and {rhs.dtype}.")
         if lhs.stride() != (lhs.shape[1], 1):
             raise ValueError("AITER grouped MM lhs must be row-major.")
         if group_sizes.device != lhs.device:
