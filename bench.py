@@ -254,6 +254,23 @@ def other_workload(name, pkg, lib, dev, args):
                 p.grad = None
             x.grad = weights.grad = None
             layer(x, idx, weights).backward(dy)
+    elif name == "moe_q4k_separated":  # configs[2] through the reference's own order: base launches + separate grouped LoRA products
+        cfg = CFG
+        layer, x, idx, weights, dy = build_workload(pkg, dev, cfg)
+        layer.get_base_layer().experts_implementation = pkg.fast_moe_lora.SEPARATED_EXPERTS_IMPLEMENTATION
+        fl = algorithmic_flops(cfg)
+        flops = fl["total"]
+        launch_flops, launches_per_step = fl["base_total"] / 4, 4
+        workload = ("configs[2] in the reference's order (fast_moe_lora.py:685-770): packed-weight launches without the LoRA term, each LoRA delta as "
+                    "two grouped bf16 products (gmm) added afterwards, factor gradients by ptgmm, gather / activation / combine as separate nodes")
+        metric = "fwd+bwd TFLOP/s, Q4_K grouped-MoE LoRA, separated order"
+        params = list(layer.parameters())
+
+        def step():
+            for p in params:
+                p.grad = None
+            x.grad = weights.grad = None
+            layer(x, idx, weights).backward(dy)
     else:
         sys.exit(f"unknown workload {name!r}")
 
@@ -290,7 +307,7 @@ def other_workload(name, pkg, lib, dev, args):
 
 def main() -> None:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--workload", default="moe_q4k", choices=["moe_q4k", "dense_q4k", "lmhead_q6k", "moe_iq2xxs"],
+    ap.add_argument("--workload", default="moe_q4k", choices=["moe_q4k", "dense_q4k", "lmhead_q6k", "moe_iq2xxs", "moe_q4k_separated"],
                     help="moe_q4k (default) is the headline configuration; the others are timed for reference")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
