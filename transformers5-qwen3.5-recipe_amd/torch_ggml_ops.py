@@ -12,9 +12,10 @@ FakeTensorMode and ``torch.compile``), the four forward entries carry registered
 grad-input entry, and the grad-input entries reject differentiation (higher-order gradients).  The Python functions exported
 here are differentiable in the activations, like the wheel's.
 
-What the reference's files need beyond this namespace stays theirs to provide: ``fast_moe_lora.py`` also imports AITER's
-``gmm`` / ``ptgmm`` and ``peft`` (fast_moe_lora.py:22-24), ``gguf_liger_loss.py`` imports ``liger_kernel`` (:16-25), and all of
-them the transformers ``gguf`` fork.  The package's own modules of the same names replace those files without these imports.
+What the reference's files need beyond this namespace: ``fast_moe_lora.py`` also imports AITER's ``gmm`` / ``ptgmm``
+(fast_moe_lora.py:22), for which ``grouped_mm.install_as_aiter_gmm()`` installs stand-ins on this library, and ``peft`` (:23-24);
+``gguf_liger_loss.py`` imports ``liger_kernel`` (:16-25), and all of them the transformers ``gguf`` fork: those stay theirs to
+provide.  The package's own modules of the same names replace those files without these imports.
 """
 
 from __future__ import annotations
