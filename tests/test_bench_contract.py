@@ -25,5 +25,5 @@ def test_algorithmic_figures_of_the_headline_configuration():
     assert abs(fl["total"] / 1e9 - 430.0) < 0.5                      # GFLOP per step
     assert bench.packed_weight_bytes(bench.CFG) == 256 * (1024 * 2048 + 2048 * 512) * 144 // 256
     ap_help = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--help"], capture_output=True, text=True, timeout=300).stdout
-    for name in ("moe_q4k", "dense_q4k", "lmhead_q6k", "moe_iq2xxs"):
+    for name in ("moe_q4k", "dense_q4k", "lmhead_q6k", "moe_iq2xxs", "moe_q4k_separated"):
         assert name in ap_help
