@@ -99,6 +99,24 @@ def test_half_precision_operands(pkg, dev):
     close(planes_d.grad, want["drhs"], mag["drhs"], "autograd d planes fp16")
 
 
+def test_degenerate_sizes(pkg, dev):
+    """No rows, no contraction, no columns: nothing faults, and what is defined is zero."""
+    gm = pkg.grouped_mm
+    bf = lambda *shape: torch.ones(*shape, dtype=torch.bfloat16, device=dev)
+    gs = torch.tensor([0, 0, 0], dtype=torch.int32, device=dev)
+    assert gm.gmm(bf(0, 8), bf(3, 8, 5), gs).shape == (0, 5)
+    assert gm.gmm(bf(4, 8), bf(3, 8, 0), torch.tensor([1, 2, 1], dtype=torch.int32, device=dev)).shape == (4, 0)
+    out = gm.gmm(bf(4, 0), bf(3, 0, 5), torch.tensor([1, 2, 1], dtype=torch.int32, device=dev))   # an empty contraction sums to zero
+    assert out.shape == (4, 5) and torch.count_nonzero(out) == 0
+    planes = gm.ptgmm(bf(0, 8).T, bf(0, 5), gs)
+    assert planes.shape == (3, 8, 5) and torch.count_nonzero(planes) == 0
+    out = gm.gmm(bf(4, 8), bf(3, 8, 5), gs)                                                        # rows, but no group owns any
+    assert torch.count_nonzero(out) == 0
+    neg = gm.gmm(bf(4, 8), bf(2, 8, 5), torch.tensor([-3, 4], dtype=torch.int32, device=dev))      # a negative size counts as zero
+    assert torch.equal(neg, (bf(4, 8).float() @ bf(8, 5).float()).to(torch.bfloat16))
+    torch.cuda.synchronize()
+
+
 def test_unaligned_bases_take_the_element_path(pkg, dev):
     gm = pkg.grouped_mm
     gen = torch.Generator().manual_seed(5)
