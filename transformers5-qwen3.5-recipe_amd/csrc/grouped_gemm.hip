@@ -169,7 +169,6 @@ struct GroupedGemmParams {
     bf16_t* out;          // gmm: [m, n]; ptgmm: [E][k][n]
     const int32_t* plan;  // row_offsets[E + 2] (the last group holds the rows past every expert's), then tile_prefix[E + 2]
     int m, k, n, experts;
-    int rhs_k_contiguous;
 };
 
 // Cumulative row offsets of the groups (clipped to m; negative sizes count as zero) and cumulative counts of their
@@ -310,7 +309,7 @@ int grouped_gemm(const void* lhs, const void* rhs, const int32_t* group_sizes, v
     if (m == 0 || n == 0) return GGQ_OK;
     GroupedGemmParams p;
     p.lhs = (const bf16_t*)lhs, p.rhs = (const bf16_t*)rhs, p.out = (bf16_t*)out, p.plan = (const int32_t*)ws;
-    p.m = (int)m, p.k = (int)k, p.n = (int)n, p.experts = (int)experts, p.rhs_k_contiguous = rhs_k_contiguous;
+    p.m = (int)m, p.k = (int)k, p.n = (int)n, p.experts = (int)experts;
     hipLaunchKernelGGL(grouped_gemm_plan_kernel, dim3(1), dim3(256), 0, stream, group_sizes, (int)experts, (int)m, (int32_t*)ws);
     if (int rc = check_launch("grouped_gemm_plan")) return rc;
     const int64_t row_tiles = (m + kT - 1) / kT + experts + 1, col_tiles = (n + kT - 1) / kT;
@@ -329,7 +328,7 @@ int grouped_gemm_transposed(const void* lhs, const void* grad_out, const int32_t
     if (k == 0 || n == 0) return GGQ_OK;
     GroupedGemmParams p;
     p.lhs = (const bf16_t*)lhs, p.rhs = (const bf16_t*)grad_out, p.out = (bf16_t*)out, p.plan = (const int32_t*)ws;
-    p.m = (int)m, p.k = (int)k, p.n = (int)n, p.experts = (int)experts, p.rhs_k_contiguous = 0;
+    p.m = (int)m, p.k = (int)k, p.n = (int)n, p.experts = (int)experts;
     hipLaunchKernelGGL(grouped_gemm_plan_kernel, dim3(1), dim3(256), 0, stream, group_sizes, (int)experts, (int)m, (int32_t*)ws);
     if (int rc = check_launch("grouped_gemm_plan")) return rc;
     const int64_t tiles = experts * ((k + kT - 1) / kT) * ((n + kT - 1) / kT);
