@@ -58,74 +58,68 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int* chunk_hist, int ch
                                                          int* end_offsets, int64_t* active_ids, int* active_end,
                                                          int* num_active, int* expert_base, const int* chunk_bad) {
     __shared__ int scan[256];
-    __shared__ int carry_rows, carry_active;
-    const int tid = threadIdx.x;
-    if (tid == 0) carry_rows = 0, carry_active = 0;
-    __syncthreads();
+    __shared__ int totals[2][2][4];  // [round parity][rows / active][wave]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int carry_rows = 0, carry_active = 0;  // the same values in every thread
+    int flip = 0;
     for (int e0 = 0; e0 < num_experts; e0 += 256) {
         const int e = e0 + tid;
         int total = 0;
         if (e < num_experts) {
-            // sixteen chunk counts are loaded together (one dependent load per chunk would cost a memory
+            // sixty-four chunk counts are loaded together (one dependent load per chunk would cost a memory
             // round trip each); every count is replaced by the chunk's base inside the expert
-            for (int c0 = 0; c0 < chunks; c0 += 16) {
-                int v[16];
+            for (int c0 = 0; c0 < chunks; c0 += 64) {
+                int v[64];
 #pragma unroll
-                for (int i = 0; i < 16; i++) v[i] = c0 + i < chunks ? chunk_hist[(int64_t)(c0 + i) * num_experts + e] : 0;
+                for (int i = 0; i < 64; i++) v[i] = c0 + i < chunks ? chunk_hist[(int64_t)(c0 + i) * num_experts + e] : 0;
 #pragma unroll
-                for (int i = 0; i < 16; i++) {
+                for (int i = 0; i < 64; i++) {
                     if (c0 + i < chunks) chunk_hist[(int64_t)(c0 + i) * num_experts + e] = total;
                     total += v[i];
                 }
             }
             counts[e] = total;
         }
-        // prefix over experts: rows
-        scan[tid] = total;
-        __syncthreads();
-        for (int off = 1; off < 256; off <<= 1) {
-            int v = tid >= off ? scan[tid - off] : 0;
-            __syncthreads();
-            scan[tid] += v;
-            __syncthreads();
-        }
-        const int end = carry_rows + scan[tid];
-        const int chunk_rows = scan[255];
-        __syncthreads();
-        // prefix over experts: active flags
+        // prefix sums over the 256 experts of the round, rows and active flags together: a shuffle scan inside each
+        // wave, the wave totals through LDS (one barrier; the next round writes the other half of `totals`)
         const int active = total > 0 ? 1 : 0;
-        scan[tid] = active;
+        int rows_incl = total, act_incl = active;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int ur = __shfl_up(rows_incl, off, 64), ua = __shfl_up(act_incl, off, 64);
+            if (lane >= off) rows_incl += ur, act_incl += ua;
+        }
+        if (lane == 63) totals[flip][0][wave] = rows_incl, totals[flip][1][wave] = act_incl;
         __syncthreads();
-        for (int off = 1; off < 256; off <<= 1) {
-            int v = tid >= off ? scan[tid - off] : 0;
-            __syncthreads();
-            scan[tid] += v;
-            __syncthreads();
+        int rows_before = 0, act_before = 0, round_rows = 0, round_active = 0;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const int tr = totals[flip][0][w], ta = totals[flip][1][w];
+            if (w < wave) rows_before += tr, act_before += ta;
+            round_rows += tr, round_active += ta;
         }
         if (e < num_experts) {
+            const int end = carry_rows + rows_before + rows_incl;
             end_offsets[e] = end;
             expert_base[e] = end - total;
             if (active) {
-                const int slot = carry_active + scan[tid] - 1;
+                const int slot = carry_active + act_before + act_incl - 1;
                 active_ids[slot] = e;
                 active_end[slot] = end;
             }
         }
-        const int chunk_active = scan[255];
-        __syncthreads();
-        if (tid == 0) carry_rows += chunk_rows, carry_active += chunk_active;
-        __syncthreads();
+        carry_rows += round_rows, carry_active += round_active;
+        flip ^= 1;
     }
     // status word pair: number of active experts, and whether any id was outside [0, num_experts)
     // (such ids are clamped so that no access leaves the buffers; the caller decides what to do).
     int bad = 0;
     for (int c = tid; c < chunks; c += 256) bad |= chunk_bad[c];
-    scan[tid] = bad;
+    if (lane == 0) scan[wave] = __any(bad) ? 1 : 0;
     __syncthreads();
     if (tid == 0) {
-        for (int j = 1; j < 256; j++) bad |= scan[j];
         num_active[0] = carry_active;
-        num_active[1] = bad;
+        num_active[1] = scan[0] | scan[1] | scan[2] | scan[3];
     }
     // unused tail of the compact lists: repeat the total so that "offsets" stay monotone
     for (int s = carry_active + tid; s < num_experts; s += 256) {
