@@ -101,7 +101,7 @@ int ggq_lora_mmq_backward(const void* dy, const void* packed, int qt, int64_t m,
 int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void* packed2, const int64_t* expert_ids,
                                  const int32_t* end_offsets, int64_t groups, int64_t experts, int qt, int64_t rows, int64_t n,
                                  int64_t k, const void* lora_a, const void* lora_b, int r, float scale, void* xa_out, void* y1,
-                                 void* y2, void* ws, int64_t ws_bytes, void* stream);
+                                 void* y2, const void* group_tables, void* ws, int64_t ws_bytes, void* stream);
 
 /* torch.ops.torch_ggml_ops.grouped_mmq_grad_input / grouped_mmq_pair_grad_input
  * (fast_moe_lora.py:255-262, 364-375: both cotangents of a pair land in one fp32 accumulator and are
@@ -111,8 +111,20 @@ int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void*
 int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* packed1, const void* packed2,
                                   const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts, int qt,
                                   int64_t rows, int64_t n, int64_t k, const void* x, const void* xa, const void* lora_a,
-                                  const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b, void* ws,
-                                  int64_t ws_bytes, void* stream);
+                                  const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b,
+                                  const void* group_tables, void* ws, int64_t ws_bytes, void* stream);
+
+/* Row-tile tables of one grouping, built once for the launches that share it (no counterpart in the reference: its ops take
+ * expert ids and offsets only, docs/plan_qwen3.5.md:32).  Every grouped call turns (expert_ids, end_offsets) into tables of
+ * row tiles on the device before its kernels run; the four packed-weight calls of an expert layer's step see the same
+ * grouping, so a caller may build the tables once (ggq_group_tables_build, into ggq_group_tables_bytes(rows, groups,
+ * experts) bytes of device memory, 16-byte aligned) and pass them as `group_tables` to the grouped calls made with the same
+ * expert_ids / end_offsets / groups / experts / rows while the offsets are unchanged.  group_tables = NULL: the call builds
+ * its own, as before.  The tables serve the Q4_K decoding-wave kernels; a call that runs another kernel shape ignores them
+ * and builds its own.  Results are bit-identical either way. */
+int64_t ggq_group_tables_bytes(int64_t rows, int64_t groups, int64_t experts);
+int ggq_group_tables_build(const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts, int64_t rows,
+                           void* tables, int64_t tables_bytes, void* stream);
 
 /* The two calls above over rows that are never materialised: the reference gathers the routed rows first
  * (prepare_expert_routing, fast_moe_routing.py:379-420: _RouteGather.apply(hidden_states, permutation, ...)) and hands the
@@ -125,14 +137,14 @@ int ggq_grouped_forward_reads_indexed_rows(int qt, int64_t rows, int64_t groups,
 int ggq_grouped_lora_mmq_forward_indexed(const void* x, int64_t x_rows, const int64_t* row_index, int index_div, const void* packed1,
                                          const void* packed2, const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups,
                                          int64_t experts, int qt, int64_t rows, int64_t n, int64_t k, const void* lora_a,
-                                         const void* lora_b, int r, float scale, void* xa_out, void* y1, void* y2, void* ws,
-                                         int64_t ws_bytes, void* stream);
+                                         const void* lora_b, int r, float scale, void* xa_out, void* y1, void* y2,
+                                         const void* group_tables, void* ws, int64_t ws_bytes, void* stream);
 int ggq_grouped_lora_mmq_backward_indexed(const void* dy1, const void* dy2, const void* packed1, const void* packed2,
                                           const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts,
                                           int qt, int64_t rows, int64_t n, int64_t k, const void* x, int64_t x_rows,
                                           const int64_t* row_index, int index_div, const void* xa, const void* lora_a,
                                           const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b,
-                                          void* ws, int64_t ws_bytes, void* stream);
+                                          const void* group_tables, void* ws, int64_t ws_bytes, void* stream);
 
 /* torch_ggml_ops.fixed_grouped_mmq (deepseek_v4_lora.py:91-124: DeepSeek's frozen eight-group output projection) and
  * its input gradient: x [rows, groups, k] bf16, packed_groups [groups, n_group, row bytes], y [rows, groups, n_group];
@@ -193,7 +205,8 @@ int ggq_grouped_lora_mmq_backward_routed_output(const void* grad_out, int64_t to
                                                 const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts,
                                                 int qt, int64_t rows, int64_t n, int64_t k, const void* x, const void* xa,
                                                 const void* lora_a, const void* lora_b, int r, float scale, void* dx_unscaled,
-                                                void* d_lora_a, void* d_lora_b, void* ws, int64_t ws_bytes, void* stream);
+                                                void* d_lora_a, void* d_lora_b, const void* group_tables, void* ws, int64_t ws_bytes,
+                                                void* stream);
 
 /* The second half of that backward: dh_unweighted [rows, inter] is dx_unscaled above, the cotangent of
  * h = silu(gate) * up (limit > 0: the clamped form) before the routing weight.  Writes dgate, dup for the cotangent

@@ -416,3 +416,40 @@ def test_fused_gated_down_combine_against_the_separate_nodes(pkg, dev, monkeypat
             assert max_rel(a, b) <= 2e-2, name
         else:
             assert a is None and b is None
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("qt_gu,qt_d", [(gb.Q4_K, gb.Q4_K), (gb.Q4_K, gb.Q6_K), (gb.Q8_0, gb.Q4_K)])
+def test_shared_group_tables_give_the_same_bits(pkg, dev, monkeypatch, fused, qt_gu, qt_d):
+    # the row-tile tables built once per step (ggq_group_tables_build) against tables built by every call: same bits in
+    # every output and gradient, also where only some of the calls run the kernels the tables serve
+    ml, G = pkg.fast_moe_lora, pkg.gguf.GGUFQuantizedTensor
+    monkeypatch.setattr(ml, "FUSE_GATED_DOWN_COMBINE", fused)
+    tokens, hidden, inter, experts, k, r = 300, 512, 256, 16, 8, 16
+    pg, pu, _, x, idx, w, a_gu, b_gu, a_d, b_d, dy = _layer_case(777, tokens, hidden, inter, experts, k, r, qt_gu)
+    pd = _layer_case(778, tokens, hidden, inter, experts, k, r, qt_d)[2]
+    mod = ml.GGUFExperts(G(torch.from_numpy(pg).to(dev), qt_gu, (experts, inter, hidden)), G(torch.from_numpy(pu).to(dev), qt_gu, (experts, inter, hidden)),
+                         G(torch.from_numpy(pd).to(dev), qt_d, (experts, hidden, inter)))
+    layer = ml.FastGGUFMoeLora(mod, r=r, lora_alpha=32)
+    with torch.no_grad():
+        layer.lora_A["default"].weight.copy_(a_gu.to(dev)); layer.lora_B["default"].weight.copy_(b_gu.to(dev))
+        layer.lora_A_down["default"].weight.copy_(a_d.to(dev)); layer.lora_B_down["default"].weight.copy_(b_d.to(dev))
+    results = []
+    for shared in (True, False):
+        monkeypatch.setattr(ml, "SHARE_GROUP_TABLES", shared)
+        for p in layer.parameters():
+            p.grad = None
+        xd, wd = x.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+        out = layer(xd, idx.to(dev), wd)
+        out.backward(dy.to(dev))
+        results.append([out.detach(), xd.grad, wd.grad] + [p.grad.clone() for p in layer.parameters()])
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    lib = pkg._lib.load()
+    ids = torch.arange(experts, dtype=torch.int64, device=dev)
+    ends = torch.full((experts,), 10, dtype=torch.int32, device=dev).cumsum(0).int()
+    need = lib.ggq_group_tables_bytes(160, experts, experts)
+    buf = torch.empty(need + 16, dtype=torch.uint8, device=dev)
+    assert lib.ggq_group_tables_build(ids.data_ptr(), ends.data_ptr(), experts, experts, 160, buf.data_ptr(), need - 1, None) == -6
+    assert lib.ggq_group_tables_build(ids.data_ptr(), ends.data_ptr(), experts, experts, 160, buf.data_ptr() + 8, need, None) == -3
+    assert lib.ggq_group_tables_bytes(-1, experts, experts) == -1

@@ -35,11 +35,13 @@ SIGNATURES: dict[str, tuple] = {
     "ggq_lora_workspace_bytes": (_L, [_L, _L, _L, _L, _L, _I]),
     "ggq_lora_mmq_forward": (_I, [_P, _P, _I, _L, _L, _L, _P, _P, _I, _F, _P, _P, _P, _L, _P]),
     "ggq_lora_mmq_backward": (_I, [_P, _P, _I, _L, _L, _L, _P, _P, _P, _P, _I, _F, _P, _P, _P, _P, _L, _P]),
-    "ggq_grouped_lora_mmq_forward": (_I, [_P, _P, _P, _P, _P, _L, _L, _I, _L, _L, _L, _P, _P, _I, _F, _P, _P, _P, _P, _L, _P]),
-    "ggq_grouped_lora_mmq_backward": (_I, [_P, _P, _P, _P, _P, _P, _L, _L, _I, _L, _L, _L, _P, _P, _P, _P, _I, _F, _P, _P, _P, _P, _L, _P]),
+    "ggq_grouped_lora_mmq_forward": (_I, [_P, _P, _P, _P, _P, _L, _L, _I, _L, _L, _L, _P, _P, _I, _F, _P, _P, _P, _P, _P, _L, _P]),
+    "ggq_grouped_lora_mmq_backward": (_I, [_P, _P, _P, _P, _P, _P, _L, _L, _I, _L, _L, _L, _P, _P, _P, _P, _I, _F, _P, _P, _P, _P, _P, _L, _P]),
+    "ggq_group_tables_bytes": (_L, [_L, _L, _L]),
+    "ggq_group_tables_build": (_I, [_P, _P, _L, _L, _L, _P, _L, _P]),
     "ggq_grouped_forward_reads_indexed_rows": (_I, [_I, _L, _L, _L, _L]),
-    "ggq_grouped_lora_mmq_forward_indexed": (_I, [_P, _L, _P, _I, _P, _P, _P, _P, _L, _L, _I, _L, _L, _L, _P, _P, _I, _F, _P, _P, _P, _P, _L, _P]),
-    "ggq_grouped_lora_mmq_backward_indexed": (_I, [_P, _P, _P, _P, _P, _P, _L, _L, _I, _L, _L, _L, _P, _L, _P, _I, _P, _P, _P, _I, _F, _P, _P, _P, _P, _L, _P]),
+    "ggq_grouped_lora_mmq_forward_indexed": (_I, [_P, _L, _P, _I, _P, _P, _P, _P, _L, _L, _I, _L, _L, _L, _P, _P, _I, _F, _P, _P, _P, _P, _P, _L, _P]),
+    "ggq_grouped_lora_mmq_backward_indexed": (_I, [_P, _P, _P, _P, _P, _P, _L, _L, _I, _L, _L, _L, _P, _L, _P, _I, _P, _P, _P, _I, _F, _P, _P, _P, _P, _P, _L, _P]),
     "ggq_route_plan_workspace_bytes": (_L, [_L, _I, _I]),
     "ggq_route_plan": (_I, [_P, _I, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _P]),
     "ggq_route_plan_static": (_I, [_P, _I, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
@@ -54,7 +56,7 @@ SIGNATURES: dict[str, tuple] = {
     "ggq_swiglu_clamped_backward": (_I, [_P, _P, _P, _P, _P, _L, _F, _P]),
     "ggq_swiglu_backward_routed": (_I, [_P, _P, _P, _P, _I, _P, _P, _P, _P, _L, _I, _F, _P]),
     "ggq_grouped_lora_mmq_backward_routed_output": (_I, [_P, _L, _P, _I, _P, _I, _P, _P, _P, _L, _L, _I, _L, _L, _L, _P, _P, _P, _P, _I, _F, _P, _P, _P,
-                                                         _P, _L, _P]),
+                                                         _P, _P, _L, _P]),
     "ggq_gmm_workspace_bytes": (_L, [_L]),
     "ggq_gmm": (_I, [_P, _P, _P, _P, _L, _L, _L, _L, _I, _I, _P, _L, _P]),
     "ggq_ptgmm": (_I, [_P, _P, _P, _P, _L, _L, _L, _L, _I, _P, _L, _P]),

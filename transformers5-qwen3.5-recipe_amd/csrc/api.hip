@@ -126,24 +126,24 @@ int ggq_lora_mmq_forward(const void* x, const void* packed, int qt, int64_t m, i
                          const void* lora_b, int r, float scale, void* xa_out, void* y, void* ws, int64_t ws_bytes,
                          void* stream) {
     return ggq_grouped_lora_mmq_forward(x, packed, nullptr, nullptr, nullptr, 0, 1, qt, m, n, k, lora_a, lora_b, r,
-                                        scale, xa_out, y, nullptr, ws, ws_bytes, stream);
+                                        scale, xa_out, y, nullptr, nullptr, ws, ws_bytes, stream);
 }
 
 int ggq_lora_mmq_backward(const void* dy, const void* packed, int qt, int64_t m, int64_t n, int64_t k, const void* x,
                           const void* xa, const void* lora_a, const void* lora_b, int r, float scale, void* dx,
                           void* d_lora_a, void* d_lora_b, void* ws, int64_t ws_bytes, void* stream) {
     return ggq_grouped_lora_mmq_backward(dy, nullptr, packed, nullptr, nullptr, nullptr, 0, 1, qt, m, n, k, x, xa, lora_a,
-                                         lora_b, r, scale, dx, d_lora_a, d_lora_b, ws, ws_bytes, stream);
+                                         lora_b, r, scale, dx, d_lora_a, d_lora_b, nullptr, ws, ws_bytes, stream);
 }
 
 int ggq_mmq(const void* x, const void* packed, int qt, int64_t m, int64_t n, int64_t k, void* y, void* stream) {
     return ggq_grouped_lora_mmq_forward(x, packed, nullptr, nullptr, nullptr, 0, 1, qt, m, n, k, nullptr, nullptr, 0, 0.f,
-                                        nullptr, y, nullptr, nullptr, 0, stream);
+                                        nullptr, y, nullptr, nullptr, nullptr, 0, stream);
 }
 
 int ggq_mmq_grad_input(const void* dy, const void* packed, int qt, int64_t m, int64_t n, int64_t k, void* dx, void* stream) {
     return ggq_grouped_lora_mmq_backward(dy, nullptr, packed, nullptr, nullptr, nullptr, 0, 1, qt, m, n, k, nullptr, nullptr,
-                                         nullptr, nullptr, 0, 0.f, dx, nullptr, nullptr, nullptr, 0, stream);
+                                         nullptr, nullptr, 0, 0.f, dx, nullptr, nullptr, nullptr, nullptr, 0, stream);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -180,6 +180,47 @@ int ggq_fixed_grouped_mmq_grad_input(const void* dy, const void* packed_groups, 
     return fixed_grouped("fixed_grouped_mmq_grad_input", kModeNN, dy, packed_groups, qt, rows, groups, n_group, k, dx, as_stream(stream));
 }
 
+// Row-tile tables of one grouping, built once (ggq_group_tables_build) and handed to the launches that share it: the
+// main table in group order and sorted by size, the 64-row table of the LoRA side kernels, the two tile counts, the
+// per-expert row ranges.  Only the decoding-wave kernels' tile height is covered; a launch of another shape builds its own.
+struct GroupTablesView {
+    TileDesc *t_main, *t_sorted, *t64;
+    int* counts;
+    int* ranges;
+    int max_main, max64;
+};
+static int64_t group_tables_layout(void* base, int64_t rows, int64_t groups, int64_t experts, GroupTablesView& v) {
+    Bump b{(char*)base, INT64_MAX, 0};
+    v.max_main = (int)(rows / kDirectBM + groups), v.max64 = (int)(rows / 64 + groups);
+    v.t_main = (TileDesc*)b.take((int64_t)v.max_main * sizeof(TileDesc));
+    v.t_sorted = (TileDesc*)b.take((int64_t)v.max_main * sizeof(TileDesc));
+    v.t64 = (TileDesc*)b.take((int64_t)v.max64 * sizeof(TileDesc));
+    v.counts = (int*)b.take(16);
+    v.ranges = (int*)b.take(experts * 2 * 4);
+    return b.used;
+}
+
+int64_t ggq_group_tables_bytes(int64_t rows, int64_t groups, int64_t experts) {
+    if (rows < 0 || groups < 1 || experts < 1 || rows >= (1ll << 31)) return -1;
+    GroupTablesView v;
+    return group_tables_layout(nullptr, rows, groups, experts, v);
+}
+
+int ggq_group_tables_build(const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts, int64_t rows, void* tables,
+                           int64_t tables_bytes, void* stream) {
+    if (!expert_ids || !end_offsets || !tables) return set_error(GGQ_ERR_NULL, "group_tables_build: null pointer");
+    if (!aligned16(tables)) return set_error(GGQ_ERR_ALIGN, "group_tables_build: the table buffer must be 16-byte aligned");
+    const int64_t need = ggq_group_tables_bytes(rows, groups, experts);
+    if (need < 0) return set_error(GGQ_ERR_SHAPE, "group_tables_build: bad sizes rows=%lld groups=%lld experts=%lld", (long long)rows, (long long)groups, (long long)experts);
+    if (tables_bytes < need) return set_error(GGQ_ERR_WORKSPACE, "group_tables_build: buffer of %lld bytes, %lld needed", (long long)tables_bytes, (long long)need);
+    GroupTablesView v;
+    group_tables_layout(tables, rows, groups, experts, v);
+    RowTileTables tb{};
+    tb.add(kDirectBM, 0, 0x7FFFFFFF, v.t_main, v.counts, v.t_sorted);
+    tb.add(64, 0, 0x7FFFFFFF, v.t64, v.counts + 1);
+    return build_row_tile_tables(expert_ids, end_offsets, (int)groups, tb, v.ranges, (int)experts, as_stream(stream));
+}
+
 // Forward of one projection (or a gate/up pair) over expert-sorted rows, optional LoRA fused.
 // groups == 0 means dense: one group of all rows using expert 0.
 // The forward launch reads its rows through an index when the source matrix stays under 4 GiB (the lane offsets of its
@@ -196,8 +237,9 @@ int ggq_grouped_forward_reads_indexed_rows(int qt, int64_t rows, int64_t groups,
 static int grouped_forward(const char* what, const void* x, RowIndex x_index, const void* packed1, const void* packed2, const int64_t* expert_ids,
                            const int32_t* end_offsets, int64_t groups, int64_t experts, int qt, int64_t rows, int64_t n,
                            int64_t k, const void* lora_a, const void* lora_b, int r, float scale, void* xa_out, void* y1,
-                           void* y2, void* ws, int64_t ws_bytes, void* stream) {
+                           void* y2, const void* group_tables, void* ws, int64_t ws_bytes, void* stream) {
     hipStream_t s = as_stream(stream);
+    if (group_tables && !aligned16(group_tables)) return set_error(GGQ_ERR_ALIGN, "%s: group tables must be 16-byte aligned", what);
     if (rows < 0 || n <= 0 || k <= 0 || rows >= (1ll << 31) || n >= (1ll << 30) || k >= (1ll << 30)) return set_error(GGQ_ERR_SHAPE, "%s: bad shape rows=%lld n=%lld k=%lld", what, (long long)rows, (long long)n, (long long)k);
     if (int rc = check_weights(what, qt, packed1, k)) return rc;
     if (packed2 && !aligned16(packed2)) return set_error(GGQ_ERR_ALIGN, "%s: packed weights must be 16-byte aligned", what);
@@ -227,7 +269,13 @@ static int grouped_forward(const char* what, const void* x, RowIndex x_index, co
     TileDesc* t_tall = nullptr;
     const int* n_tall = nullptr;
     int max_tall = 0;
-    if (groups > 0) {
+    if (groups > 0 && group_tables && p.shape == kShapeDirect) {  // tables the caller built once for this grouping
+        GroupTablesView v;
+        group_tables_layout(const_cast<void*>(group_tables), rows, groups, experts, v);
+        max_tiles64 = v.max64;
+        p.expert_ids = expert_ids, p.tiles = v.t_sorted, p.num_tiles = v.counts, p.max_row_tiles = v.max_main;
+        tiles64 = v.t64, num_tiles64 = v.counts + 1;
+    } else if (groups > 0) {
         // Wide shape: groups of at most 128 rows take one wide tile each, larger groups go to a second,
         // tall launch (a second wide tile for a few dozen leftover rows would cost a whole decode pass).
         const bool wide = p.shape == kShapeWide;
@@ -275,9 +323,9 @@ static int grouped_forward(const char* what, const void* x, RowIndex x_index, co
 int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void* packed2, const int64_t* expert_ids,
                                  const int32_t* end_offsets, int64_t groups, int64_t experts, int qt, int64_t rows, int64_t n,
                                  int64_t k, const void* lora_a, const void* lora_b, int r, float scale, void* xa_out, void* y1,
-                                 void* y2, void* ws, int64_t ws_bytes, void* stream) {
+                                 void* y2, const void* group_tables, void* ws, int64_t ws_bytes, void* stream) {
     return grouped_forward("grouped_lora_mmq_forward", x, RowIndex{}, packed1, packed2, expert_ids, end_offsets, groups, experts, qt, rows, n, k,
-                           lora_a, lora_b, r, scale, xa_out, y1, y2, ws, ws_bytes, stream);
+                           lora_a, lora_b, r, scale, xa_out, y1, y2, group_tables, ws, ws_bytes, stream);
 }
 
 // The same forward over rows that are not materialised: row i of the expert-sorted layout is row
@@ -285,26 +333,27 @@ int ggq_grouped_lora_mmq_forward(const void* x, const void* packed1, const void*
 int ggq_grouped_lora_mmq_forward_indexed(const void* x, int64_t x_rows, const int64_t* row_index, int index_div, const void* packed1,
                                          const void* packed2, const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups,
                                          int64_t experts, int qt, int64_t rows, int64_t n, int64_t k, const void* lora_a,
-                                         const void* lora_b, int r, float scale, void* xa_out, void* y1, void* y2, void* ws,
-                                         int64_t ws_bytes, void* stream) {
+                                         const void* lora_b, int r, float scale, void* xa_out, void* y1, void* y2, const void* group_tables,
+                                         void* ws, int64_t ws_bytes, void* stream) {
     const char* what = "grouped_lora_mmq_forward_indexed";
     if (!row_index) return set_error(GGQ_ERR_NULL, "%s: null row index", what);
     if (x_rows <= 0 || x_rows >= (1ll << 31) || index_div <= 0) return set_error(GGQ_ERR_SHAPE, "%s: bad x_rows=%lld or index_div=%d", what, (long long)x_rows, index_div);
     return grouped_forward(what, x, RowIndex{row_index, index_div, (int)x_rows}, packed1, packed2, expert_ids, end_offsets, groups, experts, qt,
-                           rows, n, k, lora_a, lora_b, r, scale, xa_out, y1, y2, ws, ws_bytes, stream);
+                           rows, n, k, lora_a, lora_b, r, scale, xa_out, y1, y2, group_tables, ws, ws_bytes, stream);
 }
 
 // Backward: dx = dy . W (+ LoRA term), and the factor gradients over all `experts` planes.
 static int grouped_backward(const char* what, const void* dy1, const void* dy2, const void* packed1, const void* packed2,
                             const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts, int qt,
                             int64_t rows, int64_t n, int64_t k, const void* x, RowIndex x_index, const void* xa, const void* lora_a,
-                            const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b, void* ws,
-                            int64_t ws_bytes, void* stream, RowIndex dy_index = RowIndex{}, const void* row_weights = nullptr,
+                            const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b, const void* group_tables,
+                            void* ws, int64_t ws_bytes, void* stream, RowIndex dy_index = RowIndex{}, const void* row_weights = nullptr,
                             int row_weights_are_bf16 = 0) {
     // dy_index: row i of the launch is row dy_index.source(i) of dy1 (one cotangent matrix), and, with row_weights, stands
     // for weights[dy_index.row_index[i]] times that row: dx comes out WITHOUT that factor (the caller applies it), the
     // factor gradients with it (it is put on their small operand, dy.B or xa)
     hipStream_t s = as_stream(stream);
+    if (group_tables && !aligned16(group_tables)) return set_error(GGQ_ERR_ALIGN, "%s: group tables must be 16-byte aligned", what);
     if (dy_index.on() && (dy2 || (uint64_t)dy_index.index_rows * (uint64_t)n * 2 >= (1ull << 32)))
         return set_error(GGQ_ERR_SHAPE, "%s: an indexed cotangent is one matrix under 4 GiB", what);
     if (rows < 0 || n <= 0 || k <= 0 || rows >= (1ll << 31) || n >= (1ll << 30) || k >= (1ll << 30)) return set_error(GGQ_ERR_SHAPE, "%s: bad shape rows=%lld n=%lld k=%lld", what, (long long)rows, (long long)n, (long long)k);
@@ -338,7 +387,13 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
     TileDesc* t_tall = nullptr;
     const int* n_tall = nullptr;
     int max_tall = 0;
-    if (groups > 0) {
+    if (groups > 0 && group_tables && p.shape == kShapeDirect) {  // tables the caller built once for this grouping
+        GroupTablesView v;
+        group_tables_layout(const_cast<void*>(group_tables), rows, groups, experts, v);
+        max_tiles64 = v.max64;
+        p.expert_ids = expert_ids, p.tiles = v.t_sorted, p.num_tiles = v.counts, p.max_row_tiles = v.max_main;
+        tiles64 = v.t64, num_tiles64 = v.counts + 1, ranges = v.ranges;
+    } else if (groups > 0) {
         const bool wide = p.shape == kShapeWide;  // small groups: wide tiles; larger ones: a second, tall launch
         const int bm_main = p.shape == kShapeDirect ? kDirectBM : p.shape == kShapeTall ? kBM : kWideBM;
         const int max128 = wide ? (int)groups : (int)(rows / bm_main + groups);
@@ -416,10 +471,10 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
 int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* packed1, const void* packed2,
                                   const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts, int qt,
                                   int64_t rows, int64_t n, int64_t k, const void* x, const void* xa, const void* lora_a,
-                                  const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b, void* ws,
-                                  int64_t ws_bytes, void* stream) {
+                                  const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b,
+                                  const void* group_tables, void* ws, int64_t ws_bytes, void* stream) {
     return grouped_backward("grouped_lora_mmq_backward", dy1, dy2, packed1, packed2, expert_ids, end_offsets, groups, experts, qt, rows, n, k, x,
-                            RowIndex{}, xa, lora_a, lora_b, r, scale, dx, d_lora_a, d_lora_b, ws, ws_bytes, stream);
+                            RowIndex{}, xa, lora_a, lora_b, r, scale, dx, d_lora_a, d_lora_b, group_tables, ws, ws_bytes, stream);
 }
 
 // The backward of the indexed forward: x is the [x_rows, k] matrix the forward read through row_index (it is only
@@ -429,13 +484,13 @@ int ggq_grouped_lora_mmq_backward_indexed(const void* dy1, const void* dy2, cons
                                           int qt, int64_t rows, int64_t n, int64_t k, const void* x, int64_t x_rows,
                                           const int64_t* row_index, int index_div, const void* xa, const void* lora_a,
                                           const void* lora_b, int r, float scale, void* dx, void* d_lora_a, void* d_lora_b,
-                                          void* ws, int64_t ws_bytes, void* stream) {
+                                          const void* group_tables, void* ws, int64_t ws_bytes, void* stream) {
     const char* what = "grouped_lora_mmq_backward_indexed";
     if (!row_index) return set_error(GGQ_ERR_NULL, "%s: null row index", what);
     if (x_rows <= 0 || x_rows >= (1ll << 31) || index_div <= 0) return set_error(GGQ_ERR_SHAPE, "%s: bad x_rows=%lld or index_div=%d", what, (long long)x_rows, index_div);
     return grouped_backward(what, dy1, dy2, packed1, packed2, expert_ids, end_offsets, groups, experts, qt, rows, n, k, x,
-                            RowIndex{row_index, index_div, (int)x_rows}, xa, lora_a, lora_b, r, scale, dx, d_lora_a, d_lora_b, ws, ws_bytes,
-                            stream);
+                            RowIndex{row_index, index_div, (int)x_rows}, xa, lora_a, lora_b, r, scale, dx, d_lora_a, d_lora_b, group_tables, ws,
+                            ws_bytes, stream);
 }
 
 // The backward of a projection whose output rows were scaled by routing weights and summed per token (the expert FFN's
@@ -447,12 +502,13 @@ int ggq_grouped_lora_mmq_backward_routed_output(const void* grad_out, int64_t to
                                                 const int64_t* expert_ids, const int32_t* end_offsets, int64_t groups, int64_t experts,
                                                 int qt, int64_t rows, int64_t n, int64_t k, const void* x, const void* xa,
                                                 const void* lora_a, const void* lora_b, int r, float scale, void* dx_unscaled,
-                                                void* d_lora_a, void* d_lora_b, void* ws, int64_t ws_bytes, void* stream) {
+                                                void* d_lora_a, void* d_lora_b, const void* group_tables, void* ws, int64_t ws_bytes,
+                                                void* stream) {
     const char* what = "grouped_lora_mmq_backward_routed_output";
     if (!permutation || !weights) return set_error(GGQ_ERR_NULL, "%s: null permutation or weights", what);
     if (tokens <= 0 || tokens >= (1ll << 31) || top_k <= 0 || rows != tokens * top_k) return set_error(GGQ_ERR_SHAPE, "%s: rows must be tokens * top_k", what);
     return grouped_backward(what, grad_out, nullptr, packed, nullptr, expert_ids, end_offsets, groups, experts, qt, rows, n, k, x, RowIndex{}, xa,
-                            lora_a, lora_b, r, scale, dx_unscaled, d_lora_a, d_lora_b, ws, ws_bytes, stream,
+                            lora_a, lora_b, r, scale, dx_unscaled, d_lora_a, d_lora_b, group_tables, ws, ws_bytes, stream,
                             RowIndex{permutation, top_k, (int)tokens}, weights, weights_are_bf16);
 }
 

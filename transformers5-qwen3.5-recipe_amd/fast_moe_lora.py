@@ -58,8 +58,21 @@ def _lora_ws(device, rows, groups, experts, n_total, k, r):
     return torch.empty(nbytes, dtype=torch.uint8, device=device)
 
 
-def _grouped_forward(x, p1, p2, expert_indices, expert_offsets, quant_type, n, lora_a, lora_b, scaling, row_index=None, index_div=1):
-    """``row_index`` (int64, one entry per expert-sorted row) makes row i of the launch row ``row_index[i] // index_div`` of x."""
+def build_group_tables(expert_indices: torch.Tensor, expert_offsets: torch.Tensor, rows: int, experts: int) -> torch.Tensor:
+    """The row-tile tables of one grouping (``ggq_group_tables_build``), for the grouped calls of a step that share it: every
+    such call otherwise builds the same tables in a launch of its own."""
+    lib = _lib.load()
+    groups = expert_indices.numel()
+    tables = torch.empty(int(lib.ggq_group_tables_bytes(rows, groups, experts)), dtype=torch.uint8, device=expert_indices.device)
+    _lib.check(lib.ggq_group_tables_build(expert_indices.data_ptr(), expert_offsets.data_ptr(), groups, experts, rows, tables.data_ptr(),
+                                          tables.numel(), _lib.stream_handle(expert_indices.device)))
+    return tables
+
+
+def _grouped_forward(x, p1, p2, expert_indices, expert_offsets, quant_type, n, lora_a, lora_b, scaling, row_index=None, index_div=1,
+                     group_tables=None):
+    """``row_index`` (int64, one entry per expert-sorted row) makes row i of the launch row ``row_index[i] // index_div`` of x.
+    ``group_tables``: what ``build_group_tables`` returned for these expert_indices / expert_offsets / rows."""
     k = x.shape[1]
     rows = x.shape[0] if row_index is None else row_index.numel()
     experts = p1.shape[0]
@@ -84,7 +97,7 @@ def _grouped_forward(x, p1, p2, expert_indices, expert_offsets, quant_type, n, l
         ws = _lora_ws(x.device, rows, expert_indices.numel(), experts, nseg * n, k, r)
         tail = (p1.data_ptr(), _lib.ptr(p2), expert_indices.data_ptr(), expert_offsets.data_ptr(), expert_indices.numel(),
                 experts, quant_type, rows, n, k, _lib.ptr(lora_a), _lib.ptr(lora_b), r, float(scaling), _lib.ptr(xa), y1.data_ptr(),
-                _lib.ptr(y2), ws.data_ptr(), ws.numel(), _lib.stream_handle(x.device))
+                _lib.ptr(y2), _lib.ptr(group_tables), ws.data_ptr(), ws.numel(), _lib.stream_handle(x.device))
         if row_index is None:
             _lib.check(_lib.load().ggq_grouped_lora_mmq_forward(x.data_ptr(), *tail))
         else:
@@ -93,7 +106,7 @@ def _grouped_forward(x, p1, p2, expert_indices, expert_offsets, quant_type, n, l
 
 
 def _grouped_backward(dy1, dy2, p1, p2, expert_indices, expert_offsets, quant_type, k, x, xa, lora_a, lora_b, scaling, want_da, want_db,
-                      row_index=None, index_div=1):
+                      row_index=None, index_div=1, group_tables=None):
     rows, n = dy1.shape
     experts = p1.shape[0]
     _check_grouped(dy1, p1, expert_indices, expert_offsets, quant_type, n, k, "grouped_mmq_grad_input")
@@ -107,8 +120,8 @@ def _grouped_backward(dy1, dy2, p1, p2, expert_indices, expert_offsets, quant_ty
     ws = _lora_ws(dy1.device, rows, expert_indices.numel(), experts, nseg * n, k, r)
     head = (dy1.data_ptr(), _lib.ptr(dy2), p1.data_ptr(), _lib.ptr(p2), expert_indices.data_ptr(), expert_offsets.data_ptr(),
             expert_indices.numel(), experts, quant_type, rows, n, k, _lib.ptr(x))
-    tail = (_lib.ptr(xa), _lib.ptr(lora_a), _lib.ptr(lora_b), r, float(scaling), dx.data_ptr(), _lib.ptr(da), _lib.ptr(db), ws.data_ptr(),
-            ws.numel(), _lib.stream_handle(dy1.device))
+    tail = (_lib.ptr(xa), _lib.ptr(lora_a), _lib.ptr(lora_b), r, float(scaling), dx.data_ptr(), _lib.ptr(da), _lib.ptr(db),
+            _lib.ptr(group_tables), ws.data_ptr(), ws.numel(), _lib.stream_handle(dy1.device))
     if row_index is None:
         _lib.check(_lib.load().ggq_grouped_lora_mmq_backward(*head, *tail))
     else:
@@ -135,8 +148,10 @@ class _GroupedLoraProjection(torch.autograd.Function):
     """One expert projection (or a gate/up pair) with the LoRA delta fused in."""
 
     @staticmethod
-    def forward(ctx, x, p1, p2, expert_indices, expert_offsets, quant_type, n, lora_a, lora_b, scaling):
-        y1, y2, xa = _grouped_forward(x, p1, p2, expert_indices, expert_offsets, quant_type, n, lora_a, lora_b, scaling)
+    def forward(ctx, x, p1, p2, expert_indices, expert_offsets, quant_type, n, lora_a, lora_b, scaling, group_tables=None):
+        y1, y2, xa = _grouped_forward(x, p1, p2, expert_indices, expert_offsets, quant_type, n, lora_a, lora_b, scaling,
+                                      group_tables=group_tables)
+        ctx.group_tables = group_tables
         tensors = [x, expert_indices, expert_offsets, p1]
         ctx.has_pair, ctx.has_lora = p2 is not None, lora_a is not None
         if ctx.has_pair:
@@ -163,7 +178,7 @@ class _GroupedLoraProjection(torch.autograd.Function):
         g2 = grads[1] if ctx.has_pair else None
         if ctx.has_pair and (g1 is None or g2 is None):
             if g1 is None and g2 is None:
-                return (None,) * 10
+                return (None,) * 11
             like = g1 if g1 is not None else g2
             g1 = torch.zeros_like(like) if g1 is None else g1
             g2 = torch.zeros_like(like) if g2 is None else g2
@@ -171,8 +186,8 @@ class _GroupedLoraProjection(torch.autograd.Function):
         g2 = g2.contiguous() if g2 is not None else None
         want_da, want_db = ctx.needs_input_grad[7], ctx.needs_input_grad[8]
         dx, da, db = _grouped_backward(g1, g2, p1, p2, expert_indices, expert_offsets, quant_type, x.shape[1], x, xa, lora_a, lora_b,
-                                       scaling, want_da, want_db)
-        return (dx if ctx.needs_input_grad[0] else None), None, None, None, None, None, None, da, db, None
+                                       scaling, want_da, want_db, group_tables=ctx.group_tables)
+        return (dx if ctx.needs_input_grad[0] else None), None, None, None, None, None, None, da, db, None, None
 
 
 class _RoutedGroupedLoraProjection(torch.autograd.Function):
@@ -182,9 +197,10 @@ class _RoutedGroupedLoraProjection(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, hidden_states, permutation, inverse_permutation, top_k, p1, p2, expert_indices, expert_offsets, quant_type, n,
-                lora_a, lora_b, scaling):
+                lora_a, lora_b, scaling, group_tables=None):
         y1, y2, xa = _grouped_forward(hidden_states, p1, p2, expert_indices, expert_offsets, quant_type, n, lora_a, lora_b, scaling,
-                                      row_index=permutation, index_div=top_k)
+                                      row_index=permutation, index_div=top_k, group_tables=group_tables)
+        ctx.group_tables = group_tables
         tensors = [hidden_states, permutation, inverse_permutation, expert_indices, expert_offsets, p1]
         ctx.has_pair, ctx.has_lora = p2 is not None, lora_a is not None
         if ctx.has_pair:
@@ -211,7 +227,7 @@ class _RoutedGroupedLoraProjection(torch.autograd.Function):
         g2 = grads[1] if ctx.has_pair else None
         if ctx.has_pair and (g1 is None or g2 is None):
             if g1 is None and g2 is None:
-                return (None,) * 13
+                return (None,) * 14
             like = g1 if g1 is not None else g2
             g1 = torch.zeros_like(like) if g1 is None else g1
             g2 = torch.zeros_like(like) if g2 is None else g2
@@ -220,13 +236,14 @@ class _RoutedGroupedLoraProjection(torch.autograd.Function):
         want_da, want_db = ctx.needs_input_grad[10], ctx.needs_input_grad[11]
         tokens, k = hidden_states.shape
         d_selected, da, db = _grouped_backward(g1, g2, p1, p2, expert_indices, expert_offsets, quant_type, k, hidden_states, xa, lora_a,
-                                               lora_b, scaling, want_da, want_db, row_index=permutation, index_div=top_k)
+                                               lora_b, scaling, want_da, want_db, row_index=permutation, index_div=top_k,
+                                               group_tables=ctx.group_tables)
         d_hidden = None
         if ctx.needs_input_grad[0]:
             d_hidden = torch.empty(tokens, k, dtype=d_selected.dtype, device=d_selected.device)
             _lib.check(_lib.load().ggq_route_gather_backward(d_selected.data_ptr(), inverse_permutation.data_ptr(), d_hidden.data_ptr(),
                                                              tokens, top_k, k, _lib.stream_handle(d_selected.device)))
-        return (d_hidden,) + (None,) * 9 + (da, db, None)
+        return (d_hidden,) + (None,) * 9 + (da, db, None, None)
 
 
 def routed_projection_reads_tokens_in_place(quant_type: int, routes: int, groups: int, tokens: int, in_features: int) -> bool:
@@ -302,6 +319,8 @@ def swiglu(gate: torch.Tensor, up: torch.Tensor, limit: float | None = None) -> 
 
 # set to False to run the activation, the down projection and the combine as three autograd nodes (the reference's structure)
 FUSE_GATED_DOWN_COMBINE = True
+# set to False to let every grouped call of the layer build its own row-tile tables
+SHARE_GROUP_TABLES = True
 
 
 class _RoutedGatedDownProjection(torch.autograd.Function):
@@ -315,7 +334,7 @@ class _RoutedGatedDownProjection(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, gate, up, limit, payload, expert_indices, expert_offsets, quant_type, out_features, lora_a, lora_b, scaling,
-                routing_weights, permutation, inverse_permutation):
+                routing_weights, permutation, inverse_permutation, group_tables=None):
         _lib.require_device_tensor(gate, "gate", torch.bfloat16)
         _lib.require_device_tensor(up, "up", torch.bfloat16)
         lib, stream = _lib.load(), _lib.stream_handle(gate.device)
@@ -324,7 +343,9 @@ class _RoutedGatedDownProjection(torch.autograd.Function):
             _lib.check(lib.ggq_swiglu_forward(gate.data_ptr(), up.data_ptr(), act.data_ptr(), gate.numel(), stream))
         else:
             _lib.check(lib.ggq_swiglu_clamped_forward(gate.data_ptr(), up.data_ptr(), act.data_ptr(), gate.numel(), float(limit), stream))
-        y, _, xa = _grouped_forward(act, payload, None, expert_indices, expert_offsets, quant_type, out_features, lora_a, lora_b, scaling)
+        y, _, xa = _grouped_forward(act, payload, None, expert_indices, expert_offsets, quant_type, out_features, lora_a, lora_b, scaling,
+                                    group_tables=group_tables)
+        ctx.group_tables = group_tables
         tokens, top_k = routing_weights.shape
         out = torch.empty(tokens, out_features, dtype=y.dtype, device=y.device)
         _lib.check(lib.ggq_route_combine_forward(y.data_ptr(), routing_weights.data_ptr(), int(routing_weights.dtype == torch.bfloat16),
@@ -358,13 +379,13 @@ class _RoutedGatedDownProjection(torch.autograd.Function):
         _lib.check(lib.ggq_grouped_lora_mmq_backward_routed_output(
             grad_out.data_ptr(), tokens, permutation.data_ptr(), top_k, routing_weights.data_ptr(), w_bf16, payload.data_ptr(),
             expert_indices.data_ptr(), expert_offsets.data_ptr(), expert_indices.numel(), experts, quant_type, rows, n, k, act.data_ptr(),
-            _lib.ptr(xa), _lib.ptr(lora_a), _lib.ptr(lora_b), r, scaling, d_act.data_ptr(), _lib.ptr(da), _lib.ptr(db), ws.data_ptr(),
-            ws.numel(), stream))
+            _lib.ptr(xa), _lib.ptr(lora_a), _lib.ptr(lora_b), r, scaling, d_act.data_ptr(), _lib.ptr(da), _lib.ptr(db),
+            _lib.ptr(ctx.group_tables), ws.data_ptr(), ws.numel(), stream))
         dgate, dup = torch.empty_like(gate), torch.empty_like(up)
         dw = torch.empty_like(routing_weights) if ctx.needs_input_grad[11] else None
         _lib.check(lib.ggq_swiglu_backward_routed(gate.data_ptr(), up.data_ptr(), d_act.data_ptr(), routing_weights.data_ptr(), w_bf16,
                                                   permutation.data_ptr(), dgate.data_ptr(), dup.data_ptr(), _lib.ptr(dw), rows, k, limit, stream))
-        return dgate, dup, None, None, None, None, None, None, da, db, None, dw, None, None
+        return dgate, dup, None, None, None, None, None, None, da, db, None, dw, None, None, None
 
 
 # ------------------------------------------------------------------------------------------------
@@ -474,27 +495,32 @@ def qwen3_5_moe_gguf_mmq_lora_forward(self: GGUFExperts, hidden_states: torch.Te
     expert_indices, expert_offsets = execution_plan.expert_indices, execution_plan.offsets
     lw = lora_weights
     s = lw.scaling if lw is not None else 0.0
+    # the four packed-weight calls of the step see one grouping: its row-tile tables are built once (the calls whose kernels
+    # take another tile shape ignore them and build their own)
+    tables = None
+    if SHARE_GROUP_TABLES and (int(self.gate_proj.quant_type) == 12 or int(self.down_proj.quant_type) == 12):
+        tables = build_group_tables(expert_indices, expert_offsets, tokens * top_k, self.num_experts)
 
     if in_place:
         gate, up = _RoutedGroupedLoraProjection.apply(
             compute_hidden_states, routing_plan.permutation, routing_plan.inverse_permutation, top_k, _as_payload(self.gate_proj),
             _as_payload(self.up_proj), expert_indices, expert_offsets, int(self.gate_proj.quant_type), self.intermediate_dim,
-            lw.gate_up_a if lw else None, lw.gate_up_b if lw else None, s)
+            lw.gate_up_a if lw else None, lw.gate_up_b if lw else None, s, tables)
     else:
         gate, up = _GroupedLoraProjection.apply(
             selected, _as_payload(self.gate_proj), _as_payload(self.up_proj), expert_indices, expert_offsets,
-            int(self.gate_proj.quant_type), self.intermediate_dim, lw.gate_up_a if lw else None, lw.gate_up_b if lw else None, s)
+            int(self.gate_proj.quant_type), self.intermediate_dim, lw.gate_up_a if lw else None, lw.gate_up_b if lw else None, s, tables)
     if (FUSE_GATED_DOWN_COMBINE and execution_plan.output_mask is None and type(self)._apply_split_gate is GGUFExperts._apply_split_gate
             and routing_plan.routing_weights.is_contiguous()):
         combined = _RoutedGatedDownProjection.apply(
             gate, up, self.swiglu_limit, _as_payload(self.down_proj), expert_indices, expert_offsets, int(self.down_proj.quant_type),
             self.hidden_dim, lw.down_a if lw else None, lw.down_b if lw else None, s, routing_plan.routing_weights, routing_plan.permutation,
-            routing_plan.inverse_permutation)
+            routing_plan.inverse_permutation, tables)
         return combined.to(hidden_states.dtype).reshape(hidden_states.shape)
     intermediate = self._apply_split_gate(gate, up)
     output = _GroupedLoraProjection.apply(
         intermediate, _as_payload(self.down_proj), None, expert_indices, expert_offsets, int(self.down_proj.quant_type),
-        self.hidden_dim, lw.down_a if lw else None, lw.down_b if lw else None, s)
+        self.hidden_dim, lw.down_a if lw else None, lw.down_b if lw else None, s, tables)
     return finalize_expert_routing(output, hidden_states, routing_plan, execution_plan.output_mask).reshape(hidden_states.shape)
 
 
