@@ -39,6 +39,34 @@ def test_library_exports_every_declared_symbol(pkg):
     assert set(pkg._lib.SIGNATURES) == set(declared_symbols())
 
 
+def declared_parameter_counts() -> dict[str, int]:
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    counts = {}
+    for name, params in re.findall(r"\b(ggq_\w+)\s*\(([^)]*)\)\s*;", text):
+        params = params.strip()
+        counts[name] = 0 if params in ("", "void") else params.count(",") + 1
+    return counts
+
+
+def test_signature_table_has_the_arity_and_kinds_the_header_declares(pkg):
+    """A ctypes table that is one argument short of the C declaration calls the function with garbage in that slot without
+    any error: every entry has as many argument types as the header declares parameters, pointers where it declares pointers."""
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    counts = declared_parameter_counts()
+    assert set(counts) == set(pkg._lib.SIGNATURES)
+    for name, (restype, argtypes) in pkg._lib.SIGNATURES.items():
+        assert len(argtypes) == counts[name], f"{name}: {len(argtypes)} argument types for {counts[name]} declared parameters"
+        params = re.search(r"\b" + name + r"\s*\(([^)]*)\)\s*;", text).group(1)
+        if counts[name] == 0:
+            continue
+        for i, (decl, ctype) in enumerate(zip([p.strip() for p in params.split(",")], argtypes)):
+            is_pointer = "*" in decl
+            assert is_pointer == (ctype is ctypes.c_void_p), f"{name} parameter {i} ({decl!r}) against {ctype}"
+            if not is_pointer:
+                want = ctypes.c_float if decl.startswith("float") else ctypes.c_int64 if decl.startswith("int64_t") else ctypes.c_int
+                assert ctype is want, f"{name} parameter {i} ({decl!r}) against {ctype}"
+
+
 def test_host_only_helpers(pkg):
     lib = pkg._lib.load()
     for qt, (elems, nbytes) in gb.QUANT_SIZES.items():
