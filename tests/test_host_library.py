@@ -56,6 +56,9 @@ def test_signature_table_has_the_arity_and_kinds_the_header_declares(pkg):
     assert set(counts) == set(pkg._lib.SIGNATURES)
     for name, (restype, argtypes) in pkg._lib.SIGNATURES.items():
         assert len(argtypes) == counts[name], f"{name}: {len(argtypes)} argument types for {counts[name]} declared parameters"
+        returns = re.search(r"([\w \*]+?)\s*\b" + name + r"\s*\(", text).group(1).strip()
+        want_ret = ctypes.c_char_p if "char" in returns else ctypes.c_int64 if returns.endswith("int64_t") else ctypes.c_int
+        assert restype is want_ret, f"{name} returns {returns!r}, the table says {restype}"
         params = re.search(r"\b" + name + r"\s*\(([^)]*)\)\s*;", text).group(1)
         if counts[name] == 0:
             continue
