@@ -61,7 +61,7 @@ int ggq_measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64
 }
 
 int ggq_debug_force_grouped_shape(int shape) {
-    if (shape != -1 && shape != kShapeTall && shape != kShapeWide && shape != kShapeDirect) return set_error(GGQ_ERR_SHAPE, "debug_force_grouped_shape: unknown shape %d", shape);
+    if (shape != -1 && shape != kShapeTall && shape != kShapeWide && shape != kShapeDirect && shape != kShapeSmall) return set_error(GGQ_ERR_SHAPE, "debug_force_grouped_shape: unknown shape %d", shape);
     g_shape_override = shape;
     return GGQ_OK;
 }
@@ -109,6 +109,14 @@ static int direct_tiles_per_wg(int64_t rows, int64_t groups, int col_tiles, int 
     return per_wg;
 }
 
+// Small shape: a workgroup stages the decoder's tables and its row tile's LoRA rows once, so it walks up to four column
+// tiles while that still leaves every compute unit eight workgroups.
+static int small_tiles_per_wg(int64_t groups, int col_tiles) {
+    int per_wg = 4;
+    while (per_wg > 1 && groups * ((col_tiles + per_wg - 1) / per_wg) < 2048) per_wg >>= 1;
+    return per_wg;
+}
+
 // A dense layer's factor gradients deal their rows to at most this many workgroups per column block (fp32 partial sums
 // in the workspace).
 constexpr int64_t kDenseFactorSplits = 32;
@@ -117,7 +125,7 @@ int64_t ggq_lora_workspace_bytes(int64_t rows, int64_t groups, int64_t experts, 
     const int rp = rank_pad(r > 0 ? r : 1);
     if (experts < 1) experts = 1;
     const int64_t tiles = rows / 64 + groups + 2;
-    return 3 * align256(tiles * (int64_t)sizeof(TileDesc)) + align256(16) + align256(experts * 2 * 4) +
+    return 4 * align256(tiles * (int64_t)sizeof(TileDesc)) + align256(16) + align256(experts * 2 * 4) +
            align256(experts * n_total * rp * 2) * 2 + align256(experts * k * rp * 2) + align256(rows * rp * 2) + 4096 +
            (groups == 0 ? align256(kDenseFactorSplits * std::max(n_total, k) * rp * 4) : 0);
 }
@@ -269,6 +277,8 @@ static int grouped_forward(const char* what, const void* x, RowIndex x_index, co
     TileDesc* t_tall = nullptr;
     const int* n_tall = nullptr;
     int max_tall = 0;
+    TileDesc* t_small = nullptr;
+    const int* n_small = nullptr;
     if (groups > 0 && group_tables && p.shape == kShapeDirect) {  // tables the caller built once for this grouping
         GroupTablesView v;
         group_tables_layout(const_cast<void*>(group_tables), rows, groups, experts, v);
@@ -288,15 +298,19 @@ static int grouped_forward(const char* what, const void* x, RowIndex x_index, co
         TileDesc* t_sorted = direct ? (TileDesc*)bump.take((int64_t)max128 * sizeof(TileDesc)) : nullptr;
         t_tall = wide ? (TileDesc*)bump.take((int64_t)max_tall * sizeof(TileDesc)) : nullptr;
         TileDesc* t64 = lora_a ? (TileDesc*)bump.take((int64_t)max_tiles64 * sizeof(TileDesc)) : nullptr;
+        // IQ2_XXS: the groups of at most 128 rows leave the wide table for a launch of their own (decoding waves)
+        const bool small = wide && qt == 16 /* GGML IQ2_XXS */ && direct_ok && g_shape_override != kShapeWide;
+        t_small = small ? (TileDesc*)bump.take((int64_t)groups * sizeof(TileDesc)) : nullptr;
         int* counts = (int*)bump.take(16);
-        if (!t128 || !counts || (lora_a && !t64) || (wide && !t_tall) || (direct && !t_sorted)) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
+        if (!t128 || !counts || (lora_a && !t64) || (wide && !t_tall) || (direct && !t_sorted) || (small && !t_small)) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
         RowTileTables tb{};
-        tb.add(bm_main, 0, wide ? kWideBM : 0x7FFFFFFF, t128, counts, t_sorted);
+        tb.add(bm_main, small ? kSmallBM : 0, wide ? kWideBM : 0x7FFFFFFF, t128, counts, t_sorted);
         if (direct) t128 = t_sorted;
         if (wide) tb.add(kBM, kWideBM, 0x7FFFFFFF, t_tall, counts + 2), n_tall = counts + 2;
         if (lora_a) tb.add(64, 0, 0x7FFFFFFF, t64, counts + 1);
+        if (small) tb.add(kSmallBM, 0, kSmallBM, t_small, counts + 3), n_small = counts + 3;
         if (int rc = build_row_tile_tables(expert_ids, end_offsets, (int)groups, tb, nullptr, 0, s)) return rc;
-        p.expert_ids = expert_ids, p.tiles = t128, p.num_tiles = counts, p.max_row_tiles = max128;
+        p.expert_ids = expert_ids, p.tiles = t128, p.num_tiles = counts, p.max_row_tiles = small ? 0 : max128;  // (small: the wide table stays empty)
         tiles64 = t64, num_tiles64 = counts + 1;
     }
     if (lora_a) {
@@ -315,6 +329,12 @@ static int grouped_forward(const char* what, const void* x, RowIndex x_index, co
             lb = padded;
         }
         p.la = (const bf16_t*)xa_out, p.lb = lb, p.lb_expert_elems = (int64_t)nseg * n * rp, p.r_pad = rp, p.lora_scale = scale;
+    }
+    if (t_small) {
+        MmqParams ps = p;
+        ps.tiles = t_small, ps.num_tiles = n_small, ps.max_row_tiles = (int)groups, ps.shape = kShapeSmall;
+        ps.col_tiles_per_wg = small_tiles_per_wg(groups, nseg * p.col_tiles_per_seg);
+        if (int rc = launch_mmq_small(ps, s)) return rc;
     }
     if (t_tall) return launch_wide_and_tall(qt, kModeNT, p, (int)rows, (int)n, (int)k, nseg, t_tall, n_tall, max_tall, s);
     return launch_mmq(qt, kModeNT, kEpiStore, p, s);

@@ -2,6 +2,7 @@
 #include "mmq_tile.h"
 #include "mmq_direct8.h"
 #include "mmq_direct8_nn.h"
+#include "mmq_small_iq2.h"
 #include "launch.h"
 
 #include <stdarg.h>
@@ -262,6 +263,35 @@ static int launch_mixed_mode(const MmqParams& p, hipStream_t s) {
     hipLaunchKernelGGL((mmq_mixed_kernel<QT, MODE, kEpiStore>), dim3((unsigned)grid), dim3(kThreads), kSmemBytes, s, p);
     if (t) (void)hipEventRecord(t->stop, s);
     return check_launch("mmq_mixed_kernel");
+}
+
+// IQ2_XXS, forward, store epilogue: tiles of up to kSmallBM rows (p.tiles) on the decoding-wave kernel.
+int launch_mmq_small(const MmqParams& p, hipStream_t s) {
+    const int col_tiles = p.nseg * p.col_tiles_per_seg;
+    if (p.col_tiles_per_wg < 1) return set_error(GGQ_ERR_SHAPE, "mmq: column tiles per workgroup must be at least 1");
+    if (p.steps_per_seg & 3) return set_error(GGQ_ERR_SHAPE, "mmq: the small-group kernel needs a contraction of whole 256-wide blocks");
+    // row tiles are dealt round-robin over the eight XCDs; each XCD walks its row tiles' column-tile runs
+    const int64_t total = (int64_t)((p.max_row_tiles + 7) / 8) * ((col_tiles + p.col_tiles_per_wg - 1) / p.col_tiles_per_wg);
+    if (total <= 0) return GGQ_OK;
+    const int64_t grid = total * 8;
+    if (grid > 0x7FFFFFF0) return set_error(GGQ_ERR_SHAPE, "mmq: too many tiles for one launch");
+    TimedLaunch* t = nullptr;
+    if (g_timing && g_timed_count < kMaxTimedLaunches) {
+        t = &g_timed[g_timed_count];
+        if (hipEventCreate(&t->start) != hipSuccess || hipEventCreate(&t->stop) != hipSuccess) return set_error(GGQ_ERR_RUNTIME, "mmq: event creation failed");
+        t->qt = kIQ2_XXS, t->mode = kModeNT, t->epi = kEpiStore, t->shape = kShapeSmall;
+        g_timed_count++;
+        (void)hipEventRecord(t->start, s);
+    }
+    static bool attr_set = false;
+    if (!attr_set) {
+        if (hipFuncSetAttribute((const void*)mmq_small_iq2xxs_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SmallIq2::kLdsBytes) != hipSuccess)
+            return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", SmallIq2::kLdsBytes);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(mmq_small_iq2xxs_kernel, dim3((unsigned)grid), dim3(SmallIq2::kThreadsWG), SmallIq2::kLdsBytes, s, p);
+    if (t) (void)hipEventRecord(t->stop, s);
+    return check_launch("mmq_small_iq2xxs_kernel");
 }
 
 int launch_mmq_mixed(int qt, int mode, const MmqParams& p, hipStream_t s) {

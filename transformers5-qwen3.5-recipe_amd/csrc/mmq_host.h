@@ -64,7 +64,9 @@ struct FactorGradParams {
 constexpr int kBM = 256, kBN = 128, kBK = 64;  // the tall tile shape (dense launches, large expert groups)
 constexpr int kWideBM = 128, kWideBN = 256;    // the wide tile shape (Q4_K expert groups of about a hundred rows)
 constexpr int kDirectBM = 192, kDirectBN = 256;  // the direct shape (Q4_K expert groups: the MFMA waves decode the weights themselves)
+constexpr int kSmallBM = 128, kSmallBN = 256;   // the small shape (IQ2_XXS forward, expert groups of at most 128 rows: decoding waves)
 constexpr int kShapeTall = 0, kShapeWide = 1, kShapeDirect = 3;
+constexpr int kShapeSmall = 5;  // (a launch beside the wide and tall tiles of a call, never the shape of a whole call)
 constexpr int kShapeMixed = 4;  // (profile records only: one launch of wide and tall tiles)
 constexpr int kLdsStride = kBK + 8;  // bf16 elements per LDS row: 144 bytes keeps 128-bit reads conflict-free
 constexpr int kThreads = 1024;  // waves 0..7 run the MFMAs, waves 8..15 load and decode
@@ -118,6 +120,7 @@ int measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64_t e
 const char* last_error();
 int launch_mmq(int qt, int mode, int epi, const MmqParams& p, hipStream_t s);
 int launch_mmq_mixed(int qt, int mode, const MmqParams& p, hipStream_t s);  // Q4_K, store epilogue, tiles + tiles2
+int launch_mmq_small(const MmqParams& p, hipStream_t s);  // IQ2_XXS forward, store epilogue, tiles of kSmallBM rows
 int init_params(MmqParams& p, int qt, int mode, int m, int n, int k, int nseg, int shape = kShapeTall);
 
 int pad_factor(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int r, int r_pad, bool transpose, hipStream_t s);
@@ -128,15 +131,15 @@ int factor_grad(const FactorGradParams& p, int r_pad, int64_t experts, hipStream
 
 // Builds the row-tile table of an expert-sorted layout on the device (no host sync):
 // tiles[0..*num_tiles) in group order, tile height bm; optionally per-expert row ranges.
-// Up to three row-tile tables built by one launch (one workgroup each).
+// Up to four row-tile tables built by one launch (one workgroup each).
 struct RowTileTables {
     int count;
-    int bm[3], min_rows[3], max_rows[3];
-    TileDesc* tiles[3];
-    int* num_tiles[3];
+    int bm[4], min_rows[4], max_rows[4];
+    TileDesc* tiles[4];
+    int* num_tiles[4];
     // not null: the table also goes here ordered by descending number of 32-row blocks (ties in group order), so that
     // workgroups dispatched in table order take the most expensive tiles first
-    TileDesc* by_size[3];
+    TileDesc* by_size[4];
     void add(int bm_, int min_rows_, int max_rows_, TileDesc* tiles_, int* num_tiles_, TileDesc* by_size_ = nullptr) {
         bm[count] = bm_, min_rows[count] = min_rows_, max_rows[count] = max_rows_, tiles[count] = tiles_, num_tiles[count] = num_tiles_;
         by_size[count] = by_size_;
