@@ -39,6 +39,8 @@ def kernel_name(qt: int, mode: int, epi: int, shape: int) -> str:
         return "mmq_direct8_q4k_kernel (Q4_K, forward)" if mode == 0 else "mmq_direct8_nn_q4k_kernel (Q4_K, grad_input)"
     if shape == 4:
         return f"mmq_mixed_kernel<{_TYPE_NAMES.get(qt, qt)}, {direction}, store>"
+    if shape == 5:
+        return "mmq_small_iq2xxs_kernel (IQ2_XXS, forward)"
     return f"mmq_tile_kernel<{_TYPE_NAMES.get(qt, qt)}, {direction}, {'store' if epi == 0 else 'accumulate_f32'}, {'tall' if shape == 0 else 'wide'}>"
 
 

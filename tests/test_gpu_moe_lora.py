@@ -154,6 +154,42 @@ def test_grouped_lora_projection_all_gradients(pkg, dev, qt, r, shape, n, force_
     assert_close_bf16(bd2.grad, want1["db"], "single dB")
 
 
+@pytest.mark.parametrize("sizes,n,k,r,pair", [
+    ([1, 32, 33, 64, 65, 96, 97, 128, 129, 0, 7], 256, 512, 16, True),   # every count of live 32-row blocks; 129 rows: a tall tile beside them
+    ([64, 64, 50, 3], 72, 256, 0, False),                                    # one block of the contraction; columns end inside a wave's 32
+    ([40, 100, 128], 520, 768, 32, False),                                   # three column tiles, the last one 8 wide; rank 32
+    ([5, 90], 8, 1024, 4, True),                                             # fewer columns than one wave owns; rank padded to 16
+    ([128] * 3 + [1] * 5, 512, 256, 64, False),                              # rank 64
+])
+def test_iq2xxs_forward_of_small_groups(pkg, dev, sizes, n, k, r, pair):
+    # IQ2_XXS groups of at most 128 rows run the forward kernel whose MFMA waves decode the packed bytes themselves
+    # (mmq_small_iq2xxs_kernel); larger groups of the same call stay on the tile kernel.  Against the oracle, with and
+    # without LoRA, as a pair and as a single projection.
+    ml = pkg.fast_moe_lora
+    qt = gb.IQ2_XXS
+    e_total, rows = len(sizes), sum(sizes)
+    ids = torch.arange(e_total, dtype=torch.int64)
+    ends = torch.tensor(np.cumsum(sizes), dtype=torch.int32)
+    gen = torch.Generator().manual_seed(97 + n + k + r)
+    segs = 2 if pair else 1
+    payloads = [_expert_payload(700 + 100 * j, qt, e_total, n, k) for j in range(segs)]
+    w = torch.cat([ref.weights_bf16(pl, qt) for pl in payloads], dim=1)
+    x = bf16_randn(gen, rows, k)
+    a = bf16_randn(gen, e_total, r, k, std=k ** -0.5) if r else None
+    b = bf16_randn(gen, e_total, segs * n, r, std=0.02) if r else None
+    want = ref.grouped_lora_linear(x, w, ids, ends, a, b, 2.0) if r else ref.grouped_lora_linear(x, w, ids, ends)
+    pd = [torch.from_numpy(pl).to(dev) for pl in payloads]
+    if pair and r:
+        ys = ml.grouped_lora_mmq_pair(x.to(dev), pd[0], pd[1], ids.to(dev), ends.to(dev), qt, n, a.to(dev), b.to(dev), 2.0)
+    elif pair:
+        ys = ml.grouped_mmq_pair(x.to(dev), pd[0], pd[1], ids.to(dev), ends.to(dev), qt, n)
+    elif r:
+        ys = (ml.grouped_lora_mmq(x.to(dev), pd[0], ids.to(dev), ends.to(dev), qt, n, a.to(dev), b.to(dev), 2.0),)
+    else:
+        ys = (ml.grouped_mmq(x.to(dev), pd[0], ids.to(dev), ends.to(dev), qt, n),)
+    assert_close_bf16(torch.cat(list(ys), dim=1), want["y"], "Y")
+
+
 @pytest.mark.parametrize("top_k,rank,pair,qt,shape", [(8, 16, True, gb.Q4_K, ""), (3, 4, True, gb.Q4_K, ""), (1, 16, False, gb.Q4_K, ""),
                                                       (8, 0, True, gb.Q4_K, ""), (8, 16, True, gb.Q4_K, "1"), (3, 16, True, gb.Q4_K, "0"),
                                                       (2, 8, True, gb.Q4_K, "0"), (8, 16, True, gb.Q6_K, ""), (3, 4, False, gb.IQ2_XXS, "")])

@@ -112,6 +112,9 @@ static int direct_tiles_per_wg(int64_t rows, int64_t groups, int col_tiles, int 
 // Small shape: a workgroup stages the decoder's tables and its row tile's LoRA rows once, so it walks up to four column
 // tiles while that still leaves every compute unit eight workgroups.
 static int small_tiles_per_wg(int64_t groups, int col_tiles) {
+#ifdef GGQ_X_PERWG
+    return GGQ_X_PERWG;
+#endif
     int per_wg = 4;
     while (per_wg > 1 && groups * ((col_tiles + per_wg - 1) / per_wg) < 2048) per_wg >>= 1;
     return per_wg;
@@ -125,7 +128,7 @@ int64_t ggq_lora_workspace_bytes(int64_t rows, int64_t groups, int64_t experts, 
     const int rp = rank_pad(r > 0 ? r : 1);
     if (experts < 1) experts = 1;
     const int64_t tiles = rows / 64 + groups + 2;
-    return 4 * align256(tiles * (int64_t)sizeof(TileDesc)) + align256(16) + align256(experts * 2 * 4) +
+    return 5 * align256(tiles * (int64_t)sizeof(TileDesc)) + align256(16) + align256(experts * 2 * 4) +
            align256(experts * n_total * rp * 2) * 2 + align256(experts * k * rp * 2) + align256(rows * rp * 2) + 4096 +
            (groups == 0 ? align256(kDenseFactorSplits * std::max(n_total, k) * rp * 4) : 0);
 }
@@ -301,14 +304,15 @@ static int grouped_forward(const char* what, const void* x, RowIndex x_index, co
         // IQ2_XXS: the groups of at most 128 rows leave the wide table for a launch of their own (decoding waves)
         const bool small = wide && qt == 16 /* GGML IQ2_XXS */ && direct_ok && g_shape_override != kShapeWide;
         t_small = small ? (TileDesc*)bump.take((int64_t)groups * sizeof(TileDesc)) : nullptr;
+        TileDesc* t_small_sorted = small ? (TileDesc*)bump.take((int64_t)groups * sizeof(TileDesc)) : nullptr;  // most row blocks first
         int* counts = (int*)bump.take(16);
-        if (!t128 || !counts || (lora_a && !t64) || (wide && !t_tall) || (direct && !t_sorted) || (small && !t_small)) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
+        if (!t128 || !counts || (lora_a && !t64) || (wide && !t_tall) || (direct && !t_sorted) || (small && (!t_small || !t_small_sorted))) return set_error(GGQ_ERR_WORKSPACE, "%s: workspace too small", what);
         RowTileTables tb{};
         tb.add(bm_main, small ? kSmallBM : 0, wide ? kWideBM : 0x7FFFFFFF, t128, counts, t_sorted);
         if (direct) t128 = t_sorted;
         if (wide) tb.add(kBM, kWideBM, 0x7FFFFFFF, t_tall, counts + 2), n_tall = counts + 2;
         if (lora_a) tb.add(64, 0, 0x7FFFFFFF, t64, counts + 1);
-        if (small) tb.add(kSmallBM, 0, kSmallBM, t_small, counts + 3), n_small = counts + 3;
+        if (small) tb.add(kSmallBM, 0, kSmallBM, t_small, counts + 3, t_small_sorted), n_small = counts + 3, t_small = t_small_sorted;
         if (int rc = build_row_tile_tables(expert_ids, end_offsets, (int)groups, tb, nullptr, 0, s)) return rc;
         p.expert_ids = expert_ids, p.tiles = t128, p.num_tiles = counts, p.max_row_tiles = small ? 0 : max128;  // (small: the wide table stays empty)
         tiles64 = t64, num_tiles64 = counts + 1;

@@ -122,8 +122,8 @@ struct SmallIq2 {
             issue_q(q[2], 2);
             issue_a(2, 2);
             issue_q(q[3], 3);
-            // Table reads run one group of 8 weights ahead of the MFMAs, over the step boundaries too: the selectors and sign
-            // words of the first group of step 0 are asked for here, once its run has landed.
+            // Table reads run two groups of 8 weights ahead of the MFMAs, over the step boundaries too: the selectors and sign
+            // words of the first two groups of step 0 are asked for here, once its run has landed.
             const uint4* const sel = (const uint4*)tables;
             const uint4* const flip = sel + 256;
             // (the registers a wait covers are operands of the wait itself: their readers cannot be moved ahead of it)
@@ -136,7 +136,12 @@ struct SmallIq2 {
                 asm volatile("v_mov_b32 %0, %2\n\tv_mov_b32 %1, %3" : "=&v"(cur_idx), "=&v"(cur_aux) : "v"(qr.x), "v"(qr.y));
             };
             take_run(q[0]);
-            uint4 e = sel[cur_idx & 0xFFu], f = flip[cur_aux & 127u];
+            uint4 e[2], f[2];  // selectors and sign words of the next two groups
+            auto ask = [&](int slot, int l) __attribute__((always_inline)) {
+                e[slot] = sel[(cur_idx >> (8 * l)) & 0xFFu], f[slot] = flip[(cur_aux >> (7 * l)) & 127u];
+            };
+            ask(0, 0);
+            ask(1, 1);
             for (int t0 = 0; t0 < steps; t0 += 4) {
                 auto step = [&](auto s_c) __attribute__((always_inline)) {
                     constexpr int S = decltype(s_c)::value;
@@ -159,24 +164,35 @@ struct SmallIq2 {
                     // the three products a weight can be, as bf16: bytes 0..5 of {hi : lo}
                     const uint32_t lo = pack_bf16(db * 8.0f, db * 25.0f), hi = pack_bf16(db * 43.0f, 0.0f);
                     const uint8_t* src = a_row + S * kStageBytes;
+                    // the step's scale leaves cur_aux here: group 2 below moves the next run's words in
+                    constexpr int kFirst = LIVE < 4 ? LIVE : 2;  // (four row blocks: the A operands come in two halves, for registers)
+                    constexpr bool kAhead = LIVE <= 2;           // (few row blocks: the A operands of a group are read during the group before)
+                    bf16x8_t a[kFirst], a_next[kFirst];
+                    if (kAhead) {
+#pragma unroll
+                        for (int rb = 0; rb < kFirst; rb++) a_next[rb] = *(const bf16x8_t*)(src + a_koff0 + rb * 32 * 128);
+                    }
 #pragma unroll
                     for (int l = 0; l < 4; l++) {
-                        constexpr int kFirst = LIVE < 4 ? LIVE : 2;  // (four row blocks: the A operands come in two halves, for registers)
-                        bf16x8_t a[kFirst];
+                        if (kAhead) {
 #pragma unroll
-                        for (int rb = 0; rb < kFirst; rb++) a[rb] = *(const bf16x8_t*)(src + (a_koff0 ^ (16 * l)) + rb * 32 * 128);
-                        uint4 e_next, f_next;
-                        if (l < 3) {
-                            e_next = sel[(cur_idx >> (8 * (l + 1))) & 0xFFu], f_next = flip[(cur_aux >> (7 * (l + 1))) & 127u];
+                            for (int rb = 0; rb < kFirst; rb++) a[rb] = a_next[rb];
+                            if (l < 3) {
+#pragma unroll
+                                for (int rb = 0; rb < kFirst; rb++) a_next[rb] = *(const bf16x8_t*)(src + (a_koff0 ^ (16 * (l + 1))) + rb * 32 * 128);
+                            }
                         } else {
-                            take_run(q[(S + 1) & 3]);
-                            e_next = sel[cur_idx & 0xFFu], f_next = flip[cur_aux & 127u];
+#pragma unroll
+                            for (int rb = 0; rb < kFirst; rb++) a[rb] = *(const bf16x8_t*)(src + (a_koff0 ^ (16 * l)) + rb * 32 * 128);
                         }
                         u32x4_t w;
-                        w[0] = __builtin_amdgcn_perm(hi, lo, e.x) ^ f.x;
-                        w[1] = __builtin_amdgcn_perm(hi, lo, e.y) ^ f.y;
-                        w[2] = __builtin_amdgcn_perm(hi, lo, e.z) ^ f.z;
-                        w[3] = __builtin_amdgcn_perm(hi, lo, e.w) ^ f.w;
+                        w[0] = __builtin_amdgcn_perm(hi, lo, e[l & 1].x) ^ f[l & 1].x;
+                        w[1] = __builtin_amdgcn_perm(hi, lo, e[l & 1].y) ^ f[l & 1].y;
+                        w[2] = __builtin_amdgcn_perm(hi, lo, e[l & 1].z) ^ f[l & 1].z;
+                        w[3] = __builtin_amdgcn_perm(hi, lo, e[l & 1].w) ^ f[l & 1].w;
+                        // the slot is free: the group two ahead, which from group 2 on belongs to the next step's run
+                        if (l == 2) take_run(q[(S + 1) & 3]);
+                        ask(l & 1, (l + 2) & 3);
                         const bf16x8_t b = __builtin_bit_cast(bf16x8_t, w);
 #pragma unroll
                         for (int rb = 0; rb < kFirst; rb++) acc[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, a[rb], acc[rb], 0, 0, 0);
@@ -187,7 +203,6 @@ struct SmallIq2 {
 #pragma unroll
                             for (int rb = 0; rb < 2; rb++) acc[rb + 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, a[rb], acc[rb + 2], 0, 0, 0);
                         }
-                        e = e_next, f = f_next;
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 };
@@ -196,7 +211,7 @@ struct SmallIq2 {
                 step(std::integral_constant<int, 2>{});
                 step(std::integral_constant<int, 3>{});
             }
-            asm volatile("" ::"v"(e.x), "v"(f.x));  // (the table reads past the last step)
+            asm volatile("" ::"v"(e[0].x), "v"(f[0].x), "v"(e[1].x), "v"(f[1].x));  // (the table reads past the last step)
             // every request has landed (the ones past the last step repeat it); every wave is done with the ring
             asm volatile("s_waitcnt vmcnt(0)" : "+v"(q[0]), "+v"(q[1]), "+v"(q[2]), "+v"(q[3]), "+v"(d_next) : : "memory");
             lds_barrier();
