@@ -50,10 +50,11 @@ int ggq_profile_end(float* ms, int* qt, int* mode, int* epilogue, int* shape, in
  * MFMA-bound ceiling.  Synchronous: allocates 256 bytes, times `iters` loop trips with HIP events on `stream` and waits. */
 int ggq_measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64_t elems, int iters, float* tflops_out, void* stream);
 
-/* Test aid with no counterpart in the reference: force the kernel family of the grouped Q4_K launches that follow (0 = tall
- * tiles, 1 = the wide / tall tile mix, 3 = the kernels whose MFMA waves decode the weights themselves, wherever their operand
- * conditions hold; -1 = the library's own choice, the default).  A process-wide setting, not thread safe; results are the
- * same to the stated tolerances whatever is chosen. */
+/* Test aid with no counterpart in the reference: force the kernel family of the grouped launches that follow (0 = tall
+ * tiles, 1 = the wide / tall tile mix and nothing else, 3 = the Q4_K kernels whose MFMA waves decode the weights themselves,
+ * 5 = the wide / tall mix with the IQ2_XXS forward of groups of up to 128 rows on its decoding-wave kernel, which is also what
+ * IQ2_XXS calls get by default, each wherever its operand conditions hold; -1 = the library's own choice, the default).  A
+ * process-wide setting, not thread safe; results are the same to the stated tolerances whatever is chosen. */
 int ggq_debug_force_grouped_shape(int shape);
 
 /* fast_lora.py:24-31 (_NATIVE_MMQ_QUANT_TYPES / supports_native_mmq): 1 if this library has kernels

@@ -161,10 +161,12 @@ def test_grouped_lora_projection_all_gradients(pkg, dev, qt, r, shape, n, force_
     ([5, 90], 8, 1024, 4, True),                                             # fewer columns than one wave owns; rank padded to 16
     ([128] * 3 + [1] * 5, 512, 256, 64, False),                              # rank 64
 ])
-def test_iq2xxs_forward_of_small_groups(pkg, dev, sizes, n, k, r, pair):
+@pytest.mark.parametrize("shape", ["", "1"])
+def test_iq2xxs_forward_of_small_groups(pkg, dev, sizes, n, k, r, pair, shape, force_grouped_shape):
     # IQ2_XXS groups of at most 128 rows run the forward kernel whose MFMA waves decode the packed bytes themselves
     # (mmq_small_iq2xxs_kernel); larger groups of the same call stay on the tile kernel.  Against the oracle, with and
-    # without LoRA, as a pair and as a single projection.
+    # without LoRA, as a pair and as a single projection.  Shape "1": the same calls on wide / tall tiles only.
+    force_grouped_shape(shape)
     ml = pkg.fast_moe_lora
     qt = gb.IQ2_XXS
     e_total, rows = len(sizes), sum(sizes)

@@ -112,9 +112,6 @@ static int direct_tiles_per_wg(int64_t rows, int64_t groups, int col_tiles, int 
 // Small shape: a workgroup stages the decoder's tables and its row tile's LoRA rows once, so it walks up to four column
 // tiles while that still leaves every compute unit eight workgroups.
 static int small_tiles_per_wg(int64_t groups, int col_tiles) {
-#ifdef GGQ_X_PERWG
-    return GGQ_X_PERWG;
-#endif
     int per_wg = 4;
     while (per_wg > 1 && groups * ((col_tiles + per_wg - 1) / per_wg) < 2048) per_wg >>= 1;
     return per_wg;
