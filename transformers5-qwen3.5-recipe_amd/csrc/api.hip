@@ -299,7 +299,8 @@ static int grouped_forward(const char* what, const void* x, RowIndex x_index, co
         t_tall = wide ? (TileDesc*)bump.take((int64_t)max_tall * sizeof(TileDesc)) : nullptr;
         TileDesc* t64 = lora_a ? (TileDesc*)bump.take((int64_t)max_tiles64 * sizeof(TileDesc)) : nullptr;
         // IQ2_XXS: the groups of at most 128 rows leave the wide table for a launch of their own (decoding waves)
-        const bool small = wide && qt == 16 /* GGML IQ2_XXS */ && direct_ok && g_shape_override != kShapeWide;
+        // (its lanes address a weight plane with 32-bit offsets)
+        const bool small = wide && qt == 16 /* GGML IQ2_XXS */ && direct_ok && p.w_expert_bytes < (1ll << 32) && g_shape_override != kShapeWide;
         t_small = small ? (TileDesc*)bump.take((int64_t)groups * sizeof(TileDesc)) : nullptr;
         TileDesc* t_small_sorted = small ? (TileDesc*)bump.take((int64_t)groups * sizeof(TileDesc)) : nullptr;  // most row blocks first
         int* counts = (int*)bump.take(16);
