@@ -9,9 +9,34 @@ import bench
 pytestmark = pytest.mark.gpu
 
 
-def test_expert_layer_step_replays_from_a_hip_graph(pkg, dev):
-    cfg = dict(bench.CFG, tokens=512, experts=32)
-    layer, x, idx, weights, dy = bench.build_workload(pkg, dev, cfg)
+def _iq2xxs_workload(pkg, dev, cfg):
+    """A small expert layer on IQ2_XXS weights: 64 rows per expert on average, so the forward launches run the kernel for
+    small groups and the grad-input launches wide tiles."""
+    g = torch.Generator(device=dev).manual_seed(4242)
+    e, h, i, r = cfg["experts"], cfg["hidden"], cfg["inter"], cfg["rank"]
+    G = pkg.gguf.GGUFQuantizedTensor
+    gate = G(pkg.gguf.random_iq2_xxs((e, i, h), g, dev), 16, (e, i, h))
+    up = G(pkg.gguf.random_iq2_xxs((e, i, h), g, dev), 16, (e, i, h))
+    down = G(pkg.gguf.random_iq2_xxs((e, h, i), g, dev), 16, (e, h, i))
+    layer = pkg.fast_moe_lora.FastGGUFMoeLora(pkg.fast_moe_lora.GGUFExperts(gate, up, down), r=r, lora_alpha=cfg["alpha"])
+    with torch.no_grad():
+        for name, p in layer.named_parameters():
+            p.copy_((torch.randn(p.shape, generator=g, device=dev) * (p.shape[-1] ** -0.5 if "lora_A" in name else 0.01)).to(p.dtype))
+    x = torch.randn(cfg["tokens"], h, generator=g, device=dev).to(torch.bfloat16).requires_grad_(True)
+    top = torch.topk(torch.randn(cfg["tokens"], e, generator=g, device=dev), cfg["top_k"], dim=-1)
+    weights = torch.softmax(top.values, dim=-1).requires_grad_(True)
+    dy = torch.randn(cfg["tokens"], h, generator=g, device=dev).to(torch.bfloat16)
+    return layer, x, top.indices.clone(), weights, dy
+
+
+@pytest.mark.parametrize("kind", ["q4k", "iq2xxs"])
+def test_expert_layer_step_replays_from_a_hip_graph(pkg, dev, kind):
+    if kind == "q4k":
+        cfg = dict(bench.CFG, tokens=512, experts=32)
+        layer, x, idx, weights, dy = bench.build_workload(pkg, dev, cfg)
+    else:
+        cfg = dict(bench.CFG, tokens=256, experts=16, hidden=512, inter=256, top_k=4)
+        layer, x, idx, weights, dy = _iq2xxs_workload(pkg, dev, cfg)
     params = list(layer.parameters())
     out_static = None
 
