@@ -10,16 +10,20 @@
 //   * the A tile (rows x 128 bytes) goes global -> LDS directly, three steps ahead, through a ring of four stages (one
 //     instruction per wave and 64 rows; rows unpadded with XOR-swizzled 16-byte slots, a_slot);
 //   * lane (column lane % 32, half h = lane / 32) loads the 8 bytes of run 2 step + h of its column's packed row, four
-//     steps ahead, into one of four register sets (and a block's scale one block ahead), decodes the run's 32 weights in registers
-//     (Fmt<kIQ2_XXS>::decode, selector and sign tables in LDS) and feeds group i of the run to MFMA i of the step: an MFMA
-//     sums its 16 contraction slots in any order, so the lane half reads the matching 16-byte slot (4 h + i) of the A row.
-//     No decoded weight touches LDS.
-// All requests of the loop are inline-asm loads the compiler does not track: two per wave and step and a third on the first
-// step of a block, in a fixed order, waited for with exact counts (vector memory operations complete in issue order).  The workgroup keeps 74 KB of LDS and
-// at most 128 registers per lane, so two workgroups share a compute unit and cover each other's barriers.
-// The weights are the MFMA's first operand, so a lane's accumulator registers hold four consecutive columns of one row; a
-// finished row block goes through a wave-private LDS block (in the ring, idle by then) and leaves as 64-byte row pieces, the
-// LoRA term added there.
+//     steps ahead, into one of four register sets (and a block's scale one block ahead), decodes the run's 32 weights in
+//     registers (the selector and sign tables of Fmt<kIQ2_XXS> in LDS, read two groups of 8 weights ahead of their use) and
+//     feeds group i of the run to MFMA i of the step: an MFMA sums its 16 contraction slots in any order, so the lane half
+//     reads the matching 16-byte slot (4 h + i) of the A row.  No decoded weight touches LDS.
+// All requests of the loop are inline-asm loads the compiler does not track: one per 64 rows and one run per wave and step,
+// and a scale on the first step of a block, in a fixed order, waited for with exact counts (vector memory operations
+// complete in issue order).  A register such a load writes must not be touched before its wait: the waits name the
+// registers they cover as operands, and a landed run moves to registers of its own through an instruction the compiler
+// cannot fold away, so that its register pair is dead until the next request names it (the compiler otherwise carries
+// the pair into the next loop iteration with a copy made while the load is still on its way).
+// The workgroup keeps 74 KB of LDS and at most 128 registers per lane, so two workgroups share a compute unit and cover
+// each other's barriers.  The weights are the MFMA's first operand, so a lane's accumulator registers hold four consecutive
+// columns of one row; a finished row block goes through a wave-private LDS block (in the ring, idle by then) and leaves as
+// 64-byte row pieces, the LoRA term added there.
 #pragma once
 #include "mmq_direct.h"
 
@@ -37,7 +41,7 @@ struct SmallIq2 {
     static constexpr int kLaBase = kTableBase + Fmt<kIQ2_XXS>::kTableWords * 4;     // + 6 KB: then the row tile's LA rows, 32 bytes each
     static constexpr int kLdsBytes = kLaBase + kTM * 32;                            // + 4 KB = 74 KB
     static constexpr int kOutBase = 0;  // eight 2 KB staging blocks of the epilogue: over the ring, which a finished tile no longer needs
-    
+
     using RowCtx = Direct::RowCtx;
 
     template <int LIVE>
