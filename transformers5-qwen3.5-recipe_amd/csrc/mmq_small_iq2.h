@@ -20,7 +20,7 @@
 // registers they cover as operands, and a landed run moves to registers of its own through an instruction the compiler
 // cannot fold away, so that its register pair is dead until the next request names it (the compiler otherwise carries
 // the pair into the next loop iteration with a copy made while the load is still on its way).
-// The workgroup keeps 74 KB of LDS and at most 128 registers per lane, so two workgroups share a compute unit and cover
+// The workgroup keeps 74 KB of LDS (68 KB dynamic, the tables static) and at most 128 registers per lane, so two workgroups share a compute unit and cover
 // each other's barriers.  The weights are the MFMA's first operand, so a lane's accumulator registers hold four consecutive
 // columns of one row; a finished row block goes through a wave-private LDS block (in the ring, idle by then) and leaves as
 // 64-byte row pieces, the LoRA term added there.
@@ -37,15 +37,15 @@ struct SmallIq2 {
     static constexpr int kWaves = 8;
     static constexpr int kThreadsWG = 64 * kWaves;
     static constexpr int kStageBytes = kTM * 128;                                   // 16 KB
-    static constexpr int kTableBase = kStages * kStageBytes;                        // 64 KB: then the decoder's tables
-    static constexpr int kLaBase = kTableBase + Fmt<kIQ2_XXS>::kTableWords * 4;     // + 6 KB: then the row tile's LA rows, 32 bytes each
-    static constexpr int kLdsBytes = kLaBase + kTM * 32;                            // + 4 KB = 74 KB
+    static constexpr int kLaBase = kStages * kStageBytes;                           // 64 KB: then the row tile's LA rows, 32 bytes each
+    static constexpr int kLdsBytes = kLaBase + kTM * 32;                            // + 4 KB = 68 KB of dynamic LDS
+    // (the decoder's tables, 6 KB, are a static array: it sits at LDS address 0, which the compiler then folds into the lookups)
     static constexpr int kOutBase = 0;  // eight 2 KB staging blocks of the epilogue: over the ring, which a finished tile no longer needs
 
     using RowCtx = Direct::RowCtx;
 
     template <int LIVE>
-    static __device__ __forceinline__ void work(const MmqParams& p, const RowCtx& c, int ct0, int ct1) {
+    static __device__ __forceinline__ void work(const MmqParams& p, const RowCtx& c, int ct0, int ct1, uint32_t* table_words) {
         extern __shared__ __attribute__((aligned(16))) uint8_t smem_raw[];
         const int tid = threadIdx.x, lane = tid & 63;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -53,11 +53,8 @@ struct SmallIq2 {
         const int steps = p.steps_per_seg;  // a multiple of 4: the contraction is a whole number of 256-wide blocks
         const int out_cols = p.n;
         const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem_raw;
-        {
-            uint32_t* words = (uint32_t*)(smem_raw + kTableBase);
-            for (int i = tid; i < Fmt<kIQ2_XXS>::kTableWords; i += kThreadsWG) words[i] = Fmt<kIQ2_XXS>::table_word(i, i < 1024 ? d_iq2xxs_grid_mm[i >> 2] : 0);
-        }
-        const uint2* const tables = (const uint2*)(smem_raw + kTableBase);
+        for (int i = tid; i < Fmt<kIQ2_XXS>::kTableWords; i += kThreadsWG) table_words[i] = Fmt<kIQ2_XXS>::table_word(i, i < 1024 ? d_iq2xxs_grid_mm[i >> 2] : 0);
+        const uint2* const tables = (const uint2*)table_words;
         // the row tile's LA rows stay in LDS for all the column tiles of this workgroup (ranks up to 16)
         const bool la_resident = p.r_pad == 16;
         if (la_resident) {
@@ -300,11 +297,13 @@ struct SmallIq2 {
         }
         c.rows_valid = row_end - c.row_begin;
         const int ct0 = chunk * p.col_tiles_per_wg, ct1 = min(col_tiles, ct0 + p.col_tiles_per_wg);
+        // the decoder's tables: the kernel's one static LDS array, so it sits at LDS address 0 and the lookups need no base
+        __shared__ __attribute__((aligned(16))) uint32_t table_words[Fmt<kIQ2_XXS>::kTableWords];
         switch ((c.rows_valid + 31) >> 5) {
-            case 1: work<1>(p, c, ct0, ct1); break;
-            case 2: work<2>(p, c, ct0, ct1); break;
-            case 3: work<3>(p, c, ct0, ct1); break;
-            default: work<4>(p, c, ct0, ct1); break;
+            case 1: work<1>(p, c, ct0, ct1, table_words); break;
+            case 2: work<2>(p, c, ct0, ct1, table_words); break;
+            case 3: work<3>(p, c, ct0, ct1, table_words); break;
+            default: work<4>(p, c, ct0, ct1, table_words); break;
         }
     }
 };
