@@ -37,8 +37,8 @@ const char* ggq_last_error(void);
  * between begin and end every launch of a packed-weight matmul kernel is bracketed by HIP events on
  * its stream.  ggq_profile_end synchronises on them and fills host arrays (milliseconds, GGML type id,
  * mode 0 = forward / 1 = grad-input, epilogue id 0 = store / 1 = fp32 accumulate, and - unless `shape` is NULL - the kernel
- * family: 0 = tall tiles, 1 = wide tiles, 3 = the kernels whose MFMA waves decode the weights, 4 = one launch of wide and
- * tall tiles) for up to `capacity` launches; returns the number written or a negative error.  Not thread safe; at most
+ * family: 0 = tall tiles, 1 = wide tiles, 3 = the Q4_K kernels whose MFMA waves decode the weights, 4 = one launch of wide and
+ * tall tiles, 5 = the IQ2_XXS forward of small groups) for up to `capacity` launches; returns the number written or a negative error.  Not thread safe; at most
  * 8192 launches are recorded. */
 int ggq_profile_begin(void);
 int ggq_profile_end(float* ms, int* qt, int* mode, int* epilogue, int* shape, int capacity);
