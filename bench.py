@@ -82,10 +82,11 @@ def device_ceilings(pkg, lib, dev, x_samples, w_samples):
     n = min(x_samples.numel(), w_samples.numel()) // 8 * 8
     a, b = x_samples.reshape(-1)[:n].contiguous(), w_samples.reshape(-1)[:n].contiguous()
     st = pkg._lib.stream_handle(dev)
-    if lib.ggq_measure_mfma_ceiling(a.data_ptr(), b.data_ptr(), n, 20000, ctypes.byref(tf), st) == 0:
+    sink = torch.zeros(64, dtype=torch.float32, device=dev)  # 256 bytes the measuring kernel may write
+    if lib.ggq_measure_mfma_ceiling(a.data_ptr(), b.data_ptr(), n, 20000, sink.data_ptr(), ctypes.byref(tf), st) == 0:
         out["mfma_bf16_tflops_workload_values"] = tf.value
     z = torch.zeros(n, dtype=torch.bfloat16, device=dev)
-    if lib.ggq_measure_mfma_ceiling(z.data_ptr(), z.data_ptr(), n, 20000, ctypes.byref(tf), st) == 0:
+    if lib.ggq_measure_mfma_ceiling(z.data_ptr(), z.data_ptr(), n, 20000, sink.data_ptr(), ctypes.byref(tf), st) == 0:
         out["mfma_bf16_tflops_zero_values"] = tf.value
     src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
     dst = torch.empty_like(src)
@@ -98,6 +99,55 @@ def device_ceilings(pkg, lib, dev, x_samples, w_samples):
     torch.cuda.synchronize()
     out["device_copy_gb_per_s"] = 5 * 2 * src.numel() / (e0.elapsed_time(e1) * 1e-3) / 1e9  # bytes read + bytes written
     return out
+
+def timed_tflops(fn, flops, iters=30):
+    for _ in range(3):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return flops * iters / (e0.elapsed_time(e1) * 1e-3) / 1e12
+
+
+def library_gemm_ceilings(pkg, dev, cfg, layer, x):
+    """What the framework's tuned dense bf16 GEMMs (hipBLASLt through torch.matmul / torch.bmm) reach on this box with the
+    workload's values and shapes, weights already DECODED to bf16: the share of the gap to the MFMA peak that belongs to the GEMM structure
+    (operands through LDS, tile edges, 128-row groups), as opposed to decoding packed weights and ragged grouping.
+    configs[2] as a batched product over equal groups of 128 rows (the packed-weight kernels see 128 +- 11 rows and decode
+    as they go); configs[1] as one dense product.  Not part of the timed step."""
+    out = {}
+    e, h, i = cfg["experts"], cfg["hidden"], cfg["inter"]
+    rows = cfg["tokens"] * cfg["top_k"] // e
+    with torch.no_grad():
+        base = layer.base_layer
+        w_gate = pkg.gguf.dequantize_gguf_tensor(base.gate_proj, 12, torch.bfloat16)  # [e, i, h]
+        w_up = pkg.gguf.dequantize_gguf_tensor(base.up_proj, 12, torch.bfloat16)
+        w_gu = torch.cat([w_gate, w_up], dim=1)  # [e, 2i, h]
+        del w_gate, w_up
+        w_down = pkg.gguf.dequantize_gguf_tensor(base.down_proj, 12, torch.bfloat16)  # [e, h, i]
+        xs = x.detach()[: e * rows // 8].repeat(8, 1).reshape(e, rows, h).contiguous()  # token rows, as the routed rows are
+        dgu = torch.randn(e, rows, 2 * i, device=dev, dtype=torch.bfloat16)
+        hs = torch.randn(e, rows, i, device=dev, dtype=torch.bfloat16)
+        dys = torch.randn(e, rows, h, device=dev, dtype=torch.bfloat16)
+        f_gu, f_d = 2.0 * e * rows * 2 * i * h, 2.0 * e * rows * h * i
+        out["bmm_gate_up_forward_tflops"] = timed_tflops(lambda: torch.bmm(xs, w_gu.transpose(1, 2)), f_gu)
+        out["bmm_gate_up_grad_input_tflops"] = timed_tflops(lambda: torch.bmm(dgu, w_gu), f_gu)
+        out["bmm_down_forward_tflops"] = timed_tflops(lambda: torch.bmm(hs, w_down.transpose(1, 2)), f_d)
+        out["bmm_down_grad_input_tflops"] = timed_tflops(lambda: torch.bmm(dys, w_down), f_d)
+        out["bmm_shapes"] = f"{e} groups x {rows} rows: [{rows}x{h}]x[{h}x{2 * i}] and [{rows}x{i}]x[{i}x{h}], forward (weights [n][k]) and grad-input"
+        # configs[1]: X [4096, 2048] x W [4096, 2048]^T and dY [4096, 4096] x W
+        wd = w_gu.reshape(-1, h)[:4096].contiguous()
+        xd = x.detach()[:4096].contiguous()
+        dyd = torch.randn(4096, 4096, device=dev, dtype=torch.bfloat16)
+        f = 2.0 * 4096 * 4096 * h
+        out["matmul_dense_forward_tflops"] = timed_tflops(lambda: torch.matmul(xd, wd.t()), f)
+        out["matmul_dense_grad_input_tflops"] = timed_tflops(lambda: torch.matmul(dyd, wd), f)
+        out["matmul_shapes"] = "configs[1]: [4096x2048]x[2048x4096] forward, [4096x4096]x[4096x2048] grad-input"
+    return out
+
 
 CFG = dict(tokens=4096, hidden=2048, inter=512, experts=256, top_k=8, rank=16, alpha=32.0)
 
@@ -395,6 +445,7 @@ def main() -> None:
     with torch.no_grad():
         w_samples = pkg.gguf.dequantize_gguf_tensor(layer.base_layer.gate_proj.as_subclass(torch.Tensor)[0].contiguous(), 12, torch.bfloat16)
     ceilings = device_ceilings(pkg, lib, dev, x.detach(), w_samples)
+    ceilings["library_bf16_gemm_on_decoded_weights"] = library_gemm_ceilings(pkg, dev, cfg, layer, x)
 
     result = {
         "metric": "fwd+bwd TFLOP/s and weight GB/s, Q4_K grouped-MoE LoRA; % of MI355X roofline",

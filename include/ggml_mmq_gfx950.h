@@ -47,14 +47,17 @@ int ggq_profile_end(float* ms, int* qt, int* mode, int* epilogue, int* shape, in
  * register-only loop of 32x32x16 MFMAs sustains on this device when its operands are drawn from the two device sample
  * buffers (`elems` bf16 values each, at least 4096, 16-byte aligned).  The device is power limited and its clock depends on
  * the operand values, so this - measured with a workload's own activations and decoded weights - is that workload's
- * MFMA-bound ceiling.  Synchronous: allocates 256 bytes, times `iters` loop trips with HIP events on `stream` and waits. */
-int ggq_measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64_t elems, int iters, float* tflops_out, void* stream);
+ * MFMA-bound ceiling.  `sink` is a device buffer of at least 256 bytes that the kernel may write (nothing is allocated
+ * here).  Synchronous: times `iters` loop trips with HIP events on `stream` and waits. */
+int ggq_measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64_t elems, int iters, void* sink, float* tflops_out, void* stream);
 
 /* Test aid with no counterpart in the reference: force the kernel family of the grouped launches that follow (0 = tall
  * tiles, 1 = the wide / tall tile mix and nothing else, 3 = the Q4_K kernels whose MFMA waves decode the weights themselves,
  * 5 = the wide / tall mix with the IQ2_XXS forward of groups of up to 128 rows on its decoding-wave kernel, which is also what
- * IQ2_XXS calls get by default, each wherever its operand conditions hold; -1 = the library's own choice, the default).  A
- * process-wide setting, not thread safe; results are the same to the stated tolerances whatever is chosen. */
+ * IQ2_XXS calls get by default, each wherever its operand conditions hold; -1 = the library's own choice, the default).
+ * FOR TESTS ONLY: a process-wide setting that stays until it is set back to -1 and changes the kernel choice of every later
+ * caller in the process; not thread safe (no launch may run in another thread while it changes); results are the same to
+ * the stated tolerances whatever is chosen. */
 int ggq_debug_force_grouped_shape(int shape);
 
 /* fast_lora.py:24-31 (_NATIVE_MMQ_QUANT_TYPES / supports_native_mmq): 1 if this library has kernels

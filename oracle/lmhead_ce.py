@@ -8,7 +8,7 @@ reduction "mean"; ignored rows give zero loss and zero gradient), then dHidden =
 (:172-177) and loss = sum of the per-row losses (:179).  Chunking does not change any value.
 ``n_non_ignore == 0`` divides by zero in the reference (:87,154); defined here as loss 0, grad 0.
 
-The textbook identity pins it: tests/test_oracle_ce.py compares with
+The textbook identity pins it: tests/test_oracle_lmhead.py compares with
 ``torch.nn.functional.cross_entropy(..., ignore_index, reduction)`` and its autograd.
 """
 

@@ -52,6 +52,20 @@ def test_route_plan_all_routes_to_one_expert_and_bad_ids(pkg, dev):
         pkg.fast_moe_routing.VALIDATE_EXPERT_IDS = False
 
 
+@pytest.mark.parametrize("bad_routes", [[300], [70 * 256 + 5], [256 * c + (c % 7) for c in range(1, 70)], [256 * 63 + 255], [20479]])
+def test_route_plan_reports_a_bad_id_in_any_chunk(pkg, dev, bad_routes):
+    """The flag must be raised wherever the id sits: the sort works in chunks of 256 routes whose flags one workgroup
+    gathers with a wave vote, so ids in chunks 1, 63, 70 and in every chunk of a run are tried, negative ones too."""
+    idx = _indices(86420, 2560, 8, 16).reshape(-1)
+    *_, status = pkg.fast_moe_routing.build_route_plan(idx.reshape(2560, 8).to(dev), 16)
+    assert int(status[1]) == 0
+    for n, r in enumerate(bad_routes):
+        idx[r] = 16 if n % 2 == 0 else -1
+    sorted_ids, *_, status = pkg.fast_moe_routing.build_route_plan(idx.reshape(2560, 8).to(dev), 16)
+    assert int(status[1]) == 1
+    assert int(sorted_ids.min()) >= 0 and int(sorted_ids.max()) < 16  # clamped: no access leaves the buffers
+
+
 @pytest.mark.parametrize("tokens,k,hidden", [(2048, 8, 2048), (257, 6, 4096), (8, 4, 2048), (64, 8, 4096), (5, 1, 256)])
 def test_gather_forward_backward_exact(pkg, dev, tokens, k, hidden):
     g = torch.Generator().manual_seed(2468)

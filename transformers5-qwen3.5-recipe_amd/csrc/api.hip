@@ -56,8 +56,8 @@ int ggq_profile_end(float* ms, int* qt, int* mode, int* epilogue, int* shape, in
     return profile_end(ms, qt, mode, epilogue, shape, capacity);
 }
 
-int ggq_measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64_t elems, int iters, float* tflops_out, void* stream) {
-    return measure_mfma_ceiling(a_samples, b_samples, elems, iters, tflops_out, as_stream(stream));
+int ggq_measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64_t elems, int iters, void* sink, float* tflops_out, void* stream) {
+    return measure_mfma_ceiling(a_samples, b_samples, elems, iters, sink, tflops_out, as_stream(stream));
 }
 
 int ggq_debug_force_grouped_shape(int shape) {

@@ -28,15 +28,14 @@ __global__ __launch_bounds__(512) void mfma_ceiling_kernel(const bf16_t* a_sampl
     if (s == 1.2345e-30f) sink[0] = s;  // keeps the loop alive without a store in practice
 }
 
-int measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64_t elems, int iters, float* tflops_out, hipStream_t s) {
-    if (!a_samples || !b_samples || !tflops_out) return set_error(GGQ_ERR_NULL, "measure_mfma_ceiling: null pointer");
+int measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64_t elems, int iters, void* sink_buffer, float* tflops_out, hipStream_t s) {
+    if (!a_samples || !b_samples || !tflops_out || !sink_buffer) return set_error(GGQ_ERR_NULL, "measure_mfma_ceiling: null pointer");
     if (elems < 4096 || iters < 1 || (((uintptr_t)a_samples | (uintptr_t)b_samples) & 15)) return set_error(GGQ_ERR_SHAPE, "measure_mfma_ceiling: needs at least 4096 aligned samples and iters >= 1");
     int device = 0, cus = 0;
     if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0)
         return set_error(GGQ_ERR_RUNTIME, "measure_mfma_ceiling: cannot query the device");
-    float* sink = nullptr;
+    float* sink = (float*)sink_buffer;  // the caller's: nothing is allocated here
     hipEvent_t e0, e1;
-    if (hipMalloc(&sink, 256) != hipSuccess) return set_error(GGQ_ERR_RUNTIME, "measure_mfma_ceiling: allocation failed");
     if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return set_error(GGQ_ERR_RUNTIME, "measure_mfma_ceiling: event creation failed");
     hipLaunchKernelGGL(mfma_ceiling_kernel, dim3(cus), dim3(512), 0, s, (const bf16_t*)a_samples, (const bf16_t*)b_samples, elems, 64, sink);  // warm-up
     (void)hipEventRecord(e0, s);
@@ -44,7 +43,7 @@ int measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64_t e
     (void)hipEventRecord(e1, s);
     float ms = 0.0f;
     const bool ok = hipEventSynchronize(e1) == hipSuccess && hipEventElapsedTime(&ms, e0, e1) == hipSuccess && ms > 0.0f;
-    (void)hipEventDestroy(e0), (void)hipEventDestroy(e1), (void)hipFree(sink);
+    (void)hipEventDestroy(e0), (void)hipEventDestroy(e1);
     if (!ok) return set_error(GGQ_ERR_RUNTIME, "measure_mfma_ceiling: timing failed");
     *tflops_out = (float)((double)cus * 8 /* waves */ * iters * 8 * 32768.0 / (ms * 1e-3) / 1e12);
     return check_launch("mfma_ceiling_kernel");

@@ -107,7 +107,7 @@ __device__ __forceinline__ int a_slot(int r, int kc) { return kc ^ ((r >> 1) & 7
 // lds + 16 * lane (lds is wave-uniform).  The data never passes through registers; the instruction
 // counts as one outstanding vector-memory load of the wave.
 __device__ __forceinline__ void load16_to_lds(uint32_t lds, uint32_t voff, const void* sbase) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(voff), "s"(sbase) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(voff), "s"(sbase) : "memory");
 }
 #endif
 

@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace ggq {
 
 enum : int {
@@ -17,6 +19,23 @@ enum : int {
 
 int set_error(int code, const char* fmt, ...);
 int check_launch(const char* what);
+
+// A kernel that needs more than 64 KB of dynamic LDS has that limit raised once per device (the attribute belongs to the
+// function as it is loaded on a device).  One static LdsLimit per kernel; any thread may call: the bit of a device is set
+// only after the attribute has been set there, and setting it twice is harmless.
+struct LdsLimit {
+    std::atomic<uint64_t> devices_done{0};
+};
+inline int raise_lds_limit(LdsLimit& state, const void* kernel, int bytes, const char* what) {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0) return set_error(GGQ_ERR_RUNTIME, "%s: no current device", what);
+    const uint64_t bit = device < 64 ? 1ull << device : 0;  // (devices past 63 set the attribute on every launch)
+    if (state.devices_done.load(std::memory_order_acquire) & bit) return GGQ_OK;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
+        return set_error(GGQ_ERR_RUNTIME, "%s: could not raise the dynamic LDS limit to %d bytes", what, bytes);
+    state.devices_done.fetch_or(bit, std::memory_order_release);
+    return GGQ_OK;
+}
 
 inline bool block_multiple(int qt, int64_t k) {
     switch (qt) {

@@ -514,12 +514,8 @@ int transpose_factor(const bf16_t* src, bf16_t* dst, int64_t experts, int c, int
 template <int JB, bool FNAT>
 static int launch_skinny_direct(const SkinnyNtParams& p, int grid_tiles, hipStream_t s) {
     constexpr int kSmem = 4 * 2 * (32 * 128 + JB * 16 * 128);
-    static bool attr_set = false;
-    if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)skinny_nt_direct_kernel<JB, FNAT>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmem) != hipSuccess)
-            return set_error(GGQ_ERR_RUNTIME, "skinny_nt: could not raise the dynamic LDS limit to %d bytes", kSmem);
-        attr_set = true;
-    }
+    static LdsLimit lds_limit;  // per instantiation
+    if (int rc = raise_lds_limit(lds_limit, (const void*)skinny_nt_direct_kernel<JB, FNAT>, kSmem, "skinny_nt")) return rc;
     hipLaunchKernelGGL((skinny_nt_direct_kernel<JB, FNAT>), dim3(((unsigned)grid_tiles + 7u) & ~7u), dim3(256), kSmem, s, p);
     return check_launch("skinny_nt_direct");
 }

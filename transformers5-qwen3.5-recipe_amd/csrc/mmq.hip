@@ -191,11 +191,8 @@ static int launch_one(const MmqParams& p, hipStream_t s) {
     }
     constexpr int kSmemBytes = Tile<SH>::kTileLdsBytes + (QT == kIQ2_XXS ? Fmt<kIQ2_XXS>::kTableWords * 4 : 0) +
                                (EPI != kEpiStore ? Tile<SH>::kTM * 16 : 0);
-    static bool attr_set = false;  // per instantiation; the attribute is a property of the function
-    if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)mmq_tile_kernel<QT, MODE, EPI, SH>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess) return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", kSmemBytes);
-        attr_set = true;
-    }
+    static LdsLimit lds_limit;  // per instantiation
+    if (int rc = raise_lds_limit(lds_limit, (const void*)mmq_tile_kernel<QT, MODE, EPI, SH>, kSmemBytes, "mmq")) return rc;
     hipLaunchKernelGGL((mmq_tile_kernel<QT, MODE, EPI, SH>), dim3((unsigned)grid), dim3(kThreads), kSmemBytes, s, p);
     if (t) (void)hipEventRecord(t->stop, s);
     return check_launch("mmq_tile_kernel");
@@ -223,12 +220,8 @@ static int launch_direct(const MmqParams& p, hipStream_t s) {
     }
     constexpr int kSmemBytes = MODE == kModeNT ? Direct8::kLdsBytes : Direct8NN::kLdsBytes;
     const void* fn = MODE == kModeNT ? (const void*)mmq_direct8_q4k_kernel : (const void*)mmq_direct8_nn_q4k_kernel;
-    static bool attr_set = false;  // per instantiation
-    if (!attr_set) {
-        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess)
-            return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", kSmemBytes);
-        attr_set = true;
-    }
+    static LdsLimit lds_limit;  // per instantiation
+    if (int rc = raise_lds_limit(lds_limit, fn, kSmemBytes, "mmq")) return rc;
     if (MODE == kModeNT) hipLaunchKernelGGL(mmq_direct8_q4k_kernel, dim3((unsigned)grid), dim3(Direct8::kThreadsWG), kSmemBytes, s, p);
     else hipLaunchKernelGGL(mmq_direct8_nn_q4k_kernel, dim3((unsigned)grid), dim3(Direct8NN::kThreadsWG), kSmemBytes, s, p);
     if (t) (void)hipEventRecord(t->stop, s);
@@ -254,12 +247,8 @@ static int launch_mixed_mode(const MmqParams& p, hipStream_t s) {
     }
     constexpr int kSmemBytes = (Tile<kShapeWide>::kTileLdsBytes > Tile<kShapeTall>::kTileLdsBytes ? Tile<kShapeWide>::kTileLdsBytes : Tile<kShapeTall>::kTileLdsBytes) +
                                (QT == kIQ2_XXS ? Fmt<kIQ2_XXS>::kTableWords * 4 : 0);
-    static bool attr_set = false;  // per instantiation
-    if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)mmq_mixed_kernel<QT, MODE, kEpiStore>, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes) != hipSuccess)
-            return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", kSmemBytes);
-        attr_set = true;
-    }
+    static LdsLimit lds_limit;  // per instantiation
+    if (int rc = raise_lds_limit(lds_limit, (const void*)mmq_mixed_kernel<QT, MODE, kEpiStore>, kSmemBytes, "mmq")) return rc;
     hipLaunchKernelGGL((mmq_mixed_kernel<QT, MODE, kEpiStore>), dim3((unsigned)grid), dim3(kThreads), kSmemBytes, s, p);
     if (t) (void)hipEventRecord(t->stop, s);
     return check_launch("mmq_mixed_kernel");
@@ -283,12 +272,8 @@ int launch_mmq_small(const MmqParams& p, hipStream_t s) {
         g_timed_count++;
         (void)hipEventRecord(t->start, s);
     }
-    static bool attr_set = false;
-    if (!attr_set) {
-        if (hipFuncSetAttribute((const void*)mmq_small_iq2xxs_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SmallIq2::kLdsBytes) != hipSuccess)
-            return set_error(GGQ_ERR_RUNTIME, "mmq: could not raise the dynamic LDS limit to %d bytes", SmallIq2::kLdsBytes);
-        attr_set = true;
-    }
+    static LdsLimit lds_limit;
+    if (int rc = raise_lds_limit(lds_limit, (const void*)mmq_small_iq2xxs_kernel, SmallIq2::kLdsBytes, "mmq")) return rc;
     hipLaunchKernelGGL(mmq_small_iq2xxs_kernel, dim3((unsigned)grid), dim3(SmallIq2::kThreadsWG), SmallIq2::kLdsBytes, s, p);
     if (t) (void)hipEventRecord(t->stop, s);
     return check_launch("mmq_small_iq2xxs_kernel");

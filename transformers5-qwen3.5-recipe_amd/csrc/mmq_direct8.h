@@ -99,9 +99,9 @@ struct Direct8 {
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 const int row = 16 * j + (lane >> 2), kc = (lane & 3) ^ ((row >> 1) & 3);
-                wq_voff[j] = (uint32_t)(min(32 * wave + row, out_cols - 1 - col0) * (int)p.w_row_bytes + 16 * kc);
+                wq_voff[j] = (uint32_t)min(32 * wave + row, out_cols - 1 - col0) * (uint32_t)p.w_row_bytes + 16u * kc;
             }
-            wh_voff = (uint32_t)(min(32 * wave + lane_c, out_cols - 1 - col0) * (int)p.w_row_bytes);
+            wh_voff = (uint32_t)min(32 * wave + lane_c, out_cols - 1 - col0) * (uint32_t)p.w_row_bytes;
         };
         w_cursor_rows();
         int w_wr = 0;  // byte offset (inside the wave's ring) of the buffer the next request fills
@@ -168,7 +168,7 @@ struct Direct8 {
         };
         auto request_a = [&](auto i_c) __attribute__((always_inline)) {
             constexpr int I = decltype(i_c)::value;
-            if (I < NI) load16_to_lds(ph_dst + I * 8192, a_voff[I], ph_src);
+            if constexpr (I < NI) load16_to_lds(ph_dst + I * 8192, a_voff[I], ph_src);
         };
         issue_w_half(std::integral_constant<int, 0>{});  // phase 0: the first half of block 1, A of step 3
         phase_open();
@@ -357,6 +357,7 @@ struct Direct8 {
             c.expert = 0;
         }
         c.rows_valid = row_end - c.row_begin;
+        if (c.rows_valid <= 0) return;  // (the table builders emit no empty tile; a descriptor that is one must not index row -1)
         const int ct0 = chunk * p.col_tiles_per_wg, ct1 = min(col_tiles, ct0 + p.col_tiles_per_wg);
         switch ((c.rows_valid + 31) >> 5) {
             case 1: work<1>(p, c, ct0, ct1); break;

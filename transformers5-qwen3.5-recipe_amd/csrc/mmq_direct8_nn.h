@@ -118,7 +118,7 @@ struct Direct8NN {
         };
         auto request_a = [&](auto i_c) __attribute__((always_inline)) {
             constexpr int I = decltype(i_c)::value;
-            if (I < NI) load16_to_lds(ph_dst + I * 8192, a_voff[I], ph_src);
+            if constexpr (I < NI) load16_to_lds(ph_dst + I * 8192, a_voff[I], ph_src);
         };
         auto request_w = [&]() __attribute__((always_inline)) {
             const uint8_t* src = step_src_w(w_tile_i, w_step_i);
@@ -407,6 +407,7 @@ struct Direct8NN {
             c.expert = 0;
         }
         c.rows_valid = row_end - c.row_begin;
+        if (c.rows_valid <= 0) return;  // (the table builders emit no empty tile; a descriptor that is one must not index row -1)
         const int ct0 = chunk * p.col_tiles_per_wg, ct1 = min(col_tiles, ct0 + p.col_tiles_per_wg);
         switch ((c.rows_valid + 31) >> 5) {
             case 1: work<1>(p, c, ct0, ct1); break;

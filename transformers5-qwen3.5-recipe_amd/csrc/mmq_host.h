@@ -116,7 +116,7 @@ struct MmqParams {
 constexpr int kMaxTimedLaunches = 8192;
 int profile_begin();
 int profile_end(float* ms, int* qt, int* mode, int* epi, int* shape, int capacity);
-int measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64_t elems, int iters, float* tflops_out, hipStream_t s);
+int measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64_t elems, int iters, void* sink_buffer, float* tflops_out, hipStream_t s);
 const char* last_error();
 int launch_mmq(int qt, int mode, int epi, const MmqParams& p, hipStream_t s);
 int launch_mmq_mixed(int qt, int mode, const MmqParams& p, hipStream_t s);  // Q4_K, store epilogue, tiles + tiles2

@@ -102,7 +102,7 @@ struct SmallIq2 {
             // packed row of this lane's column (columns past the end repeat the last one; their results are never stored):
             // run 2 step + h sits at block (step / 4) * 66 + 2 + 8 (2 (step % 4) + h), the block's scale at its first two bytes
             const uint8_t* const w_base = (seg ? p.w[1] : p.w[0]) + c.expert * p.w_expert_bytes;
-            const uint32_t wd_voff = (uint32_t)(min(col0 + 32 * wave + lane_c, out_cols - 1) * (int)p.w_row_bytes);
+            const uint32_t wd_voff = (uint32_t)min(col0 + 32 * wave + lane_c, out_cols - 1) * (uint32_t)p.w_row_bytes;  // (unsigned: a weight plane may pass 2 GiB)
             const uint32_t wq_voff = wd_voff + 2 + 8 * lane_h;
             dw_u32x2_t q[4];  // the runs of steps 4 b .. 4 b + 3, each reloaded for the next block as soon as it is decoded
             uint32_t d_cur = 0, d_next;  // the scales of this block and of the next
@@ -296,6 +296,7 @@ struct SmallIq2 {
             c.expert = 0;
         }
         c.rows_valid = row_end - c.row_begin;
+        if (c.rows_valid <= 0) return;  // (the table builders emit no empty tile; a descriptor that is one must not index row -1)
         const int ct0 = chunk * p.col_tiles_per_wg, ct1 = min(col_tiles, ct0 + p.col_tiles_per_wg);
         // the decoder's tables: the kernel's one static LDS array, so it sits at LDS address 0 and the lookups need no base
         __shared__ __attribute__((aligned(16))) uint32_t table_words[Fmt<kIQ2_XXS>::kTableWords];

@@ -180,7 +180,7 @@ static __device__ __forceinline__ void a_issue(const ALoader& a, const MmqParams
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                          :
                          : "s"(lds + j * (kCW * 1024)), "v"(a.voff[j]), "s"(sbase)
-                         : "memory", "m0");
+                         : "memory");
 }
 
 // Issue schedule shared by all waves of the consumer octet: steps 0 and 1 before the first barrier,

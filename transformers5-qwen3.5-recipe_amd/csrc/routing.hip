@@ -115,7 +115,8 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int* chunk_hist, int ch
     // (such ids are clamped so that no access leaves the buffers; the caller decides what to do).
     int bad = 0;
     for (int c = tid; c < chunks; c += 256) bad |= chunk_bad[c];
-    if (lane == 0) scan[wave] = __any(bad) ? 1 : 0;
+    const int wave_bad = __any(bad) ? 1 : 0;  // the vote is taken by all 64 lanes, outside any divergent branch
+    if (lane == 0) scan[wave] = wave_bad;
     __syncthreads();
     if (tid == 0) {
         num_active[0] = carry_active;
