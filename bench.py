@@ -280,32 +280,84 @@ def other_workload(name, pkg, lib, dev, args):
         def step():
             hs.grad = None
             pkg.gguf_liger_loss.packed_linear_cross_entropy(hs, payload, labels, 14, vocab, chunk).backward()
-    elif name == "moe_iq2xxs":  # configs[4], routed experts
-        tokens, hidden, inter, e, top_k, r = 2048, 4096, 2048, 256, 8, 16
+    elif name == "moe_iq2xxs":  # configs[4]: routed IQ2_XXS experts plus the shared Q8_0 expert
+        tokens, hidden, inter, e, top_k, r, s_lora = 2048, 4096, 2048, 256, 8, 16, 2.0
         G = pkg.gguf.GGUFQuantizedTensor
-        gate = G(pkg.gguf.random_iq2_xxs((e, inter, hidden), gd, dev), 16, (e, inter, hidden))
-        up = G(pkg.gguf.random_iq2_xxs((e, inter, hidden), gd, dev), 16, (e, inter, hidden))
-        down = G(pkg.gguf.random_iq2_xxs((e, hidden, inter), gd, dev), 16, (e, hidden, inter))
+
+        def quantized_experts(n_out, k_in):
+            # every expert drawn from N(0, 0.02^2) on the device (1.6 G weights per projection) and quantized there by the
+            # restatement of the oracle's IQ2_XXS quantizer (bit-checked against it in tests/test_gpu_dequant.py)
+            out = torch.empty(e, n_out, k_in // 256 * 66, dtype=torch.uint8, device=dev)
+            for j in range(e):
+                out[j] = pkg.gguf.quantize_iq2_xxs(torch.randn(n_out, k_in, generator=gd, device=dev) * 0.02)
+            return G(out, 16, (e, n_out, k_in))
+
+        gate, up, down = quantized_experts(inter, hidden), quantized_experts(inter, hidden), quantized_experts(hidden, inter)
         layer = pkg.fast_moe_lora.FastGGUFMoeLora(pkg.fast_moe_lora.GGUFExperts(gate, up, down), r=r, lora_alpha=32)
         with torch.no_grad():
             for pname, p in layer.named_parameters():
                 p.copy_(bf(*p.shape, std=p.shape[-1] ** -0.5 if "lora_A" in pname else 0.01))
+        # the shared expert: gate / up / down of the same shapes in Q8_0, a rank-16 LoRA on each, run as a SiLU FFN on every token
+        shared = {}
+        for pname, (n_out, k_in) in (("gate", (inter, hidden)), ("up", (inter, hidden)), ("down", (hidden, inter))):
+            shared[pname] = (pkg.gguf.quantize_q8_0(host_randn(g, n_out, k_in, std=0.02, device=dev)), n_out,
+                             bf(r, k_in, std=k_in ** -0.5).requires_grad_(True), bf(n_out, r, std=0.01).requires_grad_(True))
+        shared_params = [t for v in shared.values() for t in v[2:]]
+
+        def shared_ffn(h):
+            g_, u_ = (pkg.fast_lora.lora_mmq(h, shared[n][0], 8, shared[n][1], shared[n][2], shared[n][3], s_lora) for n in ("gate", "up"))
+            return pkg.fast_lora.lora_mmq(pkg.fast_moe_lora.swiglu(g_, u_), shared["down"][0], 8, hidden, shared["down"][2], shared["down"][3], s_lora)
+
         x = bf(tokens, hidden).requires_grad_(True)
         top = torch.topk(host_randn(g, tokens, e), top_k, dim=-1)
         idx, weights = top.indices.to(dev), torch.softmax(top.values, dim=-1).to(dev).requires_grad_(True)
         dy = bf(tokens, hidden)
         routes = tokens * top_k
-        flops = 2 * 2 * routes * (2 * inter * hidden + hidden * inter) + 3 * 2 * routes * r * ((hidden + 2 * inter) + (inter + hidden))
-        launch_flops, launches_per_step = 2 * routes * (2 * inter * hidden + hidden * inter) / 2, 4
-        workload = "configs[4] routed experts: grouped-MoE IQ2_XXS LoRA fwd+bwd, 2048 tokens x top-8, hidden 4096, 256 experts, gate_up [4096x4096], down [4096x2048], r=16 alpha=32"
-        metric = "fwd+bwd TFLOP/s, IQ2_XXS grouped-MoE LoRA"
+        per_row = 2 * inter * hidden + hidden * inter
+        lora_per_row = 3 * 2 * r * ((hidden + 2 * inter) + (inter + hidden))
+        flops_routed = 2 * 2 * routes * per_row + routes * lora_per_row
+        flops_shared = 2 * 2 * tokens * per_row + tokens * lora_per_row
+        flops = flops_routed + flops_shared
+        launch_flops, launches_per_step = None, None  # routed and shared launches differ; per-kernel figures are in `by_kernel_ms_per_step`
+        workload = ("configs[4]: grouped-MoE IQ2_XXS LoRA fwd+bwd, 2048 tokens x top-8, hidden 4096, 256 routed experts quantized from N(0, 0.02^2), gate_up [4096x4096], "
+                    "down [4096x2048], plus the shared Q8_0 expert of the same shapes on every token, r=16 alpha=32 on all projections")
+        metric = "fwd+bwd TFLOP/s, IQ2_XXS grouped-MoE LoRA with the shared Q8_0 expert"
         params = list(layer.parameters())
 
-        def step():
+        def step_routed():
             for p in params:
                 p.grad = None
             x.grad = weights.grad = None
             layer(x, idx, weights).backward(dy)
+
+        def step_shared():
+            for p in shared_params:
+                p.grad = None
+            x.grad = None
+            shared_ffn(x).backward(dy)
+
+        def step():
+            for p in params + shared_params:
+                p.grad = None
+            x.grad = weights.grad = None
+            (layer(x, idx, weights) + shared_ffn(x)).backward(dy)
+
+        def timed(fn, n):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / n * 1e3
+
+        extra = {"routed_experts_ms_per_step": timed(step_routed, args.steps), "shared_expert_ms_per_step": timed(step_shared, args.steps),
+                 "routed_experts_tflops": None, "shared_expert_tflops": None}
+        # algorithmic flops of a direction's packed-weight launches per step, by the block format in the launch record
+        extra["_direction_flops"] = {"IQ2_XXS": 2 * routes * per_row, "Q8_0": 2 * tokens * per_row}
+        extra["routed_experts_tflops"] = flops_routed / (extra["routed_experts_ms_per_step"] * 1e-3) / 1e12
+        extra["shared_expert_tflops"] = flops_shared / (extra["shared_expert_ms_per_step"] * 1e-3) / 1e12
     elif name == "moe_q4k_separated":  # configs[2] through the reference's own order: base launches + separate grouped LoRA products
         cfg = CFG
         layer, x, idx, weights, dy = build_workload(pkg, dev, cfg)
@@ -326,6 +378,7 @@ def other_workload(name, pkg, lib, dev, args):
     else:
         sys.exit(f"unknown workload {name!r}")
 
+    extra = locals().get("extra", {})
     for _ in range(max(args.warmup, 1)):
         step()
     torch.cuda.synchronize()
@@ -346,6 +399,19 @@ def other_workload(name, pkg, lib, dev, args):
     for nm, t in launches:
         by_kernel.setdefault(nm, []).append(t)
     roofline = None
+    direction_flops = extra.pop("_direction_flops", None)
+    if direction_flops and by_kernel:
+        # per kernel: the direction's algorithmic flops over the time its launches take per step; `roofline` = the dominant one
+        fracs = {}
+        for nm, ts in by_kernel.items():
+            fl_dir = next((v for k, v in direction_flops.items() if f"{k}," in nm), None)
+            if fl_dir and sum(ts) / prof_steps > 0.1:  # (a launch whose tile table came out empty on the device is no measurement)
+                fracs[nm] = fl_dir / (sum(ts) / prof_steps * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS
+        extra["kernel_frac_of_mfma_peak"] = fracs
+        dominant = max(by_kernel, key=lambda k: sum(by_kernel[k]))
+        if dominant in fracs:
+            roofline = {"bound": "mfma", "kernel": dominant, "achieved": fracs[dominant] * MFMA_BF16_PEAK_TFLOPS, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                        "frac": fracs[dominant], "traffic": None, "avg_launch_ms": sum(by_kernel[dominant]) / len(by_kernel[dominant]), "launches_timed": len(by_kernel[dominant])}
     if launch_flops is not None and n_l:
         avg_ms = tile_ms / launches_per_step
         achieved = launch_flops / (avg_ms * 1e-3) / 1e12
@@ -354,7 +420,8 @@ def other_workload(name, pkg, lib, dev, args):
     print(json.dumps({
         "metric": metric, "value": flops / (ms_per_step * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": workload, "launch": "eager"}, "roofline": roofline, "tile_kernel_ms_per_step": tile_ms, "tile_kernel_launches_per_step": n_l / prof_steps}))
+        "config": {"workload": workload, "launch": "eager"}, "roofline": roofline, "tile_kernel_ms_per_step": tile_ms, "tile_kernel_launches_per_step": n_l / prof_steps,
+        "by_kernel_ms_per_step": {k: sum(v) / prof_steps for k, v in by_kernel.items()}, **extra}))
 
 
 def main() -> None:

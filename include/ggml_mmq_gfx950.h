@@ -51,6 +51,14 @@ int ggq_profile_end(float* ms, int* qt, int* mode, int* epilogue, int* shape, in
  * here).  Synchronous: times `iters` loop trips with HIP events on `stream` and waits. */
 int ggq_measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64_t elems, int iters, void* sink, float* tflops_out, void* stream);
 
+/* Tuning switch with no counterpart in the reference.  A grouped backward call that returns factor gradients enqueues
+ * its grad-input launch on the caller's stream and the dA / dB launches on a stream of the library's own (one per device,
+ * default priority, created on the first such call outside a stream capture), forked behind the rank-sized product they
+ * read and joined back before the call returns: to the caller the call stays one ordered piece of work on `stream`, under
+ * stream capture the fork and join become graph edges, and the results are bit-identical either way.  0 keeps every launch
+ * on the caller's stream; 1 (the default) forks.  Process-wide. */
+int ggq_set_factor_gradient_overlap(int enabled);
+
 /* Test aid with no counterpart in the reference: force the kernel family of the grouped launches that follow (0 = tall
  * tiles, 1 = the wide / tall tile mix and nothing else, 3 = the Q4_K kernels whose MFMA waves decode the weights themselves,
  * 5 = the wide / tall mix with the IQ2_XXS forward of groups of up to 128 rows on its decoding-wave kernel, which is also what

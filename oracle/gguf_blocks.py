@@ -416,10 +416,15 @@ def _q_iq2_xxs(x: np.ndarray) -> np.ndarray:
     neg = neg ^ flip
     with np.errstate(divide="ignore", invalid="ignore"):
         t = np.where(db[:, :, None, None] > 0, mag / db[:, :, None, None], 0).astype(np.float32)
-    grid = _GRID_BYTES.astype(np.float32)                   # [256,8]
-    # nearest codebook point: argmin |t|^2 - 2 t.g + |g|^2
-    score = (grid * grid).sum(axis=1)[None, :] - 2.0 * t.reshape(-1, 8) @ grid.T
-    idx = score.argmin(axis=1).astype(np.uint8).reshape(nb, 8, 4)
+    grid = _GRID_BYTES.astype(np.float64)                   # [256,8]
+    # nearest codebook point: argmin |t|^2 - 2 t.g + |g|^2, in double precision (so that a restatement whose products are
+    # summed in another order picks the same point), a million groups at a time
+    norms = (grid * grid).sum(axis=1)[None, :]
+    tt = t.reshape(-1, 8)
+    idx = np.empty(tt.shape[0], dtype=np.uint8)
+    for lo in range(0, tt.shape[0], 1 << 20):
+        idx[lo:lo + (1 << 20)] = (norms - 2.0 * (tt[lo:lo + (1 << 20)].astype(np.float64) @ grid.T)).argmin(axis=1)
+    idx = idx.reshape(nb, 8, 4)
     sign7 = (neg[..., 0:7].astype(np.uint32) << np.arange(7, dtype=np.uint32)).sum(axis=3)   # [nb,8,4]
     aux1 = (ls << 28) | (sign7 << (7 * np.arange(4, dtype=np.uint32))).sum(axis=2).astype(np.uint32)
     out = np.empty((nb, 66), dtype=np.uint8)

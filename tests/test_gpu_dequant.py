@@ -39,6 +39,24 @@ def test_dequantize_expert_stack_and_constant_payload(pkg, dev):
     assert np.array_equal(bf16_bits(got), gb.to_bf16_bits(gb.dequantize(payload, gb.IQ2_XXS)))
 
 
+def test_device_iq2_xxs_quantizer_matches_the_oracle_quantizer_bit_for_bit(pkg, dev):
+    """The torch quantizer that manufactures BASELINE's "N(0, 0.02^2), then quantized" IQ2_XXS experts on the device against
+    the oracle's, on the same fp32 weights: identical bytes (scale codes, codebook indices, sign bits), including blocks
+    with an all-zero group, an all-zero block and a group whose minus signs are odd in number."""
+    rng = np.random.default_rng(20260817)
+    w = (rng.standard_normal((512, 4096)) * 0.02).astype(np.float32)
+    w[0, :256] = 0.0          # a whole block of zeros
+    w[1, 32:64] = 0.0         # one group of zeros
+    w[2, :8] = np.abs(w[2, :8]) * np.array([-1, 1, 1, 1, 1, 1, 1, 1], dtype=np.float32)  # one minus sign: the weakest weight flips
+    w[3] *= 40.0              # large values
+    want = gb.quantize(w, gb.IQ2_XXS)
+    got = pkg.gguf.quantize_iq2_xxs(torch.from_numpy(w).to(dev), chunk_groups=1000)
+    assert got.dtype == torch.uint8 and tuple(got.shape) == want.shape
+    assert np.array_equal(got.cpu().numpy(), want)
+    # and the table it reads back through the decoder is the oracle's codebook
+    assert np.array_equal(pkg.gguf._iq2xxs_grid(dev).cpu().numpy(), gb._GRID_BYTES.astype(np.float64))
+
+
 def test_dequantize_rejects_bad_operands(pkg, dev):
     p = torch.zeros(4, 144, dtype=torch.uint8, device=dev)
     with pytest.raises(ValueError):

@@ -308,7 +308,8 @@ def test_iq2_xxs_experts_quantized_from_gaussian_weights_and_the_shared_ffn_at_f
         for name, (n_out, k_in) in (("gate", (inter, hidden)), ("up", (inter, hidden)), ("down", (hidden, inter))):
             w = (rng.standard_normal((n_out, k_in)) * 0.02).astype(np.float32)
             packed = gb.quantize(w, gb.IQ2_XXS)
-            payloads[name][e] = torch.from_numpy(packed).to(dev)
+            payloads[name][e] = pkg.gguf.quantize_iq2_xxs(torch.from_numpy(w).to(dev))  # the device quantizer the bench uses ...
+            assert np.array_equal(payloads[name][e].cpu().numpy(), packed), f"device IQ2_XXS quantizer differs from the oracle's on {name}[{e}]"  # ... is the oracle's, bit for bit
             oracle_decoded[(name, e)] = gb.dequantize_bf16(packed, gb.IQ2_XXS)
     gate, up, down = (G(payloads[n], 16, shape) for n, shape in (("gate", (e_total, inter, hidden)), ("up", (e_total, inter, hidden)),
                                                                   ("down", (e_total, hidden, inter))))
@@ -346,23 +347,75 @@ def test_iq2_xxs_experts_quantized_from_gaussian_weights_and_the_shared_ffn_at_f
     a, b = layer.lora_A["default"].weight.detach(), layer.lora_B["default"].weight.detach()
     ad, bd = layer.lora_A_down["default"].weight.detach(), layer.lora_B_down["default"].weight.detach()
     sel = plan.selected_hidden_states
-    y1, y2 = ml.grouped_lora_mmq_pair(sel, gate, up, ids, plan.expert_end_offsets, 16, inter, a, b, s)
-    act = ml.swiglu(y1, y2)
-    yd = ml.grouped_lora_mmq(act, down, ids, plan.expert_end_offsets, 16, hidden, ad, bd, s)
-    dyd = torch.randn(sel.shape[0], hidden, generator=gen).to(torch.bfloat16).to(dev)
+    rows = sel.shape[0]
+
+    def leaf(t):
+        return t.detach().clone().requires_grad_(True)
+
+    al, bl, adl, bdl = leaf(a), leaf(b), leaf(ad), leaf(bd)
+    sel_l = leaf(sel)
+    dy1 = torch.randn(rows, inter, generator=gen).to(torch.bfloat16).to(dev)
+    dy2 = torch.randn(rows, inter, generator=gen).to(torch.bfloat16).to(dev)
+    y1, y2 = ml.grouped_lora_mmq_pair(sel_l, gate, up, ids, plan.expert_end_offsets, 16, inter, al, bl, s)
+    torch.autograd.backward((y1, y2), (dy1, dy2))
+    act = leaf(ml.swiglu(y1.detach(), y2.detach()))
+    yd = ml.grouped_lora_mmq(act, down, ids, plan.expert_end_offsets, 16, hidden, adl, bdl, s)
+    dyd = torch.randn(rows, hidden, generator=gen).to(torch.bfloat16).to(dev)
+    yd.backward(dyd)
     dact = ml.grouped_mmq_grad_input(dyd, down, ids, plan.expert_end_offsets, 16, inter)
     ends = plan.expert_end_offsets.cpu().tolist()
+    f = lambda t: t.detach().float()
     for e in quantized:
         r0, r1 = _expert_rows(ends, e)
         assert r1 > r0
         wg, wu, wd = (torch.from_numpy(oracle_decoded[(n, e)]).to(dev) for n in ("gate", "up", "down"))
-        xe = sel[r0:r1].float()
-        xa = _bf16(xe @ a[e].float().T)
-        assert_close_bf16(y1[r0:r1], (xe @ wg.T + s * (xa @ b[e, :inter].float().T)).double(), f"gate of quantized expert {e}")
-        assert_close_bf16(y2[r0:r1], (xe @ wu.T + s * (xa @ b[e, inter:].float().T)).double(), f"up of quantized expert {e}")
-        ae = act[r0:r1].float()
-        assert_close_bf16(yd[r0:r1], (ae @ wd.T + s * (_bf16(ae @ ad[e].float().T) @ bd[e].float().T)).double(), f"down of quantized expert {e}")
-        assert_close_bf16(dact[r0:r1], (dyd[r0:r1].float() @ wd).double(), f"down dX of quantized expert {e}")
+        xe, d1, d2 = f(sel[r0:r1]), f(dy1[r0:r1]), f(dy2[r0:r1])
+        xa = _bf16(xe @ f(a[e]).T)
+        assert_close_bf16(y1[r0:r1], (xe @ wg.T + s * (xa @ f(b[e, :inter]).T)).double(), f"gate of quantized expert {e}")
+        assert_close_bf16(y2[r0:r1], (xe @ wu.T + s * (xa @ f(b[e, inter:]).T)).double(), f"up of quantized expert {e}")
+        # gate/up input gradient WITH the LoRA term, and the factor gradients of the pair
+        dyb = _bf16(d1 @ f(b[e, :inter]) + d2 @ f(b[e, inter:]))
+        assert_close_bf16(sel_l.grad[r0:r1], (d1 @ wg + d2 @ wu + s * (dyb @ f(a[e]))).double(), f"gate/up dX of quantized expert {e}")
+        assert_close_bf16(al.grad[e], (s * (dyb.T @ xe)).double(), f"gate/up dA of quantized expert {e}")
+        assert_close_bf16(bl.grad[e], (s * (torch.cat([d1, d2], dim=1).T @ xa)).double(), f"gate/up dB of quantized expert {e}")
+        # down: forward, input gradient with and without the LoRA term, factor gradients
+        ae, dd = f(act[r0:r1]), f(dyd[r0:r1])
+        xad = _bf16(ae @ f(ad[e]).T)
+        dybd = _bf16(dd @ f(bd[e]))
+        assert_close_bf16(yd[r0:r1], (ae @ wd.T + s * (xad @ f(bd[e]).T)).double(), f"down of quantized expert {e}")
+        assert_close_bf16(act.grad[r0:r1], (dd @ wd + s * (dybd @ f(ad[e]))).double(), f"down dX (with LoRA) of quantized expert {e}")
+        assert_close_bf16(dact[r0:r1], (dd @ wd).double(), f"down dX of quantized expert {e}")
+        assert_close_bf16(adl.grad[e], (s * (dybd.T @ ae)).double(), f"down dA of quantized expert {e}")
+        assert_close_bf16(bdl.grad[e], (s * (dd.T @ xad)).double(), f"down dB of quantized expert {e}")
+    # dHidden of the launch that reads the tokens in place, for tokens routed to a quantized expert: every route's dX
+    # rounded to bf16 (the quantized experts on the ORACLE's decode), then the token's eight routes added up
+    xr = leaf(x)
+    z1, z2 = ml._RoutedGroupedLoraProjection.apply(xr, plan.permutation, plan.inverse_permutation, top_k, gate.as_subclass(torch.Tensor),
+                                                   up.as_subclass(torch.Tensor), ids, plan.expert_end_offsets, 16, inter, a, b, s)
+    assert torch.equal(z1, y1) and torch.equal(z2, y2)
+    torch.autograd.backward((z1, z2), (dy1, dy2))
+    inverse = plan.inverse_permutation.cpu().reshape(-1, top_k)
+    idx_rows = idx.cpu()
+
+    def decoded(name, t, e):
+        if (name, e) in oracle_decoded:
+            return torch.from_numpy(oracle_decoded[(name, e)]).to(dev)
+        return pkg.gguf.dequantize_gguf_tensor(t[e:e + 1], 16, torch.bfloat16)[0].float()
+
+    for q in quantized:
+        t = int((idx_rows == q).any(dim=1).nonzero()[0])
+        want = torch.zeros(hidden, dtype=torch.float64, device=dev)
+        magnitude = torch.zeros(hidden, dtype=torch.float64, device=dev)
+        for k in range(top_k):
+            row, e = int(inverse[t, k]), int(idx_rows[t, k])
+            d1, d2 = dy1[row].float(), dy2[row].float()
+            dyb = _bf16(d1 @ f(b[e, :inter]) + d2 @ f(b[e, inter:]))
+            term = _bf16(d1 @ decoded("gate", gate, e) + d2 @ decoded("up", up, e) + s * (dyb @ f(a[e]))).double()
+            want += term
+            magnitude += term.abs()
+        err = (xr.grad[t].double() - want).abs()
+        assert bool((err <= (top_k + 1) * 2.0 ** -9 * magnitude + 1e-6).all()), f"dHidden of token {t}"
+        assert max_rel(xr.grad[t], want) <= 2e-2
 
     # the whole block on sampled tokens (one of them routed to a quantized expert), every stage rounded to bf16 where the
     # path stores bf16

@@ -29,8 +29,42 @@ def _iq2xxs_workload(pkg, dev, cfg):
     return layer, x, top.indices.clone(), weights, dy
 
 
+@pytest.fixture
+def factor_gradient_overlap(pkg):
+    """Sets the library's switch for one test and puts the default (forked factor gradients) back."""
+    lib = pkg._lib.load()
+    yield lambda on: pkg._lib.check(lib.ggq_set_factor_gradient_overlap(int(on)))
+    lib.ggq_set_factor_gradient_overlap(1)
+
+
+def test_forked_factor_gradients_give_the_bits_of_the_single_stream_order(pkg, dev, factor_gradient_overlap):
+    """The backward calls put dA / dB on the library's side stream (forked and joined inside the call); the results must
+    not depend on it, eagerly and back to back (the second step reuses the workspace the first one's side work read)."""
+    cfg = dict(bench.CFG, tokens=512, experts=32)
+    layer, x, idx, weights, dy = bench.build_workload(pkg, dev, cfg)
+    params = list(layer.parameters())
+    results = {}
+    for on in (1, 0, 1):
+        factor_gradient_overlap(on)
+        for _ in range(3):
+            for p in params:
+                p.grad = None
+            x.grad = weights.grad = None
+            out = layer(x, idx, weights)
+            out.backward(dy)
+        torch.cuda.synchronize()
+        got = [out.detach().clone(), x.grad.clone(), weights.grad.clone()] + [p.grad.clone() for p in params]
+        if on in results:
+            assert all(torch.equal(a, b) for a, b in zip(got, results[on]))
+        results[on] = got
+    assert all(torch.equal(a, b) for a, b in zip(results[0], results[1]))
+    assert all(float(p.grad.float().abs().sum()) > 0 for p in params)
+
+
+@pytest.mark.parametrize("overlap", [1, 0])
 @pytest.mark.parametrize("kind", ["q4k", "iq2xxs"])
-def test_expert_layer_step_replays_from_a_hip_graph(pkg, dev, kind):
+def test_expert_layer_step_replays_from_a_hip_graph(pkg, dev, kind, overlap, factor_gradient_overlap):
+    factor_gradient_overlap(overlap)  # 1: the capture holds the fork and join of the factor gradients as graph edges
     if kind == "q4k":
         cfg = dict(bench.CFG, tokens=512, experts=32)
         layer, x, idx, weights, dy = bench.build_workload(pkg, dev, cfg)

@@ -23,6 +23,7 @@ SIGNATURES: dict[str, tuple] = {
     "ggq_last_error": (c_char_p, []),
     "ggq_profile_begin": (_I, []),
     "ggq_profile_end": (_I, [_P, _P, _P, _P, _P, _I]),
+    "ggq_set_factor_gradient_overlap": (_I, [_I]),
     "ggq_measure_mfma_ceiling": (_I, [_P, _P, _L, _I, _P, _P, _P]),
     "ggq_debug_force_grouped_shape": (_I, [_I]),
     "ggq_supports_quant_type": (_I, [_I]),

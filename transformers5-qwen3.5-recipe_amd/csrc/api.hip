@@ -3,6 +3,7 @@
 #include "../../include/ggml_mmq_gfx950.h"
 
 #include <algorithm>
+#include <mutex>
 
 #include "launch.h"
 #include "mmq_host.h"
@@ -28,6 +29,72 @@ struct Bump {  // carve 256-byte aligned pieces out of the caller's workspace
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 int g_shape_override = -1;  // ggq_debug_force_grouped_shape: -1 = the automatic choice
+
+// ---------------------------------------------------------------------------------------------------
+// The factor gradients dA / dB of a backward call depend on nothing the grad-input launch writes, are HBM-bound and
+// small, while the grad-input launch is MFMA-bound and leaves compute units idle at its tail: they run on a second
+// stream of the library's own, forked from the caller's stream behind the rank-sized product they read and joined back
+// into it before the call returns, so that to the caller the call is still one ordered piece of work on its stream.
+// Under stream capture the fork and the join become graph edges.  One side stream and event pair per device (default
+// priority); the lock is held while a call enqueues its forked section, so calls from several threads do not mix their
+// event records.  A stream that is being captured when the side stream does not exist yet runs the call unforked
+// (nothing is created during a capture).
+std::atomic<int> g_overlap_enabled{1};
+constexpr int kMaxDevices = 64;
+struct SideStream {
+    hipStream_t stream = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
+    bool tried = false;
+};
+SideStream g_side[kMaxDevices];
+std::mutex g_side_lock;
+
+class Forked {  // fork on construction (when allowed), join in done() or on destruction
+public:
+    explicit Forked(hipStream_t main_stream) : main_(main_stream), lock_(g_side_lock, std::defer_lock) {
+        if (!g_overlap_enabled.load(std::memory_order_relaxed)) return;
+        int device = -1;
+        if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return;
+        lock_.lock();
+        SideStream& st = g_side[device];
+        if (!st.stream) {
+            hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+            if (st.tried || hipStreamIsCapturing(main_, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+                (void)hipGetLastError();
+                lock_.unlock();
+                return;
+            }
+            st.tried = true;
+            if (hipStreamCreateWithFlags(&st.stream, hipStreamNonBlocking) != hipSuccess || hipEventCreateWithFlags(&st.fork, hipEventDisableTiming) != hipSuccess ||
+                hipEventCreateWithFlags(&st.join, hipEventDisableTiming) != hipSuccess) {
+                (void)hipGetLastError();
+                st.stream = nullptr;
+                lock_.unlock();
+                return;
+            }
+        }
+        if (hipEventRecord(st.fork, main_) != hipSuccess || hipStreamWaitEvent(st.stream, st.fork, 0) != hipSuccess) {
+            (void)hipGetLastError();
+            lock_.unlock();
+            return;
+        }
+        side_ = &st;
+    }
+    hipStream_t stream() const { return side_ ? side_->stream : main_; }  // the forked stream, or the caller's own
+    int done() {
+        if (!side_) return GGQ_OK;
+        const bool ok = hipEventRecord(side_->join, side_->stream) == hipSuccess && hipStreamWaitEvent(main_, side_->join, 0) == hipSuccess;
+        side_ = nullptr;
+        lock_.unlock();
+        return ok ? GGQ_OK : set_error(GGQ_ERR_RUNTIME, "could not join the library's side stream");
+    }
+    ~Forked() { (void)done(); }
+
+private:
+    hipStream_t main_;
+    std::unique_lock<std::mutex> lock_;
+    SideStream* side_ = nullptr;
+};
 
 int check_weights(const char* what, int qt, const void* w, int64_t k) {
     if (!w) return set_error(GGQ_ERR_NULL, "%s: packed weight pointer is null", what);
@@ -63,6 +130,11 @@ int ggq_measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64
 int ggq_debug_force_grouped_shape(int shape) {
     if (shape != -1 && shape != kShapeTall && shape != kShapeWide && shape != kShapeDirect && shape != kShapeSmall) return set_error(GGQ_ERR_SHAPE, "debug_force_grouped_shape: unknown shape %d", shape);
     g_shape_override = shape;
+    return GGQ_OK;
+}
+
+int ggq_set_factor_gradient_overlap(int enabled) {
+    g_overlap_enabled.store(enabled ? 1 : 0, std::memory_order_relaxed);
     return GGQ_OK;
 }
 
@@ -459,13 +531,21 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
             if (int rc = skinny_nt(sp, rp, max_tiles64, s)) return rc;
         }
         p.la = dyb, p.lb = (const bf16_t*)lora_a, p.lb_expert_elems = (int64_t)r * k, p.r_pad = rp, p.lora_rank = r, p.lora_scale = scale;
-        float* partials = nullptr;
-        int64_t partials_bytes = 0;
-        if (groups == 0 && (d_lora_a || d_lora_b)) {  // optional: without it the rows are not split
-            partials_bytes = kDenseFactorSplits * std::max<int64_t>(ntot, k) * rp * 4;
-            partials = (float*)bump.take(partials_bytes);
-            if (!partials) partials_bytes = 0;
-        }
+    }
+    auto grad_input = [&]() -> int {
+        if (rows == 0) return GGQ_OK;
+        if (t_tall) return launch_wide_and_tall(qt, kModeNN, p, (int)rows, (int)n, (int)k, nseg, t_tall, n_tall, max_tall, s);
+        return launch_mmq(qt, kModeNN, kEpiStore, p, s);
+    };
+    if (!lora_a || !(d_lora_a || d_lora_b)) return grad_input();
+    float* partials = nullptr;
+    int64_t partials_bytes = 0;
+    if (groups == 0) {  // optional: without it the rows are not split
+        partials_bytes = kDenseFactorSplits * std::max<int64_t>(ntot, k) * rp * 4;
+        partials = (float*)bump.take(partials_bytes);
+        if (!partials) partials_bytes = 0;
+    }
+    auto factor_gradients = [&](hipStream_t fs) -> int {
         if (d_lora_b) {
             FactorGradParams fp{};
             fp.partials = partials, fp.partials_bytes = partials_bytes;
@@ -473,21 +553,31 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
             fp.s = (const bf16_t*)xa, fp.out = (bf16_t*)d_lora_b, fp.out_expert_elems = ntot * r;
             fp.s_weights = row_weights, fp.s_weight_index = dy_index.row_index, fp.s_weights_are_bf16 = row_weights_are_bf16;
             fp.ranges = ranges, fp.m = (int)rows, fp.c = (int)n, fp.r = r, fp.nseg = nseg, fp.out_j_major = 0, fp.scale = scale;
-            if (int rc = factor_grad(fp, rp, experts, s)) return rc;
+            if (int rc = factor_grad(fp, rp, experts, fs)) return rc;
         }
         if (d_lora_a) {
             FactorGradParams fp{};
             fp.partials = partials, fp.partials_bytes = partials_bytes;
             fp.in[0] = (const bf16_t*)x, fp.ld_in = k, fp.in_rows = x_index;
-            fp.s = dyb, fp.out = (bf16_t*)d_lora_a, fp.out_expert_elems = (int64_t)r * k;
+            fp.s = (const bf16_t*)p.la, fp.out = (bf16_t*)d_lora_a, fp.out_expert_elems = (int64_t)r * k;
             fp.s_weights = row_weights, fp.s_weight_index = dy_index.row_index, fp.s_weights_are_bf16 = row_weights_are_bf16;
             fp.ranges = ranges, fp.m = (int)rows, fp.c = (int)k, fp.r = r, fp.nseg = 1, fp.out_j_major = 1, fp.scale = scale;
-            if (int rc = factor_grad(fp, rp, experts, s)) return rc;
+            if (int rc = factor_grad(fp, rp, experts, fs)) return rc;
+        }
+        return GGQ_OK;
+    };
+    if (rows > 0 && groups > 0) {
+        // Expert groups: the grad-input launch goes out first, on the caller's stream, and the factor gradients on the
+        // forked one (they read dy, x, xa and dy . B, all complete at the fork point, and write only dA / dB).
+        Forked side(s);
+        if (side.stream() != s) {
+            if (int rc = grad_input()) return rc;
+            if (int rc = factor_gradients(side.stream())) return rc;
+            return side.done();
         }
     }
-    if (rows == 0) return GGQ_OK;
-    if (t_tall) return launch_wide_and_tall(qt, kModeNN, p, (int)rows, (int)n, (int)k, nseg, t_tall, n_tall, max_tall, s);
-    return launch_mmq(qt, kModeNN, kEpiStore, p, s);
+    if (int rc = factor_gradients(s)) return rc;
+    return grad_input();
 }
 
 int ggq_grouped_lora_mmq_backward(const void* dy1, const void* dy2, const void* packed1, const void* packed2,

@@ -155,6 +155,65 @@ def quantize_q6_k(w: torch.Tensor) -> torch.Tensor:
     return out.reshape(*lead, k // 256 * 210)
 
 
+_IQ2XXS_GRID: dict = {}
+
+
+def _iq2xxs_grid(device) -> torch.Tensor:
+    """The 256 codebook points of IQ2_XXS as ``[256, 8]`` float64 magnitudes, read back through the library's own decoder
+    (eight crafted blocks: block scale 1, group scale code 1, all signs plus, codebook indices 0..255), so that the
+    quantizer below and the kernels cannot disagree about the table."""
+    key = str(device)
+    if key not in _IQ2XXS_GRID:
+        blocks = torch.zeros(8, 66, dtype=torch.uint8)
+        blocks[:, 0:2] = torch.tensor([0x00, 0x3C], dtype=torch.uint8)  # d = 1.0 in half precision
+        body = blocks[:, 2:].reshape(8, 8, 8)
+        body[:, :, 0:4] = torch.arange(256, dtype=torch.int64).reshape(8, 8, 4).to(torch.uint8)
+        body[:, :, 7] = 1 << 4  # bits 28..31 of the second word: scale code 1 -> db = 1 * (0.5 + 1) * 0.25
+        decoded = dequantize_gguf_tensor(blocks.to(device), IQ2_XXS, torch.float32)  # [8, 256]
+        _IQ2XXS_GRID[key] = (decoded.double() / 0.375).reshape(256, 8)
+    return _IQ2XXS_GRID[key]
+
+
+def quantize_iq2_xxs(w: torch.Tensor, chunk_groups: int = 1 << 20) -> torch.Tensor:
+    """IQ2_XXS payload of ``w [..., K]`` on the device the library runs on: per 32 weights a 4-bit scale code against the
+    block's half-precision scale, per 8 weights the nearest codebook point of the magnitudes and seven sign bits (the
+    weakest weight changes sign where the number of minus signs would be odd).  A nearest-point fit, not ggml's
+    importance-weighted search; it manufactures BASELINE's "drawn from N(0, 0.02^2) and quantized" weights."""
+    lead, k = w.shape[:-1], w.shape[-1]
+    if k % 256:
+        raise ValueError(f"last dimension {k} is not a multiple of 256")
+    grid = _iq2xxs_grid(w.device)
+    x = w.float().reshape(-1, 8, 32)
+    nb = x.shape[0]
+    # (divided by a device tensor: a division by a host scalar is carried out as a multiplication by its reciprocal on the
+    # device, which is not the correctly rounded quotient the format's reference arithmetic takes)
+    db_want = x.abs().amax(dim=2) / torch.full((), 33.0, dtype=torch.float32, device=w.device)
+    d = (db_want.amax(dim=1, keepdim=True) * (4.0 / 15.5)).to(torch.float16).float()
+    ls = torch.where(d > 0, (_roundf(db_want * 4 / torch.where(d > 0, d, torch.ones_like(d)) - 0.5)).clamp(0, 15), torch.zeros_like(db_want))
+    db = d * (0.5 + ls) * 0.25
+    v = x.reshape(nb, 8, 4, 8)
+    neg = v < 0
+    mag = v.abs()
+    odd = (neg.sum(dim=3) & 1).bool()
+    flip = torch.zeros_like(neg).scatter_(3, mag.argmin(dim=3, keepdim=True), odd.unsqueeze(3))
+    neg = neg ^ flip
+    dbx = db[:, :, None, None]
+    t = torch.where(dbx > 0, mag / torch.where(dbx > 0, dbx, torch.ones_like(dbx)), torch.zeros_like(mag)).reshape(-1, 8)
+    norms = (grid * grid).sum(dim=1)[None, :]
+    idx = torch.empty(t.shape[0], dtype=torch.int64, device=w.device)
+    for lo in range(0, t.shape[0], chunk_groups):  # the nearest codebook point: argmin |g|^2 - 2 t.g, in double precision
+        idx[lo:lo + chunk_groups] = (norms - 2.0 * (t[lo:lo + chunk_groups].double() @ grid.T)).argmin(dim=1)
+    sign7 = (neg[..., 0:7].to(torch.int64) << torch.arange(7, device=w.device)).sum(dim=3)  # [nb, 8, 4]
+    aux = (ls.to(torch.int64) << 28) | (sign7 << (7 * torch.arange(4, device=w.device))).sum(dim=2)  # [nb, 8]
+    out = torch.empty(nb, 66, dtype=torch.uint8, device=w.device)
+    out[:, 0:2] = _f16_bytes(d).reshape(-1, 2)
+    body = out[:, 2:].reshape(nb, 8, 8)
+    body[:, :, 0:4] = idx.reshape(nb, 8, 4).to(torch.uint8)
+    for byte in range(4):
+        body[:, :, 4 + byte] = ((aux >> (8 * byte)) & 0xFF).to(torch.uint8)
+    return out.reshape(*lead, k // 256 * 66)
+
+
 def random_iq2_xxs(shape, generator: torch.Generator | None = None, device="cpu", std: float = 0.02) -> torch.Tensor:
     """Random IQ2_XXS payload for a logical ``[..., K]`` tensor: every byte pattern is a valid block
     (any codebook index, sign pattern and 4-bit scale); the half-precision block scale is set so that
@@ -171,7 +230,7 @@ def random_iq2_xxs(shape, generator: torch.Generator | None = None, device="cpu"
 
 
 def quantize(w: torch.Tensor, quant_type: int) -> torch.Tensor:
-    fn = {Q8_0: quantize_q8_0, Q4_K: quantize_q4_k, Q6_K: quantize_q6_k}.get(int(quant_type))
+    fn = {Q8_0: quantize_q8_0, Q4_K: quantize_q4_k, Q6_K: quantize_q6_k, IQ2_XXS: quantize_iq2_xxs}.get(int(quant_type))
     if fn is None:
         raise ValueError(f"no synthetic quantizer for GGML type id {quant_type}")
     elems = GGML_QUANT_SIZES[int(quant_type)][0]
