@@ -170,13 +170,14 @@ static int pick_shape(int qt, int64_t rows, int64_t groups, bool direct_ok) {
     return kShapeWide;
 }
 
-// Direct shape: a workgroup walks a run of column tiles of its row tile as one stream of steps.  Short tiles (few
-// contraction steps) gain from runs of four (the next tile's first loads are in flight while a tile finishes); with
-// long tiles one tile per workgroup balances the compute units better (the tiles with the most rows are dispatched
-// first).  Fewer per run while that leaves compute units without work.
-static int direct_tiles_per_wg(int64_t rows, int64_t groups, int col_tiles, int steps_per_tile) {
+// Direct shape: a workgroup walks a run of column tiles of its row tile as one stream of steps, so that only the run's
+// first tile waits for its first loads.  Measured on configs[2] by alternating captured steps on one box: tiles of 32
+// steps and more want runs of two (one tile per workgroup is 0.9 % of the step slower per such launch, four 0.4 %
+// slower still); shorter tiles want runs of four in the forward launch (two and eight are both slower) and of eight in
+// the grad-input launch (four: + 0.4 %, two: + 1.3 %).  Fewer per run while that leaves compute units without work.
+static int direct_tiles_per_wg(int64_t rows, int64_t groups, int col_tiles, int steps_per_tile, int mode) {
     const int64_t row_tiles = groups > 0 ? std::max<int64_t>(groups, rows / kDirectBM) : (rows + kDirectBM - 1) / kDirectBM;
-    int per_wg = steps_per_tile >= 32 ? 1 : 4;
+    int per_wg = steps_per_tile >= 32 ? 2 : mode == kModeNN ? 8 : 4;
     while (per_wg > 1 && row_tiles * ((col_tiles + per_wg - 1) / per_wg) < 256) per_wg >>= 1;
     return per_wg;
 }
@@ -341,7 +342,7 @@ static int grouped_forward(const char* what, const void* x, RowIndex x_index, co
     p.a[0] = (const bf16_t*)x, p.lda = k, p.a_rows = x_index;
     p.w[0] = (const uint8_t*)packed1, p.w[1] = (const uint8_t*)packed2;
     p.c[0] = y1, p.c[1] = y2, p.ldc = n;
-    if (p.shape == kShapeDirect) p.col_tiles_per_wg = direct_tiles_per_wg(rows, groups, nseg * p.col_tiles_per_seg, p.steps_per_seg);
+    if (p.shape == kShapeDirect) p.col_tiles_per_wg = direct_tiles_per_wg(rows, groups, nseg * p.col_tiles_per_seg, p.steps_per_seg, kModeNT);
 
     const TileDesc* tiles64 = nullptr;
     const int* num_tiles64 = nullptr;
@@ -472,7 +473,7 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
     p.a[0] = (const bf16_t*)dy1, p.a[1] = (const bf16_t*)dy2, p.lda = n, p.a_rows = dy_index;
     p.w[0] = (const uint8_t*)packed1, p.w[1] = (const uint8_t*)packed2;
     p.c[0] = dx, p.ldc = k;
-    if (p.shape == kShapeDirect) p.col_tiles_per_wg = direct_tiles_per_wg(rows, groups, p.col_tiles_per_seg, nseg * p.steps_per_seg);
+    if (p.shape == kShapeDirect) p.col_tiles_per_wg = direct_tiles_per_wg(rows, groups, p.col_tiles_per_seg, nseg * p.steps_per_seg, kModeNN);
 
     const TileDesc* tiles64 = nullptr;
     const int* num_tiles64 = nullptr;
