@@ -52,6 +52,48 @@ __global__ __launch_bounds__(kChunk) void route_rank_kernel(const IdT* ids, int6
     }
 }
 
+// Pass 1 for up to kWaveRankMaxExperts experts, in chunks of 1024 routes: the lanes of a wave that hold the same id find
+// each other through one ballot per id bit (rank inside the wave = equal ids in lower lanes), the first of them leaves the
+// wave's count in LDS, and a route's rank inside the chunk adds the counts of the waves before its own.  Same outputs as
+// route_rank_kernel with four times fewer chunks for the scan pass to walk.
+constexpr int kWaveChunk = 1024;
+constexpr int kWaveRankMaxExperts = 1024;
+template <typename IdT>
+__global__ __launch_bounds__(kWaveChunk) void route_rank_wave_kernel(const IdT* ids, int64_t routes, int num_experts, int id_bits,
+                                                                      int* local_rank, int* chunk_hist, int* chunk_bad) {
+    extern __shared__ int wave_hist[];  // [16 waves][num_experts]
+    __shared__ int any_bad;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int i = tid; i < 16 * num_experts; i += kWaveChunk) wave_hist[i] = 0;
+    if (tid == 0) any_bad = 0;
+    __syncthreads();
+    const int64_t i = (int64_t)blockIdx.x * kWaveChunk + tid;
+    int bad = 0;
+    const int my = i < routes ? load_id(ids, i, num_experts, &bad) : -1;  // (-1 has bit id_bits set: it matches no id)
+    unsigned long long same = ~0ull;
+    for (int b = 0; b <= id_bits; b++) {
+        const int bit = (my >> b) & 1;
+        const unsigned long long set = __ballot(bit);
+        same &= bit ? set : ~set;
+    }
+    const int rank = __popcll(same & ((1ull << lane) - 1ull));
+    if (my >= 0 && rank == 0) wave_hist[wave * num_experts + my] = __popcll(same);
+    if (bad) any_bad = 1;  // benign race: every writer stores 1
+    __syncthreads();
+    if (i < routes) {
+        int before = 0;
+        for (int w = 0; w < wave; w++) before += wave_hist[w * num_experts + my];
+        local_rank[i] = before + rank;
+    }
+    for (int e = tid; e < num_experts; e += kWaveChunk) {
+        int c = 0;
+#pragma unroll
+        for (int w = 0; w < 16; w++) c += wave_hist[w * num_experts + e];
+        chunk_hist[(int64_t)blockIdx.x * num_experts + e] = c;
+    }
+    if (tid == 0) chunk_bad[blockIdx.x] = any_bad;
+}
+
 // Pass 2 (one workgroup): turn chunk histograms into chunk bases, expert counts, cumulative end
 // offsets and the compact list of active experts.
 __global__ __launch_bounds__(256) void route_scan_kernel(int* chunk_hist, int chunks, int num_experts, int* counts,
@@ -131,16 +173,98 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int* chunk_hist, int ch
 
 // Pass 3: scatter.
 template <typename IdT>
-__global__ __launch_bounds__(kChunk) void route_scatter_kernel(const IdT* ids, int64_t routes, int num_experts,
-                                                               const int* local_rank, const int* chunk_base,
-                                                               const int* expert_base, int64_t* sorted_ids,
-                                                               int64_t* permutation, int64_t* inverse) {
-    const int64_t i = (int64_t)blockIdx.x * kChunk + threadIdx.x;
+__global__ __launch_bounds__(kWaveChunk) void route_scatter_kernel(const IdT* ids, int64_t routes, int num_experts,
+                                                                   const int* local_rank, const int* chunk_base,
+                                                                   const int* expert_base, int64_t* sorted_ids,
+                                                                   int64_t* permutation, int64_t* inverse) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // a workgroup is one chunk of the rank pass
     if (i >= routes) return;
     int bad = 0;
     const int e = load_id(ids, i, num_experts, &bad);
     const int64_t pos = (int64_t)expert_base[e] + chunk_base[(int64_t)blockIdx.x * num_experts + e] + local_rank[i];
     sorted_ids[pos] = e;
+    permutation[pos] = i;
+    inverse[i] = pos;
+}
+
+// Passes 2 and 3 in one launch for the chunks of route_rank_wave_kernel (num_experts <= 1024 = one thread per expert):
+// every workgroup sums the chunk histograms itself (one batch of loads per 64 chunks; the table is a few dozen KB and
+// stays in L2) into the experts' totals and its own chunk's bases, scans the totals over the experts, and scatters its
+// chunk; workgroup 0 also writes the counts, end offsets, active list and status words.  One dependent launch fewer than
+// scan-then-scatter, and the scan no longer runs on a single compute unit while the others wait.
+template <typename IdT>
+__global__ __launch_bounds__(kWaveChunk) void route_scan_scatter_wave_kernel(const IdT* ids, int64_t routes, int num_experts, int chunks,
+                                                                              const int* local_rank, const int* chunk_hist, const int* chunk_bad,
+                                                                              int* counts, int* end_offsets, int64_t* active_ids, int* active_end,
+                                                                              int* num_active, int64_t* sorted_ids, int64_t* permutation, int64_t* inverse) {
+    __shared__ int base[kWaveRankMaxExperts];      // first sorted position of the expert, plus this chunk's base inside it
+    __shared__ int wave_totals[2][16];
+    __shared__ int any_bad;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int e = tid;
+    int total = 0, before_chunk = 0;
+    if (e < num_experts) {
+        for (int c0 = 0; c0 < chunks; c0 += 64) {
+            int v[64];
+#pragma unroll
+            for (int i = 0; i < 64; i++) v[i] = c0 + i < chunks ? chunk_hist[(int64_t)(c0 + i) * num_experts + e] : 0;
+#pragma unroll
+            for (int i = 0; i < 64; i++) {
+                if (c0 + i < (int)blockIdx.x) before_chunk += v[i];
+                total += v[i];
+            }
+        }
+    }
+    if (tid == 0) any_bad = 0;
+    // inclusive scans over the experts (rows, and active flags for the compact list): shuffles inside a wave, wave totals through LDS
+    const int active = total > 0 ? 1 : 0;
+    int rows_incl = total, act_incl = active;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int ur = __shfl_up(rows_incl, off, 64), ua = __shfl_up(act_incl, off, 64);
+        if (lane >= off) rows_incl += ur, act_incl += ua;
+    }
+    if (lane == 63) wave_totals[0][wave] = rows_incl, wave_totals[1][wave] = act_incl;
+    __syncthreads();
+    int rows_before = 0, act_before = 0, all_rows = 0, all_active = 0;
+#pragma unroll
+    for (int w = 0; w < 16; w++) {
+        const int tr = wave_totals[0][w], ta = wave_totals[1][w];
+        if (w < wave) rows_before += tr, act_before += ta;
+        all_rows += tr, all_active += ta;
+    }
+    const int end = rows_before + rows_incl;
+    if (e < num_experts) base[e] = end - total + before_chunk;
+    if (blockIdx.x == 0) {
+        if (e < num_experts) {
+            counts[e] = total;
+            end_offsets[e] = end;
+            if (active) {
+                const int slot = act_before + act_incl - 1;
+                active_ids[slot] = e;
+                active_end[slot] = end;
+            }
+        }
+        int bad = 0;
+        for (int c = tid; c < chunks; c += kWaveChunk) bad |= chunk_bad[c];
+        if (bad) any_bad = 1;  // benign race: every writer stores 1
+        // unused tail of the compact lists: repeat the total so that "offsets" stay monotone
+        for (int sl = all_active + tid; sl < num_experts; sl += kWaveChunk) {
+            active_ids[sl] = 0;
+            active_end[sl] = all_rows;
+        }
+    }
+    __syncthreads();
+    if (blockIdx.x == 0 && tid == 0) {
+        num_active[0] = all_active;
+        num_active[1] = any_bad;
+    }
+    const int64_t i = (int64_t)blockIdx.x * kWaveChunk + tid;
+    if (i >= routes) return;
+    int bad = 0;
+    const int id = load_id(ids, i, num_experts, &bad);
+    const int64_t pos = (int64_t)base[id] + local_rank[i];
+    sorted_ids[pos] = id;
     permutation[pos] = i;
     inverse[i] = pos;
 }
@@ -157,23 +281,45 @@ int route_plan(const void* topk_ids, int ids_are_int64, int64_t tokens, int top_
     if (tokens < 0 || top_k <= 0 || num_experts <= 0) return set_error(GGQ_ERR_SHAPE, "route_plan: bad shape");
     if (routes >= (int64_t)1 << 31) return set_error(GGQ_ERR_SHAPE, "route_plan: more than 2^31 routes");
     if (ws_bytes < route_plan_workspace_bytes(routes, num_experts)) return set_error(GGQ_ERR_WORKSPACE, "route_plan: workspace too small");
-    const int chunks = (int)((routes + kChunk - 1) / kChunk);
+    // chunks of 1024 routes ranked by wave ballots when the per-wave counts fit in LDS, else chunks of 256 ranked by comparison
+    const bool by_wave = num_experts <= kWaveRankMaxExperts;
+    const int chunk = by_wave ? kWaveChunk : kChunk;
+    const int chunks = (int)((routes + chunk - 1) / chunk);
     int* local_rank = (int*)ws;
     int* chunk_hist = local_rank + routes;
     int* expert_base = chunk_hist + (int64_t)chunks * num_experts;
     int* chunk_bad = expert_base + num_experts;
-    if (chunks > 0) {
+    if (chunks > 0 && by_wave) {
+        int id_bits = 0;
+        while ((1 << id_bits) < num_experts) id_bits++;
+        const int lds = 16 * num_experts * (int)sizeof(int);
+        static LdsLimit lim64, lim32;
+        if (int rc = raise_lds_limit(ids_are_int64 ? lim64 : lim32, ids_are_int64 ? (const void*)route_rank_wave_kernel<int64_t> : (const void*)route_rank_wave_kernel<int32_t>, lds, "route_plan")) return rc;
+        if (ids_are_int64)
+            hipLaunchKernelGGL(route_rank_wave_kernel<int64_t>, dim3(chunks), dim3(kWaveChunk), lds, s, (const int64_t*)topk_ids, routes, num_experts, id_bits, local_rank, chunk_hist, chunk_bad);
+        else
+            hipLaunchKernelGGL(route_rank_wave_kernel<int32_t>, dim3(chunks), dim3(kWaveChunk), lds, s, (const int32_t*)topk_ids, routes, num_experts, id_bits, local_rank, chunk_hist, chunk_bad);
+    } else if (chunks > 0) {
         if (ids_are_int64)
             hipLaunchKernelGGL(route_rank_kernel<int64_t>, dim3(chunks), dim3(kChunk), 0, s, (const int64_t*)topk_ids, routes, num_experts, local_rank, chunk_hist, chunk_bad);
         else
             hipLaunchKernelGGL(route_rank_kernel<int32_t>, dim3(chunks), dim3(kChunk), 0, s, (const int32_t*)topk_ids, routes, num_experts, local_rank, chunk_hist, chunk_bad);
     }
+    if (chunks > 0 && by_wave) {
+        if (ids_are_int64)
+            hipLaunchKernelGGL(route_scan_scatter_wave_kernel<int64_t>, dim3(chunks), dim3(kWaveChunk), 0, s, (const int64_t*)topk_ids, routes, num_experts, chunks, local_rank,
+                               chunk_hist, chunk_bad, counts, end_offsets, active_ids, active_end, num_active, sorted_ids, permutation, inverse);
+        else
+            hipLaunchKernelGGL(route_scan_scatter_wave_kernel<int32_t>, dim3(chunks), dim3(kWaveChunk), 0, s, (const int32_t*)topk_ids, routes, num_experts, chunks, local_rank,
+                               chunk_hist, chunk_bad, counts, end_offsets, active_ids, active_end, num_active, sorted_ids, permutation, inverse);
+        return check_launch("route_plan");
+    }
     hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(256), 0, s, chunk_hist, chunks, num_experts, counts, end_offsets, active_ids, active_end, num_active, expert_base, chunk_bad);
     if (chunks > 0) {
         if (ids_are_int64)
-            hipLaunchKernelGGL(route_scatter_kernel<int64_t>, dim3(chunks), dim3(kChunk), 0, s, (const int64_t*)topk_ids, routes, num_experts, local_rank, chunk_hist, expert_base, sorted_ids, permutation, inverse);
+            hipLaunchKernelGGL(route_scatter_kernel<int64_t>, dim3(chunks), dim3(chunk), 0, s, (const int64_t*)topk_ids, routes, num_experts, local_rank, chunk_hist, expert_base, sorted_ids, permutation, inverse);
         else
-            hipLaunchKernelGGL(route_scatter_kernel<int32_t>, dim3(chunks), dim3(kChunk), 0, s, (const int32_t*)topk_ids, routes, num_experts, local_rank, chunk_hist, expert_base, sorted_ids, permutation, inverse);
+            hipLaunchKernelGGL(route_scatter_kernel<int32_t>, dim3(chunks), dim3(chunk), 0, s, (const int32_t*)topk_ids, routes, num_experts, local_rank, chunk_hist, expert_base, sorted_ids, permutation, inverse);
     }
     return check_launch("route_plan");
 }
