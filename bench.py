@@ -287,9 +287,13 @@ def other_workload(name, pkg, lib, dev, args):
         def quantized_experts(n_out, k_in):
             # every expert drawn from N(0, 0.02^2) on the device (1.6 G weights per projection) and quantized there by the
             # restatement of the oracle's IQ2_XXS quantizer (bit-checked against it in tests/test_gpu_dequant.py)
+            # (--iq2-pool N < 256 quantizes N distinct experts and repeats them: every expert still has its own bytes in HBM)
             out = torch.empty(e, n_out, k_in // 256 * 66, dtype=torch.uint8, device=dev)
-            for j in range(e):
+            pool = max(1, min(e, args.iq2_pool))
+            for j in range(pool):
                 out[j] = pkg.gguf.quantize_iq2_xxs(torch.randn(n_out, k_in, generator=gd, device=dev) * 0.02)
+            for j in range(pool, e):
+                out[j] = out[j % pool]
             return G(out, 16, (e, n_out, k_in))
 
         gate, up, down = quantized_experts(inter, hidden), quantized_experts(inter, hidden), quantized_experts(hidden, inter)
@@ -320,7 +324,8 @@ def other_workload(name, pkg, lib, dev, args):
         flops = flops_routed + flops_shared
         launch_flops, launches_per_step = None, None  # routed and shared launches differ; per-kernel figures are in `by_kernel_ms_per_step`
         workload = ("configs[4]: grouped-MoE IQ2_XXS LoRA fwd+bwd, 2048 tokens x top-8, hidden 4096, 256 routed experts quantized from N(0, 0.02^2), gate_up [4096x4096], "
-                    "down [4096x2048], plus the shared Q8_0 expert of the same shapes on every token, r=16 alpha=32 on all projections")
+                    "down [4096x2048], plus the shared Q8_0 expert of the same shapes on every token, r=16 alpha=32 on all projections"
+                    + ("" if args.iq2_pool >= e else f" ({args.iq2_pool} distinct experts, repeated)"))
         metric = "fwd+bwd TFLOP/s, IQ2_XXS grouped-MoE LoRA with the shared Q8_0 expert"
         params = list(layer.parameters())
 
@@ -387,12 +392,14 @@ def other_workload(name, pkg, lib, dev, args):
         step()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    lib.ggq_set_factor_gradient_overlap(0)  # per-launch event times of a launch alone on its stream (see main())
     lib.ggq_profile_begin()
     prof_steps = min(args.steps, 5)
     for _ in range(prof_steps):
         step()
     torch.cuda.synchronize()
     launches = profiled_launches(lib)
+    lib.ggq_set_factor_gradient_overlap(1 if args.overlap else 0)
     n_l = len(launches)
     tile_ms = sum(t for _, t in launches) / prof_steps
     by_kernel = {}
@@ -431,9 +438,12 @@ def main() -> None:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--settle-ms", type=float, default=300.0, help="moe_q4k: milliseconds of untimed step replays ahead of the warm-up steps (0: none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--chunk", type=int, default=1024, help="lmhead_q6k: rows per chunk (1024 in the BASELINE configuration; from 4096 rows on the logits of a chunk are kept)")
     ap.add_argument("--graph", type=int, default=1, help="replay the step from a captured HIP graph (1) or run it eagerly (0)")
+    ap.add_argument("--iq2-pool", type=int, default=256, help="moe_iq2xxs: number of distinct experts drawn and quantized (the others repeat them)")
+    ap.add_argument("--overlap", type=int, default=1, help="factor gradients of the grouped backward calls on the library's side stream (1, the library's default) or on the launch stream (0)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (every box here has one MI355X); run with --gpus 1")
@@ -442,6 +452,7 @@ def main() -> None:
     pkg = __graft_entry__.import_package()
     lib = pkg._lib.load()
     dev = torch.device("cuda:0")
+    lib.ggq_set_factor_gradient_overlap(1 if args.overlap else 0)
     if args.workload != "moe_q4k":
         other_workload(args.workload, pkg, lib, dev, args)
         return
@@ -479,6 +490,17 @@ def main() -> None:
         else:
             step()
 
+    # Settle: the device comes out of the set-up above (host-paced quantization, capture) at idle clocks and cold
+    # translation caches, and its first few dozen steps run 5-6 % slower than the ones after them; a training run spends
+    # its life in the sustained state.  The step is replayed for --settle-ms milliseconds (untimed, like the warm-up steps
+    # that follow) so that the timed region measures that state whatever --steps is.
+    t_settle = time.perf_counter()
+    settle_steps = 0
+    while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
+        for _ in range(10):
+            run_step()
+        torch.cuda.synchronize()
+        settle_steps += 10
     for _ in range(args.warmup):
         run_step()
     torch.cuda.synchronize()
@@ -489,13 +511,17 @@ def main() -> None:
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
 
-    # per-launch durations of the tile kernel, HIP events on the launch stream, eager steps
+    # per-launch durations of the packed-weight kernels, HIP events on the launch stream, eager steps.  For these steps the
+    # factor gradients stay on the launch stream: forked (the default, and what the timed region above ran) they share the
+    # compute units with the grad-input launch, whose event pair would then time both.
+    lib.ggq_set_factor_gradient_overlap(0)
     lib.ggq_profile_begin()
     prof_steps = min(args.steps, 10)
     for _ in range(prof_steps):
         step()
     torch.cuda.synchronize()
     launches = profiled_launches(lib)
+    lib.ggq_set_factor_gradient_overlap(1 if args.overlap else 0)
     fl = algorithmic_flops(cfg)
     by_kernel = {}
     for nm, t in launches:
@@ -528,13 +554,16 @@ def main() -> None:
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "configs[2]: grouped-MoE Q4_K LoRA fwd+bwd, 4096 tokens x top-8 = 32768 routes, hidden 2048, 256 experts, gate_up [1024x2048], down [2048x512], r=16 alpha=32",
-                   "launch": "hip-graph replay" if graph is not None else "eager"},
+                   "launch": "hip-graph replay" if graph is not None else "eager",
+                   "factor_gradients": "forked onto the library's side stream" if args.overlap else "on the launch stream",
+                   "settle": f"{settle_steps} untimed steps ({args.settle_ms:.0f} ms) ahead of the {args.warmup} warm-up steps, so that the timed steps run at sustained clocks"},
         "weight_gb_per_s": 2 * packed_weight_bytes(cfg) / (ms_per_step * 1e-3) / 1e9,
         "pct_of_mfma_peak": 100.0 * fl["total"] / (ms_per_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
         "pct_of_hbm_peak_weights": 100.0 * 2 * packed_weight_bytes(cfg) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "roofline": {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic_bytes, "traffic_source": traffic_source, "avg_launch_ms": avg_ms,
-                     "launches_timed": n_launches, "flops_per_launch": flops_per_launch},
+                     "launches_timed": n_launches, "flops_per_launch": flops_per_launch,
+                     "timed_with": "HIP events around each launch, eager steps, factor gradients on the launch stream"},
         "tile_kernel_ms_per_step": kernel_ms_per_step,
         "ceilings_on_this_box": ceilings,
         "frac_of_measured_mfma_ceiling": achieved / ceilings["mfma_bf16_tflops_workload_values"] if ceilings.get("mfma_bf16_tflops_workload_values") else None,

@@ -28,7 +28,7 @@ struct Bump {  // carve 256-byte aligned pieces out of the caller's workspace
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
-int g_shape_override = -1;  // ggq_debug_force_grouped_shape: -1 = the automatic choice
+std::atomic<int> g_shape_override{-1};  // ggq_debug_force_grouped_shape (a test aid): -1 = the automatic choice
 
 // ---------------------------------------------------------------------------------------------------
 // The factor gradients dA / dB of a backward call depend on nothing the grad-input launch writes, are HBM-bound and
@@ -129,7 +129,7 @@ int ggq_measure_mfma_ceiling(const void* a_samples, const void* b_samples, int64
 
 int ggq_debug_force_grouped_shape(int shape) {
     if (shape != -1 && shape != kShapeTall && shape != kShapeWide && shape != kShapeDirect && shape != kShapeSmall) return set_error(GGQ_ERR_SHAPE, "debug_force_grouped_shape: unknown shape %d", shape);
-    g_shape_override = shape;
+    g_shape_override.store(shape);
     return GGQ_OK;
 }
 
@@ -163,7 +163,7 @@ static int launch_wide_and_tall(int qt, int mode, MmqParams& p, int rows, int n,
 // most 192 rows run the tile kernel in its wide shape, mixed with tall tiles for their larger groups; everything else runs
 // tall tiles.
 static int pick_shape(int qt, int64_t rows, int64_t groups, bool direct_ok) {
-    const int forced = g_shape_override;  // a test aid
+    const int forced = g_shape_override.load();  // a test aid
     const bool q4k = qt == 12;            // GGML Q4_K: the only block format with decoding-wave kernels
     if (q4k && direct_ok && (forced == kShapeDirect || (forced < 0 && groups > 0 && rows <= 256 * groups))) return kShapeDirect;
     if (forced == kShapeTall || !(groups > 0 && rows <= 192 * groups)) return kShapeTall;
@@ -373,7 +373,7 @@ static int grouped_forward(const char* what, const void* x, RowIndex x_index, co
         TileDesc* t64 = lora_a ? (TileDesc*)bump.take((int64_t)max_tiles64 * sizeof(TileDesc)) : nullptr;
         // IQ2_XXS: the groups of at most 128 rows leave the wide table for a launch of their own (decoding waves)
         // (its lanes address a weight plane with 32-bit offsets)
-        const bool small = wide && qt == 16 /* GGML IQ2_XXS */ && direct_ok && p.w_expert_bytes < (1ll << 32) && g_shape_override != kShapeWide;
+        const bool small = wide && qt == 16 /* GGML IQ2_XXS */ && direct_ok && p.w_expert_bytes < (1ll << 32) && g_shape_override.load() != kShapeWide;
         t_small = small ? (TileDesc*)bump.take((int64_t)groups * sizeof(TileDesc)) : nullptr;
         TileDesc* t_small_sorted = small ? (TileDesc*)bump.take((int64_t)groups * sizeof(TileDesc)) : nullptr;  // most row blocks first
         int* counts = (int*)bump.take(16);
