@@ -286,8 +286,8 @@ struct Direct8 {
             if (nl > 0) {
 #pragma unroll
                 for (int rb = 0; rb < LIVE; rb++)
-                    la0[rb] = la_resident ? *(const bf16x8_t*)(smem_raw + kLaBase + (32 * rb + lane_ce) * 32 + lane_he * 16)
-                                          : *(const bf16x8_t*)(p.la + (int64_t)(c.row_begin + min(32 * rb + lane_ce, rows_valid - 1)) * p.r_pad + lane_he * 8);
+                    la0[rb] = read_lds_or_global(la_resident, smem_raw + kLaBase + (32 * rb + lane_ce) * 32 + lane_he * 16,
+                                                 p.la + (int64_t)(c.row_begin + min(32 * rb + lane_ce, rows_valid - 1)) * p.r_pad + lane_he * 8);
             }
             // the staging block: the buffer of the pair of steps just finished (the next request into it comes with the
             // next tile's first step, after the reads below have returned their data to the stores)

@@ -346,8 +346,8 @@ struct Direct8NN {
                 lb0 = read_tr(dblk + (8 * (g4 >> 1) + (s4 >> 2)) * kDecPitch + (16 * (g4 & 1) + 4 * (s4 & 3)) * 2, kDecPitch);
 #pragma unroll
                 for (int rb = 0; rb < LIVE; rb++)
-                    la0[rb] = la_resident ? *(const bf16x8_t*)(smem_raw + kLaBase + (32 * rb + lane_ce) * 32 + lane_he * 16)
-                                          : *(const bf16x8_t*)(p.la + (int64_t)(c.row_begin + min(32 * rb + lane_ce, rows_valid - 1)) * p.r_pad + lane_he * 8);
+                    la0[rb] = read_lds_or_global(la_resident, smem_raw + kLaBase + (32 * rb + lane_ce) * 32 + lane_he * 16,
+                                                 p.la + (int64_t)(c.row_begin + min(32 * rb + lane_ce, rows_valid - 1)) * p.r_pad + lane_he * 8);
             }
             uint8_t* const stage = dblk + 32 * kDecPitch;  // 2 KB behind the factor rows
 #pragma unroll

@@ -237,7 +237,7 @@ struct SmallIq2 {
                 for (int e = 0; e < 16; e++) t[e] = 0.0f;
                 if (nl > 0) {
                     const bf16_t* la = p.la + (int64_t)(c.row_begin + min(row, rows_valid - 1)) * p.r_pad + lane_h * 8;
-                    const bf16x8_t la0 = la_resident ? *(const bf16x8_t*)(smem_raw + kLaBase + row * 32 + lane_h * 16) : *(const bf16x8_t*)la;
+                    const bf16x8_t la0 = read_lds_or_global(la_resident, smem_raw + kLaBase + row * 32 + lane_h * 16, la);
                     t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lb0, la0, t, 0, 0, 0);
 #pragma nounroll
                     for (int kk = 1; kk < nl; kk++)
