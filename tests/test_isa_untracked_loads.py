@@ -7,6 +7,12 @@ way, which copies stale data and loses the load's result: wrong numbers without 
 kernels to gfx950 assembly and replays every loop body twice against the in-order queue of vector-memory operations:
 between an inline-asm load into a VGPR and the wait that retires it, no instruction may name that VGPR.  It also checks
 that the loops hold no scratch (spill) traffic, which would drain the queue through compiler-made waits.
+
+It also guards the compiler's own LDS waits.  A load through a pointer selected between LDS and global memory is a flat
+load; the compiler never sees these kernels' inline-asm `vmcnt` waits, so it takes such a load for outstanding through
+every later loop iteration and, unable to count LDS returns past it, drains ALL of a wave's LDS reads (`lgkmcnt(0)`) where
+it needs the oldest of them: in front of the first MFMA of every sub-step.  The kernels must hold no flat memory
+instruction, and the Q4_K main loops must wait for their LDS operands with exact counts.
 """
 import pathlib
 import re
@@ -130,3 +136,29 @@ def test_the_replay_flags_a_copy_of_a_register_in_flight():
     assert [b[1] for b in bad] == ["v_mov_b32_e32 v20, v10", "v_mov_b32_e32 v20, v10"]
     ok = [("global_load_dwordx2 v[10:11], v1, s[2:3]", True), ("global_load_lds_dwordx4 v1, s[2:3]", True), ("s_waitcnt vmcnt(1)", True), ("v_mov_b32_e32 v20, v10", False)]
     assert not _replay(ok)
+
+
+@pytest.mark.parametrize("kernel", sorted(KERNELS))
+def test_no_flat_memory_instruction(assembly, kernel):
+    m = re.search(r"^(_ZN3ggq\d+" + kernel + r"\w*):", assembly, re.M)
+    body = assembly[m.end() : assembly.index(".Lfunc_end", m.end())]
+    flat = [t for t, _ in _instructions(body) if re.match(r"flat_(load|store|atomic)", t)]
+    assert not flat, f"{kernel}: {flat[:3]}"
+
+
+@pytest.mark.parametrize("kernel", ["mmq_direct8_q4k_kernel", "mmq_direct8_nn_q4k_kernel"])
+def test_main_loops_wait_for_lds_operands_with_exact_counts(assembly, kernel):
+    """In the inner loops of the tile variants with two or more row blocks, a compiler-made `lgkmcnt(0)` stands only in
+    front of the step barrier (the kernels' own wait), never in front of an MFMA."""
+    m = re.search(r"^(_ZN3ggq\d+" + kernel + r"\w*):", assembly, re.M)
+    body = assembly[m.end() : assembly.index(".Lfunc_end", m.end())]
+    checked = 0
+    for label, loop, innermost in _loops(_instructions(body)):
+        texts = [t for t, _ in loop]
+        mfmas = sum(t.startswith("v_mfma") for t in texts)
+        if not innermost or mfmas < 32:  # one-block tiles read each operand one sub-step ahead: nothing newer is in flight behind it
+            continue
+        drains = [b for a, b in zip(texts, texts[1:]) if a.startswith("s_waitcnt") and "lgkmcnt(0)" in a and b.startswith("v_mfma")]
+        assert not drains, f"{kernel} {label}: {len(drains)} of {mfmas} MFMAs wait for every LDS read"
+        checked += 1
+    assert checked >= 3

@@ -108,8 +108,8 @@ typedef __attribute__((address_space(3))) const bf16x8_t* lds_bf16x8_ptr;
 typedef __attribute__((address_space(1))) const bf16x8_t* global_bf16x8_ptr;
 __device__ __forceinline__ bf16x8_t read_lds_or_global(bool in_lds, const uint8_t* lds, const void* global) {
     bf16x8_t v;
-    if (in_lds) v = *(lds_bf16x8_ptr)(uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)lds;
-    else v = *(global_bf16x8_ptr)(uintptr_t)global;
+    if (in_lds) v = *(lds_bf16x8_ptr)lds;
+    else v = *(global_bf16x8_ptr)global;
     return v;
 }
 
