@@ -466,8 +466,9 @@ static int grouped_backward(const char* what, const void* dy1, const void* dy2, 
     Bump bump{(char*)ws, ws_bytes, 0};
 
     MmqParams p;
-    // the direct kernel moves the cotangents with aligned 16-byte accesses and takes an even number of whole 64-row steps
-    const bool direct_ok = aligned16(dy1) && (!dy2 || aligned16(dy2)) && n % 64 == 0 && (nseg * (n / 64)) % 2 == 0 && n < (1 << 22) &&
+    // the direct kernel moves the cotangents with aligned 16-byte accesses and takes an even number, four or more, of whole
+    // 64-row steps (the request of a tile's LoRA factor piece is certain to have landed behind the tile's third step)
+    const bool direct_ok = aligned16(dy1) && (!dy2 || aligned16(dy2)) && n % 64 == 0 && (nseg * (n / 64)) % 2 == 0 && nseg * (n / 64) >= 4 && n < (1 << 22) &&
                            (!lora_a || aligned16(lora_a)) && k % 8 == 0;
     if (int rc = init_params(p, qt, kModeNN, (int)rows, (int)n, (int)k, nseg, pick_shape(qt, rows, groups, direct_ok))) return rc;
     p.a[0] = (const bf16_t*)dy1, p.a[1] = (const bf16_t*)dy2, p.lda = n, p.a_rows = dy_index;

@@ -99,20 +99,6 @@ __device__ __forceinline__ void wait_loads_at_most(int n) {
     }
 }
 
-// A row of eight bf16 that sits either in LDS or in global memory.  Each source is read through a pointer typed with its own
-// address space: a load through a pointer SELECTED between the two (`in_lds ? *a : *b` compiles to that) is a flat load, and
-// as long as the compiler believes a flat load may be outstanding - it never sees the inline-asm waits of these kernels - it
-// cannot count LDS returns and waits for ALL of a wave's LDS reads (lgkmcnt(0)) wherever it needs one of them: one exposed LDS
-// round trip in front of every sub-step's first MFMA of the main loops, far away from the load that caused it.
-typedef __attribute__((address_space(3))) const bf16x8_t* lds_bf16x8_ptr;
-typedef __attribute__((address_space(1))) const bf16x8_t* global_bf16x8_ptr;
-__device__ __forceinline__ bf16x8_t read_lds_or_global(bool in_lds, const uint8_t* lds, const void* global) {
-    bf16x8_t v;
-    if (in_lds) v = *(lds_bf16x8_ptr)lds;
-    else v = *(global_bf16x8_ptr)global;
-    return v;
-}
-
 // 16-byte slot that holds contraction chunk kc (0..7) of A-tile row r.  Sixteen consecutive rows at one
 // kc cover all sixteen 16-byte bank groups exactly once.
 __device__ __forceinline__ int a_slot(int r, int kc) { return kc ^ ((r >> 1) & 7); }

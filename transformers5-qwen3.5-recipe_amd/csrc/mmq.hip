@@ -208,8 +208,8 @@ static int launch_direct(const MmqParams& p, hipStream_t s) {
     if (total <= 0) return GGQ_OK;
     const int64_t grid = total * 8;
     if (grid > 0x7FFFFFF0) return set_error(GGQ_ERR_SHAPE, "mmq: too many tiles for one launch");
-    if (MODE == kModeNN && ((p.n & 63) || ((p.nseg * p.steps_per_seg) & 1)))
-        return set_error(GGQ_ERR_SHAPE, "mmq: the direct grad-input kernel needs an even number of whole 64-row steps");
+    if (MODE == kModeNN && ((p.n & 63) || ((p.nseg * p.steps_per_seg) & 1) || p.nseg * p.steps_per_seg < 4))
+        return set_error(GGQ_ERR_SHAPE, "mmq: the direct grad-input kernel needs an even number, four or more, of whole 64-row steps");
     TimedLaunch* t = nullptr;
     if (g_timing && g_timed_count < kMaxTimedLaunches) {
         t = &g_timed[g_timed_count];

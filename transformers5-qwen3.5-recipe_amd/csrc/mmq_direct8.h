@@ -144,12 +144,12 @@ struct Direct8 {
         issue_a();
         issue_a();
         issue_a();
-        // the row tile's LA rows stay in LDS for all the column tiles of this workgroup (ranks up to 16)
-        const bool la_resident = p.r_pad == 16;
-        if (la_resident) {
+        // the first 16 rank columns of the row tile's LA rows stay in LDS for all the column tiles of this workgroup: the
+        // epilogue then reads them with LDS reads, which no pending store or request stands in front of
+        if (p.r_pad > 0) {
             for (int id = tid; id < LIVE * 64; id += kThreadsWG) {
                 const int row = id >> 1, half = id & 1;
-                *(uint4*)(smem_raw + kLaBase + row * 32 + half * 16) = *(const uint4*)(p.la + (int64_t)(c.row_begin + min(row, c.rows_valid - 1)) * 16 + half * 8);
+                *(uint4*)(smem_raw + kLaBase + row * 32 + half * 16) = *(const uint4*)(p.la + (int64_t)(c.row_begin + min(row, c.rows_valid - 1)) * p.r_pad + half * 8);
             }
         }
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI) : "memory");  // the first block's bytes and the first step's A stage have landed
@@ -202,12 +202,17 @@ struct Direct8 {
             for (int i = 0; i < LIVE; i++)
 #pragma unroll
                 for (int e = 0; e < 16; e++) acc[i][e] = 0.0f;
-            // this lane's row of the LoRA factor B (first 16 of the rank), requested ahead of the tile's steps
-            bf16x8_t lb0;
-            if (p.r_pad > 0) {
+            // This lane's row of the LoRA factor B (first 16 of the rank), requested ahead of the tile's steps with a load of
+            // the same untracked kind as the other requests (without a LoRA term: 16 bytes of the packed weights, unused).
+            // A load the compiler tracks would be waited for at its use in the epilogue with vmcnt(0): behind the next
+            // tile's first requests, and behind the stores of the row blocks before it, one round trip each.
+            u32x4_t lb0_raw;
+            {
                 int seg0, colz;
                 tile_origin(ct, seg0, colz);
-                lb0 = *(const bf16x8_t*)(p.lb + c.expert * p.lb_expert_elems + ((int64_t)seg0 * out_cols + min(colz + 32 * wave + lane_c, out_cols - 1)) * p.r_pad + lane_h * 8);
+                const void* src = p.r_pad > 0 ? (const void*)(p.lb + c.expert * p.lb_expert_elems + ((int64_t)seg0 * out_cols + min(colz + 32 * wave + lane_c, out_cols - 1)) * p.r_pad + lane_h * 8)
+                                              : (const void*)(p.w[0] + c.expert * p.w_expert_bytes);
+                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(lb0_raw) : "v"(src) : "memory");
             }
             // the first half of the next block's quant bytes goes out with a block's last sub-step, except behind a
             // tile's last block, where the store path below still uses the buffer it would fill
@@ -233,10 +238,12 @@ struct Direct8 {
                     // the barrier every wave's part has, and every wave is done reading stage S, which the next phase's
                     // requests overwrite.  Requests complete in order, so the distance matters: packed bytes come from
                     // HBM, and a wait that covered requests only one step old stalled on them.
-                    // (Behind a tile's stores, which went out inside phase 0's requests, the first two steps allow for them.)
+                    // (Behind a tile's stores and the request of the LoRA factor row, which went out inside phase 0's requests,
+                    // the first two steps allow for them.)
                     constexpr int kGroup[4] = {NI + 2, NI + 1, NI + 2, NI};
                     constexpr int kBehind = kGroup[S] + kGroup[(S + 3) & 3];
-                    if (S < 2 && kb == 0 && stores_behind) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBehind + kStores) : "memory");
+                    if (S < 2 && kb == 0 && stores_behind) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBehind + kStores + 1) : "memory");
+                    else if (S < 2 && kb == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBehind + 1) : "memory");
                     else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBehind) : "memory");
                     if (S == 3) asm volatile("" : "+v"(hn));
                     lds_barrier();
@@ -282,12 +289,14 @@ struct Direct8 {
             const int nl = p.r_pad >> 4;  // LoRA sub-steps (0: no LoRA)
             const float ls = nl > 0 ? p.lora_scale : 0.0f;
             const bf16_t* const lb_lane = p.lb + c.expert * p.lb_expert_elems + ((int64_t)seg * out_cols + min(col0 + 32 * wave + lane_ce, out_cols - 1)) * p.r_pad + lane_he * 8;
+            // (the factor row landed long ago: every step's wait leaves only the requests of two phases outstanding)
+            asm volatile("" : "+v"(lb0_raw));
+            const bf16x8_t lb0 = __builtin_bit_cast(bf16x8_t, lb0_raw);
             bf16x8_t la0[LIVE];
             if (nl > 0) {
 #pragma unroll
                 for (int rb = 0; rb < LIVE; rb++)
-                    la0[rb] = read_lds_or_global(la_resident, smem_raw + kLaBase + (32 * rb + lane_ce) * 32 + lane_he * 16,
-                                                 p.la + (int64_t)(c.row_begin + min(32 * rb + lane_ce, rows_valid - 1)) * p.r_pad + lane_he * 8);
+                    la0[rb] = *(const bf16x8_t*)(smem_raw + kLaBase + (32 * rb + lane_ce) * 32 + lane_he * 16);
             }
             // the staging block: the buffer of the pair of steps just finished (the next request into it comes with the
             // next tile's first step, after the reads below have returned their data to the stores)

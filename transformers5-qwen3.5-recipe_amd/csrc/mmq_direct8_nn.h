@@ -185,12 +185,12 @@ struct Direct8NN {
             request_a(std::integral_constant<int, 2>{});
             request_w();
         }
-        // the row tile's LA rows stay in LDS for all the column tiles of this workgroup (ranks up to 16)
-        const bool la_resident = p.r_pad == 16;
-        if (la_resident) {
+        // the first 16 rank columns of the row tile's LA rows stay in LDS for all the column tiles of this workgroup: the
+        // epilogue then reads them with LDS reads, which no pending store or request stands in front of
+        if (p.r_pad > 0) {
             for (int id = tid; id < LIVE * 64; id += kThreadsWG) {
                 const int row = id >> 1, half = id & 1;
-                *(uint4*)(smem_raw + kLaBase + row * 32 + half * 16) = *(const uint4*)(p.la + (int64_t)(c.row_begin + min(row, c.rows_valid - 1)) * 16 + half * 8);
+                *(uint4*)(smem_raw + kLaBase + row * 32 + half * 16) = *(const uint4*)(p.la + (int64_t)(c.row_begin + min(row, c.rows_valid - 1)) * p.r_pad + half * 8);
             }
         }
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 2) * kGroup) : "memory");
@@ -239,9 +239,16 @@ struct Direct8NN {
                 for (int e = 0; e < 16; e++) acc[i][e] = 0.0f;
             // rows 0..15 of the LoRA factor x this wave's 32 columns (one 16-byte piece per lane), requested ahead of
             // the tile's steps
-            uint4 lbraw = zero4();
-            if (p.r_pad > 0) lbraw = *(const uint4*)(p.lb + c.expert * p.lb_expert_elems + (int64_t)min(lane >> 2, p.lora_rank - 1) * out_cols + ct * kTN + 32 * wave + (lane & 3) * 8);
-            relax = stores_behind ? kStages - 2 : 0;
+            // (a load of the same untracked kind as the other requests; without a LoRA term: 16 bytes of the packed weights,
+            // unused.  A load the compiler tracks would be waited for at its use in the epilogue with vmcnt(0): behind the
+            // next tile's first requests, and behind the stores of the row blocks before it, one round trip each.)
+            u32x4_t lbraw;
+            {
+                const void* src = p.r_pad > 0 ? (const void*)(p.lb + c.expert * p.lb_expert_elems + (int64_t)min(lane >> 2, p.lora_rank - 1) * out_cols + min(ct * kTN + 32 * wave + (lane & 3) * 8, out_cols - 8))
+                                              : (const void*)(p.w[0] + c.expert * p.w_expert_bytes);
+                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(lbraw) : "v"(src) : "memory");
+            }
+            relax = kStages - 2;
             for (int st = 0; st < steps; st += 2) {
                 // One step.  Its B operands were read at the end of the step before; the next step's weight rows are
                 // decoded behind its MFMAs (a half of a quarter row per slot) and read back at its end.
@@ -281,10 +288,11 @@ struct Direct8NN {
                     // End of the phase: all but the requests of this phase (and, with four stages, the one before it)
                     // have landed - this wave's parts of the next step's A stage and of the packed bytes of the step
                     // after it.  Behind the barrier every wave's parts have, and every wave is done with the stages the
-                    // next phase's requests overwrite.  (Behind a tile's stores, which went out inside a phase's requests, the
-                    // steps whose awaited requests are older than that phase allow for them.)
+                    // next phase's requests overwrite.  (Behind a tile's stores and the request of the LoRA factor piece, which went out
+                    // inside a phase's requests, the steps whose awaited requests are older than that phase allow for them.)
                     constexpr int kBehind = (kStages - 2) * kGroup;
-                    if (relax > 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBehind + kStores) : "memory");
+                    if (relax > 0 && stores_behind) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBehind + kStores + 1) : "memory");
+                    else if (relax > 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBehind + 1) : "memory");
                     else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBehind) : "memory");
                     lds_barrier();
                     open_a();
@@ -341,13 +349,15 @@ struct Direct8NN {
                 // rows 0..15 of the factor x this wave's 32 columns: whole 64-byte rows into the block (rows past the rank
                 // as zeros), one transposing read back out
                 const int j = lane_e >> 2, ch = lane_e & 3;
-                *(uint4*)(dblk + j * kDecPitch + ch * 16) = j < p.lora_rank ? lbraw : zero4();
+                // The piece has landed: the first wait of the tile that no longer allows for it (step kStages - 2 <= 2) is
+                // behind us; the host launches this kernel for contractions of four steps or more.
+                asm volatile("" : "+v"(lbraw));
+                *(u32x4_t*)(dblk + j * kDecPitch + ch * 16) = j < p.lora_rank ? lbraw : u32x4_t{0u, 0u, 0u, 0u};
                 const int g4 = lane_e >> 4, s4 = lane_e & 15;
                 lb0 = read_tr(dblk + (8 * (g4 >> 1) + (s4 >> 2)) * kDecPitch + (16 * (g4 & 1) + 4 * (s4 & 3)) * 2, kDecPitch);
 #pragma unroll
                 for (int rb = 0; rb < LIVE; rb++)
-                    la0[rb] = read_lds_or_global(la_resident, smem_raw + kLaBase + (32 * rb + lane_ce) * 32 + lane_he * 16,
-                                                 p.la + (int64_t)(c.row_begin + min(32 * rb + lane_ce, rows_valid - 1)) * p.r_pad + lane_he * 8);
+                    la0[rb] = *(const bf16x8_t*)(smem_raw + kLaBase + (32 * rb + lane_ce) * 32 + lane_he * 16);
             }
             uint8_t* const stage = dblk + 32 * kDecPitch;  // 2 KB behind the factor rows
 #pragma unroll

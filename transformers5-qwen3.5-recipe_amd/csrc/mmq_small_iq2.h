@@ -55,12 +55,11 @@ struct SmallIq2 {
         const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem_raw;
         for (int i = tid; i < Fmt<kIQ2_XXS>::kTableWords; i += kThreadsWG) table_words[i] = Fmt<kIQ2_XXS>::table_word(i, i < 1024 ? d_iq2xxs_grid_mm[i >> 2] : 0);
         const uint2* const tables = (const uint2*)table_words;
-        // the row tile's LA rows stay in LDS for all the column tiles of this workgroup (ranks up to 16)
-        const bool la_resident = p.r_pad == 16;
-        if (la_resident) {
+        // the first 16 rank columns of the row tile's LA rows stay in LDS for all the column tiles of this workgroup
+        if (p.r_pad > 0) {
             for (int id = tid; id < LIVE * 64; id += kThreadsWG) {
                 const int row = id >> 1, half = id & 1;
-                *(uint4*)(smem_raw + kLaBase + row * 32 + half * 16) = *(const uint4*)(p.la + (int64_t)(c.row_begin + min(row, c.rows_valid - 1)) * 16 + half * 8);
+                *(uint4*)(smem_raw + kLaBase + row * 32 + half * 16) = *(const uint4*)(p.la + (int64_t)(c.row_begin + min(row, c.rows_valid - 1)) * p.r_pad + half * 8);
             }
         }
         __syncthreads();
@@ -237,7 +236,7 @@ struct SmallIq2 {
                 for (int e = 0; e < 16; e++) t[e] = 0.0f;
                 if (nl > 0) {
                     const bf16_t* la = p.la + (int64_t)(c.row_begin + min(row, rows_valid - 1)) * p.r_pad + lane_h * 8;
-                    const bf16x8_t la0 = read_lds_or_global(la_resident, smem_raw + kLaBase + row * 32 + lane_h * 16, la);
+                    const bf16x8_t la0 = *(const bf16x8_t*)(smem_raw + kLaBase + row * 32 + lane_h * 16);
                     t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lb0, la0, t, 0, 0, 0);
 #pragma nounroll
                     for (int kk = 1; kk < nl; kk++)
