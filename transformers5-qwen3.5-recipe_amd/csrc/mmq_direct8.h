@@ -10,7 +10,7 @@
 //     unpadded with XOR-swizzled 16-byte slots (a_slot), every wave reads all of them;
 //   * the packed quant bytes go global -> LDS directly as well, half a 256-wide block (two steps) of the wave's 32
 //     columns at a time, four lanes per row so that a row's bytes are requested by adjacent lanes, into a ring of three
-//     wave-private buffers; block headers are loaded into registers;
+//     wave-private buffers; a block's 16-byte headers follow the same way, one lane per column, a block ahead;
 //   * a lane reads its 16 quant bytes of the step from its wave's buffer and decodes them in registers into the operands
 //     of the step's four MFMA sub-steps (mmq_direct.h).  No decoded weight ever touches LDS.
 // A single wave issues at most one instruction per four to five cycles, whatever its kind, so a step's decode
@@ -38,7 +38,8 @@ struct Direct8 {
     static constexpr int kWBufBytes = 32 * 64, kWBufs = 3;
     static constexpr int kWBase = kRingBytes;
     static constexpr int kLaBase = kWBase + kWaves * kWBufs * kWBufBytes;  // + 48 KB: then the row tile's LA rows (rank <= 16), 32 bytes each
-    static constexpr int kLdsBytes = kLaBase + kTM * 32;                   // + 6 KB = 150 KB
+    static constexpr int kHdrBase = kLaBase + kTM * 32;                    // + 6 KB: then per wave the 16-byte headers of a block of its 32 columns
+    static constexpr int kLdsBytes = kHdrBase + kWaves * 512;              // + 4 KB = 154 KB
 
     using Scales = Direct::Scales;
     using RowCtx = Direct::RowCtx;
@@ -114,8 +115,13 @@ struct Direct8 {
             for (int j = 0; j < 2; j++) load16_to_lds(w_lds + w_wr + j * 1024, wq_voff[j], src);
             w_wr = w_wr == (kWBufs - 1) * kWBufBytes ? 0 : w_wr + kWBufBytes;
         };
-        auto issue_w_header = [&](u32x4_t& h) __attribute__((always_inline)) {
-            asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(h) : "v"(wh_voff), "s"(w_next + w_blk * 144) : "memory");
+        // The headers of the cursor's block go global -> LDS as well, one lane per column (a load of 64 lanes that names
+        // each of 32 addresses twice costs the vector cache twice the accesses), into the wave's one header buffer: a
+        // block's headers are read out of it (below) a whole step before the request of the next block's goes out.
+        const uint32_t hdr_lds = lds_base + kHdrBase + wave * 512;
+        const uint8_t* const hdr_row = smem_raw + kHdrBase + wave * 512 + lane_c * 16;
+        auto issue_w_header = [&]() __attribute__((always_inline)) {
+            if (lane_h == 0) load16_to_lds(hdr_lds, wh_voff, w_next + w_blk * 144);
         };
         auto w_cursor_advance = [&]() __attribute__((always_inline)) {  // past the last block of the last tile the cursor stays
             if (w_blk + 1 < blocks) w_blk++;
@@ -137,7 +143,7 @@ struct Direct8 {
 
         u32x4_t qc, qn;  // quant bytes of the current / next step
         u32x4_t hc, hn;  // headers of the current / next block
-        issue_w_header(hc);
+        issue_w_header();
         issue_w_half(std::integral_constant<int, 0>{});
         issue_w_half(std::integral_constant<int, 1>{});
         w_cursor_advance();
@@ -153,8 +159,9 @@ struct Direct8 {
             }
         }
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NI) : "memory");  // the first block's bytes and the first step's A stage have landed
-        asm volatile("" : "+v"(hc));
         lds_barrier();
+        hc = *(const u32x4_t*)hdr_row;
+        asm volatile("" : "+v"(hc));  // (read out before the request below refills the buffer)
         // Phase p = the last sub-step of step p - 1 and the first three of step p: it reads A stage p only, and its
         // requests (behind the barrier that opens it) fill the stage of step p - 1.  A phase's first A instruction goes
         // out in its first sub-step, the others in the next step's first two; ph_dst / ph_src carry them across.
@@ -170,7 +177,8 @@ struct Direct8 {
             constexpr int I = decltype(i_c)::value;
             if constexpr (I < NI) load16_to_lds(ph_dst + I * 8192, a_voff[I], ph_src);
         };
-        issue_w_half(std::integral_constant<int, 0>{});  // phase 0: the first half of block 1, A of step 3
+        issue_w_half(std::integral_constant<int, 0>{});  // phase 0: the first half of block 1 and its headers, A of step 3
+        issue_w_header();
         phase_open();
         request_a(std::integral_constant<int, 0>{});
         qc = *(const u32x4_t*)(w_rows + w_roff[0]);
@@ -219,12 +227,13 @@ struct Direct8 {
             if (ct > ct0) issue_w_half(std::integral_constant<int, 0>{});
             for (int kb = 0; kb < blocks; kb++) {
                 // Requests per phase P (= step index % 4): the A stage three steps on [NI]; P = 0: the first half of the
-                // next block's quant bytes [2]; P = 1: its header [1]; P = 2: the second half [2].
+                // next block's quant bytes [2] and its headers [1]; P = 2: the second half [2].
                 auto step = [&](auto s_c) __attribute__((always_inline)) {
                     constexpr int S = decltype(s_c)::value;
                     // the quant bytes of the next step: second step of this buffer, or the first of the next one
                     const int w_rd_next = w_rd == (kWBufs - 1) * kWBufBytes ? 0 : w_rd + kWBufBytes;
                     qn = *(const u32x4_t*)(w_rows + ((S & 1) ? w_rd_next + w_roff[0] : w_rd + w_roff[1]));
+                    if (S == 3) hn = *(const u32x4_t*)hdr_row;  // the next block's headers: requested a block ago, landed by the last step's wait
                     const int a_rd_next = a_rd == (kStages - 1) * kStageBytes ? 0 : a_rd + kStageBytes;
                     __builtin_amdgcn_sched_barrier(0);
                     sub_step(bx, a_rd, 1, [&](auto k_c) __attribute__((always_inline)) { Direct::decode_half<1, decltype(k_c)::value>(qc, sc, by); },
@@ -240,12 +249,11 @@ struct Direct8 {
                     // HBM, and a wait that covered requests only one step old stalled on them.
                     // (Behind a tile's stores and the request of the LoRA factor row, which went out inside phase 0's requests,
                     // the first two steps allow for them.)
-                    constexpr int kGroup[4] = {NI + 2, NI + 1, NI + 2, NI};
+                    constexpr int kGroup[4] = {NI + 3, NI, NI + 2, NI};
                     constexpr int kBehind = kGroup[S] + kGroup[(S + 3) & 3];
                     if (S < 2 && kb == 0 && stores_behind) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBehind + kStores + 1) : "memory");
                     else if (S < 2 && kb == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBehind + 1) : "memory");
                     else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBehind) : "memory");
-                    if (S == 3) asm volatile("" : "+v"(hn));
                     lds_barrier();
                     phase_open();
                     // behind the last sub-step's MFMAs: the first operand of the next step (of the next tile behind a
@@ -256,7 +264,7 @@ struct Direct8 {
                         Direct::decode_half<0, K>(qn, sc, bx);
                     }, [&]() __attribute__((always_inline)) {
                         if (S == 3 && kb + 1 < blocks) issue_w_half(std::integral_constant<int, 0>{});
-                        if (S == 0) issue_w_header(hn);
+                        if (S == 3) issue_w_header();  // (behind the barrier: every read of the buffer's last contents has returned)
                         if (S == 1) issue_w_half(std::integral_constant<int, 1>{});
                         request_a(std::integral_constant<int, 0>{});
                     });
