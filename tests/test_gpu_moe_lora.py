@@ -108,6 +108,8 @@ def test_constant_byte_iq2_xxs_experts(pkg, dev):
 
 
 @pytest.mark.parametrize("qt,r,shape,n", [(gb.Q4_K, 16, "", 192), (gb.Q4_K, 16, "", 256), (gb.Q4_K, 16, "3", 256), (gb.Q4_K, 16, "1", 256), (gb.Q4_K, 16, "0", 192),
+                                          (gb.Q4_K, 16, "3", 128),  # the pair's grad-input: four steps, the fewest the decoding-wave kernel takes; the single projection's two: tiles
+                                          (gb.Q4_K, 32, "3", 256),  # a rank beyond the 16 columns of the LoRA rows the kernels keep in LDS
                                           (gb.Q8_0, 4, "", 192), (gb.Q6_K, 8, "", 192), (gb.IQ2_XXS, 16, "", 192)])
 def test_grouped_lora_projection_all_gradients(pkg, dev, qt, r, shape, n, force_grouped_shape):
     # ragged groups including empty experts, a group larger than one 128-row tile, and inactive planes.
