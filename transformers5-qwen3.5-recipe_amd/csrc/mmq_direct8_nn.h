@@ -72,7 +72,7 @@ struct Direct8NN {
         constexpr int NI = (LIVE + 1) / 2;        // direct-to-LDS instructions per A stage and wave
         constexpr int kStages = LIVE <= 4 ? 4 : 3;
         constexpr int kStageBytes = NI * 8192;
-        constexpr int kGroup = NI + 2;            // requests per phase and wave: A [NI], quant bytes [1], headers [1]
+        constexpr int kGroup = NI + 1;            // requests per phase and wave: A [NI], quant bytes [1]; wave 0 one more: the headers
         constexpr int kStores = 2 * LIVE - 1;     // 16-byte store instructions a tile certainly issues per wave
         const int tid = threadIdx.x, lane = tid & 63;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -93,9 +93,17 @@ struct Direct8NN {
         }
         // packed bytes of a step: lane t of the workgroup moves quant chunk (t % 8) ^ swizzle of weight row t / 8
         // (the 16-byte chunks of a row are XOR-swizzled like an A row's: the per-row reads below meet no bank conflict);
-        // lanes 0..7 of wave w move the headers of rows 8 w .. 8 w + 7
+        // wave 0 moves the 64 headers of the step with one request (eight requests of eight lanes each, one per wave, cost
+        // 1.9 % of the configs[2] step more: what a request costs is its issue, not its bytes)
         const uint32_t wq_voff = (uint32_t)((tid >> 3) * (int)p.w_row_bytes + 16 + 16 * ((tid & 7) ^ (((tid >> 3) >> 1) & 7)));
-        const uint32_t wh_voff = (uint32_t)((8 * wave + (lane & 7)) * (int)p.w_row_bytes);
+        const uint32_t wh_voff = (uint32_t)(lane * (int)p.w_row_bytes);
+        const bool hdr_wave = wave == 0;
+        // waits: at most `behind` phases of requests (and `extra` other operations) of this wave outstanding
+        auto wait_behind = [&](auto extra_c) __attribute__((always_inline)) {
+            constexpr int X = decltype(extra_c)::value;
+            if (hdr_wave) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 2) * (kGroup + 1) + X) : "memory");
+            else asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 2) * kGroup + X) : "memory");
+        };
         // Cursors: (column tile, step) of the next A stage / packed-byte stage to request; past the last tile they
         // stay on it (what they request again is never used).
         int a_step_i = 0, a_wr = 0;
@@ -124,7 +132,7 @@ struct Direct8NN {
             const uint8_t* src = step_src_w(w_tile_i, w_step_i);
             const uint32_t dst = lds_base + kRawBase + w_wr;
             load16_to_lds(dst + wave * 1024, wq_voff, src);
-            if (lane < 8) load16_to_lds(dst + 64 * 128 + wave * 128, wh_voff, src);
+            if (hdr_wave) load16_to_lds(dst + 64 * 128, wh_voff, src);
             w_wr = w_wr == (kStages - 1) * kRawStageBytes ? 0 : w_wr + kRawStageBytes;
             if (++w_step_i == steps) {
                 w_step_i = 0;
@@ -193,7 +201,7 @@ struct Direct8NN {
                 *(uint4*)(smem_raw + kLaBase + row * 32 + half * 16) = *(const uint4*)(p.la + (int64_t)(c.row_begin + min(row, c.rows_valid - 1)) * p.r_pad + half * 8);
             }
         }
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 2) * kGroup) : "memory");
+        wait_behind(std::integral_constant<int, 0>{});
         lds_barrier();
         int a_rd = 0;   // byte offset of the A stage of the current step
         int w_rd = 0;   // byte offset of the packed-byte stage of the step being decoded (one ahead of the A stage)
@@ -290,10 +298,9 @@ struct Direct8NN {
                     // after it.  Behind the barrier every wave's parts have, and every wave is done with the stages the
                     // next phase's requests overwrite.  (Behind a tile's stores and the request of the LoRA factor piece, which went out
                     // inside a phase's requests, the steps whose awaited requests are older than that phase allow for them.)
-                    constexpr int kBehind = (kStages - 2) * kGroup;
-                    if (relax > 0 && stores_behind) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBehind + kStores + 1) : "memory");
-                    else if (relax > 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBehind + 1) : "memory");
-                    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBehind) : "memory");
+                    if (relax > 0 && stores_behind) wait_behind(std::integral_constant<int, kStores + 1>{});
+                    else if (relax > 0) wait_behind(std::integral_constant<int, 1>{});
+                    else wait_behind(std::integral_constant<int, 0>{});
                     lds_barrier();
                     open_a();
                     bf16x8_t* bn = bops[P ^ 1];
